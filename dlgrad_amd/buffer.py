@@ -1,0 +1,422 @@
+"""Buffer: a pointer plus shape metadata, and the place where ops pick a runtime.
+
+Same role and method names as dlgrad/buffer.py:35-565, with one deliberate
+difference that is part of the device boundary: the reference hard-wires many
+ops to Device.CPU (creation ops, masked_fill, mean, permute, rsqrt, clamp,
+where, argmax, comparisons, cross-entropy and embedding helpers; buffer.py:48,
+:104-130, :204, :292-297, :322-328, :367-400, :454-528), which only works where
+host and device share memory.  Here *every* op goes to `self.device`, so a
+Buffer that lives in HBM never needs a host round trip.
+
+`ptr` is opaque to this file: the runtime that made it knows what it is (a
+`DevicePtr` for HIP).  Python floats that enter an expression become 0-d
+Buffers whose `ptr` is a `HostScalar`; runtimes receive those by value instead
+of uploading four bytes (the reference keeps them in a host `float[1]`,
+buffer.py:86-90).  Buffers are always contiguous: `stride` is derived from
+`shape`, and permutations materialise, exactly as in the reference.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+
+from dlgrad_amd.device import Device, as_device
+from dlgrad_amd.dispatch import dispatcher
+from dlgrad_amd.dtype import CDataPtr, DType, Scalar
+from dlgrad_amd.helpers import (
+    BinaryOps,
+    BufferOps,
+    CustomOps,
+    UnaryOps,
+    broadcast_shapes,
+    cal_sum_max_out_shape,
+    calculate_stride,
+    check_broadcast,
+    get_broadcast_shape,
+    prod_,
+)
+
+
+class HostScalar:
+    """One fp32 value that lives on the host and is passed to kernels by value."""
+    __slots__ = ("value",)
+
+    def __init__(self, value: float) -> None:
+        self.value = np.float32(value)
+
+    def __float__(self) -> float:
+        return float(self.value)
+
+    def __repr__(self) -> str:
+        return f"HostScalar({float(self.value)!r})"
+
+
+@dataclass
+class BufferMetadata:
+    shape: tuple
+    numel: int
+    stride: tuple
+    ndim: int
+    dtype: DType
+    device: Device
+    nbytes: int
+
+
+def _is_scalar(v) -> bool:
+    return isinstance(v, (int, float, np.floating)) and not isinstance(v, bool)
+
+
+# 0-d host values never reach a device: scalar-with-scalar arithmetic is done here in
+# fp32 (the reference runs its zero-loop C kernels on them, cpu_kernel.py:47-48).
+_f32 = np.float32
+_HOST_BINARY = {
+    BinaryOps.ADD: lambda a, b: a + b, BinaryOps.SUB: lambda a, b: a - b,
+    BinaryOps.MUL: lambda a, b: a * b, BinaryOps.DIV: lambda a, b: a / b,
+    BinaryOps.GT: lambda a, b: _f32(a > b), BinaryOps.GTE: lambda a, b: _f32(a >= b),
+    BinaryOps.EQT: lambda a, b: _f32(a == b),
+}
+_HOST_UNARY = {
+    UnaryOps.NEG: lambda v: -v,
+    UnaryOps.EXP: lambda v: _f32(np.exp(np.float64(v))),
+    UnaryOps.LOG: lambda v: _f32(np.log(np.float64(v))),
+    UnaryOps.SQRT: lambda v: np.sqrt(v),
+    UnaryOps.RSQRT: lambda v: _f32(1.0) / np.sqrt(v),
+    UnaryOps.POW: lambda v, val: _f32(np.float64(v) ** int(val)),
+    UnaryOps.CLAMP: lambda v, min_val, max_val: _f32(
+        min(max(v, v if min_val is None else _f32(min_val)), v if max_val is None else _f32(max_val))),
+}
+
+
+class Buffer:
+    def __init__(self, data: CDataPtr, shape: tuple, device: str | Device | None = Device.CPU,
+                 dtype: str | DType | None = None, **kwargs) -> None:
+        self.ptr = data
+        shape = tuple(shape)
+        dtype = DType.from_str(dtype) if isinstance(dtype, str) else (dtype or DType.FLOAT32)
+        n = prod_(shape)
+        self.metadata = BufferMetadata(
+            shape=shape, numel=n, stride=kwargs.get("stride", calculate_stride(shape)),
+            ndim=kwargs.get("ndim", len(shape)), dtype=dtype, device=as_device(device),
+            nbytes=n * DType.get_n_bytes(dtype))
+
+    # ---- plumbing -------------------------------------------------------------------
+    def _dispatch(self, op, **kw):
+        return dispatcher.dispatch(op=op, device=self.device, **kw)
+
+    def _like(self, ptr, shape: tuple | None = None, **kw) -> "Buffer":
+        return Buffer(data=ptr, shape=self.shape if shape is None else shape,
+                      device=self.device, dtype=self.dtype, **kw)
+
+    @property
+    def is_host_scalar(self) -> bool:
+        return isinstance(self.ptr, HostScalar)
+
+    def _set_shape(self, shape: tuple) -> None:
+        md = self.metadata
+        md.shape = tuple(shape)
+        md.numel = prod_(shape)
+        md.stride = calculate_stride(shape)
+        md.ndim = len(shape)
+
+    # ---- host boundary ----------------------------------------------------------------
+    @staticmethod
+    def from_numpy(arr: np.ndarray, device: Device) -> "Buffer":
+        """H2D upload (the reference aliases the numpy memory, tensor.py:112-115)."""
+        device = as_device(device)
+        return Buffer(data=dispatcher.dispatch(op=BufferOps.CREATE, device=device, data=arr),
+                      shape=arr.shape, device=device, dtype=DType.FLOAT32, ndim=arr.ndim)
+
+    def numpy(self) -> np.ndarray:
+        """D2H copy with this Buffer's shape (buffer.py:67-84 returns a host view)."""
+        if self.is_host_scalar:
+            return np.array(self.ptr.value, dtype=np.float32).reshape(self.shape)
+        return self._dispatch(CustomOps.TO_HOST, x=self)
+
+    def show(self) -> None:
+        self._dispatch(CustomOps.PRINT, x=self)
+
+    @staticmethod
+    def from_scalar(val: Scalar) -> "Buffer":
+        return Buffer(data=HostScalar(val), shape=(), device=Device.CPU, dtype=DType.FLOAT32)
+
+    # ---- creation -----------------------------------------------------------------------
+    @staticmethod
+    def uniform(shape: tuple, device: Device, dtype: DType | str, **kwargs) -> "Buffer":
+        dtype = DType.from_str(dtype) if isinstance(dtype, str) else dtype
+        device = as_device(device)
+        if dtype is not DType.FLOAT32:
+            raise NotImplementedError("dlgrad only supports float32")
+        if not isinstance(shape, tuple):
+            raise ValueError("Shape must be a tuple")
+        return Buffer(data=dispatcher.dispatch(op=BufferOps.UNIFORM, device=device, shape=shape, **kwargs),
+                      shape=shape, device=device, dtype=dtype)
+
+    @staticmethod
+    def full(shape: tuple, fill_value: Scalar, device: Device, dtype: DType = DType.FLOAT32) -> "Buffer":
+        device = as_device(device)
+        return Buffer(data=dispatcher.dispatch(op=BufferOps.FULL, device=device, shape=shape,
+                                               fill_value=fill_value),
+                      shape=shape, device=device, dtype=dtype)
+
+    @staticmethod
+    def arange(shape: tuple, device: Device, dtype: DType = DType.FLOAT32) -> "Buffer":
+        device = as_device(device)
+        return Buffer(data=dispatcher.dispatch(op=BufferOps.ARANGE, device=device, shape=shape),
+                      shape=shape, device=device, dtype=dtype)
+
+    # ---- views (metadata only) --------------------------------------------------------------
+    def reshape(self, new_shape: tuple) -> "Buffer":
+        new_shape = tuple(new_shape)
+        if -1 in new_shape:
+            known = -prod_(new_shape)
+            new_shape = tuple(self.numel // known if d == -1 else d for d in new_shape)
+        if prod_(new_shape) != self.numel:
+            raise ValueError(f"Cannot reshape {self.shape} ({self.numel} elements) to {new_shape} "
+                             f"({prod_(new_shape)} elements)")
+        return self._like(self.ptr, new_shape)
+
+    def unsqueeze(self, dim: list[int] | int) -> None:
+        """In place, like the reference (buffer.py:134-151); dim == -1 means 0."""
+        if dim == -1:
+            dim = 0
+        dims = [dim] if isinstance(dim, int) else list(dim)
+        if len(set(dims)) != len(dims):
+            raise AssertionError(f"duplicate dims not allowed in unsqueeze: {dim}")
+        shape = list(self.shape)
+        for d in dims:
+            assert d <= len(shape), f"Cannot unsqueeze {dim} from {self.shape}"
+        for d in sorted(dims, reverse=True):
+            shape.insert(d, 1)
+        self._set_shape(tuple(shape))
+
+    def squeeze(self, dim: list[int] | int) -> None:
+        """In place; dims that are not of extent 1 are left alone (buffer.py:153-165)."""
+        for d in ([dim] if isinstance(dim, int) else dim):
+            if self.shape[d] == 1:
+                shape = list(self.shape)
+                del shape[d]
+                self._set_shape(tuple(shape))
+
+    # ---- reductions -------------------------------------------------------------------------
+    def _reduce(self, op: UnaryOps, dim: int, keepdim: bool) -> "Buffer":
+        out_shape = cal_sum_max_out_shape(ndim=self.ndim, dim=dim, inp_shape=self.shape, keepdim=keepdim)
+        if dim == -1 and keepdim:
+            # helpers.py:205-206 reports the *input* shape here although one element is
+            # produced; a shape of ones is what that element can back.
+            out_shape = (1,) * self.ndim
+        ndim = self.ndim if keepdim else (0 if dim == -1 else self.ndim - 1)
+        return self._like(self._dispatch(op, x=self, dim=dim), out_shape, ndim=ndim)
+
+    def sum(self, dim: int = -1, keepdim: bool = False) -> "Buffer":
+        return self._reduce(UnaryOps.SUM, dim, keepdim)
+
+    def mean(self, dim: int = -1, keepdim: bool = False) -> "Buffer":
+        return self._reduce(UnaryOps.MEAN, dim, keepdim)
+
+    def max(self, dim: int = -1, out: "Buffer" = None, keepdim: bool = False) -> "Buffer":
+        return self._reduce(UnaryOps.MAX, dim, keepdim)
+
+    def argmax(self, dim: int) -> "Buffer":
+        assert self.ndim == 2, "currently dlgrad supports argmax for 2d only"
+        shape = {0: (1, self.shape[1]), 1: (self.shape[0], 1)}.get(dim, (1, 1))
+        return self._like(self._dispatch(UnaryOps.ARGMAX, x=self, dim=dim), shape)
+
+    # ---- matmul / layout ----------------------------------------------------------------------
+    def matmul(self, other: "Buffer") -> "Buffer":
+        p1, p2, out_shape = broadcast_shapes(self.shape, other.shape)
+        x = self if self.shape == p1 else self._like(self.ptr, p1)
+        y = other if other.shape == p2 else other._like(other.ptr, p2)
+        return self._like(self._dispatch(BinaryOps.MATMUL, x=x, y=y), out_shape)
+
+    def permute(self, order: tuple) -> "Buffer":
+        order = tuple(order)
+        return self._like(self._dispatch(UnaryOps.PERMUTE, x=self, order=order),
+                          tuple(self.shape[i] for i in order))
+
+    def transpose(self, dim0: int, dim1: int) -> "Buffer":
+        order = list(range(self.ndim))
+        order[dim0], order[dim1] = order[dim1], order[dim0]
+        return self.permute(tuple(order))
+
+    # ---- unary --------------------------------------------------------------------------------
+    def _unary(self, op: UnaryOps, **kw) -> "Buffer":
+        if self.is_host_scalar and op in _HOST_UNARY:
+            with np.errstate(all="ignore"):
+                return self._like(HostScalar(_HOST_UNARY[op](self.ptr.value, **kw)))
+        return self._like(self._dispatch(op, x=self, **kw))
+
+    def exp(self) -> "Buffer":
+        return self._unary(UnaryOps.EXP)
+
+    def log(self) -> "Buffer":
+        return self._unary(UnaryOps.LOG)
+
+    def sqrt(self) -> "Buffer":
+        return self._unary(UnaryOps.SQRT)
+
+    def rsqrt(self) -> "Buffer":
+        return self._unary(UnaryOps.RSQRT)
+
+    def clamp(self, min: int | None = None, max: int | None = None) -> "Buffer":
+        return self._unary(UnaryOps.CLAMP, min_val=min, max_val=max)
+
+    def __neg__(self) -> "Buffer":
+        return self._unary(UnaryOps.NEG)
+
+    def __pow__(self, val: Scalar) -> "Buffer":
+        return self._unary(UnaryOps.POW, val=val)
+
+    # compositions, same formulas as buffer.py:338-362
+    def relu(self) -> "Buffer":
+        return self.where(inp=self, other=0.0)
+
+    def leaky_relu(self, neg_slope: Scalar = 0.01) -> "Buffer":
+        return self.where(inp=self, other=self * neg_slope)
+
+    def sigmoid(self) -> "Buffer":
+        e = self.exp()
+        return e / (e + 1.0)
+
+    def tanh(self) -> "Buffer":
+        p, n = self.exp(), (-self).exp()
+        return (p - n) / (p + n)
+
+    def softmax(self, dim: int) -> "Buffer":
+        """Fused row softmax (one kernel instead of max, sub, exp, sum, div)."""
+        return self._unary(CustomOps.SOFTMAX, dim=dim)
+
+    def log_softmax(self, dim: int) -> "Buffer":
+        return self._unary(CustomOps.LOG_SOFTMAX, dim=dim)
+
+    # ---- selects ----------------------------------------------------------------------------------
+    def where(self, inp: "Buffer | Scalar", other: "Buffer | Scalar") -> "Buffer":
+        inp = Buffer.from_scalar(inp) if _is_scalar(inp) else inp
+        other = Buffer.from_scalar(other) if _is_scalar(other) else other
+        return self._like(self._dispatch(UnaryOps.WHERE, cond=self, x=inp, y=other))
+
+    @staticmethod
+    def masked_fill(x: "Buffer", mask: "Buffer", val: Scalar) -> "Buffer":
+        out_shape = get_broadcast_shape(x.shape, mask.shape)
+        return x._like(x._dispatch(UnaryOps.MASKED_FILL, x=x, mask=mask, val=val, out_shape=out_shape),
+                       out_shape)
+
+    # ---- cross-entropy and embedding helpers ---------------------------------------------------------
+    @staticmethod
+    def ce_forward(x: "Buffer", y: "Buffer") -> "Buffer":
+        return x._like(x._dispatch(CustomOps.CE_FORWARD, x=x, y=y), (1, x.shape[0]))
+
+    @staticmethod
+    def ce_backward(**kwargs) -> None:
+        """Same calling convention as buffer.py:397-400 (op and device arrive as kwargs);
+        the target device is the one of `x`."""
+        kwargs.pop("device", None)
+        op = kwargs.pop("op")
+        kwargs["x"]._dispatch(op, **kwargs)
+
+    def embedding(self, idx: "Buffer", backward: bool = False, upstream_grad: "Buffer" = None) -> "Buffer":
+        if backward:
+            return self._like(self._dispatch(CustomOps.EMBEDDING, x=self, idx=idx, out_numel=self.numel,
+                                             backward=True, upstream_grad=upstream_grad))
+        out_shape = idx.shape + (self.shape[-1],)
+        return self._like(self._dispatch(CustomOps.EMBEDDING, x=self, idx=idx, out_numel=prod_(out_shape)),
+                          out_shape)
+
+    # ---- binary -----------------------------------------------------------------------------------------
+    def _binary_op(self, other: "Buffer", op: BinaryOps) -> "Buffer":
+        """x is the operand with more elements and fixes the output shape (buffer.py:402-448).
+        A smaller left operand of SUB is handled as -(other - self), as there."""
+        check_broadcast(self.shape, other.shape)
+        if self.is_host_scalar and other.is_host_scalar:
+            with np.errstate(all="ignore"):
+                return self._like(HostScalar(_HOST_BINARY[op](self.ptr.value, other.ptr.value)))
+        big, small = (self, other) if self.numel >= other.numel else (other, self)
+        dev = small.device if big.is_host_scalar else big.device
+        ptr = dispatcher.dispatch(op=op, device=dev, x=big, y=small)
+        out = Buffer(data=ptr, shape=big.shape, device=dev, dtype=self.dtype)
+        if op == BinaryOps.SUB and big is not self:
+            out = -out
+        return out
+
+    @staticmethod
+    def _coerce(v) -> "Buffer":
+        return Buffer.from_scalar(v) if _is_scalar(v) else v
+
+    def __add__(self, other) -> "Buffer":
+        return self._binary_op(Buffer._coerce(other), BinaryOps.ADD)
+
+    def __sub__(self, other) -> "Buffer":
+        return self._binary_op(Buffer._coerce(other), BinaryOps.SUB)
+
+    def __mul__(self, other) -> "Buffer":
+        return self._binary_op(Buffer._coerce(other), BinaryOps.MUL)
+
+    def __truediv__(self, other) -> "Buffer":
+        other = Buffer._coerce(other)
+        if self.numel >= other.numel:
+            return self._binary_op(other, BinaryOps.DIV)
+        return self._binary_op(other ** -1, BinaryOps.MUL)       # small / big = big**-1 * small
+
+    def __rsub__(self, other: Scalar) -> "Buffer":
+        return -(self._binary_op(Buffer._coerce(other), BinaryOps.SUB))
+
+    __radd__ = __add__
+    __rmul__ = __mul__
+
+    def __le__(self, other: "Buffer") -> "Buffer":
+        out_shape = get_broadcast_shape(self.shape, other.shape)
+        return self._like(self._dispatch(BinaryOps.CMP, x=self, y=other, out_shape=out_shape, mode="<="),
+                          out_shape)
+
+    def _compare(self, op: BinaryOps, other) -> "Buffer":
+        other = Buffer._coerce(other)
+        if self.is_host_scalar and other.is_host_scalar:
+            return self._like(HostScalar(_HOST_BINARY[op](self.ptr.value, other.ptr.value)))
+        return self._like(self._dispatch(op, x=self, y=other))
+
+    def __gt__(self, other) -> "Buffer":
+        return self._compare(BinaryOps.GT, other)
+
+    def __ge__(self, other) -> "Buffer":
+        return self._compare(BinaryOps.GTE, other)
+
+    def __eq__(self, other) -> "Buffer":  # type: ignore[override]
+        return self._compare(BinaryOps.EQT, other)
+
+    __hash__ = object.__hash__
+
+    def __matmul__(self, other: "Buffer") -> "Buffer":
+        return self.matmul(other)
+
+    # ---- metadata -----------------------------------------------------------------------------------------
+    @property
+    def T(self) -> "Buffer":  # noqa: N802
+        return self.transpose(0, 1)
+
+    @property
+    def numel(self) -> int:
+        return self.metadata.numel
+
+    @property
+    def shape(self) -> tuple:
+        return self.metadata.shape
+
+    @property
+    def stride(self) -> tuple:
+        return self.metadata.stride
+
+    @property
+    def ndim(self) -> int:
+        return self.metadata.ndim
+
+    @property
+    def dtype(self) -> DType:
+        return self.metadata.dtype
+
+    @property
+    def device(self) -> Device:
+        return self.metadata.device
+
+    @property
+    def nbytes(self) -> int:
+        return self.metadata.nbytes

@@ -1,0 +1,414 @@
+// libdlgrad_hip.so -- device layer under dlgrad's `device="hip"` runtime.
+//
+// Host-only C++ (no device code lives here: kernels arrive as HIP source strings
+// from dlgrad_amd/codegen/hip_kernel.py and are compiled by hiprtc for gfx950).
+// Implements include/dlgrad_hip.h: a size-bucketed caching allocator over
+// hipMalloc, synchronous transfers, hiprtc compile, code-object load, kernel
+// launch from a packed argument block, events and error strings.
+//
+// One device, one default-priority stream, one process.  The allocator hands a
+// freed block to the next request of the same bucket without waiting for the
+// GPU: that is safe because every consumer of the block was enqueued on the
+// same stream before the free and every producer is enqueued after it.
+
+#include "../../include/dlgrad_hip.h"
+
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+namespace {
+
+thread_local std::string g_err;
+thread_local std::string g_log;
+
+std::mutex g_mu;
+bool g_inited = false;
+int g_device = -1;
+hipStream_t g_stream = nullptr;
+
+struct Kernel {
+    hipModule_t module;
+    hipFunction_t fn;
+};
+std::vector<Kernel> g_kernels;                   // handle = index + 1
+std::vector<hipModule_t> g_modules;
+
+// ---- allocator state --------------------------------------------------------
+std::map<size_t, std::vector<void *>> g_free;    // bucket size -> cached blocks
+std::unordered_map<void *, size_t> g_live;       // block -> bucket size
+uint64_t g_bytes_in_use = 0, g_bytes_cached = 0, g_device_allocs = 0;
+
+int fail(const char *what, hipError_t e) {
+    char buf[512];
+    std::snprintf(buf, sizeof buf, "%s: %s (%d)", what, hipGetErrorString(e), (int)e);
+    g_err = buf;
+    return -(int)e - 1000;
+}
+int fail_msg(int code, const std::string &msg) {
+    g_err = msg;
+    return code;
+}
+#define HIP_TRY(expr)                                   \
+    do {                                                \
+        hipError_t e__ = (expr);                        \
+        if (e__ != hipSuccess) return fail(#expr, e__); \
+    } while (0)
+
+#define NEED_INIT()                                                          \
+    do {                                                                     \
+        if (!g_inited) return fail_msg(-2, "dlg_hip_init has not succeeded"); \
+    } while (0)
+
+size_t bucket_of(size_t n) {
+    if (n < 256) n = 256;
+    if (n <= (size_t(1) << 20)) {             // up to 1 MiB: next power of two
+        size_t b = 256;
+        while (b < n) b <<= 1;
+        return b;
+    }
+    const size_t mib = size_t(1) << 20;       // above: whole MiB
+    return (n + mib - 1) / mib * mib;
+}
+
+void trim_locked() {
+    for (auto &kv : g_free)
+        for (void *p : kv.second) (void)hipFree(p);
+    g_free.clear();
+    g_bytes_cached = 0;
+}
+
+int alloc_locked(size_t nbytes, void **out) {
+    size_t b = bucket_of(nbytes);
+    auto it = g_free.find(b);
+    if (it != g_free.end() && !it->second.empty()) {
+        *out = it->second.back();
+        it->second.pop_back();
+        g_bytes_cached -= b;
+    } else {
+        void *p = nullptr;
+        hipError_t e = hipMalloc(&p, b);
+        if (e != hipSuccess) {                // give cached blocks back and retry once
+            (void)hipGetLastError();
+            (void)hipStreamSynchronize(g_stream);
+            trim_locked();
+            e = hipMalloc(&p, b);
+        }
+        if (e != hipSuccess || p == nullptr) {
+            (void)hipGetLastError();
+            *out = nullptr;
+            char buf[160];
+            std::snprintf(buf, sizeof buf, "Failed to allocate %zu bytes of device memory", nbytes);
+            return fail_msg(-3, buf);
+        }
+        ++g_device_allocs;
+        *out = p;
+    }
+    g_live[*out] = b;
+    g_bytes_in_use += b;
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *dlg_hip_last_error(void) { return g_err.c_str(); }
+const char *dlg_hip_compile_log(void) { return g_log.c_str(); }
+
+int dlg_hip_device_count(int *count) {
+    if (!count) return fail_msg(-1, "count is NULL");
+    *count = 0;
+    hipError_t e = hipGetDeviceCount(count);
+    if (e != hipSuccess) {
+        *count = 0;
+        return fail("hipGetDeviceCount", e);
+    }
+    return 0;
+}
+
+int dlg_hip_init(int device) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_inited) {
+        if (device == g_device) return 0;
+        return fail_msg(-4, "already initialised on another device");
+    }
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return fail_msg(-5, "no HIP device available");
+    }
+    if (device < 0 || device >= n) return fail_msg(-6, "device index out of range");
+    HIP_TRY(hipSetDevice(device));
+    HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+    g_device = device;
+    g_inited = true;
+    return 0;
+}
+
+int dlg_hip_shutdown(void) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_inited) return 0;
+    (void)hipStreamSynchronize(g_stream);
+    trim_locked();
+    for (hipModule_t m : g_modules) (void)hipModuleUnload(m);
+    g_modules.clear();
+    g_kernels.clear();
+    (void)hipStreamDestroy(g_stream);
+    g_stream = nullptr;
+    g_inited = false;
+    g_device = -1;
+    return 0;
+}
+
+int dlg_hip_props(dlg_hip_props_t *out) {
+    NEED_INIT();
+    if (!out) return fail_msg(-1, "out is NULL");
+    hipDeviceProp_t p;
+    HIP_TRY(hipGetDeviceProperties(&p, g_device));
+    std::memset(out, 0, sizeof *out);
+    std::snprintf(out->name, sizeof out->name, "%s", p.name);
+    std::snprintf(out->arch, sizeof out->arch, "%s", p.gcnArchName);
+    out->compute_units = p.multiProcessorCount;
+    out->wavefront_size = p.warpSize;
+    out->clock_khz = p.clockRate;
+    out->mem_clock_khz = p.memoryClockRate;
+    out->mem_bus_bits = p.memoryBusWidth;
+    out->lds_bytes = (int32_t)p.sharedMemPerBlock;
+    out->l2_bytes = p.l2CacheSize;
+    out->total_mem = p.totalGlobalMem;
+    return 0;
+}
+
+// ---- memory -------------------------------------------------------------------
+
+int dlg_hip_alloc(size_t nbytes, void **out) {
+    NEED_INIT();
+    if (!out) return fail_msg(-1, "out is NULL");
+    std::lock_guard<std::mutex> lk(g_mu);
+    return alloc_locked(nbytes, out);
+}
+
+int dlg_hip_alloc_zero(size_t nbytes, void **out) {
+    NEED_INIT();
+    if (!out) return fail_msg(-1, "out is NULL");
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        int rc = alloc_locked(nbytes, out);
+        if (rc) return rc;
+    }
+    if (nbytes) HIP_TRY(hipMemsetAsync(*out, 0, nbytes, g_stream));
+    return 0;
+}
+
+int dlg_hip_fill_f32(void *dst, float value, size_t count) {
+    NEED_INIT();
+    if (!count) return 0;
+    uint32_t bits;
+    std::memcpy(&bits, &value, 4);
+    HIP_TRY(hipMemsetD32Async((hipDeviceptr_t)dst, (int)bits, count, g_stream));
+    return 0;
+}
+
+int dlg_hip_free(void *ptr) {
+    if (!ptr) return 0;
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_inited) return 0;                  // after shutdown the driver owns nothing
+    auto it = g_live.find(ptr);
+    if (it == g_live.end()) return fail_msg(-7, "dlg_hip_free: pointer was not allocated here");
+    size_t b = it->second;
+    g_live.erase(it);
+    g_bytes_in_use -= b;
+    g_free[b].push_back(ptr);
+    g_bytes_cached += b;
+    return 0;
+}
+
+int dlg_hip_pool_stats(uint64_t *in_use, uint64_t *cached, uint64_t *n_allocs) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (in_use) *in_use = g_bytes_in_use;
+    if (cached) *cached = g_bytes_cached;
+    if (n_allocs) *n_allocs = g_device_allocs;
+    return 0;
+}
+
+int dlg_hip_pool_trim(void) {
+    NEED_INIT();
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    std::lock_guard<std::mutex> lk(g_mu);
+    trim_locked();
+    return 0;
+}
+
+// ---- transfers ------------------------------------------------------------------
+
+int dlg_hip_h2d(void *dst, const void *src, size_t n) {
+    NEED_INIT();
+    if (!n) return 0;
+    HIP_TRY(hipMemcpyAsync(dst, src, n, hipMemcpyHostToDevice, g_stream));
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    return 0;
+}
+
+int dlg_hip_d2h(void *dst, const void *src, size_t n) {
+    NEED_INIT();
+    if (!n) return 0;
+    HIP_TRY(hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToHost, g_stream));
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    return 0;
+}
+
+int dlg_hip_d2d(void *dst, const void *src, size_t n) {
+    NEED_INIT();
+    if (!n) return 0;
+    HIP_TRY(hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToDevice, g_stream));
+    return 0;
+}
+
+// ---- kernels ----------------------------------------------------------------------
+
+int dlg_hip_compile(const char *source, const char *name, const char *const *options,
+                    int n_options, void **code, size_t *code_size) {
+    if (!source || !code || !code_size) return fail_msg(-1, "NULL argument");
+    *code = nullptr;
+    *code_size = 0;
+    g_log.clear();
+    hiprtcProgram prog;
+    hiprtcResult r = hiprtcCreateProgram(&prog, source, name ? name : "kernel.hip", 0, nullptr, nullptr);
+    if (r != HIPRTC_SUCCESS)
+        return fail_msg(-10, std::string("hiprtcCreateProgram: ") + hiprtcGetErrorString(r));
+    r = hiprtcCompileProgram(prog, n_options, const_cast<const char **>(options));
+    size_t log_size = 0;
+    if (hiprtcGetProgramLogSize(prog, &log_size) == HIPRTC_SUCCESS && log_size > 1) {
+        g_log.resize(log_size);
+        (void)hiprtcGetProgramLog(prog, &g_log[0]);
+    }
+    if (r != HIPRTC_SUCCESS) {
+        (void)hiprtcDestroyProgram(&prog);
+        return fail_msg(-11, std::string("Compilation failed: ") + hiprtcGetErrorString(r));
+    }
+    size_t sz = 0;
+    r = hiprtcGetCodeSize(prog, &sz);
+    if (r != HIPRTC_SUCCESS || sz == 0) {
+        (void)hiprtcDestroyProgram(&prog);
+        return fail_msg(-12, "hiprtcGetCodeSize failed");
+    }
+    void *buf = std::malloc(sz);
+    if (!buf) {
+        (void)hiprtcDestroyProgram(&prog);
+        return fail_msg(-13, "out of host memory for code object");
+    }
+    r = hiprtcGetCode(prog, (char *)buf);
+    (void)hiprtcDestroyProgram(&prog);
+    if (r != HIPRTC_SUCCESS) {
+        std::free(buf);
+        return fail_msg(-14, "hiprtcGetCode failed");
+    }
+    *code = buf;
+    *code_size = sz;
+    return 0;
+}
+
+int dlg_hip_code_free(void *code) {
+    std::free(code);
+    return 0;
+}
+
+int dlg_hip_module_load(const void *code, size_t code_size, const char *kernel_name,
+                        uint64_t *handle) {
+    NEED_INIT();
+    if (!code || !code_size || !kernel_name || !handle) return fail_msg(-1, "NULL argument");
+    hipModule_t mod;
+    HIP_TRY(hipModuleLoadData(&mod, code));
+    hipFunction_t fn;
+    hipError_t e = hipModuleGetFunction(&fn, mod, kernel_name);
+    if (e != hipSuccess) {
+        (void)hipModuleUnload(mod);
+        return fail(kernel_name, e);
+    }
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_modules.push_back(mod);
+    g_kernels.push_back({mod, fn});
+    *handle = (uint64_t)g_kernels.size();
+    return 0;
+}
+
+int dlg_hip_launch(uint64_t handle, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx,
+                   uint32_t by, uint32_t bz, uint32_t shared_bytes, const void *args,
+                   size_t args_size) {
+    NEED_INIT();
+    if (handle == 0 || handle > g_kernels.size()) return fail_msg(-20, "bad kernel handle");
+    if (!gx || !gy || !gz || !bx || !by || !bz) return fail_msg(-21, "empty grid or block");
+    if ((uint64_t)bx * by * bz > 1024) return fail_msg(-22, "block larger than 1024 threads");
+    void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void *>(args),
+                      HIP_LAUNCH_PARAM_BUFFER_SIZE, &args_size, HIP_LAUNCH_PARAM_END};
+    HIP_TRY(hipModuleLaunchKernel(g_kernels[handle - 1].fn, gx, gy, gz, bx, by, bz, shared_bytes,
+                                  g_stream, nullptr, config));
+    return 0;
+}
+
+int dlg_hip_kernel_attrs(uint64_t handle, int32_t *num_regs, int32_t *lds_bytes,
+                         int32_t *scratch_bytes, int32_t *max_threads) {
+    NEED_INIT();
+    if (handle == 0 || handle > g_kernels.size()) return fail_msg(-20, "bad kernel handle");
+    hipFunction_t fn = g_kernels[handle - 1].fn;
+    int v = 0;
+    if (num_regs) { HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_NUM_REGS, fn)); *num_regs = v; }
+    if (lds_bytes) { HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES, fn)); *lds_bytes = v; }
+    if (scratch_bytes) { HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, fn)); *scratch_bytes = v; }
+    if (max_threads) { HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_MAX_THREADS_PER_BLOCK, fn)); *max_threads = v; }
+    return 0;
+}
+
+// ---- ordering and timing ------------------------------------------------------------
+
+int dlg_hip_sync(void) {
+    NEED_INIT();
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    return 0;
+}
+
+int dlg_hip_event_create(uint64_t *event) {
+    NEED_INIT();
+    if (!event) return fail_msg(-1, "event is NULL");
+    hipEvent_t ev;
+    HIP_TRY(hipEventCreate(&ev));
+    *event = (uint64_t)(uintptr_t)ev;
+    return 0;
+}
+
+int dlg_hip_event_record(uint64_t event) {
+    NEED_INIT();
+    HIP_TRY(hipEventRecord((hipEvent_t)(uintptr_t)event, g_stream));
+    return 0;
+}
+
+int dlg_hip_event_sync(uint64_t event) {
+    NEED_INIT();
+    HIP_TRY(hipEventSynchronize((hipEvent_t)(uintptr_t)event));
+    return 0;
+}
+
+int dlg_hip_event_elapsed_ms(uint64_t start, uint64_t stop, float *ms) {
+    NEED_INIT();
+    if (!ms) return fail_msg(-1, "ms is NULL");
+    HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)(uintptr_t)start, (hipEvent_t)(uintptr_t)stop));
+    return 0;
+}
+
+int dlg_hip_event_destroy(uint64_t event) {
+    NEED_INIT();
+    HIP_TRY(hipEventDestroy((hipEvent_t)(uintptr_t)event));
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,185 @@
+"""Op enums and the shape/stride rules kernels are launched with.
+
+The enum members and the function names are the ones the reference's Buffer and
+runtimes use (dlgrad/helpers.py:18-58, :114-212, :276-334) so a runtime written
+against one works against the other.  The bodies are this package's own.
+Two extra enum members exist only here: `BufferOps.CREATE` is given a meaning
+(host array -> device buffer) and `CustomOps.TO_HOST` is new (device buffer ->
+host array); the reference needs neither because its pointers are host memory.
+"""
+from __future__ import annotations
+
+import itertools
+import os
+from collections.abc import Iterable
+from enum import Enum, auto
+from math import prod
+
+
+class UnaryOps(Enum):
+    SUM = auto()
+    MAX = auto()
+    NEG = auto()
+    EXP = auto()
+    LOG = auto()
+    POW = auto()
+    SQRT = auto()
+    RSQRT = auto()
+    TRANSPOSE = auto()
+    RELU = auto()
+    ARGMAX = auto()
+    WHERE = auto()
+    MEAN = auto()
+    CLAMP = auto()
+    MASKED_FILL = auto()
+    PERMUTE = auto()
+
+
+class BufferOps(Enum):
+    CREATE = auto()
+    UNIFORM = auto()
+    ARANGE = auto()
+    FULL = auto()
+
+
+class BinaryOps(Enum):
+    ADD = auto()
+    SUB = auto()
+    MUL = auto()
+    DIV = auto()
+    MATMUL = auto()
+    GT = auto()
+    GTE = auto()
+    EQT = auto()
+    CMP = auto()
+
+
+class CustomOps(Enum):
+    INDEX = auto()
+    CE_FORWARD = auto()
+    CE_BACKWARD = auto()
+    PRINT = auto()
+    EMBEDDING = auto()
+    TO_HOST = auto()
+    # fused row kernels (no counterpart in the reference, which composes them
+    # from max/sub/exp/sum/div: tensor.py:634-669, ops.py:337-370)
+    SOFTMAX = auto()
+    LOG_SOFTMAX = auto()
+
+
+def prod_(x: Iterable) -> int:
+    return prod(x) if x else 1
+
+
+def calculate_stride(shape: tuple | list) -> tuple:
+    """Row-major element strides; () for a 0-d shape (helpers.py:176-187)."""
+    out, acc = [], 1
+    for d in reversed(tuple(shape)):
+        out.append(acc)
+        acc *= d
+    return tuple(reversed(out))
+
+
+def check_broadcast(x_shape: tuple, y_shape: tuple) -> bool:
+    """True, or AssertionError when a trailing-aligned pair of dims is neither
+    equal nor 1 (helpers.py:64-82)."""
+    for a, b in itertools.zip_longest(reversed(x_shape), reversed(y_shape), fillvalue=1):
+        if a != b and a != 1 and b != 1:
+            raise AssertionError(
+                f"Cannot broadcast {y_shape} to {x_shape}, the dimensions {a} and {b} dont match")
+    return True
+
+
+def broadcast_shapes_2(s1: tuple, s2: tuple) -> tuple:
+    """numpy-style broadcast of two shapes (helpers.py:311-334)."""
+    n = max(len(s1), len(s2))
+    a = (1,) * (n - len(s1)) + tuple(s1)
+    b = (1,) * (n - len(s2)) + tuple(s2)
+    out = []
+    for d1, d2 in zip(a, b):
+        if d1 != d2 and d1 != 1 and d2 != 1:
+            raise ValueError(f"Operands could not be broadcast together with shapes {s1} {s2}")
+        out.append(d2 if d1 == 1 else d1)
+    return tuple(out)
+
+
+get_broadcast_shape = broadcast_shapes_2   # helpers.py:135-155 computes the same thing
+
+
+def get_broadcast_strides_2(out_shape: tuple, in_shape: tuple, in_stride: tuple) -> tuple:
+    """Strides of `in` viewed at `out_shape`: 0 wherever a size-1 (or missing
+    leading) dim is stretched (helpers.py:276-309)."""
+    pad = len(out_shape) - len(in_shape)
+    shape = (1,) * pad + tuple(in_shape)
+    stride = (0,) * pad + tuple(in_stride)
+    res = []
+    for o, i, s in zip(out_shape, shape, stride):
+        if i == o:
+            res.append(s)
+        elif i == 1:
+            res.append(0)
+        else:
+            raise ValueError(f"Shape mismatch: cannot broadcast {in_shape} to {out_shape}")
+    return tuple(res)
+
+
+def broadcast_shapes(s1: tuple, s2: tuple) -> tuple[tuple, tuple, tuple]:
+    """Matmul operand alignment: left-pad both to equal rank, broadcast the batch
+    dims, check the inner dims; returns (padded1, padded2, out) (helpers.py:114-133)."""
+    n = max(len(s1), len(s2))
+    p1 = (1,) * (n - len(s1)) + tuple(s1)
+    p2 = (1,) * (n - len(s2)) + tuple(s2)
+    batch = []
+    for d1, d2 in zip(p1[:-2], p2[:-2]):
+        if d1 != d2 and 1 not in (d1, d2):
+            raise ValueError(f"Cannot broadcast batch dims: {s1} and {s2}")
+        batch.append(max(d1, d2))
+    if p1[-1] != p2[-2]:
+        raise ValueError(f"Matrix inner dims must match: {s1} and {s2}")
+    return p1, p2, tuple(batch) + (p1[-2], p2[-1])
+
+
+def cal_sum_max_out_shape(ndim: int, dim: int, inp_shape: tuple, keepdim: bool = False) -> tuple:
+    """Output shape of sum/max/mean; dim == -1 means "all elements" (helpers.py:204-212)."""
+    if dim == -1:
+        return tuple(inp_shape) if keepdim else ()
+    t = list(inp_shape)
+    if keepdim:
+        t[dim] = 1
+    else:
+        del t[dim]
+    return tuple(t)
+
+
+def collapse_dims(shape: tuple, *strides: tuple) -> tuple[tuple, list[tuple]]:
+    """Merge adjacent dims that every operand walks contiguously.
+
+    `shape` is the iteration space, each `strides[k]` one operand's element strides
+    over it (0 = broadcast).  Dims of extent 1 vanish; dims d, d+1 merge when
+    stride[d] == stride[d+1] * shape[d+1] for every operand.  Returns the reduced
+    shape and strides (at least one dim).  This is what lets a 4-D broadcast such
+    as (16,4,128,128) * (16,4,128,1) run as a 2-D rows-by-columns kernel.
+    """
+    dims = [(n, tuple(s[i] for s in strides)) for i, n in enumerate(shape) if n != 1]
+    if not dims:
+        return (1,), [(0,) for _ in strides]
+    merged = [dims[0]]
+    for n, st in dims[1:]:
+        pn, pst = merged[-1]
+        if all(ps == s * n for ps, s in zip(pst, st)):
+            merged[-1] = (pn * n, st)
+        else:
+            merged.append((n, st))
+    out_shape = tuple(n for n, _ in merged)
+    out_strides = [tuple(st[k] for _, st in merged) for k in range(len(strides))]
+    return out_shape, out_strides
+
+
+CACHE_DIR = os.environ.get(
+    "DLGRAD_HIP_CACHE_DIR",
+    os.path.join(os.path.dirname(os.path.abspath(__file__)), "_kcache"))
+
+# Reference quirks that live inside a kernel's contract (int-truncated `full` and
+# `pow` arguments, dlgrad/runtime/cpu.py:252 and :500) are reproduced when this is
+# on, which is the default because parity is judged against that behaviour.
+STRICT_REFERENCE = os.environ.get("DLGRAD_STRICT_REFERENCE", "1") != "0"

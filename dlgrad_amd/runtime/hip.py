@@ -1,0 +1,438 @@
+"""The `hip` runtime: one static method per (op, Device.HIP) pair of the dispatch table.
+
+Plays the part dlgrad/runtime/cpu.py:43-1061 plays for the CPU: allocate the
+output, pick the kernel for the ranks/shapes at hand, pack its arguments, call
+it, return the bare pointer.  The differences are the MI355X ones:
+
+* kernels are HIP sources from `dlgrad_amd.codegen.hip_kernel`, compiled for
+  gfx950 by hiprtc through libdlgrad_hip.so and cached as code objects on disk
+  (the reference caches .so files per source hash, cpu.py:64-78, and stats the
+  file on every call, cpu.py:268; here the handle lookup is an in-process dict);
+* outputs come from a pooled device allocator and are returned to it by the
+  `DevicePtr` finaliser (the reference uses ffi.gc(ptr, free_ptr), cpu.py:102);
+* launches are asynchronous on one stream; only `TO_HOST` waits;
+* Python floats arrive by value, never through memory.
+
+Nothing here falls back to another device: a missing library or GPU raises.
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+import struct
+
+import numpy as np
+
+from dlgrad_amd import ffi as _ffi
+from dlgrad_amd.buffer import Buffer, HostScalar
+from dlgrad_amd.codegen import hip_kernel as K
+from dlgrad_amd.device import Device
+from dlgrad_amd.dispatch import dispatcher
+from dlgrad_amd.helpers import (
+    CACHE_DIR,
+    STRICT_REFERENCE,
+    BinaryOps,
+    BufferOps,
+    CustomOps,
+    UnaryOps,
+    broadcast_shapes_2,
+    calculate_stride,
+    collapse_dims,
+    get_broadcast_strides_2,
+    prod_,
+)
+
+_state = {"lib": None, "ready": False, "props": None}
+_handles: dict = {}            # (generator, params) -> (kernel handle, struct.Struct)
+launch_count = 0               # launches issued since import (read by the benchmarks)
+
+# Ahead-of-time mode for the build step: no device is touched, every kernel a workload
+# asks for is compiled into the on-disk cache and listed, launches are skipped and
+# results are meaningless.  It exists so a machine without a GPU can compile exactly the
+# code objects a later GPU run will load; it is never a way to compute anything.
+COMPILE_ONLY = os.environ.get("DLGRAD_HIP_COMPILE_ONLY") == "1"
+requested_kernels: set = set()  # (generator name, params) seen by kernel()
+compiled_now: list = []         # kernels that missed the on-disk cache in this process
+
+
+class _CompileOnlyLib:
+    """Stands where HipLib stands when COMPILE_ONLY is set: compiles, never runs."""
+
+    def __init__(self, real: _ffi.HipLib) -> None:
+        import sys
+        print("dlgrad_amd: DLGRAD_HIP_COMPILE_ONLY=1 -- kernels are compiled, nothing is executed",
+              file=sys.stderr)
+        self._real, self._next = real, 0x7F0000000000
+
+    def compile(self, *a):
+        return self._real.compile(*a)
+
+    def alloc(self, nbytes: int, zero: bool = False) -> int:
+        a = self._next
+        self._next += (nbytes + 255) // 256 * 256
+        return a
+
+    def d2h(self, host_addr: int, src: int, nbytes: int) -> None:
+        import ctypes
+        ctypes.memset(host_addr, 0, nbytes)
+
+    def module_load(self, code: bytes, name: str) -> int:
+        return 1
+
+    def props(self) -> dict:
+        return {"name": "compile-only", "arch": K.ARCH, "compute_units": 256, "wavefront_size": 64,
+                "clock_khz": 2400000, "mem_clock_khz": 0, "mem_bus_bits": 8192, "lds_bytes": 163840,
+                "l2_bytes": 4 << 20, "total_mem": 288 << 30}
+
+    def event_create(self) -> int:
+        return 1
+
+    def event_elapsed_ms(self, a: int, b: int) -> float:
+        return 1.0
+
+    def pool_stats(self) -> tuple:
+        return (0, 0, 0)
+
+    def __getattr__(self, name: str):           # free, h2d, launch, sync, fill_f32, events ...
+        return lambda *a, **k: None
+
+
+def lib() -> _ffi.HipLib:
+    """The loaded library with the device initialised; raises when there is no GPU."""
+    if not _state["ready"]:
+        l = _ffi.get_lib()
+        if COMPILE_ONLY:
+            l = _CompileOnlyLib(l)
+        else:
+            l.init(int(os.environ.get("DLGRAD_HIP_DEVICE", "0")))
+        _state["lib"], _state["ready"] = l, True
+    return _state["lib"]
+
+
+def available() -> bool:
+    try:
+        return _ffi.get_lib().device_count() > 0
+    except Exception:
+        return False
+
+
+def props() -> dict:
+    if _state["props"] is None:
+        _state["props"] = lib().props()
+    return _state["props"]
+
+
+class DevicePtr:
+    """An address in HBM.  Owning pointers give their block back to the pool when
+    collected; views (`ptr + n_elements`, as tensor.py:816-821 slices) keep their
+    base alive instead."""
+    __slots__ = ("addr", "nbytes", "base", "__weakref__")
+
+    def __init__(self, addr: int, nbytes: int, base: "DevicePtr | None" = None) -> None:
+        self.addr, self.nbytes, self.base = addr, nbytes, base
+
+    def __add__(self, n_elements: int) -> "DevicePtr":
+        off = 4 * int(n_elements)
+        if off < 0 or off > self.nbytes:
+            raise IndexError(f"offset {n_elements} elements outside a {self.nbytes}-byte block")
+        return DevicePtr(self.addr + off, self.nbytes - off, self.base or self)
+
+    def __del__(self) -> None:
+        if self.base is None and self.addr:
+            l = _state["lib"]
+            if l is not None:
+                try:
+                    l.free(self.addr)
+                except Exception:      # interpreter shutdown
+                    pass
+
+    def __repr__(self) -> str:
+        return f"DevicePtr(0x{self.addr:x}, {self.nbytes} B{', view' if self.base else ''})"
+
+
+def alloc(numel: int, zero: bool = False) -> DevicePtr:
+    nbytes = 4 * max(int(numel), 1)
+    return DevicePtr(lib().alloc(nbytes, zero), nbytes)
+
+
+# ---- kernel cache -----------------------------------------------------------------------
+
+def code_object(src: str, name: str, l: _ffi.HipLib | None = None) -> bytes:
+    """Code object for `src`: from the on-disk cache, else hiprtc.  Needs no GPU."""
+    opts = list(K.COMPILE_OPTIONS)
+    key = hashlib.sha256((src + "\0" + " ".join(opts)).encode()).hexdigest()[:20]
+    path = os.path.join(CACHE_DIR, f"{name}_{key}.hsaco")
+    try:
+        with open(path, "rb") as f:
+            return f.read()
+    except FileNotFoundError:
+        pass
+    code = (l or _ffi.get_lib()).compile(src, name + ".hip", opts)
+    compiled_now.append(name)
+    os.makedirs(CACHE_DIR, exist_ok=True)
+    tmp = f"{path}.{os.getpid()}.tmp"
+    with open(tmp, "wb") as f:
+        f.write(code)
+    os.replace(tmp, path)
+    return code
+
+
+def kernel(gen, *params):
+    key = (gen, params)
+    h = _handles.get(key)
+    if h is None:
+        src, name, fmt = gen(*params)
+        requested_kernels.add((gen.__name__, params))
+        l = lib()
+        h = _handles[key] = (l.module_load(code_object(src, name, l), name), struct.Struct(fmt))
+    return h
+
+
+def launch(k, grid, block, *args) -> None:
+    global launch_count
+    launch_count += 1
+    handle, st = k
+    g = grid if isinstance(grid, tuple) else (grid, 1, 1)
+    b = block if isinstance(block, tuple) else (block, 1, 1)
+    _state["lib"].launch(handle, g + (1,) * (3 - len(g)), b + (1,) * (3 - len(b)), st.pack(*args))
+
+
+def _addr(b: Buffer) -> int:
+    return b.ptr.addr
+
+
+def _pad4(t: tuple, fill: int) -> tuple:
+    return (fill,) * (4 - len(t)) + tuple(t)
+
+
+# ---- element-wise launcher ------------------------------------------------------------------
+
+def _map(tag: str, expr: str, operands: list[Buffer], out_shape: tuple, svals: tuple = (),
+         out: DevicePtr | None = None) -> DevicePtr:
+    """Runs `expr` over `operands` broadcast to `out_shape`.
+
+    Collapses the iteration space jointly over all operands; if what is left is a
+    row-major (R, C) grid on which each operand is whole, one-per-row, one-row or a
+    single value, the vectorised `map_kernel` runs, otherwise the strided one."""
+    if len(out_shape) > 4:
+        raise ValueError("dlgrad only supports upto 4D tensors")
+    n = prod_(out_shape)
+    if n >= 2 ** 31:
+        raise ValueError(f"{n} elements exceed the 32-bit index range of the kernels")
+    out = out or alloc(n)
+    if n == 0:
+        return out
+    tens = [b for b in operands if not b.is_host_scalar]
+    t_strides = [get_broadcast_strides_2(out_shape, b.shape, b.stride) for b in tens]
+    cshape, cstr = collapse_dims(out_shape, calculate_stride(out_shape), *t_strides)
+    modes: list | None = []
+    C = cshape[-1] if len(cshape) == 2 else 1
+    it = iter(cstr[1:])
+    if len(cshape) <= 2:
+        full = (C, 1) if len(cshape) == 2 else (1,)
+        for b in operands:
+            if b.is_host_scalar:
+                modes.append("sval")
+                continue
+            st = next(it)
+            if st == full:
+                modes.append("vec")
+            elif not any(st):
+                modes.append("sptr")
+            elif st == (1, 0):
+                modes.append("row")
+            elif st == (0, 1):
+                modes.append("col")
+            else:
+                modes = None
+                break
+    else:
+        modes = None
+    vals = tuple(float(s) for s in svals)
+    if modes is not None:
+        wide = all(_addr(b) % 16 == 0 for b, m in zip(operands, modes) if m in ("vec", "col")) \
+            and out.addr % 16 == 0 and (C % 4 == 0 or not any(m in ("row", "col") for m in modes))
+        vec = 4 if wide else 1
+        k = kernel(K.map_kernel, tag, expr, tuple(modes), vec, len(vals))
+        args = [float(b.ptr.value) if b.is_host_scalar else _addr(b) for b in operands]
+        launch(k, K.map_grid(n, vec), 256, *args, *vals, out.addr, n, C)
+    else:
+        sval = tuple(b.is_host_scalar for b in operands)
+        k = kernel(K.strided_map_kernel, tag, expr, len(operands), sval, len(vals))
+        args = [float(b.ptr.value) if b.is_host_scalar else _addr(b) for b in operands]
+        st_args = [x for st in t_strides for x in _pad4(st, 0)]
+        launch(k, (n + 1023) // 1024, 256, *args, *vals, out.addr, n, *_pad4(out_shape, 1), *st_args)
+    return out
+
+
+class HIP:
+    """Dispatch-table entries for Device.HIP."""
+
+    # ---- host boundary ------------------------------------------------------------------------
+    @staticmethod
+    @dispatcher.register(BufferOps.CREATE, Device.HIP)
+    def create(data: np.ndarray) -> DevicePtr:
+        a = np.ascontiguousarray(data, dtype=np.float32)
+        p = alloc(a.size)
+        if a.size:
+            lib().h2d(p.addr, a.ctypes.data, a.nbytes)
+        return p
+
+    @staticmethod
+    @dispatcher.register(CustomOps.TO_HOST, Device.HIP)
+    def to_host(x: Buffer) -> np.ndarray:
+        out = np.empty(x.shape, dtype=np.float32)
+        if x.numel:
+            lib().d2h(out.ctypes.data, _addr(x), 4 * x.numel)
+        return out
+
+    @staticmethod
+    @dispatcher.register(CustomOps.PRINT, Device.HIP)
+    def show(x: Buffer) -> None:
+        print(HIP.to_host(x))
+
+    # ---- creation -------------------------------------------------------------------------------
+    _rng = np.random.default_rng()
+
+    @staticmethod
+    def manual_seed(seed: int) -> None:
+        HIP._rng = np.random.default_rng(seed)
+
+    @staticmethod
+    @dispatcher.register(BufferOps.UNIFORM, Device.HIP)
+    def uniform(shape: tuple, low: float = 0.0, high: float = 1.0) -> DevicePtr:
+        """U[low, high) drawn on the host and uploaded.  The reference's generator
+        (PCG32 reseeded from /dev/random per call, cpu_kernel.py:774-874) cannot be
+        reproduced value for value; only range and moments are comparable."""
+        u = HIP._rng.random(shape, dtype=np.float32)
+        return HIP.create(np.float32(low) + (np.float32(high) - np.float32(low)) * u)
+
+    @staticmethod
+    @dispatcher.register(BufferOps.FULL, Device.HIP)
+    def full(shape: tuple, fill_value: float) -> DevicePtr:
+        # cpu.py:252 hands the C kernel int(fill_value)
+        v = float(int(fill_value)) if STRICT_REFERENCE else float(fill_value)
+        return _map("full", "s0", [], tuple(shape), (v,))
+
+    @staticmethod
+    @dispatcher.register(BufferOps.ARANGE, Device.HIP)
+    def arange(shape: tuple) -> DevicePtr:
+        return _map("arange", "(float)i", [], tuple(shape))
+
+    # ---- binary -----------------------------------------------------------------------------------
+    @staticmethod
+    def _binary_op(x: Buffer, y: Buffer, op: str) -> DevicePtr:
+        return _map(op, K.BINARY_EXPR[op], [x, y], broadcast_shapes_2(x.shape, y.shape))
+
+    @staticmethod
+    @dispatcher.register(BinaryOps.ADD, Device.HIP)
+    def add(x: Buffer, y: Buffer) -> DevicePtr:
+        return HIP._binary_op(x, y, "add")
+
+    @staticmethod
+    @dispatcher.register(BinaryOps.SUB, Device.HIP)
+    def sub(x: Buffer, y: Buffer) -> DevicePtr:
+        return HIP._binary_op(x, y, "sub")
+
+    @staticmethod
+    @dispatcher.register(BinaryOps.MUL, Device.HIP)
+    def mul(x: Buffer, y: Buffer) -> DevicePtr:
+        return HIP._binary_op(x, y, "mul")
+
+    @staticmethod
+    @dispatcher.register(BinaryOps.DIV, Device.HIP)
+    def div(x: Buffer, y: Buffer) -> DevicePtr:
+        return HIP._binary_op(x, y, "div")
+
+    @staticmethod
+    @dispatcher.register(BinaryOps.GT, Device.HIP)
+    def gt(x: Buffer, y: Buffer) -> DevicePtr:
+        return HIP._binary_op(x, y, "gt")
+
+    @staticmethod
+    @dispatcher.register(BinaryOps.GTE, Device.HIP)
+    def gte(x: Buffer, y: Buffer) -> DevicePtr:
+        return HIP._binary_op(x, y, "gte")
+
+    @staticmethod
+    @dispatcher.register(BinaryOps.EQT, Device.HIP)
+    def eqt(x: Buffer, y: Buffer) -> DevicePtr:
+        return HIP._binary_op(x, y, "eq")
+
+    @staticmethod
+    @dispatcher.register(BinaryOps.CMP, Device.HIP)
+    def cmp(x: Buffer, y: Buffer, out_shape: tuple, mode: str) -> DevicePtr:
+        if mode != "<=":
+            raise ValueError(f"unsupported comparison {mode!r}")   # cpu.py:839-840 knows only "<="
+        return _map("le", K.BINARY_EXPR["le"], [x, y], tuple(out_shape))
+
+    # ---- unary ---------------------------------------------------------------------------------------
+    @staticmethod
+    def _unary(x: Buffer, tag: str, expr: str, svals: tuple = ()) -> DevicePtr:
+        return _map(tag, expr, [x], x.shape, svals)
+
+    @staticmethod
+    @dispatcher.register(UnaryOps.NEG, Device.HIP)
+    def neg(x: Buffer) -> DevicePtr:
+        return HIP._unary(x, "neg", K.UNARY_EXPR["neg"])
+
+    @staticmethod
+    @dispatcher.register(UnaryOps.EXP, Device.HIP)
+    def exp(x: Buffer) -> DevicePtr:
+        return HIP._unary(x, "exp", K.UNARY_EXPR["exp"])
+
+    @staticmethod
+    @dispatcher.register(UnaryOps.LOG, Device.HIP)
+    def log(x: Buffer) -> DevicePtr:
+        return HIP._unary(x, "log", K.UNARY_EXPR["log"])
+
+    @staticmethod
+    @dispatcher.register(UnaryOps.SQRT, Device.HIP)
+    def sqrt(x: Buffer) -> DevicePtr:
+        return HIP._unary(x, "sqrt", K.UNARY_EXPR["sqrt"])
+
+    @staticmethod
+    @dispatcher.register(UnaryOps.RSQRT, Device.HIP)
+    def rsqrt(x: Buffer) -> DevicePtr:
+        return HIP._unary(x, "rsqrt", K.UNARY_EXPR["rsqrt"])
+
+    @staticmethod
+    @dispatcher.register(UnaryOps.RELU, Device.HIP)
+    def relu(x: Buffer) -> DevicePtr:
+        return HIP._unary(x, "relu", K.UNARY_EXPR["relu"])
+
+    @staticmethod
+    @dispatcher.register(UnaryOps.POW, Device.HIP)
+    def pow(x: Buffer, val: float) -> DevicePtr:
+        # cpu.py:500 truncates the exponent to int before the call
+        if STRICT_REFERENCE or float(val).is_integer():
+            n = int(val)
+            return HIP._unary(x, f"pow{n}".replace("-", "m"), K.pow_expr(n))
+        return HIP._unary(x, "powf", "powf(x0, s0)", (val,))
+
+    @staticmethod
+    @dispatcher.register(UnaryOps.CLAMP, Device.HIP)
+    def clamp(x: Buffer, min_val: float | None, max_val: float | None) -> DevicePtr:
+        lo, hi = min_val is not None, max_val is not None
+        # the reference's two ifs in order (cpu_kernel.py:335-339): v<min -> min, then v>max -> max
+        expr, sv = "x0", []
+        if lo:
+            expr = "((x0 < s0) ? s0 : x0)"
+            sv.append(min_val)
+        if hi:
+            expr = f"(({expr} > s{len(sv)}) ? s{len(sv)} : {expr})"
+            sv.append(max_val)
+        return HIP._unary(x, f"clamp{int(lo)}{int(hi)}", expr, tuple(sv))
+
+    # ---- selects ----------------------------------------------------------------------------------------
+    @staticmethod
+    @dispatcher.register(UnaryOps.WHERE, Device.HIP)
+    def where(cond: Buffer, x: Buffer, y: Buffer) -> DevicePtr:
+        out_shape = broadcast_shapes_2(broadcast_shapes_2(x.shape, y.shape), cond.shape)
+        return _map("where", "(x0 > 0.0f) ? x1 : x2", [cond, x, y], out_shape)
+
+    @staticmethod
+    @dispatcher.register(UnaryOps.MASKED_FILL, Device.HIP)
+    def masked_fill(x: Buffer, mask: Buffer, val: float, out_shape: tuple) -> DevicePtr:
+        out_shape = broadcast_shapes_2(x.shape, mask.shape)
+        return _map("mfill", "(x1 > 0.0f) ? s0 : x0", [x, mask], out_shape, (val,))

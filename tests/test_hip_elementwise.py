@@ -1,0 +1,141 @@
+"""GPU parity: element-wise, broadcast, select and fill kernels against the C oracle.
+
+Tolerances are the ones the task states: bit-exact for selects/masks/fills and for
++ - * (single IEEE operations), 1e-6 relative for division and the transcendental
+unary ops.  The shape matrix is the reference's (test/test_ops.py:29-75, :347-384)."""
+import numpy as np
+import pytest
+
+from dlgrad_amd.buffer import Buffer
+from dlgrad_amd.device import Device
+from oracle import cref
+from tests.hip_util import check, dev, require_gpu
+
+pytestmark = pytest.mark.gpu
+RNG = np.random.default_rng(11)
+
+
+def f32(*shape):
+    return RNG.standard_normal(shape).astype(np.float32)
+
+
+def bcast_cases(shape):
+    return [tuple(1 if (m >> i) & 1 else d for i, d in enumerate(shape)) for m in range(2 ** len(shape))]
+
+
+OPS = {"add": lambda a, b: a + b, "sub": lambda a, b: a - b, "mul": lambda a, b: a * b,
+       "div": lambda a, b: a / b}
+
+
+@pytest.mark.parametrize("op", list(OPS))
+@pytest.mark.parametrize("shape", [(2, 3, 4, 5), (2, 3, 4), (784, 64), (1030,)])
+def test_binary_broadcast_matrix(op, shape):
+    require_gpu()
+    x = f32(*shape)
+    tol = 1e-6 if op == "div" else 0
+    for ys in bcast_cases(shape):
+        y = f32(*ys) + (3 if op == "div" else 0)
+        want = cref.binary(op, x, y)
+        check(OPS[op](dev(x), dev(y)).numpy(), want, tol, f"{op} {shape} {ys}")
+        # smaller operand on the left: Buffer swaps, negates (sub) or inverts (div)
+        if op in ("add", "mul"):
+            check(OPS[op](dev(y), dev(x)).numpy(), want, tol, f"r{op} {shape} {ys}")
+    check(OPS[op](dev(x), 2.5).numpy(), cref.binary(op, x, np.float32(2.5)), tol, f"{op} scalar")
+
+
+def test_reversed_sub_and_div():
+    require_gpu()
+    x, y = f32(6, 8), f32(1, 8) + 3
+    check((dev(y) - dev(x)).numpy(), cref.unary("neg", cref.binary("sub", x, y)), 0, "small-big")
+    check((dev(y) / dev(x)).numpy(), cref.binary("mul", cref.unary("pow", x, -1), y), 1e-6, "small/big")
+    check((3.0 - dev(x)).numpy(), np.float32(3.0) - x, 0, "scalar - x")
+
+
+@pytest.mark.parametrize("shape,ys", [((4096, 4096), (4096, 4096)), ((4096, 4096), (4096, 1)),
+                                      ((4096, 4096), (1, 4096)), ((16, 128, 128), (1, 128, 128)),
+                                      ((16, 4, 128, 128), (16, 4, 128, 1)), ((16, 128, 128), (1, 1, 128)),
+                                      ((1023, 1021), (1023, 1)), ((1023, 1021), (1, 1021))])
+def test_binary_config_shapes(shape, ys):
+    require_gpu()
+    x, y = f32(*shape), f32(*ys) + 3
+    bx, by = dev(x), dev(y)
+    for op in OPS:
+        check(OPS[op](bx, by).numpy(), cref.binary(op, x, y), 1e-6 if op == "div" else 0, f"{op} {shape}{ys}")
+
+
+def test_device_scalar_operand_and_views():
+    require_gpu()
+    x = f32(33, 17)
+    s = dev(np.float32(1.5).reshape(1, 1))
+    check((dev(x) * s).numpy(), x * np.float32(1.5), 0, "sptr")
+    # a view that starts 4 bytes into a block is not 16-byte aligned: scalar-width kernel
+    base = dev(f32(1 + 33 * 17))
+    view = Buffer(base.ptr + 1, (33, 17), Device.HIP)
+    want = base.numpy()[1:].reshape(33, 17)
+    check((view + dev(x)).numpy(), want + x, 0, "unaligned view")
+
+
+def test_comparisons_and_cmp():
+    require_gpu()
+    x = RNG.integers(-2, 3, (37, 41)).astype(np.float32)
+    y = RNG.integers(-2, 3, (37, 41)).astype(np.float32)
+    check((dev(x) == dev(y)).numpy(), cref.binary("eq", x, y), 0, "eq")
+    check((dev(x) > 0.0).numpy(), cref.binary("gt", x, np.float32(0)), 0, "gt")
+    check((dev(x) >= 1.0).numpy(), cref.binary("gte", x, np.float32(1)), 0, "gte")
+    H, W = 128, 128
+    cols, rows = np.arange(W, dtype=np.float32).reshape(1, W), np.arange(H, dtype=np.float32).reshape(H, 1)
+    check((dev(cols) <= dev(rows)).numpy(), cref.cmp_le(cols, rows, (H, W)), 0, "cmp<=")
+
+
+@pytest.mark.parametrize("n", [1, 5, 1024, 4097, 1 << 20])
+def test_unary(n):
+    require_gpu()
+    x = f32(n)
+    pos = np.abs(x) + np.float32(1e-3)
+    check((-dev(x)).numpy(), cref.unary("neg", x), 0, "neg")
+    check(dev(x).exp().numpy(), cref.unary("exp", x), 1e-6, "exp")
+    check(dev(pos).log().numpy(), cref.unary("log", pos), 1e-6, "log")
+    check(dev(pos).sqrt().numpy(), cref.unary("sqrt", pos), 1e-6, "sqrt")
+    check(dev(pos).rsqrt().numpy(), cref.unary("rsqrt", pos), 1e-6, "rsqrt")
+    for p in (2.0, 3.0, -1.0, 0.0):
+        check((dev(pos) ** p).numpy(), cref.unary("pow", pos, p), 1e-6, f"pow {p}")
+    check(dev(x).clamp(-0.5, 0.25).numpy(), cref.clamp(x, -0.5, 0.25), 0, "clamp")
+    check(dev(x).clamp(min=0).numpy(), cref.clamp(x, 0, None), 0, "clamp min")
+    check(dev(x).clamp(max=0.1).numpy(), cref.clamp(x, None, 0.1), 0, "clamp max")
+
+
+def test_exp_of_minus_inf_and_log_edge_values():
+    require_gpu()
+    x = np.array([-np.inf, -100.0, 0.0, 88.0, 1e-30], np.float32)
+    check(dev(x).exp().numpy(), np.exp(x.astype(np.float64)).astype(np.float32), 1e-6, "exp edge")
+
+
+def test_where_relu_masked_fill():
+    require_gpu()
+    c, x, y = f32(64, 50), f32(64, 50), f32(64, 50)
+    check(dev(c).where(dev(x), dev(y)).numpy(), cref.where(c, x, y), 0, "where ttt")
+    check(dev(c).where(dev(x), 0.0).numpy(), cref.where(c, x, np.float32(0)), 0, "where tts")
+    check(dev(c).where(1.0, 0.0).numpy(), cref.where(c, np.float32(1), np.float32(0)), 0, "where tss")
+    check(dev(x).relu().numpy(), cref.where(x, x, np.float32(0)), 0, "relu")
+    check(dev(x).leaky_relu(0.01).numpy(), cref.where(x, x, x * np.float32(0.01)), 0, "leaky")
+    x4 = f32(2, 3, 8, 8)
+    for ms in bcast_cases((2, 3, 8, 8)) + [(8, 8), (8,)]:
+        m = (RNG.random(ms) > 0.5).astype(np.float32)
+        for fill in (7.0, -np.inf):
+            check(Buffer.masked_fill(dev(x4), dev(m), fill).numpy(), cref.masked_fill(x4, m, fill), 0,
+                  f"masked_fill {ms} {fill}")
+    att = f32(16, 4, 128, 128)
+    mask = 1 - np.tril(np.ones((128, 128), np.float32))
+    check(Buffer.masked_fill(dev(att), dev(mask), float("-inf")).numpy(),
+          cref.masked_fill(att, mask, -np.inf), 0, "causal mask")
+
+
+def test_fills():
+    require_gpu()
+    check(Buffer.arange((128, 1), Device.HIP).numpy(), cref.arange((128, 1)), 0, "arange")
+    check(Buffer.full((3, 5), 1.0, Device.HIP).numpy(), cref.full((3, 5), 1.0), 0, "full 1")
+    check(Buffer.full((3, 5), 0.5, Device.HIP).numpy(), cref.full((3, 5), 0.5), 0, "full int-truncated")
+    check(Buffer.full((1027,), -3.0, Device.HIP).numpy(), cref.full((1027,), -3.0), 0, "full tail")
+    u = Buffer.uniform((100000,), Device.HIP, "float32", low=-2.0, high=2.0).numpy()
+    if u.any():
+        assert u.min() >= -2 and u.max() < 2 and abs(u.mean()) < 0.05
