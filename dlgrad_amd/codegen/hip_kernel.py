@@ -291,3 +291,473 @@ extern "C" __global__ __launch_bounds__(256) void {name}({', '.join(params)}) {{
 }}
 """
     return src, name, _fmt(*fmt)
+
+
+# =====================================================================================
+# reductions
+# =====================================================================================
+# (identity, combine(a, b), wave-level reduce) per op.  max starts from -FLT_MAX and
+# ignores NaN, as `if (v > val) val = v` does (cpu_kernel.py:78-81, :160-163).
+_RED = {
+    "sum": ("0.0f", "({a} + {b})", "wave_sum"),
+    "max": ("NEG_FLT_MAX", "fmaxf({a}, {b})", "wave_max"),
+}
+
+_BLOCK_REDUCE = r"""
+// 256 threads = 4 waves: per-wave DPP tree, then the four partials meet in LDS.
+static __device__ __forceinline__ float block_reduce(float v, float* sm) {
+    v = WAVE_RED(v);
+    const u32 lane = threadIdx.x & 63u, w = threadIdx.x >> 6;
+    if (lane == 0) sm[w] = v;
+    __syncthreads();
+    v = COMB(COMB(sm[0], sm[1]), COMB(sm[2], sm[3]));
+    __syncthreads();
+    return v;
+}
+"""
+
+
+def _red_defs(op: str) -> str:
+    ident, comb, wred = _RED[op]
+    return (f"#define IDENT {ident}\n#define COMB(a, b) {comb.format(a='(a)', b='(b)')}\n"
+            f"#define WAVE_RED {wred}\n")
+
+
+@cache
+def reduce_full_kernel(op: str, vec: int) -> tuple[str, str, str]:
+    """Stage kernel of the full reduction (cpu_kernel.py:150-177): every block folds a
+    grid-strided share of x into one value, out[blockIdx.x] = value / divisor.  The
+    launcher runs it once over x with G blocks and once more, with one block, over the
+    G partials; `divisor` is 1 except in the last stage of a mean."""
+    name = f"reduce_full_{op}_v{vec}"
+    if vec == 4:
+        loop = r"""
+    const u32 nv = n >> 2;
+    const float4* __restrict__ x4 = reinterpret_cast<const float4*>(x);
+    float a0 = IDENT, a1 = IDENT, a2 = IDENT, a3 = IDENT;
+    const u32 stride = gridDim.x * 256u;
+    u32 v = blockIdx.x * 256u + threadIdx.x;
+    for (; v + 3u * stride < nv; v += 4u * stride) {
+        const float4 p = x4[v], q = x4[v + stride], r = x4[v + 2u * stride], s = x4[v + 3u * stride];
+        a0 = COMB(a0, COMB(COMB(p.x, p.y), COMB(p.z, p.w)));
+        a1 = COMB(a1, COMB(COMB(q.x, q.y), COMB(q.z, q.w)));
+        a2 = COMB(a2, COMB(COMB(r.x, r.y), COMB(r.z, r.w)));
+        a3 = COMB(a3, COMB(COMB(s.x, s.y), COMB(s.z, s.w)));
+    }
+    for (; v < nv; v += stride) {
+        const float4 p = x4[v];
+        a0 = COMB(a0, COMB(COMB(p.x, p.y), COMB(p.z, p.w)));
+    }
+    float acc = COMB(COMB(a0, a1), COMB(a2, a3));
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) acc = COMB(acc, x[(nv << 2) + threadIdx.x]);
+"""
+    else:
+        loop = r"""
+    float a0 = IDENT, a1 = IDENT;
+    const u32 stride = gridDim.x * 256u;
+    u32 i = blockIdx.x * 256u + threadIdx.x;
+    for (; i + stride < n; i += 2u * stride) { a0 = COMB(a0, x[i]); a1 = COMB(a1, x[i + stride]); }
+    if (i < n) a0 = COMB(a0, x[i]);
+    float acc = COMB(a0, a1);
+"""
+    src = f"""{PRELUDE}{_red_defs(op)}{_BLOCK_REDUCE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        float* __restrict__ out, u32 n, float divisor) {{
+    __shared__ float sm[4];
+{loop}
+    acc = block_reduce(acc, sm);
+    if (threadIdx.x == 0) out[blockIdx.x] = acc / divisor;
+}}
+"""
+    return src, name, _fmt("P", "P", "I", "f")
+
+
+@cache
+def reduce_rows_kernel(op: str, vec: int, per_block: bool) -> tuple[str, str, str]:
+    """out[r] = reduce over the contiguous row r of an (R, L) view, / divisor
+    (the last-axis case of cpu_kernel.py:68-148).  Either one wavefront per row
+    (four rows per 256-thread block) or, for long rows, one block per row."""
+    name = f"reduce_rows_{op}_v{vec}_{'blk' if per_block else 'wav'}"
+    T = "256u" if per_block else "64u"
+    tid = "threadIdx.x" if per_block else "(threadIdx.x & 63u)"
+    row = "blockIdx.x" if per_block else "(blockIdx.x * 4u + (threadIdx.x >> 6))"
+    if vec == 4:
+        loop = f"""
+    const float4* __restrict__ p = reinterpret_cast<const float4*>(x + (u64)row * L);
+    const u32 nv = L >> 2;
+    float a0 = IDENT, a1 = IDENT;
+    u32 v = {tid};
+    for (; v + {T} < nv; v += 2u * {T}) {{
+        const float4 s = p[v], t = p[v + {T}];
+        a0 = COMB(a0, COMB(COMB(s.x, s.y), COMB(s.z, s.w)));
+        a1 = COMB(a1, COMB(COMB(t.x, t.y), COMB(t.z, t.w)));
+    }}
+    if (v < nv) {{ const float4 s = p[v]; a0 = COMB(a0, COMB(COMB(s.x, s.y), COMB(s.z, s.w))); }}
+    float acc = COMB(a0, a1);
+"""
+    else:
+        loop = f"""
+    const float* __restrict__ p = x + (u64)row * L;
+    float acc = IDENT;
+    for (u32 i = {tid}; i < L; i += {T}) acc = COMB(acc, p[i]);
+"""
+    if per_block:
+        fin = """    acc = block_reduce(acc, sm);
+    if (threadIdx.x == 0) out[row] = acc / divisor;"""
+        guard = ""
+    else:
+        fin = """    acc = WAVE_RED(acc);
+    if ((threadIdx.x & 63u) == 0) out[row] = acc / divisor;"""
+        guard = "    if (row >= R) return;\n"
+    src = f"""{PRELUDE}{_red_defs(op)}{_BLOCK_REDUCE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        float* __restrict__ out, u32 R, u32 L, float divisor) {{
+    __shared__ float sm[4];
+    const u32 row = {row};
+{guard}{loop}
+{fin}
+}}
+"""
+    return src, name, _fmt("P", "P", "I", "I", "f")
+
+
+@cache
+def reduce_cols_kernel(op: str, vec: int) -> tuple[str, str, str]:
+    """out[o, c, i] = reduce over l in chunk c of x[o, l, i] for an (O, L, I) view, / divisor
+    (the non-last-axis case of cpu_kernel.py:68-148, e.g. axis 0 of a matrix).
+
+    The reference walks each column with stride I.  Here a 64x4 block owns 64*vec
+    adjacent columns: lanes read consecutive addresses of one row (coalesced), the
+    four thread rows take every fourth row of the chunk, and LDS joins them.  L is
+    split into `chunks` so that tall, narrow inputs still fill the chip; the launcher
+    reduces the (O, chunks, I) partials with a second call."""
+    name = f"reduce_cols_{op}_v{vec}"
+    if vec == 4:
+        defs = """#define VT float4
+#define LD(l) (reinterpret_cast<const float4*>(xp + (u64)(l) * I)[0])
+#define ACC(a, t) { a.x = COMB(a.x, t.x); a.y = COMB(a.y, t.y); a.z = COMB(a.z, t.z); a.w = COMB(a.w, t.w); }
+#define VINIT make_float4(IDENT, IDENT, IDENT, IDENT)
+#define STORE(p, r) { r.x /= divisor; r.y /= divisor; r.z /= divisor; r.w /= divisor; reinterpret_cast<float4*>(p)[0] = r; }
+"""
+    else:
+        defs = """#define VT float
+#define LD(l) (xp[(u64)(l) * I])
+#define ACC(a, t) { a = COMB(a, t); }
+#define VINIT IDENT
+#define STORE(p, r) { (p)[0] = r / divisor; }
+"""
+    src = f"""{PRELUDE}{_red_defs(op)}{defs}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        float* __restrict__ out, u32 L, u32 I, u32 chunk, float divisor) {{
+    __shared__ VT sm[4][64];
+    const u32 tx = threadIdx.x, ty = threadIdx.y, o = blockIdx.z;
+    const u32 col = (blockIdx.x * 64u + tx) * {vec}u;
+    const u32 l0 = blockIdx.y * chunk, l1 = min(L, l0 + chunk);
+    VT a0 = VINIT, a1 = VINIT, a2 = VINIT, a3 = VINIT;
+    if (col < I) {{
+        const float* __restrict__ xp = x + (u64)o * L * I + col;
+        u32 l = l0 + ty;
+        for (; l + 12u < l1; l += 16u) {{
+            const VT t0 = LD(l), t1 = LD(l + 4u), t2 = LD(l + 8u), t3 = LD(l + 12u);
+            ACC(a0, t0) ACC(a1, t1) ACC(a2, t2) ACC(a3, t3)
+        }}
+        for (; l < l1; l += 4u) {{ const VT t0 = LD(l); ACC(a0, t0) }}
+        ACC(a0, a1) ACC(a2, a3) ACC(a0, a2)
+    }}
+    sm[ty][tx] = a0;
+    __syncthreads();
+    if (ty == 0 && col < I) {{
+        VT r = sm[0][tx];
+        #pragma unroll
+        for (int k = 1; k < 4; ++k) {{ const VT t = sm[k][tx]; ACC(r, t) }}
+        STORE(out + ((u64)o * gridDim.y + blockIdx.y) * I + col, r)
+    }}
+}}
+"""
+    return src, name, _fmt("P", "P", "I", "I", "I", "f")
+
+
+@cache
+def argmax_kernel(rows: bool) -> tuple[str, str, str]:
+    """Index (as float) of the first maximum along L of an (O, L, I) view
+    (cpu_kernel.py:459-517: strict '>', start value -FLT_MAX at index 0).
+    rows=True handles I == 1 with one wavefront per row; otherwise one thread per
+    output column walks L.  Ties resolve to the lowest index in both."""
+    if rows:
+        name = "argmax_rows"
+        src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        float* __restrict__ out, u32 R, u32 L) {{
+    const u32 row = blockIdx.x * 4u + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    if (row >= R) return;
+    const float* __restrict__ p = x + (u64)row * L;
+    float best = NEG_FLT_MAX; u32 bi = 0;
+    for (u32 i = lane; i < L; i += 64u) {{ const float v = p[i]; if (v > best) {{ best = v; bi = i; }} }}
+    #pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {{
+        const float ov = __shfl_xor(best, off, WAVE);
+        const u32 oi = __shfl_xor(bi, off, WAVE);
+        if (ov > best || (ov == best && oi < bi)) {{ best = ov; bi = oi; }}
+    }}
+    if (lane == 0) out[row] = (float)bi;
+}}
+"""
+        return src, name, _fmt("P", "P", "I", "I")
+    name = "argmax_cols"
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        float* __restrict__ out, u32 O, u32 L, u32 I) {{
+    const u32 t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= O * I) return;
+    const u32 o = t / I, i = t % I;
+    const float* __restrict__ p = x + (u64)o * L * I + i;
+    float best = NEG_FLT_MAX; u32 bi = 0;
+    for (u32 l = 0; l < L; ++l) {{ const float v = p[(u64)l * I]; if (v > best) {{ best = v; bi = l; }} }}
+    out[t] = (float)bi;
+}}
+"""
+    return src, name, _fmt("P", "P", "I", "I", "I")
+
+
+# =====================================================================================
+# permute
+# =====================================================================================
+
+@cache
+def permute_gather_kernel(vec: int) -> tuple[str, str, str]:
+    """out (contiguous, <=4-D, padded on the left) <- x read through permuted strides
+    (cpu_kernel.py:179-215), for permutations that keep the innermost dim innermost:
+    both sides are then contiguous along that dim and each thread moves `vec` floats.
+    vec=4 needs the inner extent, every input stride and both bases to be multiples of 4."""
+    name = f"permute_gather_v{vec}"
+    if vec == 4:
+        move = ("reinterpret_cast<float4*>(out)[i] = "
+                "reinterpret_cast<const float4*>(x + off)[0];")
+        scale = "const u32 c3 = (r % shape.d[3]) << 2; r /= shape.d[3];"   # shape.d[3] is in float4 units
+    else:
+        move = "out[i] = x[off];"
+        scale = "const u32 c3 = r % shape.d[3]; r /= shape.d[3];"
+    src = f"""{PRELUDE}
+struct Dims4 {{ u32 d[4]; }};
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        float* __restrict__ out, u32 n, Dims4 shape, Dims4 st) {{
+    const u32 i0 = blockIdx.x * 1024u + threadIdx.x;
+    #pragma unroll
+    for (int u = 0; u < 4; ++u) {{
+        const u32 i = i0 + u * 256u;
+        if (i < n) {{
+            u32 r = i;
+            {scale}
+            const u32 c2 = r % shape.d[2]; r /= shape.d[2];
+            const u32 c1 = r % shape.d[1];
+            const u32 c0 = r / shape.d[1];
+            const u64 off = (u64)c0 * st.d[0] + (u64)c1 * st.d[1] + (u64)c2 * st.d[2] + c3;
+            {move}
+        }}
+    }}
+}}
+"""
+    return src, name, _fmt("P", "P", "I", "4I", "4I")
+
+
+@cache
+def permute_tiled_kernel() -> tuple[str, str, str]:
+    """Permutations that move another dim into the innermost position, e.g. (.., a, b) ->
+    (.., b, a) or (B,T,h,d) -> (B,h,d,T).  Out dims are (p, q, t, b) after padding where
+    b is the out-innermost dim and t is the out dim whose *input* stride is 1.  A 32x32
+    tile of the (t, b) plane goes through LDS (33-float rows, no bank conflicts) so that
+    reads run along t and writes along b, both coalesced; p and q only offset the tile.
+    The reference reads with the large stride directly (cpu_kernel.py:207-212)."""
+    name = "permute_tiled"
+    src = f"""{PRELUDE}
+struct PArgs {{ u32 np, nq, nt, nb;        // extents: two carried dims, tile dims t and b
+               u32 ip, iq, ib;            // input strides of p, q, b (t has input stride 1)
+               u32 op, oq, ot; }};        // output strides of p, q, t (b has output stride 1)
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        float* __restrict__ out, PArgs a) {{
+    __shared__ float tile[32][33];
+    const u32 tb = (a.nb + 31u) >> 5, tt = (a.nt + 31u) >> 5;
+    u32 r = blockIdx.x;
+    const u32 bb = r % tb; r /= tb;
+    const u32 bt = r % tt; r /= tt;
+    const u32 q = r % a.nq, p = r / a.nq;
+    const float* __restrict__ xi = x + (u64)p * a.ip + (u64)q * a.iq;
+    float* __restrict__ oo = out + (u64)p * a.op + (u64)q * a.oq;
+    const u32 tx = threadIdx.x & 31u, ty = threadIdx.x >> 5;
+    #pragma unroll
+    for (u32 k = 0; k < 32u; k += 8u) {{
+        const u32 t = bt * 32u + tx, b = bb * 32u + ty + k;
+        if (t < a.nt && b < a.nb) tile[ty + k][tx] = xi[(u64)b * a.ib + t];
+    }}
+    __syncthreads();
+    #pragma unroll
+    for (u32 k = 0; k < 32u; k += 8u) {{
+        const u32 t = bt * 32u + ty + k, b = bb * 32u + tx;
+        if (t < a.nt && b < a.nb) oo[(u64)t * a.ot + b] = tile[tx][ty + k];
+    }}
+}}
+"""
+    return src, name, _fmt("P", "P", "10I")
+
+
+# =====================================================================================
+# embedding, cross-entropy helpers, fused softmax
+# =====================================================================================
+
+@cache
+def embedding_kernel() -> tuple[str, str, str]:
+    """Gather: out[i, :] = x[(int)(idx[i] * W) + 0..W) (cpu_kernel.py:217-229; the
+    offset is formed in float and truncated, exactly as there).  One wavefront per
+    index; 16-byte moves when W and the offset allow it."""
+    name = "embedding_gather"
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        const float* __restrict__ idx, float* __restrict__ out, u32 n_idx, u32 W, u32 aligned) {{
+    const u32 i = blockIdx.x * 4u + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    if (i >= n_idx) return;
+    const int x_idx = (int)(idx[i] * (float)W);
+    const float* __restrict__ src = x + (long long)x_idx;
+    float* __restrict__ dst = out + (u64)i * W;
+    if (aligned && ((x_idx & 3) == 0)) {{
+        for (u32 v = lane; v < (W >> 2); v += 64u)
+            reinterpret_cast<float4*>(dst)[v] = reinterpret_cast<const float4*>(src)[v];
+    }} else {{
+        for (u32 j = lane; j < W; j += 64u) dst[j] = src[j];
+    }}
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "I", "I", "I")
+
+
+@cache
+def embedding_backward_kernel() -> tuple[str, str, str]:
+    """Scatter-add: out[(int)idx[i], j] += g[i, j] into a zeroed (V, W) table
+    (cpu_kernel.py:231-243).  The row index is formed in integers; the reference forms
+    idx*W + j in float, which is the same number wherever that product is exact
+    (below 2^24) and a wrong column above.  Hardware fp32 atomics, one wavefront per
+    index row, so duplicate ids accumulate in an unspecified order."""
+    name = "embedding_scatter_add"
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out,
+        const float* __restrict__ g, const float* __restrict__ idx, u32 n_idx, u32 W) {{
+    const u32 i = blockIdx.x * 4u + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    if (i >= n_idx) return;
+    float* __restrict__ dst = out + (long long)((int)idx[i]) * W;
+    const float* __restrict__ src = g + (u64)i * W;
+    for (u32 j = lane; j < W; j += 64u) unsafeAtomicAdd(dst + j, src[j]);
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "I", "I")
+
+
+@cache
+def ce_kernel(backward: bool) -> tuple[str, str, str]:
+    """ce_forward: out[i] = x[(int)target[i] + stride0*i]; ce_backward: that element -= 1,
+    in place (cpu_kernel.py:430-457)."""
+    if backward:
+        name = "ce_backward"
+        src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(float* x, const float* __restrict__ target,
+        u32 rows, u32 stride0) {{
+    const u32 i = blockIdx.x * 256u + threadIdx.x;
+    if (i < rows) x[(long long)(int)target[i] + (u64)stride0 * i] -= 1.0f;
+}}
+"""
+        return src, name, _fmt("P", "P", "I", "I")
+    name = "ce_forward"
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        const float* __restrict__ target, float* __restrict__ out, u32 rows, u32 stride0) {{
+    const u32 i = blockIdx.x * 256u + threadIdx.x;
+    if (i < rows) out[i] = x[(long long)(int)target[i] + (u64)stride0 * i];
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "I", "I")
+
+
+@cache
+def softmax_rows_kernel(log: bool, vec: int, per_block: bool) -> tuple[str, str, str]:
+    """Row softmax / log-softmax over the contiguous last axis of an (R, L) view in one
+    pass over HBM: max, exp-sum and the normalised write all read the row from
+    registers-or-L2 instead of materialising max, x-max, exp and sum as the reference's
+    five kernels do (tensor.py:634-669).  Same formula: e = exp(x - max); e / sum(e)
+    (or (x - max) - log(sum)).  One wavefront per row, or one block per long row."""
+    name = f"{'log_' if log else ''}softmax_rows_v{vec}_{'blk' if per_block else 'wav'}"
+    T = "256u" if per_block else "64u"
+    tid = "threadIdx.x" if per_block else "(threadIdx.x & 63u)"
+    row = "blockIdx.x" if per_block else "(blockIdx.x * 4u + (threadIdx.x >> 6))"
+    red_max = "block_max(m, sm)" if per_block else "wave_max(m)"
+    red_sum = "block_sum(s, sm)" if per_block else "wave_sum(s)"
+    outexpr = "(V - m) - ls" if log else "expf(V - m) / s"
+    if vec == 4:
+        body = f"""
+    const float4* __restrict__ p = reinterpret_cast<const float4*>(x + (u64)row * L);
+    float4* __restrict__ q = reinterpret_cast<float4*>(out + (u64)row * L);
+    const u32 nv = L >> 2;
+    float m = NEG_FLT_MAX;
+    for (u32 v = {tid}; v < nv; v += {T}) {{ const float4 t = p[v]; m = fmaxf(fmaxf(m, fmaxf(t.x, t.y)), fmaxf(t.z, t.w)); }}
+    m = {red_max};
+    float s = 0.0f;
+    for (u32 v = {tid}; v < nv; v += {T}) {{ const float4 t = p[v]; s += (expf(t.x - m) + expf(t.y - m)) + (expf(t.z - m) + expf(t.w - m)); }}
+    s = {red_sum};
+    const float ls = logf(s); (void)ls;
+    for (u32 v = {tid}; v < nv; v += {T}) {{
+        const float4 t = p[v]; float4 o;
+        #define V t.x
+        o.x = {outexpr};
+        #undef V
+        #define V t.y
+        o.y = {outexpr};
+        #undef V
+        #define V t.z
+        o.z = {outexpr};
+        #undef V
+        #define V t.w
+        o.w = {outexpr};
+        #undef V
+        q[v] = o;
+    }}
+"""
+    else:
+        body = f"""
+    const float* __restrict__ p = x + (u64)row * L;
+    float* __restrict__ q = out + (u64)row * L;
+    float m = NEG_FLT_MAX;
+    for (u32 i = {tid}; i < L; i += {T}) m = fmaxf(m, p[i]);
+    m = {red_max};
+    float s = 0.0f;
+    for (u32 i = {tid}; i < L; i += {T}) s += expf(p[i] - m);
+    s = {red_sum};
+    const float ls = logf(s); (void)ls;
+    for (u32 i = {tid}; i < L; i += {T}) {{
+        #define V p[i]
+        q[i] = {outexpr};
+        #undef V
+    }}
+"""
+    src = f"""{PRELUDE}
+static __device__ __forceinline__ float block_max(float v, float* sm) {{
+    v = wave_max(v);
+    if ((threadIdx.x & 63u) == 0) sm[threadIdx.x >> 6] = v;
+    __syncthreads();
+    v = fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3]));
+    __syncthreads();
+    return v;
+}}
+static __device__ __forceinline__ float block_sum(float v, float* sm) {{
+    v = wave_sum(v);
+    if ((threadIdx.x & 63u) == 0) sm[threadIdx.x >> 6] = v;
+    __syncthreads();
+    v = (sm[0] + sm[1]) + (sm[2] + sm[3]);
+    __syncthreads();
+    return v;
+}}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        float* __restrict__ out, u32 R, u32 L) {{
+    __shared__ float sm[4];
+    const u32 row = {row};
+    {'' if per_block else 'if (row >= R) return;'}
+{body}
+}}
+"""
+    return src, name, _fmt("P", "P", "I", "I")

@@ -436,3 +436,194 @@ class HIP:
     def masked_fill(x: Buffer, mask: Buffer, val: float, out_shape: tuple) -> DevicePtr:
         out_shape = broadcast_shapes_2(x.shape, mask.shape)
         return _map("mfill", "(x1 > 0.0f) ? s0 : x0", [x, mask], out_shape, (val,))
+
+    # ---- reductions ------------------------------------------------------------------------------------
+    @staticmethod
+    def _reduce_full_into(kop: str, x_addr: int, n: int, divisor: float, out_addr: int) -> None:
+        vec = 4 if x_addr % 16 == 0 else 1
+        G = max(1, min(2048, n // (256 * 4 * 4)))
+        if G == 1:
+            launch(kernel(K.reduce_full_kernel, kop, vec), 1, 256, x_addr, out_addr, n, float(divisor))
+            return
+        part = alloc(G)
+        launch(kernel(K.reduce_full_kernel, kop, vec), G, 256, x_addr, part.addr, n, 1.0)
+        launch(kernel(K.reduce_full_kernel, kop, 4), 1, 256, part.addr, out_addr, G, float(divisor))
+
+    @staticmethod
+    def _reduce_cols(kop: str, x_addr: int, O: int, L: int, I: int, divisor: float, out_addr: int) -> None:
+        vec = 4 if (I % 4 == 0 and x_addr % 16 == 0 and out_addr % 16 == 0) else 1
+        bx = (I + 64 * vec - 1) // (64 * vec)
+        chunks = max(1, min(2048 // max(1, bx * O), L // 32))
+        chunk = (L + chunks - 1) // chunks
+        chunk = (chunk + 3) // 4 * 4
+        chunks = (L + chunk - 1) // chunk
+        k = kernel(K.reduce_cols_kernel, kop, vec)
+        if chunks == 1:
+            launch(k, (bx, 1, O), (64, 4, 1), x_addr, out_addr, L, I, L, float(divisor))
+            return
+        part = alloc(O * chunks * I)
+        launch(k, (bx, chunks, O), (64, 4, 1), x_addr, part.addr, L, I, chunk, 1.0)
+        HIP._reduce_cols(kop, part.addr, O, chunks, I, divisor, out_addr)
+
+    @staticmethod
+    def _reduce(x: Buffer, dim: int, op: str) -> DevicePtr:
+        """sum / max / mean over everything (dim -1 or None) or over one axis
+        (cpu.py:604-761).  The (outer, L, inner) view of the contiguous input decides
+        the kernel: inner == 1 reduces contiguous rows, otherwise columns."""
+        kop = "sum" if op == "mean" else op
+        if x.numel >= 2 ** 31:
+            raise ValueError("tensor too large for 32-bit indexing")
+        if dim is None or dim == -1:
+            out = alloc(1)
+            HIP._reduce_full_into(kop, _addr(x), x.numel, x.numel if op == "mean" else 1.0, out.addr)
+            return out
+        if dim < 0:
+            dim += x.ndim
+        O, L, I = prod_(x.shape[:dim]), x.shape[dim], prod_(x.shape[dim + 1:])
+        divisor = float(L) if op == "mean" else 1.0
+        out = alloc(O * I)
+        if O * I == 0 or L == 0:
+            return out
+        if I == 1:
+            if O < 64 and L >= (1 << 16):                  # a few very long rows: full reduction each
+                for r in range(O):
+                    HIP._reduce_full_into(kop, _addr(x) + 4 * r * L, L, divisor, out.addr + 4 * r)
+                return out
+            vec = 4 if (L % 4 == 0 and _addr(x) % 16 == 0) else 1
+            blk = L >= 2048
+            launch(kernel(K.reduce_rows_kernel, kop, vec, blk), O if blk else (O + 3) // 4, 256,
+                   _addr(x), out.addr, O, L, divisor)
+        else:
+            if O > 65535:
+                raise ValueError("outer extent too large for the column reduction grid")
+            HIP._reduce_cols(kop, _addr(x), O, L, I, divisor, out.addr)
+        return out
+
+    @staticmethod
+    @dispatcher.register(UnaryOps.SUM, Device.HIP)
+    def sum(x: Buffer, dim: int) -> DevicePtr:
+        return HIP._reduce(x, dim, "sum")
+
+    @staticmethod
+    @dispatcher.register(UnaryOps.MEAN, Device.HIP)
+    def mean(x: Buffer, dim: int) -> DevicePtr:
+        return HIP._reduce(x, dim, "mean")
+
+    @staticmethod
+    @dispatcher.register(UnaryOps.MAX, Device.HIP)
+    def max(x: Buffer, dim: int, out: Buffer = None) -> DevicePtr:
+        return HIP._reduce(x, dim, "max")
+
+    @staticmethod
+    @dispatcher.register(UnaryOps.ARGMAX, Device.HIP)
+    def argmax(x: Buffer, dim: int) -> DevicePtr:
+        if dim is None:
+            O, L, I = 1, x.numel, 1                       # cpu.py:913-918 flattens
+        else:
+            if dim < 0:
+                dim += x.ndim
+            O, L, I = prod_(x.shape[:dim]), x.shape[dim], prod_(x.shape[dim + 1:])
+        out = alloc(O * I)
+        if I == 1:
+            launch(kernel(K.argmax_kernel, True), (O + 3) // 4, 256, _addr(x), out.addr, O, L)
+        else:
+            launch(kernel(K.argmax_kernel, False), (O * I + 255) // 256, 256, _addr(x), out.addr, O, L, I)
+        return out
+
+    # ---- permute ---------------------------------------------------------------------------------------------
+    @staticmethod
+    @dispatcher.register(UnaryOps.PERMUTE, Device.HIP)
+    def permute(x: Buffer, order: tuple) -> DevicePtr:
+        """Materialised permutation (cpu.py:333-368).  After merging dims that stay
+        adjacent, either the innermost dim is still innermost (strided row copy) or
+        another dim became innermost (LDS-tiled transpose of that pair of dims)."""
+        out_shape = tuple(x.shape[i] for i in order)
+        in_str = tuple(x.stride[i] for i in order)
+        n = x.numel
+        out = alloc(n)
+        if n == 0:
+            return out
+        cshape, (cout, cin) = collapse_dims(out_shape, calculate_stride(out_shape), in_str)
+        if n == 1 or cin[-1] == 1:
+            wide = (cshape[-1] % 4 == 0 and all(s % 4 == 0 for s in cin[:-1])
+                    and _addr(x) % 16 == 0 and out.addr % 16 == 0)
+            vec = 4 if wide else 1
+            shape4 = list(_pad4(cshape, 1))
+            shape4[3] //= vec
+            launch(kernel(K.permute_gather_kernel, vec), (n // vec + 1023) // 1024, 256,
+                   _addr(x), out.addr, n // vec, *shape4, *_pad4(cin, 0))
+            return out
+        t = cin.index(1)
+        others = [d for d in range(len(cshape) - 1) if d != t]
+        ext = [cshape[d] for d in others]
+        i_st = [cin[d] for d in others]
+        o_st = [cout[d] for d in others]
+        while len(ext) < 2:
+            ext.insert(0, 1), i_st.insert(0, 0), o_st.insert(0, 0)
+        nt, nb = cshape[t], cshape[-1]
+        grid = ((nb + 31) // 32) * ((nt + 31) // 32) * ext[0] * ext[1]
+        launch(kernel(K.permute_tiled_kernel), grid, 256, _addr(x), out.addr,
+               ext[0], ext[1], nt, nb, i_st[0], i_st[1], cin[-1], o_st[0], o_st[1], cout[t])
+        return out
+
+    # ---- embedding and cross-entropy helpers ----------------------------------------------------------------------
+    @staticmethod
+    @dispatcher.register(CustomOps.EMBEDDING, Device.HIP)
+    def embedding(x: Buffer, idx: Buffer, out_numel: int, backward: bool = False,
+                  upstream_grad: Buffer = None) -> DevicePtr:
+        W, n_idx = x.shape[-1], idx.numel
+        if backward:
+            out = alloc(x.numel, zero=True)                    # init_with_scalar(0), cpu.py:1031
+            if n_idx:
+                launch(kernel(K.embedding_backward_kernel), (n_idx + 3) // 4, 256,
+                       out.addr, _addr(upstream_grad), _addr(idx), n_idx, W)
+            return out
+        out = alloc(out_numel)
+        if n_idx:
+            aligned = int(W % 4 == 0 and _addr(x) % 16 == 0 and out.addr % 16 == 0)
+            launch(kernel(K.embedding_kernel), (n_idx + 3) // 4, 256,
+                   _addr(x), _addr(idx), out.addr, n_idx, W, aligned)
+        return out
+
+    @staticmethod
+    @dispatcher.register(CustomOps.CE_FORWARD, Device.HIP)
+    def ce_forward(x: Buffer, y: Buffer) -> DevicePtr:
+        rows = x.shape[0]
+        out = alloc(rows)
+        launch(kernel(K.ce_kernel, False), (rows + 255) // 256, 256, _addr(x), _addr(y), out.addr,
+               rows, x.stride[0])
+        return out
+
+    @staticmethod
+    @dispatcher.register(CustomOps.CE_BACKWARD, Device.HIP)
+    def ce_backward(x: Buffer, target: Buffer) -> None:
+        rows = x.shape[0]
+        launch(kernel(K.ce_kernel, True), (rows + 255) // 256, 256, _addr(x), _addr(target), rows, x.stride[0])
+
+    # ---- fused row softmax ---------------------------------------------------------------------------------------------
+    @staticmethod
+    def _softmax(x: Buffer, dim: int, log: bool) -> DevicePtr:
+        if dim < 0:
+            dim += x.ndim
+        if dim != x.ndim - 1:
+            raise ValueError("the fused softmax kernel reduces the last axis only")
+        L = x.shape[-1]
+        R = x.numel // max(L, 1)
+        out = alloc(x.numel)
+        if x.numel == 0:
+            return out
+        vec = 4 if (L % 4 == 0 and _addr(x) % 16 == 0 and out.addr % 16 == 0) else 1
+        blk = L > 2048
+        launch(kernel(K.softmax_rows_kernel, log, vec, blk), R if blk else (R + 3) // 4, 256,
+               _addr(x), out.addr, R, L)
+        return out
+
+    @staticmethod
+    @dispatcher.register(CustomOps.SOFTMAX, Device.HIP)
+    def softmax(x: Buffer, dim: int) -> DevicePtr:
+        return HIP._softmax(x, dim, False)
+
+    @staticmethod
+    @dispatcher.register(CustomOps.LOG_SOFTMAX, Device.HIP)
+    def log_softmax(x: Buffer, dim: int) -> DevicePtr:
+        return HIP._softmax(x, dim, True)

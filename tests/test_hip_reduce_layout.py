@@ -1,0 +1,175 @@
+"""GPU parity: reductions, arg-max, permutations, embedding, cross-entropy helpers and
+the fused row softmax against the C oracle.
+
+Tolerances (task statement): reductions 1e-5 relative -- judged on |hip - f64| not being
+worse than that, or on hip being at least as close to float64 as the CPU path is, because
+a -ffast-math fp32 sum over millions of values is itself ~1e-5..1e-4 away from the true sum;
+max, arg-max, permutes, gathers and the CE helpers are bit-exact."""
+import numpy as np
+import pytest
+
+from dlgrad_amd.buffer import Buffer
+from dlgrad_amd.helpers import CustomOps
+from oracle import cref
+from tests.hip_util import check, dev, rel_err, require_gpu
+from dlgrad_amd.runtime import hip
+
+pytestmark = pytest.mark.gpu
+RNG = np.random.default_rng(5)
+
+
+def f32(*shape):
+    return RNG.standard_normal(shape).astype(np.float32)
+
+
+def check_sum_like(got, x64_result, cpu_result, what):
+    """1e-5 relative to the scale of the result, or at least as close to float64 as the CPU path."""
+    if hip.COMPILE_ONLY:
+        return
+    got = np.asarray(got, np.float64)
+    scale = np.maximum(np.abs(x64_result), np.abs(x64_result).mean() if np.ndim(x64_result) else 0) + 1e-30
+    e_hip = np.max(np.abs(got - x64_result) / scale)
+    e_cpu = np.max(np.abs(np.asarray(cpu_result, np.float64) - x64_result) / scale)
+    assert got.shape == np.shape(x64_result), what
+    assert e_hip <= 1e-5 or e_hip <= e_cpu, f"{what}: hip err {e_hip:.2e}, cpu err {e_cpu:.2e}"
+
+
+SHAPES = [(5,), (4, 7), (3, 4, 5), (2, 3, 4, 5), (64, 1000), (1000, 64), (1024, 1024), (16, 4, 128, 128),
+          (16, 128, 128), (4097, 3), (3, 4099), (2048, 65), (70000, 2), (2, 300000)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_sum_mean_max_every_axis(shape):
+    require_gpu()
+    x = f32(*shape)
+    x64 = x.astype(np.float64)
+    b = dev(x)
+    check_sum_like(b.sum().numpy(), x64.sum(), cref.reduce("sum", x), f"sum all {shape}")
+    check_sum_like(b.mean().numpy(), x64.mean(), cref.reduce("mean", x), f"mean all {shape}")
+    check(b.max().numpy(), cref.reduce("max", x), 0, f"max all {shape}")
+    for d in range(len(shape)):
+        for keep in (False, True):
+            want_shape = tuple(1 if i == d else s for i, s in enumerate(shape)) if keep else \
+                tuple(s for i, s in enumerate(shape) if i != d)
+            check_sum_like(b.sum(d, keepdim=keep).numpy(), x64.sum(d).reshape(want_shape),
+                           cref.reduce("sum", x, d).reshape(want_shape), f"sum {shape} axis {d}")
+        check_sum_like(b.mean(d).numpy(), x64.mean(d), cref.reduce("mean", x, d), f"mean {shape} axis {d}")
+        check(b.max(d).numpy(), cref.reduce("max", x, d), 0, f"max {shape} axis {d}")
+
+
+@pytest.mark.parametrize("shape", [(4096, 4096), (16384, 8192)])
+def test_reductions_at_bench_sizes(shape):
+    require_gpu()
+    x = f32(*shape)
+    b = dev(x)
+    x64 = x.astype(np.float64)
+    check_sum_like(b.sum().numpy(), x64.sum(), cref.reduce("sum", x), "sum all")
+    check(b.max().numpy(), x.max(), 0, "max all")
+    for d in (0, 1):
+        check_sum_like(b.sum(d).numpy(), x64.sum(d), cref.reduce("sum", x, d), f"sum axis {d}")
+        check(b.max(d).numpy(), x.max(d), 0, f"max axis {d}")
+
+
+def test_max_of_minus_inf_rows_matches_reference_start_value():
+    require_gpu()
+    x = np.full((5, 130), -np.inf, np.float32)
+    x[2, 7] = 3.0
+    check(dev(x).max(1).numpy(), cref.reduce("max", x, 1), 0, "max rows -inf")
+    check(dev(x).max(0).numpy(), cref.reduce("max", x, 0), 0, "max cols -inf")
+    check(dev(x[:2]).max().numpy(), cref.reduce("max", x[:2]), 0, "max all -inf")
+
+
+@pytest.mark.parametrize("shape", [(128, 10), (10000, 10), (1, 65), (1, 50304), (7, 1000), (300, 257)])
+def test_argmax_bit_exact_with_ties(shape):
+    require_gpu()
+    x = RNG.integers(0, 5, shape).astype(np.float32)         # few distinct values: many ties
+    for d in (0, 1):
+        want = cref.argmax(x, d).reshape((1, shape[1]) if d == 0 else (shape[0], 1))
+        check(dev(x).argmax(d).numpy(), want, 0, f"argmax {shape} dim {d}")
+    y = f32(*shape)
+    check(dev(y).argmax(1).numpy(), y.argmax(1).astype(np.float32).reshape(-1, 1), 0, "argmax random")
+
+
+PERMS = [((4, 7), (1, 0)), ((64, 784), (1, 0)), ((10, 64), (1, 0)), ((128, 128), (1, 0)), ((512, 128), (1, 0)),
+         ((2, 3, 4), (0, 2, 1)), ((2, 3, 4), (2, 0, 1)), ((2, 3, 4), (1, 0, 2)), ((2, 3, 4, 5), (0, 2, 1, 3)),
+         ((2, 3, 4, 5), (0, 1, 3, 2)), ((2, 3, 4, 5), (3, 2, 1, 0)), ((2, 3, 4, 5), (1, 3, 0, 2)),
+         ((16, 128, 4, 32), (0, 2, 1, 3)), ((16, 4, 128, 32), (0, 1, 3, 2)), ((16, 4, 128, 32), (0, 2, 1, 3)),
+         ((1000, 333), (1, 0)), ((3, 1, 5), (2, 1, 0)), ((5,), (0,)), ((2, 3, 4, 6), (0, 1, 2, 3))]
+
+
+@pytest.mark.parametrize("shape,order", PERMS)
+def test_permute_bit_exact(shape, order):
+    require_gpu()
+    x = f32(*shape)
+    check(dev(x).permute(order).numpy(), cref.permute(x, order), 0, f"permute {shape} {order}")
+
+
+def test_transpose_helpers():
+    require_gpu()
+    x = f32(6, 9)
+    check(dev(x).T.numpy(), x.T, 0, "T")
+    x4 = f32(2, 3, 4, 5)
+    check(dev(x4).transpose(1, 2).numpy(), x4.transpose(0, 2, 1, 3), 0, "transpose(1,2)")
+
+
+@pytest.mark.parametrize("V,W,idx_shape", [(100, 32, (4, 16)), (65, 128, (16, 128)), (128, 128, (128,)),
+                                          (50, 7, (33,)), (1000, 768, (64,))])
+def test_embedding_gather_bit_exact_and_scatter_add(V, W, idx_shape):
+    require_gpu()
+    table = f32(V, W)
+    idx = RNG.integers(0, V, idx_shape).astype(np.float32)
+    check(dev(table).embedding(dev(idx)).numpy(), cref.embedding(table, idx), 0, "gather")
+    g = f32(*idx_shape, W)
+    got = dev(table).embedding(dev(idx), backward=True, upstream_grad=dev(g)).numpy()
+    want = cref.embedding_backward((V, W), idx, g)
+    if not hip.COMPILE_ONLY:
+        np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
+def test_embedding_scatter_with_heavy_collisions():
+    require_gpu()
+    V, W, n = 50, 64, 4096
+    idx = np.minimum(RNG.zipf(1.1, n) - 1, V - 1).astype(np.float32)    # most ids are 0..3
+    g = f32(n, W)
+    got = dev(f32(V, W)).embedding(dev(idx), backward=True, upstream_grad=dev(g)).numpy()
+    want = np.zeros((V, W))
+    np.add.at(want, idx.astype(int), g.astype(np.float64))
+    if not hip.COMPILE_ONLY:
+        np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+
+
+def test_cross_entropy_helpers_bit_exact():
+    require_gpu()
+    lsm = f32(2048, 65)
+    t = RNG.integers(0, 65, (2048, 1)).astype(np.float32)
+    check(Buffer.ce_forward(dev(lsm), dev(t)).numpy(), cref.ce_forward(lsm, t).reshape(1, -1), 0, "ce_forward")
+    p = dev(lsm)
+    Buffer.ce_backward(op=CustomOps.CE_BACKWARD, device=p.device, x=p, target=dev(t))
+    want = lsm.copy()
+    cref.ce_backward_(want, t)
+    check(p.numpy(), want, 0, "ce_backward in place")
+
+
+@pytest.mark.parametrize("shape", [(8, 10), (16, 4, 128, 128), (2048, 65), (96, 1024), (4, 50304), (5, 4099), (3, 2052)])
+def test_fused_softmax_matches_the_five_kernel_composition(shape):
+    require_gpu()
+    x = f32(*shape) * 3
+    m = cref.reduce("max", x, len(shape) - 1)[..., None]
+    e = cref.unary("exp", cref.binary("sub", x, m))
+    s = cref.reduce("sum", e, len(shape) - 1)[..., None]
+    check(dev(x).softmax(len(shape) - 1).numpy(), cref.binary("div", e, s), 2e-6, f"softmax {shape}")
+    lsm = cref.binary("sub", cref.binary("sub", x, m), cref.unary("log", s))
+    got = dev(x).log_softmax(len(shape) - 1).numpy()
+    if not hip.COMPILE_ONLY:
+        np.testing.assert_allclose(got, lsm, rtol=2e-6, atol=2e-6)
+
+
+def test_softmax_with_causal_minus_inf_mask_gives_exact_zeros():
+    require_gpu()
+    att = f32(2, 4, 128, 128)
+    mask = 1 - np.tril(np.ones((128, 128), np.float32))
+    filled = Buffer.masked_fill(dev(att), dev(mask), float("-inf"))
+    p = filled.softmax(3).numpy()
+    if not hip.COMPILE_ONLY:
+        assert np.all(p[..., np.triu_indices(128, 1)[0], np.triu_indices(128, 1)[1]] == 0)
+        np.testing.assert_allclose(p.sum(-1), 1.0, rtol=1e-5)
