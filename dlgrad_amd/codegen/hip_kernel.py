@@ -761,3 +761,201 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 }}
 """
     return src, name, _fmt("P", "P", "I", "I")
+
+
+# =====================================================================================
+# matmul
+# =====================================================================================
+
+@cache
+def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb: bool) -> tuple[str, str, str]:
+    """C[z] = A[z] . B[z], fp32, row-major, on the matrix cores (v_mfma_f32_32x32x2_f32).
+
+    Replaces the i-k-j loops of cpu_kernel.py:351-428.  Batched over blockIdx.z with two
+    batch extents (z = zb * nbc + zc) whose operand strides may be 0, which is how the
+    reference broadcasts a batch or channel dim (cpu.py:519-532, :553-559).
+
+    Tiling.  A block of WM x WN wavefronts owns a (32*MI*WM) x (32*NJ*WN) tile of C; each
+    wavefront owns MI x NJ MFMA tiles of 32x32, i.e. 16*MI*NJ accumulator registers.  The
+    K loop advances BK at a time through double-buffered LDS (one barrier per step; the
+    next A/B tiles are in flight in registers while the current ones are multiplied).
+
+    Operand layout chosen for 16-byte LDS traffic:
+      * A sits in LDS as [m][k] with a 4-float pad per row.  One 32x32x2 MFMA consumes,
+        per lane, A[m = lane%32][k = lane/32].  The k order inside a group of 8 is
+        permuted (lane half h takes k = 8*blk + 4*h + s at step s, for A and B alike), so
+        one ds_read_b128 per lane feeds four MFMA steps.
+      * the NJ column tiles of a wavefront interleave: lane c of column tile j owns
+        column NJ*c + j.  One read of NJ consecutive floats of B[k][...] then feeds NJ
+        MFMAs, and in the epilogue each lane holds NJ adjacent columns of a row: one
+        dwordx4 store for NJ = 4, a fully coalesced 512-byte row segment per half wave.
+    veca / vecb: 16-byte global loads of A (needs K % 4 == 0) and of B plus 16-byte
+    stores of C (needs N % 4 == 0); bases and batch strides are then 16-byte aligned.
+    Out-of-range rows, columns and k are read as zero and never written.
+    Blocks are renumbered so that the eight XCDs (round-robin dispatch) each work on a
+    contiguous band of C tiles, walked in groups of 8 tile rows for L2 reuse."""
+    BM, BN, T = 32 * MI * WM, 32 * NJ * WN, 64 * WM * WN
+    AKQ, BNQ = BK // 4, BN // 4
+    assert T % AKQ == 0 and T % BNQ == 0 and BK % 8 == 0
+    ROWS_A, ROWS_B = T // AKQ, T // BNQ
+    PA, PB = max(1, BM // ROWS_A), max(1, BK // ROWS_B)
+    assert BM % ROWS_A == 0 or ROWS_A > BM
+    assert BK % ROWS_B == 0 or ROWS_B > BK
+    guard_a = ROWS_A > BM      # more loader threads than A rows: extra threads idle
+    guard_b = ROWS_B > BK
+    name = f"matmul_{BM}x{BN}x{BK}_w{WM}x{WN}_{'a4' if veca else 'a1'}{'b4' if vecb else 'b1'}"
+    LDA, LDB = BK + 4, BN
+    bvec = {1: "float", 2: "float2", 4: "float4"}[NJ]
+    comp = ["x", "y", "z", "w"]
+
+    if veca:
+        load_a = """            ra[p] = (m < g.M && k < g.K) ? *reinterpret_cast<const float4*>(A + (u64)m * g.K + k)
+                                         : make_float4(0.f, 0.f, 0.f, 0.f);"""
+    else:
+        load_a = """            const float* __restrict__ s = A + (u64)m * g.K + k;
+            const bool okm = m < g.M;
+            ra[p].x = (okm && k + 0u < g.K) ? s[0] : 0.f;
+            ra[p].y = (okm && k + 1u < g.K) ? s[1] : 0.f;
+            ra[p].z = (okm && k + 2u < g.K) ? s[2] : 0.f;
+            ra[p].w = (okm && k + 3u < g.K) ? s[3] : 0.f;"""
+    if vecb:
+        load_b = """            rb[p] = (k < g.K && n < g.N) ? *reinterpret_cast<const float4*>(B + (u64)k * g.N + n)
+                                         : make_float4(0.f, 0.f, 0.f, 0.f);"""
+    else:
+        load_b = """            const float* __restrict__ s = B + (u64)k * g.N + n;
+            const bool okk = k < g.K;
+            rb[p].x = (okk && n + 0u < g.N) ? s[0] : 0.f;
+            rb[p].y = (okk && n + 1u < g.N) ? s[1] : 0.f;
+            rb[p].z = (okk && n + 2u < g.N) ? s[2] : 0.f;
+            rb[p].w = (okk && n + 3u < g.N) ? s[3] : 0.f;"""
+
+    mfma = ""
+    for s in range(4):
+        mfma += f"            {{ const {bvec} b = *reinterpret_cast<const {bvec}*>(&Bs[buf][kb + 4u * h + {s}u][wn0 + {NJ}u * r]);\n"
+        for i in range(MI):
+            for j in range(NJ):
+                bj = "b" if NJ == 1 else f"b.{comp[j]}"
+                mfma += (f"              acc[{i}][{j}] = __builtin_amdgcn_mfma_f32_32x32x2f32("
+                         f"a[{i}].{comp[s]}, {bj}, acc[{i}][{j}], 0, 0, 0);\n")
+        mfma += "            }\n"
+
+    if vecb and NJ == 4:
+        store = """                    if (col + 3u < g.N) {
+                        *reinterpret_cast<float4*>(crow + col) =
+                            make_float4(acc[i][0][e], acc[i][1][e], acc[i][2][e], acc[i][3][e]);
+                    } else {
+                        #pragma unroll
+                        for (int j = 0; j < NJ; ++j) if (col + j < g.N) crow[col + j] = acc[i][j][e];
+                    }"""
+    else:
+        store = """                    #pragma unroll
+                    for (int j = 0; j < NJ; ++j) if (col + j < g.N) crow[col + j] = acc[i][j][e];"""
+
+    src = f"""{PRELUDE}
+typedef float f16v __attribute__((ext_vector_type(16)));
+struct MMArgs {{ u32 M, N, K, nbc, sa0, sa1, sb0, sb1; }};
+#define BM {BM}u
+#define BN {BN}u
+#define BK {BK}u
+#define MI {MI}
+#define NJ {NJ}
+extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict__ A,
+        const float* __restrict__ B, float* __restrict__ C, MMArgs g) {{
+    __shared__ __attribute__((aligned(16))) float As[2][{BM}][{LDA}];
+    __shared__ __attribute__((aligned(16))) float Bs[2][{BK}][{LDB}];
+
+    // ---- which C tile: XCD-contiguous renumbering, then groups of 8 tile rows
+    const u32 tiles_m = (g.M + BM - 1u) / BM, tiles_n = (g.N + BN - 1u) / BN;
+    const u32 nblk = tiles_m * tiles_n;
+    u32 pid = blockIdx.x;
+    if ((nblk & 7u) == 0u) pid = (pid & 7u) * (nblk >> 3) + (pid >> 3);
+    const u32 width = 8u * tiles_n;
+    const u32 first_m = (pid / width) * 8u;
+    const u32 gsz = min(tiles_m - first_m, 8u);
+    const u32 tm = first_m + (pid % width) % gsz, tn = (pid % width) / gsz;
+    const u32 m0 = tm * BM, n0 = tn * BN;
+
+    const u32 zb = blockIdx.z / g.nbc, zc = blockIdx.z % g.nbc;
+    A += (u64)zb * g.sa0 + (u64)zc * g.sa1;
+    B += (u64)zb * g.sb0 + (u64)zc * g.sb1;
+    C += (u64)blockIdx.z * g.M * g.N;
+
+    const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const u32 r = lane & 31u, h = lane >> 5;
+    const u32 wm0 = (wave / {WN}u) * {32 * MI}u, wn0 = (wave % {WN}u) * {32 * NJ}u;
+    const u32 a_kq = tid % {AKQ}u, a_m = tid / {AKQ}u;
+    const u32 b_nq = tid % {BNQ}u, b_k = tid / {BNQ}u;
+
+    f16v acc[MI][NJ];
+    #pragma unroll
+    for (int i = 0; i < MI; ++i)
+        #pragma unroll
+        for (int j = 0; j < NJ; ++j)
+            #pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    float4 ra[{PA}], rb[{PB}];
+    auto load_tiles = [&](u32 k0) {{
+        #pragma unroll
+        for (u32 p = 0; p < {PA}u; ++p) {{
+            const u32 m = m0 + a_m + p * {ROWS_A}u, k = k0 + 4u * a_kq;
+{load_a}
+        }}
+        #pragma unroll
+        for (u32 p = 0; p < {PB}u; ++p) {{
+            const u32 k = k0 + b_k + p * {ROWS_B}u, n = n0 + 4u * b_nq;
+{load_b}
+        }}
+    }};
+    auto stash_tiles = [&](u32 buf) {{
+        #pragma unroll
+        for (u32 p = 0; p < {PA}u; ++p)
+            {'if (a_m < BM)' if guard_a else ''} *reinterpret_cast<float4*>(&As[buf][a_m + p * {ROWS_A}u][4u * a_kq]) = ra[p];
+        #pragma unroll
+        for (u32 p = 0; p < {PB}u; ++p)
+            {'if (b_k < BK)' if guard_b else ''} *reinterpret_cast<float4*>(&Bs[buf][b_k + p * {ROWS_B}u][4u * b_nq]) = rb[p];
+    }};
+
+    const u32 nk = (g.K + BK - 1u) / BK;
+    load_tiles(0u);
+    stash_tiles(0u);
+    __syncthreads();
+    for (u32 kt = 0; kt < nk; ++kt) {{
+        const u32 buf = kt & 1u;
+        if (kt + 1u < nk) load_tiles((kt + 1u) * BK);
+        #pragma unroll
+        for (u32 kb = 0; kb < BK; kb += 8u) {{
+            float4 a[MI];
+            #pragma unroll
+            for (int i = 0; i < MI; ++i)
+                a[i] = *reinterpret_cast<const float4*>(&As[buf][wm0 + 32u * i + r][kb + 4u * h]);
+{mfma}        }}
+        if (kt + 1u < nk) stash_tiles(buf ^ 1u);
+        __syncthreads();
+    }}
+
+    // ---- epilogue: accumulator e of tile (i, j) is C[8*(e/4) + 4*h + e%4][lane%32]
+    #pragma unroll
+    for (int i = 0; i < MI; ++i)
+        #pragma unroll
+        for (int e = 0; e < 16; ++e) {{
+            const u32 row = m0 + wm0 + 32u * i + 8u * (e >> 2) + 4u * h + (e & 3);
+            if (row < g.M) {{
+                float* __restrict__ crow = C + (u64)row * g.N;
+                const u32 col = n0 + wn0 + {NJ}u * r;
+{store}
+            }}
+        }}
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "8I")
+
+
+# name -> (WM, WN, MI, NJ, BK): block tile = (32*MI*WM) x (32*NJ*WN), 64*WM*WN threads
+MATMUL_CONFIGS = {
+    "128x128": (4, 1, 1, 4, 32),
+    "128x256": (2, 2, 2, 4, 16),
+    "64x128": (2, 1, 1, 4, 32),
+    "64x64": (2, 2, 1, 1, 16),
+    "32x32": (1, 1, 1, 1, 16),
+}

@@ -1,0 +1,50 @@
+"""Layers: compositions of Tensor ops, parameter shapes and initial distributions as in
+dlgrad/nn/__init__.py:8-41."""
+import math
+
+from dlgrad_amd.device import Device
+from dlgrad_amd.nn import optim, utils  # noqa: F401
+from dlgrad_amd.tensor import Tensor
+
+
+class Linear:
+    """y = x @ W^T + b with W (out, in) and b (1, out), both U(-1/sqrt(in), 1/sqrt(in))."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, device: Device = Device.CPU) -> None:
+        bound = 1 / math.sqrt(in_features)
+        self.weight = Tensor.uniform((out_features, in_features), low=-bound, high=bound,
+                                     requires_grad=True, device=device)
+        self.bias = Tensor.uniform((1, out_features), low=-bound, high=bound,
+                                   requires_grad=True, device=device) if bias else None
+
+    def __call__(self, x: Tensor) -> Tensor:
+        return x.linear(self.weight, self.bias)
+
+
+class Embedding:
+    """Row lookup in a (num_embeddings, embedding_dim) table initialised U[0, 1); indices
+    are fp32-encoded integers."""
+
+    def __init__(self, num_embeddings: int, embedding_dim: int, device: Device = Device.CPU) -> None:
+        self.num_embeddings, self.embedding_dim = num_embeddings, embedding_dim
+        self.weight = Tensor.uniform((num_embeddings, embedding_dim), requires_grad=True, device=device)
+
+    def __call__(self, idx: Tensor) -> Tensor:
+        return Tensor.embedding(self.weight, idx)
+
+
+class RMSNorm:
+    """x * rsqrt(mean(x^2, last, keepdim) + eps) * weight, weight (1, dim) of ones."""
+
+    def __init__(self, dim: int, eps: float = 1e-6, elementwise_affine: bool = True,
+                 device: Device = Device.CPU) -> None:
+        self.eps = eps
+        self.weight = Tensor.ones((1, dim), device=device, requires_grad=True) if elementwise_affine else None
+
+    def _norm(self, x: Tensor) -> Tensor:
+        ms = (x ** 2).mean(x.ndim - 1, keepdim=True)
+        return x * (ms + self.eps).rsqrt()
+
+    def __call__(self, x: Tensor) -> Tensor:
+        y = self._norm(x)
+        return y if self.weight is None else y * self.weight

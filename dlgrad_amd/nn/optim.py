@@ -1,0 +1,58 @@
+"""Optimizers as Tensor expressions (dlgrad/nn/optim.py:4-70): every update is a handful
+of element-wise kernels per parameter and rebinds `param.data` to the new buffer."""
+from dlgrad_amd.tensor import Tensor
+
+
+class Optimizer:
+    def __init__(self, params: list[Tensor], lr: float = 1e-1) -> None:
+        self.params = params
+        self.lr = lr
+
+    def step(self) -> None:
+        for p in self.params:
+            assert p.shape == p.grad.shape, f"The shape of the parameter {p.shape} and its grad {p.grad.shape} do not match"
+            p.data = (p - p.grad * self.lr).data
+
+    def zero_grad(self) -> None:
+        for p in self.params:
+            p.grad = None
+
+
+class SGD(Optimizer):
+    def __init__(self, params: list[Tensor], lr: float = 1e-3, momentum: float = 0.0) -> None:
+        super().__init__(params, lr)
+        self.momentum = momentum
+        self.velocities = {id(p): Tensor.zeros_like(p) for p in params} if momentum else {}
+
+    def step(self) -> None:
+        for p in self.params:
+            if p.grad is None:
+                continue
+            assert p.shape == p.grad.shape, f"The shape of the parameter {p.shape} and its grad {p.grad.shape} do not match"
+            upd = p.grad
+            if self.momentum != 0:
+                upd = self.velocities[id(p)] * self.momentum + p.grad          # v = mu * v + g
+                self.velocities[id(p)] = upd
+            p.data = (p - upd * self.lr).data
+
+
+class Adam(Optimizer):
+    """m = b1 m + (1-b1) g;  v = b2 v + (1-b2) g^2;  p -= lr * m_hat / (sqrt(v_hat) + eps)."""
+
+    def __init__(self, params: list[Tensor], lr: float = 1e-3, betas: tuple[float, float] = (0.9, 0.999),
+                 eps: float = 1e-8) -> None:
+        self.params, self.lr, self.eps = params, lr, eps
+        self.beta1, self.beta2 = betas
+        self.m = {id(p): Tensor.zeros_like(p) for p in params}
+        self.v = {id(p): Tensor.zeros_like(p) for p in params}
+        self.t = 0
+
+    def step(self) -> None:
+        self.t += 1
+        c1, c2 = 1.0 - self.beta1 ** self.t, 1.0 - self.beta2 ** self.t
+        for p in self.params:
+            k, g = id(p), p.grad
+            self.m[k] = ((self.m[k] * self.beta1) + (g * (1.0 - self.beta1))).detach()
+            self.v[k] = ((self.v[k] * self.beta2) + ((g ** 2.0) * (1.0 - self.beta2))).detach()
+            m_hat, v_hat = self.m[k] / c1, self.v[k] / c2
+            p.data = (p - (m_hat / (v_hat.sqrt() + self.eps)) * self.lr).data

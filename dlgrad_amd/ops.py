@@ -1,0 +1,408 @@
+"""Autograd nodes: forward and backward of every Tensor op, written on Buffers.
+
+The formulas, and therefore the sequence of kernels a backward pass issues, are the
+ones of dlgrad/ops.py:8-462.  Two things differ on purpose:
+  * where the reference reshapes a gradient by mutating Buffer metadata in place
+    (`upstream_grad.unsqueeze(dim)`, ops.py:70, :90, :105-110), a reshaped *view* is
+    used, so a gradient shared by two consumers is never seen with the wrong shape;
+  * `Softmax` is a node of its own when the fused row kernel applies, with the
+    closed-form backward y * (g - sum(g * y)).
+"""
+from __future__ import annotations
+
+import os
+
+from dlgrad_amd.buffer import Buffer
+from dlgrad_amd.device import Device
+from dlgrad_amd.dtype import Scalar
+from dlgrad_amd.helpers import CustomOps, broadcast_shapes, check_broadcast
+from dlgrad_amd.tensor import OP
+
+# Fused row kernels (softmax, log-softmax inside cross-entropy) on the hip device.
+# Off = the reference's op-by-op compositions, kept as the parity bridge.
+FUSED = os.environ.get("DLGRAD_HIP_FUSED", "1") != "0"
+
+
+def use_fused(t, dim: int) -> bool:
+    """dim must name the last axis explicitly: -1 means "all elements" to the reference's
+    reductions (helpers.py:204-206), so softmax(dim=-1) is a global softmax there."""
+    return FUSED and t.device is Device.HIP and t.ndim >= 1 and dim == t.ndim - 1
+
+
+def _expand_at(g: Buffer, dim: int, keepdim: bool) -> Buffer:
+    """View of a reduced gradient with the reduced dim back as extent 1
+    (dim == -1, "all elements", becomes a leading 1 as Buffer.unsqueeze does)."""
+    if keepdim:
+        return g
+    d = 0 if dim == -1 else dim
+    shape = list(g.shape)
+    shape.insert(d, 1)
+    if g.is_host_scalar:
+        return g
+    return g.reshape(tuple(shape))
+
+
+# ------------------------------------------------------------------ unary
+class Pow(OP):
+    def forward(self, x: Buffer, y: float) -> Buffer:
+        self.x, self.y = x, y
+        return x ** y
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return (upstream_grad * ((self.x ** (self.y - 1.0)) * self.y),)      # g * p * x^(p-1)
+
+
+class Reshape(OP):
+    def forward(self, x: Buffer, shape: tuple) -> Buffer:
+        self.input_shape = x.shape
+        return x.reshape(shape)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return (upstream_grad.reshape(self.input_shape),)
+
+
+class Permute(OP):
+    def forward(self, x: Buffer, order: tuple) -> Buffer:
+        self.order = order
+        return x.permute(order)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        inverse = [0] * len(self.order)
+        for i, p in enumerate(self.order):
+            inverse[p] = i
+        return (upstream_grad.permute(tuple(inverse)),)
+
+
+class Transpose(OP):
+    def forward(self, x: Buffer, dim0: int, dim1: int) -> Buffer:
+        self.dims = (dim0, dim1)
+        return x.transpose(dim0, dim1)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return (upstream_grad.transpose(self.dims[1], self.dims[0]),)
+
+
+class _Reduction(OP):
+    def _remember(self, x: Buffer, dim: int, keepdim: bool) -> None:
+        self.inp_shape, self.device, self.dtype = x.shape, x.device, x.dtype
+        self.dim, self.keepdim = dim, keepdim
+
+
+class Sum(_Reduction):
+    def forward(self, x: Buffer, dim: int = -1, keepdim: bool = False) -> Buffer:
+        self._remember(x, dim, keepdim)
+        return x.sum(dim=dim, keepdim=keepdim)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        ones = Buffer.full(shape=self.inp_shape, fill_value=1.0, device=self.device, dtype=self.dtype)
+        return (ones * _expand_at(upstream_grad, self.dim, self.keepdim),)
+
+
+class Mean(_Reduction):
+    def forward(self, x: Buffer, dim: int = -1, keepdim: bool = False) -> Buffer:
+        self._remember(x, dim, keepdim)
+        self.N = x.numel if dim == -1 else x.shape[dim]
+        return x.mean(dim=dim, keepdim=keepdim)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        # ops.py:86-91.  Buffer.full hands the fill value to the runtime, which truncates
+        # it to int when reference-strict (cpu.py:252): 1/N becomes 0 there.
+        scale = Buffer.full(self.inp_shape, fill_value=1.0 / self.N, device=self.device, dtype=self.dtype)
+        return (scale * _expand_at(upstream_grad, self.dim, self.keepdim),)
+
+
+class Max(_Reduction):
+    def forward(self, x: Buffer, dim: int = -1, keepdim: bool = False) -> Buffer:
+        self._remember(x, dim, keepdim)
+        self.x = x
+        self.out = x.max(dim=dim, keepdim=keepdim)
+        return self.out
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        hit = self.x == _expand_at(self.out, self.dim, self.keepdim)           # 1.0 where x attains the max
+        return (hit * _expand_at(upstream_grad, self.dim, self.keepdim),)
+
+
+class Tril(OP):
+    def forward(self, x: Buffer, k: Buffer) -> Buffer:
+        H, W = x.shape[0], x.shape[1]                                          # 2-D only (ops.py:116-117)
+        rows = Buffer.arange((H, 1), x.device)
+        cols = Buffer.arange((1, W), x.device)
+        self.mask = cols <= (rows + k)
+        return self.mask.where(x, 0.0)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return (self.mask.where(upstream_grad, 0.0),)
+
+
+class Exp(OP):
+    def forward(self, x: Buffer) -> Buffer:
+        self.out = x.exp()
+        return self.out
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return (upstream_grad * self.out,)
+
+
+class Log(OP):
+    def forward(self, x: Buffer) -> Buffer:
+        self.x = x
+        return x.log()
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return (upstream_grad / self.x,)
+
+
+class Relu(OP):
+    def forward(self, x: Buffer) -> Buffer:
+        self.out = x.relu()
+        return self.out
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return (self.out.where(inp=1.0, other=0.0) * upstream_grad,)
+
+
+class LeakyRelu(OP):
+    def forward(self, x: Buffer, neg_slope: Scalar = 0.01) -> Buffer:
+        self.neg_slope = neg_slope
+        self.out = x.leaky_relu(neg_slope=neg_slope)
+        return self.out
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return (self.out.where(inp=1.0, other=self.neg_slope) * upstream_grad,)
+
+
+class Sigmoid(OP):
+    def forward(self, x: Buffer) -> Buffer:
+        self.out = x.sigmoid()
+        return self.out
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return ((self.out * -(self.out - 1.0)) * upstream_grad,)
+
+
+class Tanh(OP):
+    def forward(self, x: Buffer) -> Buffer:
+        self.out = x.tanh()
+        return self.out
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        ones = Buffer.full(self.out.shape, 1.0, self.out.device, self.out.dtype)
+        return ((ones - self.out ** 2) * upstream_grad,)
+
+
+class Sqrt(OP):
+    def forward(self, x: Buffer) -> Buffer:
+        self.out = x.sqrt()
+        return self.out
+
+    def backward(self, grad_output: Buffer) -> tuple:
+        return (grad_output / (self.out * 2),)
+
+
+class RSqrt(OP):
+    def forward(self, x: Buffer) -> Buffer:
+        self.out = x.rsqrt()
+        return self.out
+
+    def backward(self, grad_output: Buffer) -> tuple:
+        return (grad_output * (self.out ** 3 * -0.5),)
+
+
+class Clamp(OP):
+    def forward(self, x: Buffer, min: int | None, max: int | None) -> Buffer:
+        self.min, self.max = min, max
+        return x.clamp(min, max)
+
+    def backward(self, grad_output: Buffer) -> tuple:
+        return (grad_output.clamp(self.min, self.max),)                        # as ops.py:204-205
+
+
+class Squeeze(OP):
+    def forward(self, x: Buffer, dim: list[int] | int) -> Buffer:
+        self.dim = dim
+        x.squeeze(dim)
+        return x
+
+    def backward(self, grad_output: Buffer) -> tuple:
+        grad_output.unsqueeze(self.dim)
+        return (grad_output,)
+
+
+class Unsqueeze(OP):
+    def forward(self, x: Buffer, dim: list[int] | int) -> Buffer:
+        self.dim = dim
+        x.unsqueeze(dim)
+        return x
+
+    def backward(self, grad_output: Buffer) -> tuple:
+        grad_output.squeeze(self.dim)
+        return (grad_output,)
+
+
+# ------------------------------------------------------------------ binary
+class _Binary(OP):
+    def _keep(self, x: Buffer, y: Buffer) -> None:
+        check_broadcast(x.shape, y.shape)
+        self.x, self.y = x, y
+
+    def _to(self, g: Buffer, which: int) -> Buffer | None:
+        if not self.req_grad[which]:
+            return None
+        return self.reduce_grad_for_broadcasting(g() if callable(g) else g, (self.x, self.y)[which].shape)
+
+
+class Add(_Binary):
+    def forward(self, x: Buffer, y: Buffer) -> Buffer:
+        self._keep(x, y)
+        return x + y
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return self._to(upstream_grad, 0), self._to(upstream_grad, 1)
+
+
+class Sub(_Binary):
+    def forward(self, x: Buffer, y: Buffer) -> Buffer:
+        self._keep(x, y)
+        return x - y
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return self._to(upstream_grad, 0), self._to(lambda: -upstream_grad, 1)
+
+
+class Mul(_Binary):
+    def forward(self, x: Buffer, y: Buffer) -> Buffer:
+        self._keep(x, y)
+        return x * y
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return self._to(lambda: upstream_grad * self.y, 0), self._to(lambda: upstream_grad * self.x, 1)
+
+
+class Div(_Binary):
+    def forward(self, x: Buffer, y: Buffer) -> Buffer:
+        self._keep(x, y)
+        return x / y
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return (self._to(lambda: upstream_grad / self.y, 0),
+                self._to(lambda: (-upstream_grad * self.x) / self.y ** 2, 1))
+
+
+def unbroadcast(grad: Buffer, original_shape: tuple) -> Buffer:
+    """Sum a matmul gradient back to an operand that was batch-broadcast (ops.py:287-295)."""
+    while grad.ndim > len(original_shape):
+        grad = grad.sum(0, keepdim=False)
+    for i, (g, o) in enumerate(zip(grad.shape, original_shape)):
+        if o == 1 and g > 1:
+            grad = grad.sum(i, keepdim=True)
+    return grad
+
+
+class MatMul(OP):
+    def forward(self, x: Buffer, y: Buffer) -> Buffer:
+        self.p1, self.p2, self.out_shape = broadcast_shapes(x.shape, y.shape)
+        self.x, self.y = x, y
+        return x @ y
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        """dX = G . Y^T and dY = X^T . G with materialised transposes, then the batch
+        broadcast is summed away (ops.py:308-335)."""
+        if upstream_grad.shape != self.out_shape:
+            upstream_grad = upstream_grad.reshape(self.out_shape)
+        xr, yr = self.x.reshape(self.p1), self.y.reshape(self.p2)
+        nd = xr.ndim
+        grad_x = upstream_grad @ yr.transpose(nd - 2, nd - 1)
+        grad_y = xr.transpose(nd - 2, nd - 1) @ upstream_grad
+        return unbroadcast(grad_x, self.x.shape), unbroadcast(grad_y, self.y.shape)
+
+
+class Softmax(OP):
+    """Fused forward along the last axis; backward dx = y * (g - sum(g * y, last))."""
+
+    def forward(self, x: Buffer, dim: int) -> Buffer:
+        self.out = x.softmax(x.ndim - 1)
+        return self.out
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        gy = upstream_grad * self.out
+        return (gy - self.out * gy.sum(dim=self.out.ndim - 1, keepdim=True),)
+
+
+class CrossEntropy(OP):
+    def forward(self, logits: Buffer, target: Buffer, dim: int = 1) -> Buffer:
+        """log-softmax, gather of the target log-probs, and -SUM over rows -- not the mean
+        (ops.py:338-357); backward nevertheless scales by 1/N (ops.py:359-370)."""
+        assert logits.shape[0] == target.shape[0]
+        self.target = target
+        if FUSED and logits.device is Device.HIP and dim == logits.ndim - 1:
+            self.log_softmax = logits.log_softmax(dim)
+        else:
+            shifted = logits - logits.max(dim=dim, keepdim=True)
+            self.log_softmax = shifted - shifted.exp().sum(dim=dim, keepdim=True).log()
+        picked = Buffer.ce_forward(self.log_softmax, self.target)
+        self.N = float(logits.shape[0])
+        return -picked.sum()
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        probs = self.log_softmax.exp()
+        Buffer.ce_backward(op=CustomOps.CE_BACKWARD, device=probs.device, x=probs, target=self.target)   # p - onehot
+        return ((probs * upstream_grad) / self.N,)
+
+
+class BCEWithLogitsLoss(OP):
+    def forward(self, probs: Buffer, target: Buffer) -> Buffer:
+        assert probs.shape == target.shape, f"shape mismatch {probs.shape} vs {target.shape}"
+        self.probs, self.target = probs, target
+        m = (-probs).clamp(min=0)
+        loss = ((1.0 - target) * probs) + m + ((-m).exp() + (-(probs + m)).exp()).log()
+        return loss.mean()
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return (((self.probs.sigmoid() - self.target) * upstream_grad) / float(self.probs.numel),)
+
+
+class Embedding(OP):
+    def forward(self, weight: Buffer, idx: Buffer) -> Buffer:
+        self.weight, self.idx = weight, idx
+        return weight.embedding(idx)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return (self.weight.embedding(self.idx, backward=True, upstream_grad=upstream_grad),)
+
+
+class Where(OP):
+    def forward(self, cond: Buffer, inp: Buffer, other: Buffer) -> Buffer:
+        self.cond = cond
+        return cond.where(inp, other)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return None, self.cond.where(upstream_grad, 0.0), self.cond.where(0.0, upstream_grad)
+
+
+class MaskedFill(OP):
+    def forward(self, data: Buffer, mask: Buffer, value: Scalar) -> Buffer:
+        self.mask = mask
+        return Buffer.masked_fill(x=data, mask=mask, val=value)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return Buffer.masked_fill(x=upstream_grad, mask=self.mask, val=0.0), None, None
+
+
+class Dropout(OP):
+    def forward(self, x: Buffer, p: Scalar) -> Buffer:
+        self.p = p
+        if p == 1.0:
+            return Buffer.full(x.shape, 0.0, x.device, x.dtype)
+        if p == 0.0:
+            return x
+        self.mask = Buffer.uniform(x.shape, x.device, x.dtype, low=0.0, high=1.0) >= p
+        self.scale = 1.0 / (1.0 - p)
+        return self.mask.where(x, 0.0) * self.scale
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        if self.p == 1.0:
+            return (Buffer.full(upstream_grad.shape, 0.0, upstream_grad.device, upstream_grad.dtype),)
+        if self.p == 0.0:
+            return (upstream_grad,)
+        return (self.mask.where(upstream_grad, 0.0) * self.scale,)

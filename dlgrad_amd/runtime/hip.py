@@ -627,3 +627,56 @@ class HIP:
     @dispatcher.register(CustomOps.LOG_SOFTMAX, Device.HIP)
     def log_softmax(x: Buffer, dim: int) -> DevicePtr:
         return HIP._softmax(x, dim, True)
+
+    # ---- matmul ----------------------------------------------------------------------------------------------------------
+    MATMUL_FORCE = os.environ.get("DLGRAD_HIP_MATMUL_TILE")      # e.g. "128x128": benchmarking aid
+
+    @staticmethod
+    def _pick_tile(M: int, N: int, batch: int) -> str:
+        if HIP.MATMUL_FORCE:
+            return HIP.MATMUL_FORCE
+        for name in ("128x256", "128x128", "64x128", "64x64"):
+            bm, bn = (int(v) for v in name.split("x"))
+            if ((M + bm - 1) // bm) * ((N + bn - 1) // bn) * batch >= 512:
+                return name
+        return "64x64" if (M > 32 and N > 32) else "32x32"
+
+    @staticmethod
+    @dispatcher.register(BinaryOps.MATMUL, Device.HIP)
+    def matmul(x: Buffer, y: Buffer) -> DevicePtr:
+        """x (.., M, K) @ y (.., K, N) for operands already padded to the same rank 2..4
+        (buffer.py:231-243); batch dims of extent 1 broadcast through a zero stride as in
+        cpu.py:519-532 and :553-559.  When y carries no batch at all the batch of x is
+        folded into M: one tall GEMM instead of many small ones."""
+        assert x.ndim == y.ndim and 2 <= x.ndim <= 4
+        M, Kd, N = x.shape[-2], x.shape[-1], y.shape[-1]
+        assert y.shape[-2] == Kd
+        xb = (1,) * (4 - x.ndim) + tuple(x.shape[:-2])
+        yb = (1,) * (4 - y.ndim) + tuple(y.shape[:-2])
+        B0, B1 = max(xb[0], yb[0]), max(xb[1], yb[1])
+        out = alloc(B0 * B1 * M * N)
+        if B0 * B1 * M * N == 0:
+            return out
+        if Kd == 0:
+            lib().fill_f32(out.addr, 0.0, B0 * B1 * M * N)
+            return out
+        if yb == (1, 1):
+            M, nbc, batch = xb[0] * xb[1] * M, 1, 1
+            sa = sb = (0, 0)
+        else:
+            nbc, batch = B1, B0 * B1
+            sa = (xb[1] * M * Kd if xb[0] > 1 else 0, M * Kd if xb[1] > 1 else 0)
+            sb = (yb[1] * Kd * N if yb[0] > 1 else 0, Kd * N if yb[1] > 1 else 0)
+        if batch > 65535:
+            raise ValueError(f"{batch} batches exceed the grid limit")
+        if max(M * Kd, Kd * N, M * N) >= 2 ** 31:
+            raise ValueError("matrix too large for 32-bit indexing")
+        veca = Kd % 4 == 0 and _addr(x) % 16 == 0
+        vecb = N % 4 == 0 and _addr(y) % 16 == 0 and out.addr % 16 == 0
+        tile = HIP._pick_tile(M, N, batch)
+        bm, bn = (int(v) for v in tile.split("x"))
+        k = kernel(K.matmul_kernel, *K.MATMUL_CONFIGS[tile], veca, vecb)
+        wm, wn = K.MATMUL_CONFIGS[tile][:2]
+        grid = (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch)
+        launch(k, grid, 64 * wm * wn, _addr(x), _addr(y), out.addr, M, N, Kd, nbc, *sa, *sb)
+        return out
