@@ -1,0 +1,384 @@
+#!/usr/bin/env python3
+"""Benchmark of the hip kernel backend on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|matmul|gpt|mlp] [--no-extra]
+
+Prints ONE JSON line.  A "step" is one pass of the workload over one batch of synthetic,
+seeded input that is already resident in HBM when the timed region starts.
+
+  c2      (default)  element-wise / broadcast / reduce suite on fp32 N(0,1) tensors of
+                     16384 x 8192: add sub mul div with a same-shape, (R,1), (1,C) and scalar
+                     right operand; exp, relu on N(0,1); log, sqrt on |x|+1e-3; sum and max
+                     over axis 0, axis 1 and everything.  value = algorithmic GB/s of the suite.
+  matmul             4096^3 fp32 GEMM, entries N(0, 1/sqrt(K)).  value = TFLOP/s.
+  gpt                char-GPT (vocab 65, block 128, 6 layers, 4 heads, n_embd 128, batch 16):
+                     forward + backward + Adam step.  value = tokens/s.
+  mlp                784-64-10 MLP, batch 128: forward + backward + SGD step.  value = samples/s.
+
+Unless --no-extra is given, the default run also reports the matmul sweep, the GPT step and
+the 4096^2 / 1024^2 suites under "extra", so one run carries every headline figure.
+
+`roofline` describes the dominant kernel of the workload (same-shape add for c2, the GEMM for
+matmul/gpt): algorithmic bytes or flops per launch divided by the average launch duration,
+measured with HIP events on the stream the kernels run on, inside the timed region.
+`cpu_baseline` is the single-threaded C restatement of the reference's CPU kernels (oracle/),
+timed on this machine's host cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_FP32_PEAK_TFLOPS = 157.3  # dense fp32 MFMA
+
+
+def _imports():
+    from dlgrad_amd import Tensor, nn
+    from dlgrad_amd.buffer import Buffer
+    from dlgrad_amd.device import Device
+    from dlgrad_amd.runtime import hip
+    return Tensor, nn, Buffer, Device, hip
+
+
+class EventTimer:
+    """Per-name accumulation of kernel time from HIP events on the library's stream."""
+
+    def __init__(self, lib) -> None:
+        self.lib, self.pending, self.pool = lib, [], []
+
+    def _ev(self) -> int:
+        return self.pool.pop() if self.pool else self.lib.event_create()
+
+    def run(self, name: str, fn):
+        e0, e1 = self._ev(), self._ev()
+        self.lib.event_record(e0)
+        out = fn()
+        self.lib.event_record(e1)
+        self.pending.append((name, e0, e1))
+        return out
+
+    def collect(self) -> dict:
+        """name -> list of ms; call after a sync."""
+        res: dict = {}
+        for name, e0, e1 in self.pending:
+            res.setdefault(name, []).append(self.lib.event_elapsed_ms(e0, e1))
+            self.pool += [e0, e1]
+        self.pending = []
+        return res
+
+
+# ---------------------------------------------------------------------------------------------
+# c2: element-wise / broadcast / reduce suite
+# ---------------------------------------------------------------------------------------------
+def c2_ops(R: int, C: int):
+    """(name, callable on a dict of operands, algorithmic bytes) for every op of the suite.
+    Bytes per element: 12 same-shape binary, 8 binary with a broadcast/scalar operand
+    (+ the small operand), 8 unary, 4 per element read + 4 per output for reductions."""
+    n = R * C
+    ops = []
+    for name, f in (("add", lambda a, b: a + b), ("sub", lambda a, b: a - b),
+                    ("mul", lambda a, b: a * b), ("div", lambda a, b: a / b)):
+        ops.append((f"{name}_same", (lambda d, f=f: f(d["a"], d["b"])), 12 * n))
+        ops.append((f"{name}_rowvec", (lambda d, f=f: f(d["a"], d["col"])), 8 * n + 4 * R))   # (R,1)
+        ops.append((f"{name}_colvec", (lambda d, f=f: f(d["a"], d["row"])), 8 * n + 4 * C))   # (1,C)
+        ops.append((f"{name}_scalar", (lambda d, f=f: f(d["a"], 1.5)), 8 * n))
+    ops.append(("exp", lambda d: d["a"].exp(), 8 * n))
+    ops.append(("relu", lambda d: d["a"].relu(), 8 * n))
+    ops.append(("log", lambda d: d["pos"].log(), 8 * n))
+    ops.append(("sqrt", lambda d: d["pos"].sqrt(), 8 * n))
+    for red in ("sum", "max"):
+        ops.append((f"{red}_axis0", (lambda d, r=red: getattr(d["a"], r)(0)), 4 * n + 4 * C))
+        ops.append((f"{red}_axis1", (lambda d, r=red: getattr(d["a"], r)(1)), 4 * n + 4 * R))
+        ops.append((f"{red}_all", (lambda d, r=red: getattr(d["a"], r)()), 4 * n + 4))
+    return ops
+
+
+def c2_inputs(R: int, C: int, seed: int = 2):
+    rng = np.random.default_rng(seed)
+    a = rng.standard_normal((R, C), dtype=np.float32)
+    b = rng.standard_normal((R, C), dtype=np.float32)
+    return {"a": a, "b": b, "pos": np.abs(a) + np.float32(1e-3),
+            "col": rng.standard_normal((R, 1), dtype=np.float32) + np.float32(3),
+            "row": rng.standard_normal((1, C), dtype=np.float32) + np.float32(3)}
+
+
+def run_c2(R: int, C: int, steps: int, warmup: int) -> dict:
+    _, _, Buffer, Device, hip = _imports()
+    lib = hip.lib()
+    host = c2_inputs(R, C)
+    d = {k: Buffer.from_numpy(v, Device.HIP) for k, v in host.items()}
+    del host
+    ops = c2_ops(R, C)
+    timer = EventTimer(lib)
+    for _ in range(warmup):
+        for _, f, _ in ops:
+            f(d)
+    lib.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        for name, f, _ in ops:
+            timer.run(name, lambda f=f: f(d))
+    lib.sync()
+    wall = time.perf_counter() - t0
+    per = timer.collect()
+    total_bytes = sum(b for _, _, b in ops)
+    per_op = {name: {"ms": float(np.mean(per[name])), "GBps": b / np.mean(per[name]) / 1e6,
+                     "frac_hbm": b / np.mean(per[name]) / 1e6 / HBM_PEAK_GBS}
+              for name, _, b in ops}
+    return {"ms_per_step": wall / steps * 1e3, "GBps": total_bytes * steps / wall / 1e9,
+            "bytes_per_step": total_bytes, "per_op": per_op, "n_ops": len(ops)}
+
+
+def cpu_c2(R: int, C: int, reps: int = 2) -> dict:
+    """The same suite on the C restatement of the reference's kernels, one thread."""
+    from oracle import cref
+    host = c2_inputs(R, C)
+    n = R * C
+    work = []
+    for op in ("add", "sub", "mul", "div"):
+        work += [(lambda op=op: cref.binary(op, host["a"], host["b"]), 12 * n),
+                 (lambda op=op: cref.binary(op, host["a"], host["col"]), 8 * n + 4 * R),
+                 (lambda op=op: cref.binary(op, host["a"], host["row"]), 8 * n + 4 * C),
+                 (lambda op=op: cref.binary(op, host["a"], np.float32(1.5)), 8 * n)]
+    work += [(lambda: cref.unary("exp", host["a"]), 8 * n),
+             (lambda: cref.where(host["a"], host["a"], np.float32(0)), 8 * n),
+             (lambda: cref.unary("log", host["pos"]), 8 * n), (lambda: cref.unary("sqrt", host["pos"]), 8 * n)]
+    for red in ("sum", "max"):
+        work += [(lambda r=red: cref.reduce(r, host["a"], 0), 4 * n + 4 * C),
+                 (lambda r=red: cref.reduce(r, host["a"], 1), 4 * n + 4 * R),
+                 (lambda r=red: cref.reduce(r, host["a"]), 4 * n + 4)]
+    best = float("inf")
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        for f, _ in work:
+            f()
+        best = min(best, time.perf_counter() - t0)
+    return {"value": sum(b for _, b in work) / best / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"the same {len(work)}-op suite at {R}x{C}, single thread, min of {reps} passes "
+                      f"({best:.2f} s per pass); host has {os.cpu_count()} logical cores"}
+
+
+# ---------------------------------------------------------------------------------------------
+# matmul
+# ---------------------------------------------------------------------------------------------
+def run_matmul(M: int, N: int, K: int, steps: int, warmup: int, seed: int = 3) -> dict:
+    _, _, Buffer, Device, hip = _imports()
+    lib = hip.lib()
+    rng = np.random.default_rng(seed)
+    a = Buffer.from_numpy(rng.standard_normal((M, K), dtype=np.float32) * np.float32(K ** -0.5), Device.HIP)
+    b = Buffer.from_numpy(rng.standard_normal((K, N), dtype=np.float32) * np.float32(K ** -0.5), Device.HIP)
+    for _ in range(warmup):
+        a @ b
+    lib.sync()
+    timer = EventTimer(lib)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        timer.run("matmul", lambda: a @ b)
+    lib.sync()
+    wall = time.perf_counter() - t0
+    ms = float(np.mean(timer.collect()["matmul"]))
+    flops = 2.0 * M * N * K
+    return {"ms_per_step": wall / steps * 1e3, "kernel_ms": ms, "TFLOPs": flops / ms / 1e9,
+            "TFLOPs_wall": flops * steps / wall / 1e12, "flops": flops,
+            "bytes": 4.0 * (M * K + K * N + M * N)}
+
+
+def cpu_matmul(n: int = 512) -> dict:
+    from oracle import cref
+    rng = np.random.default_rng(3)
+    a = rng.standard_normal((n, n), dtype=np.float32)
+    b = rng.standard_normal((n, n), dtype=np.float32)
+    best = float("inf")
+    for _ in range(3):
+        t0 = time.perf_counter()
+        cref.matmul(a, b)
+        best = min(best, time.perf_counter() - t0)
+    return {"value": 2.0 * n ** 3 / best / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"{n}^3 fp32 matmul_2d (i-k-j loops), single thread, min of 3 ({best * 1e3:.1f} ms); "
+                      f"host has {os.cpu_count()} logical cores"}
+
+
+# ---------------------------------------------------------------------------------------------
+# GPT / MLP steps
+# ---------------------------------------------------------------------------------------------
+GPT_C4 = dict(vocab_size=65, block_size=128, n_layer=6, n_head=4, n_embd=128, batch_size=16)
+
+
+def make_gpt(device: str, cfg: dict, seed: int = 0):
+    Tensor, nn, *_ = _imports()
+    from examples import gpt as G
+    c = G.GPTConfig(device=device, **cfg)
+    model = G.GPT(c)
+    G.init_weights_(model, seed)
+    rng = np.random.default_rng(seed + 1)
+    idx = Tensor(rng.integers(0, c.vocab_size, (c.batch_size, c.block_size)).astype(np.float32), device=device)
+    tgt = Tensor(rng.integers(0, c.vocab_size, (c.batch_size, c.block_size)).astype(np.float32), device=device)
+    params = nn.utils.get_parameters(model)
+    opt = nn.optim.Adam(params, lr=c.learning_rate)
+
+    def step():
+        opt.zero_grad()
+        _, loss = model(idx, tgt)
+        loss.backward()
+        opt.step()
+        return loss
+    return model, step
+
+
+def run_gpt(steps: int, warmup: int, cfg: dict = GPT_C4) -> dict:
+    *_, hip = _imports()
+    lib = hip.lib()
+    _, step = make_gpt("hip", cfg)
+    for _ in range(warmup):
+        step()
+    lib.sync()
+    n0 = hip.launch_count
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = step()
+    lib.sync()
+    wall = time.perf_counter() - t0
+    tokens = cfg["batch_size"] * cfg["block_size"]
+    return {"ms_per_step": wall / steps * 1e3, "tokens_per_s": tokens * steps / wall,
+            "launches_per_step": (hip.launch_count - n0) / steps, "loss_sum": float(loss.numpy()),
+            "loss_per_token": float(loss.numpy()) / tokens}
+
+
+def cpu_gpt(cfg: dict = GPT_C4) -> dict:
+    import oracle.cpu_runtime  # noqa: F401
+    _, step = make_gpt("cpu", cfg)
+    t0 = time.perf_counter()
+    step()
+    dt = time.perf_counter() - t0
+    tokens = cfg["batch_size"] * cfg["block_size"]
+    return {"value": tokens / dt, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"one full char-GPT step (fwd+bwd+Adam, {tokens} tokens) on the C restatement, "
+                      f"single thread ({dt:.2f} s); host has {os.cpu_count()} logical cores"}
+
+
+def run_mlp(steps: int, warmup: int) -> dict:
+    Tensor, nn, _, _, hip = _imports()
+    from examples import mlp as M
+    lib = hip.lib()
+    model = M.MLP(device="hip")
+    M.init_weights_(model, 0)
+    x, y = M.synthetic_batch(1)
+    xt, yt = Tensor(x, device="hip"), Tensor(y, device="hip")
+    params = [model.fc1.weight, model.fc1.bias, model.fc2.weight, model.fc2.bias]
+    opt = nn.optim.SGD(params, lr=1e-3)
+
+    def step():
+        opt.zero_grad()
+        loss = model(xt).cross_entropy_loss(yt)
+        loss.backward()
+        opt.step()
+    for _ in range(warmup):
+        step()
+    lib.sync()
+    n0 = hip.launch_count
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    lib.sync()
+    wall = time.perf_counter() - t0
+    return {"ms_per_step": wall / steps * 1e3, "samples_per_s": 128 * steps / wall,
+            "launches_per_step": (hip.launch_count - n0) / steps}
+
+
+# ---------------------------------------------------------------------------------------------
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c2", choices=["c2", "matmul", "gpt", "mlp"])
+    ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this backend runs on one GPU; --gpus must be 1 (nothing here uses a second device)")
+    *_, hip = _imports()
+    props = hip.props()
+    base = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic"}
+    device = {"name": props["name"], "arch": props["arch"], "compute_units": props["compute_units"],
+              "clock_mhz": props["clock_khz"] / 1000}
+
+    if args.workload == "c2":
+        R, C = 16384, 8192
+        r = run_c2(R, C, args.steps, args.warmup)
+        add = r["per_op"]["add_same"]
+        out = {"metric": "elementwise/reduce HBM GB/s (1 GPU)", "value": r["GBps"], "unit": "GB/s", **base,
+               "ms_per_step": r["ms_per_step"],
+               "config": {"workload": f"C2 elementwise/broadcast/reduce suite, fp32 N(0,1), {R}x{C} "
+                                      f"({r['n_ops']} kernels per step: add/sub/mul/div x same,(R,1),(1,C),scalar; "
+                                      "exp relu log sqrt; sum/max x axis0,axis1,all)"},
+               "roofline": {"bound": "hbm", "achieved": add["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                            "frac": add["GBps"] / HBM_PEAK_GBS, "traffic": None,
+                            "kernel": "map_add_vec_vec_v4u4", "bytes_per_launch": 12 * R * C,
+                            "avg_launch_ms": add["ms"]},
+               "per_op": {k: {"GBps": round(v["GBps"], 1), "frac_hbm": round(v["frac_hbm"], 3),
+                              "ms": round(v["ms"], 4)} for k, v in r["per_op"].items()}}
+        if not args.no_cpu:
+            out["cpu_baseline"] = cpu_c2(4096, 4096)
+        if not args.no_extra:
+            extra = {}
+            for (r2, c2) in ((4096, 4096), (1024, 1024)):
+                e = run_c2(r2, c2, args.steps, args.warmup)
+                extra[f"c2_{r2}x{c2}_cache_resident"] = {
+                    "GBps": round(e["GBps"], 1), "ms_per_step": round(e["ms_per_step"], 4),
+                    "add_same_GBps": round(e["per_op"]["add_same"]["GBps"], 1)}
+            sweep = {}
+            for n in (128, 512, 1024, 2048, 4096, 8192):
+                m = run_matmul(n, n, n, max(3, min(args.steps, 10)), 2)
+                sweep[str(n)] = {"TFLOPs": round(m["TFLOPs"], 2), "kernel_ms": round(m["kernel_ms"], 4),
+                                 "frac_mfma_fp32": round(m["TFLOPs"] / MFMA_FP32_PEAK_TFLOPS, 3)}
+            for name, (M_, K_, N_) in (("16384x128.128x512", (16384, 128, 512)), ("2048x128.128x128", (2048, 128, 128))):
+                m = run_matmul(M_, N_, K_, 10, 2)
+                sweep[name] = {"TFLOPs": round(m["TFLOPs"], 2), "kernel_ms": round(m["kernel_ms"], 4)}
+            extra["matmul_fp32_TFLOPs"] = sweep
+            g = run_gpt(max(3, min(args.steps, 10)), 2)
+            extra["gpt_char_fwd_bwd_adam"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in g.items()}
+            out["extra"] = extra
+    elif args.workload == "matmul":
+        n = 4096
+        m = run_matmul(n, n, n, args.steps, args.warmup)
+        out = {"metric": "matmul fp32 TFLOPS (1 GPU)", "value": m["TFLOPs_wall"], "unit": "TFLOP/s", **base,
+               "ms_per_step": m["ms_per_step"],
+               "config": {"workload": f"C3 fp32 matmul {n}x{n}x{n}, entries N(0, 1/sqrt(K))"},
+               "roofline": {"bound": "mfma", "achieved": m["TFLOPs"], "peak": MFMA_FP32_PEAK_TFLOPS,
+                            "unit": "TFLOP/s", "frac": m["TFLOPs"] / MFMA_FP32_PEAK_TFLOPS, "traffic": None,
+                            "flops_per_launch": m["flops"], "avg_launch_ms": m["kernel_ms"]}}
+        if not args.no_cpu:
+            out["cpu_baseline"] = cpu_matmul(512)
+    elif args.workload == "gpt":
+        g = run_gpt(args.steps, args.warmup)
+        out = {"metric": "GPT fwd+bwd tokens/s (1 GPU)", "value": g["tokens_per_s"], "unit": "tokens/s", **base,
+               "ms_per_step": g["ms_per_step"],
+               "config": {"workload": "C4 char-GPT vocab 65, block 128, 6 layers, 4 heads, n_embd 128, batch 16; "
+                                      "forward + backward + Adam step (RMSNorm, ReLU MLP, no bias, as examples/gpt.py)",
+                          "launches_per_step": g["launches_per_step"], "loss_per_token": g["loss_per_token"]},
+               "roofline": None}
+        if not args.no_cpu:
+            out["cpu_baseline"] = cpu_gpt()
+    else:
+        r = run_mlp(args.steps, args.warmup)
+        out = {"metric": "MLP 784-64-10 step samples/s (1 GPU)", "value": r["samples_per_s"], "unit": "samples/s",
+               **base, "ms_per_step": r["ms_per_step"],
+               "config": {"workload": "C1 MLP 784-64-10, batch 128, fwd+bwd+SGD", "launches_per_step": r["launches_per_step"]},
+               "roofline": None}
+    out["device"] = device
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -97,6 +97,18 @@ class _CompileOnlyLib:
         return lambda *a, **k: None
 
 
+def _dump_manifest() -> None:
+    path = os.environ.get("DLGRAD_HIP_MANIFEST")
+    if path and requested_kernels:
+        from dlgrad_amd.codegen import manifest
+        manifest.merge(requested_kernels)
+
+
+if os.environ.get("DLGRAD_HIP_MANIFEST"):
+    import atexit
+    atexit.register(_dump_manifest)
+
+
 def lib() -> _ffi.HipLib:
     """The loaded library with the device initialised; raises when there is no GPU."""
     if not _state["ready"]:

@@ -1,0 +1,147 @@
+"""CPU-only checks of the C-ABI library and of the host-side logic around it:
+the library loads, exports every function include/dlgrad_hip.h declares, reports errors
+the way the boundary promises, compiles kernels for gfx950 without a GPU, and the
+shape/stride helpers the launchers rely on behave."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from dlgrad_amd import ffi, helpers
+from dlgrad_amd.buffer import Buffer
+from dlgrad_amd.codegen import hip_kernel as K
+from dlgrad_amd.codegen import manifest
+from dlgrad_amd.device import Device
+from dlgrad_amd.dispatch import dispatcher
+from dlgrad_amd.helpers import BinaryOps, BufferOps, CustomOps, UnaryOps
+from dlgrad_amd.runtime import hip
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "dlgrad_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dlg_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_functions()
+    assert len(names) >= 25
+    lib = ctypes.CDLL(ffi.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in the header but not exported"
+    assert sorted(ffi.EXPORTS) == names, "the Python binding table and the header disagree"
+
+
+def test_calls_before_init_fail_with_a_message():
+    lib = ffi.get_lib()
+    if hip.available():
+        pytest.skip("a GPU is present; the no-device error path is not reachable")
+    with pytest.raises(ffi.HipError, match="no HIP device"):
+        lib.init(0)
+    with pytest.raises(MemoryError):
+        lib.alloc(1024)
+    with pytest.raises(ffi.HipError, match="dlg_hip_init"):
+        lib.sync()
+    assert lib.device_count() == 0
+    with pytest.raises(ffi.HipError):
+        Buffer.from_numpy(np.zeros((2, 2), np.float32), Device.HIP)     # loud, no CPU fallback
+
+
+def test_hiprtc_compiles_for_gfx950_without_a_gpu_and_reports_errors():
+    lib = ffi.get_lib()
+    src, name, fmt = K.map_kernel("add", K.BINARY_EXPR["add"], ("vec", "row"), 4)
+    code = lib.compile(src, name, list(K.COMPILE_OPTIONS))
+    assert code[:4] == b"\x7fELF" and name.encode() in code
+    assert fmt == "@PPPII"
+    with pytest.raises(RuntimeError, match="Compilation failed"):
+        lib.compile('extern "C" __global__ void broken() { this is not C++; }', "broken", list(K.COMPILE_OPTIONS))
+
+
+def test_every_manifest_kernel_has_source_and_argument_format():
+    import struct
+    entries = manifest.load()
+    assert len(entries) > 50
+    for gen, params in entries:
+        src, name, fmt = getattr(K, gen)(*params)
+        assert f"void {name}(" in src
+        assert struct.calcsize(fmt) > 0
+
+
+def test_hip_runtime_registers_the_whole_operator_table():
+    want = {BufferOps.CREATE, BufferOps.UNIFORM, BufferOps.ARANGE, BufferOps.FULL,
+            BinaryOps.ADD, BinaryOps.SUB, BinaryOps.MUL, BinaryOps.DIV, BinaryOps.MATMUL, BinaryOps.GT,
+            BinaryOps.GTE, BinaryOps.EQT, BinaryOps.CMP,
+            UnaryOps.SUM, UnaryOps.MAX, UnaryOps.MEAN, UnaryOps.NEG, UnaryOps.EXP, UnaryOps.LOG, UnaryOps.POW,
+            UnaryOps.SQRT, UnaryOps.RSQRT, UnaryOps.RELU, UnaryOps.ARGMAX, UnaryOps.WHERE, UnaryOps.CLAMP,
+            UnaryOps.MASKED_FILL, UnaryOps.PERMUTE,
+            CustomOps.CE_FORWARD, CustomOps.CE_BACKWARD, CustomOps.PRINT, CustomOps.EMBEDDING,
+            CustomOps.TO_HOST, CustomOps.SOFTMAX, CustomOps.LOG_SOFTMAX}
+    assert want <= dispatcher.registered(Device.HIP)
+    with pytest.raises(KeyError):
+        dispatcher.dispatch(UnaryOps.EXP, Device.METAL, x=None)
+
+
+def test_device_names():
+    assert Device.from_str("hip") is Device.HIP and Device.from_str("CPU") is Device.CPU
+    assert Device.from_str("tpu") is None
+
+
+def test_shape_helpers():
+    assert helpers.calculate_stride((2, 3, 4)) == (12, 4, 1) and helpers.calculate_stride(()) == ()
+    assert helpers.broadcast_shapes_2((3, 1), (3, 4)) == (3, 4)
+    assert helpers.broadcast_shapes_2((4,), (2, 3, 4)) == (2, 3, 4)
+    with pytest.raises(ValueError):
+        helpers.broadcast_shapes_2((3, 2), (3, 4))
+    assert helpers.get_broadcast_strides_2((2, 3, 4), (3, 1), (1, 1)) == (0, 1, 0)
+    assert helpers.broadcast_shapes((5, 7), (4, 7, 3)) == ((1, 5, 7), (4, 7, 3), (4, 5, 3))
+    with pytest.raises(ValueError):
+        helpers.broadcast_shapes((5, 7), (6, 3))
+    assert helpers.cal_sum_max_out_shape(3, 1, (2, 3, 4)) == (2, 4)
+    assert helpers.cal_sum_max_out_shape(3, 1, (2, 3, 4), keepdim=True) == (2, 1, 4)
+    assert helpers.cal_sum_max_out_shape(3, -1, (2, 3, 4)) == ()
+    with pytest.raises(AssertionError):
+        helpers.check_broadcast((2, 3), (4, 3))
+
+
+def test_collapse_dims_finds_the_row_and_column_broadcast_patterns():
+    cd, st = helpers.collapse_dims, helpers.calculate_stride
+    # (16,4,128,128) * (16,4,128,1): rows of 128 with one value per row
+    out = (16, 4, 128, 128)
+    shape, (o, y) = cd(out, st(out), helpers.get_broadcast_strides_2(out, (16, 4, 128, 1), st((16, 4, 128, 1))))
+    assert shape == (8192, 128) and o == (128, 1) and y == (1, 0)
+    # (16,128,128) + (1,128,128): one "row" of 16384 repeated 16 times
+    out = (16, 128, 128)
+    shape, (o, y) = cd(out, st(out), helpers.get_broadcast_strides_2(out, (1, 128, 128), st((1, 128, 128))))
+    assert shape == (16, 16384) and y == (0, 1)
+    # same shapes collapse to one dim; a single value has all-zero strides
+    shape, (o, y) = cd((4, 5), (5, 1), (5, 1))
+    assert shape == (20,) and y == (1,)
+    shape, (o, y) = cd((4, 5), (5, 1), (0, 0))
+    assert shape == (20,) and y == (0,)
+    # an interleaved pattern stays multi-dimensional
+    shape, _ = cd((2, 3, 4, 5), st((2, 3, 4, 5)), (4, 0, 1, 0))
+    assert len(shape) == 4
+
+
+def test_device_pointer_views_keep_their_base_and_check_bounds():
+    base = hip.DevicePtr(0x1000, 64)
+    base.base = base          # pretend it is a view so __del__ frees nothing
+    v = base + 4
+    assert v.addr == 0x1010 and v.nbytes == 48 and v.base is base
+    with pytest.raises(IndexError):
+        base + 17
+    base.base = base
+
+
+def test_pow_expression_is_repeated_multiplication():
+    assert K.pow_expr(2) == "(x0 * x0)" or K.pow_expr(2) == "x0 * x0" or "x0" in K.pow_expr(2)
+    x0 = 1.7
+
+    def ev(n):
+        return eval(K.pow_expr(n).replace("1.0f", "1.0").replace("powf", "pow"), {"x0": x0})
+    for n in (0, 1, 2, 3, 5, 8, -1, -2):
+        assert abs(ev(n) - x0 ** n) < 1e-12
