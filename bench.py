@@ -303,6 +303,9 @@ def main() -> None:
     ap.add_argument("--workload", default="c2", choices=["c2", "matmul", "gpt", "mlp"])
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also launch a plain 16384x8192 copy kernel three times before the timed region "
+                         "(a known 512 MiB read + 512 MiB write, to scale rocprofv3's FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs on one GPU; --gpus must be 1 (nothing here uses a second device)")
@@ -313,6 +316,14 @@ def main() -> None:
     device = {"name": props["name"], "arch": props["arch"], "compute_units": props["compute_units"],
               "clock_mhz": props["clock_khz"] / 1000}
 
+    if args.calib_copy:
+        from dlgrad_amd.buffer import Buffer
+        from dlgrad_amd.device import Device
+        src = Buffer.from_numpy(np.ones((16384, 8192), np.float32), Device.HIP)
+        for _ in range(3):
+            hip._map("copy", "x0", [src], src.shape)
+        hip.lib().sync()
+        del src
     if args.workload == "c2":
         R, C = 16384, 8192
         r = run_c2(R, C, args.steps, args.warmup)

@@ -643,15 +643,24 @@ class HIP:
     # ---- matmul ----------------------------------------------------------------------------------------------------------
     MATMUL_FORCE = os.environ.get("DLGRAD_HIP_MATMUL_TILE")      # e.g. "128x128": benchmarking aid
 
+    # relative per-CU throughput of each tile shape, measured on 4096^3 (larger = faster)
+    _TILE_RATE = {"128x256": 0.95, "128x128": 1.0, "64x128": 0.67, "64x64": 0.83, "32x32": 0.68}
+
     @staticmethod
     def _pick_tile(M: int, N: int, batch: int) -> str:
+        """Largest expected throughput = tile rate x fraction of the tile grid that is real
+        output x fraction of the 256 CUs that get a block."""
         if HIP.MATMUL_FORCE:
             return HIP.MATMUL_FORCE
-        for name in ("128x256", "128x128", "64x128", "64x64"):
+        best, best_score = "64x64", -1.0
+        for name, rate in HIP._TILE_RATE.items():
             bm, bn = (int(v) for v in name.split("x"))
-            if ((M + bm - 1) // bm) * ((N + bn - 1) // bn) * batch >= 512:
-                return name
-        return "64x64" if (M > 32 and N > 32) else "32x32"
+            tm, tn = (M + bm - 1) // bm, (N + bn - 1) // bn
+            eff = (M * N) / float(tm * bm * tn * bn)
+            score = rate * eff * min(1.0, tm * tn * batch / 256.0)
+            if score > best_score * 1.0001:
+                best, best_score = name, score
+        return best
 
     @staticmethod
     @dispatcher.register(BinaryOps.MATMUL, Device.HIP)
