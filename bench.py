@@ -39,6 +39,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_FP32_PEAK_TFLOPS = 157.3  # dense fp32 MFMA
+# HBM bytes per launch of the same-shape add at 16384x8192, from two rocprofv3 --pmc runs
+# (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors a plain copy kernel of known size gives):
+# 1024.0 MiB read + 512.0 MiB written = the algorithmic 12 B per element.
+C2_ADD_TRAFFIC_BYTES = 1610612736
 
 
 def _imports():
@@ -208,6 +212,47 @@ def cpu_matmul(n: int = 512) -> dict:
 
 
 # ---------------------------------------------------------------------------------------------
+# C5 components at the scaled-GPT shapes
+# ---------------------------------------------------------------------------------------------
+def run_c5(steps: int, warmup: int) -> dict:
+    """Embedding gather / scatter-add on a 50304x768 table with 8192 Zipf(1.1) ids, fused softmax
+    on (98304, 1024), fused cross-entropy forward and backward on (8192, 50304).  GB/s are
+    algorithmic: gather 4n + 8nW; scatter 4VW + 4nW + 4n; softmax, CE fwd and CE bwd 8 B/elt."""
+    Tensor, _, Buffer, Device, hip = _imports()
+    lib = hip.lib()
+    rng = np.random.default_rng(5)
+    V, W, n = 50304, 768, 8192
+    ids = np.minimum(rng.zipf(1.1, n) - 1, V - 1).astype(np.float32)
+    table = Buffer.from_numpy(rng.standard_normal((V, W), dtype=np.float32), Device.HIP)
+    idx = Buffer.from_numpy(ids.reshape(8, 1024), Device.HIP)
+    g = Buffer.from_numpy(rng.standard_normal((8, 1024, W), dtype=np.float32), Device.HIP)
+    att = Buffer.from_numpy(rng.standard_normal((8 * 12 * 1024, 1024), dtype=np.float32), Device.HIP)
+    logits = Buffer.from_numpy(rng.standard_normal((n, V), dtype=np.float32), Device.HIP)
+    tgt = Buffer.from_numpy(ids.reshape(n, 1), Device.HIP)
+    one = Buffer.from_scalar(1.0)
+    lsm, _ = logits.log_softmax_gather(tgt)
+    work = [("embedding_gather", lambda: table.embedding(idx), 4 * n + 8 * n * W),
+            ("embedding_scatter_add", lambda: table.embedding(idx, backward=True, upstream_grad=g),
+             4 * V * W + 4 * n * W + 4 * n),
+            ("softmax_98304x1024", lambda: att.softmax(1), 8 * att.numel),
+            ("ce_forward_8192x50304", lambda: logits.log_softmax_gather(tgt), 8 * n * V),
+            ("ce_backward_8192x50304", lambda: lsm.ce_grad(tgt, one, float(n)), 8 * n * V)]
+    timer = EventTimer(lib)
+    for _ in range(warmup):
+        for _, f, _ in work:
+            f()
+    for _ in range(steps):
+        for name, f, _ in work:
+            timer.run(name, f)
+    lib.sync()
+    per = timer.collect()
+    return {name: {"ms": round(float(np.mean(per[name])), 4),
+                   "GBps": round(b / float(np.mean(per[name])) / 1e6, 1),
+                   "frac_hbm": round(b / float(np.mean(per[name])) / 1e6 / HBM_PEAK_GBS, 3)}
+            for name, _, b in work}
+
+
+# ---------------------------------------------------------------------------------------------
 # GPT / MLP steps
 # ---------------------------------------------------------------------------------------------
 GPT_C4 = dict(vocab_size=65, block_size=128, n_layer=6, n_head=4, n_embd=128, batch_size=16)
@@ -334,7 +379,7 @@ def main() -> None:
                                       f"({r['n_ops']} kernels per step: add/sub/mul/div x same,(R,1),(1,C),scalar; "
                                       "exp relu log sqrt; sum/max x axis0,axis1,all)"},
                "roofline": {"bound": "hbm", "achieved": add["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                            "frac": add["GBps"] / HBM_PEAK_GBS, "traffic": None,
+                            "frac": add["GBps"] / HBM_PEAK_GBS, "traffic": C2_ADD_TRAFFIC_BYTES,
                             "kernel": "map_add_vec_vec_v4u4", "bytes_per_launch": 12 * R * C,
                             "avg_launch_ms": add["ms"]},
                "per_op": {k: {"GBps": round(v["GBps"], 1), "frac_hbm": round(v["frac_hbm"], 3),
@@ -359,6 +404,7 @@ def main() -> None:
             extra["matmul_fp32_TFLOPs"] = sweep
             g = run_gpt(max(3, min(args.steps, 10)), 2)
             extra["gpt_char_fwd_bwd_adam"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in g.items()}
+            extra["c5_components"] = run_c5(max(3, min(args.steps, 10)), 2)
             out["extra"] = extra
     elif args.workload == "matmul":
         n = 4096

@@ -289,6 +289,15 @@ class Buffer:
     def log_softmax(self, dim: int) -> "Buffer":
         return self._unary(CustomOps.LOG_SOFTMAX, dim=dim)
 
+    def log_softmax_gather(self, target: "Buffer") -> tuple["Buffer", "Buffer"]:
+        """(log_softmax(self, last axis), its entries at the target columns as (1, N))."""
+        lsm, picked = self._dispatch(CustomOps.LOG_SOFTMAX_GATHER, x=self, target=target)
+        return self._like(lsm), self._like(picked, (1, self.shape[0]))
+
+    def ce_grad(self, target: "Buffer", upstream: "Buffer", n: float) -> "Buffer":
+        """self is a log-softmax; returns ((exp(self) - onehot(target)) * upstream) / n."""
+        return self._like(self._dispatch(CustomOps.CE_GRAD, lsm=self, target=target, upstream=upstream, n=n))
+
     # ---- selects ----------------------------------------------------------------------------------
     def where(self, inp: "Buffer | Scalar", other: "Buffer | Scalar") -> "Buffer":
         inp = Buffer.from_scalar(inp) if _is_scalar(inp) else inp

@@ -157,7 +157,7 @@ def map_kernel(tag: str, expr: str, modes: tuple[str, ...], vec: int, n_sval_ext
     params += ["float* __restrict__ out", "u32 n", "u32 C"]
     fmt += ["P", "I", "I"]
     nx = len(modes)
-    fargs = ", ".join([f"float x{k}" for k in range(nx)] + [f"float s{k}" for k in range(n_sval_extra)] + ["u32 i"])
+    fargs = ", ".join([f"float x{k}" for k in range(nx)] + [f"float s{k}" for k in range(n_sval_extra)] + ["u32 i", "u32 C"])
     extra = "".join(f"s{k}, " for k in range(n_sval_extra))
 
     def scalar_load(k: int, idx: str) -> str:
@@ -187,7 +187,7 @@ def map_kernel(tag: str, expr: str, modes: tuple[str, ...], vec: int, n_sval_ext
         for j, c in enumerate("xyzw"):
             xs = ", ".join([comp(k, c) for k in range(nx)])
             xs = (xs + ", ") if xs else ""
-            calc += f"            o.{c} = f({xs}{extra}(v << 2) + {j});\n"
+            calc += f"            o.{c} = f({xs}{extra}(v << 2) + {j}, C);\n"
         store = ("{ v4f ov = {o.x, o.y, o.z, o.w}; __builtin_nontemporal_store(ov, reinterpret_cast<v4f*>(out) + v); }" if nt_store
                  else "reinterpret_cast<float4*>(out)[v] = o;")
         tail_x = ", ".join(scalar_load(k, "i") for k in range(nx))
@@ -212,7 +212,7 @@ def map_kernel(tag: str, expr: str, modes: tuple[str, ...], vec: int, n_sval_ext
     }}
     if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {{
         const u32 i = (nv << 2) + threadIdx.x;
-        out[i] = f({tail_x}{extra}i);
+        out[i] = f({tail_x}{extra}i, C);
     }}
 """
     else:
@@ -223,7 +223,7 @@ def map_kernel(tag: str, expr: str, modes: tuple[str, ...], vec: int, n_sval_ext
     #pragma unroll
     for (int u = 0; u < {unroll}; ++u) {{
         const u32 i = i0 + u * {T}u;
-        if (i < n) out[i] = f({xs}{extra}i);
+        if (i < n) out[i] = f({xs}{extra}i, C);
     }}
 """
     src = f"""{PRELUDE}
@@ -676,46 +676,91 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 
 
 @cache
-def softmax_rows_kernel(log: bool, vec: int, per_block: bool) -> tuple[str, str, str]:
-    """Row softmax / log-softmax over the contiguous last axis of an (R, L) view in one
-    pass over HBM: max, exp-sum and the normalised write all read the row from
-    registers-or-L2 instead of materialising max, x-max, exp and sum as the reference's
-    five kernels do (tensor.py:634-669).  Same formula: e = exp(x - max); e / sum(e)
-    (or (x - max) - log(sum)).  One wavefront per row, or one block per long row."""
-    name = f"{'log_' if log else ''}softmax_rows_v{vec}_{'blk' if per_block else 'wav'}"
+def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gather: bool = False) -> tuple[str, str, str]:
+    """Row softmax / log-softmax over the contiguous last axis of an (R, L) view, replacing
+    the reference's five kernels and four temporaries (tensor.py:634-669).  Same formula:
+    e = exp(x - max); e / sum(e)   (or (x - max) - log(sum)).
+
+    One wavefront per row, or one 256-thread block per long row.  nval > 0 is the
+    register-resident form: each thread keeps its nval float4 (or float) items of the row
+    in registers, so the row is read from HBM once and written once (8 B per element, the
+    algorithmic minimum); rows of 50304 floats fit in 50 float4 per thread of a block.
+    nval = 0 streams the row three times (for rows longer than registers hold).
+    gather (log-softmax only): also writes picked[row] = out[row, (int)target[row]], the
+    ce_forward gather of cpu_kernel.py:430-441, fused."""
+    name = (f"{'log_' if log else ''}softmax_rows_v{vec}_{'blk' if per_block else 'wav'}"
+            f"{f'_r{nval}' if nval else ''}{'_g' if gather else ''}")
     T = "256u" if per_block else "64u"
     tid = "threadIdx.x" if per_block else "(threadIdx.x & 63u)"
     row = "blockIdx.x" if per_block else "(blockIdx.x * 4u + (threadIdx.x >> 6))"
     red_max = "block_max(m, sm)" if per_block else "wave_max(m)"
     red_sum = "block_sum(s, sm)" if per_block else "wave_sum(s)"
-    outexpr = "(V - m) - ls" if log else "expf(V - m) / s"
-    if vec == 4:
+
+    def outexpr(v: str) -> str:
+        return f"(({v}) - m) - ls" if log else f"expf(({v}) - m) / s"
+    comps = ("x", "y", "z", "w")
+    if nval and vec == 4:
+        body = f"""
+    const float4* __restrict__ p = reinterpret_cast<const float4*>(x + (u64)row * L);
+    float4* __restrict__ q = reinterpret_cast<float4*>(out + (u64)row * L);
+    const u32 nv = L >> 2;
+    float4 v[{nval}];
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < nv) v[k] = p[c]; }}
+    float m = NEG_FLT_MAX;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < nv)
+        m = fmaxf(fmaxf(m, fmaxf(v[k].x, v[k].y)), fmaxf(v[k].z, v[k].w));
+    m = {red_max};
+    float s = 0.0f;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < nv)
+        s += (expf(v[k].x - m) + expf(v[k].y - m)) + (expf(v[k].z - m) + expf(v[k].w - m));
+    s = {red_sum};
+    const float ls = logf(s); (void)ls;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{
+        const u32 c = {tid} + k * {T};
+        if (c < nv) {{
+            float4 o;
+{''.join(f"            o.{c} = {outexpr(f'v[k].{c}')};{chr(10)}" for c in comps)}            q[c] = o;
+        }}
+    }}
+"""
+    elif nval:
+        body = f"""
+    const float* __restrict__ p = x + (u64)row * L;
+    float* __restrict__ q = out + (u64)row * L;
+    float v[{nval}];
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < L) v[k] = p[c]; }}
+    float m = NEG_FLT_MAX;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < L) m = fmaxf(m, v[k]);
+    m = {red_max};
+    float s = 0.0f;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < L) s += expf(v[k] - m);
+    s = {red_sum};
+    const float ls = logf(s); (void)ls;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < L) q[c] = {outexpr('v[k]')}; }}
+"""
+    elif vec == 4:
         body = f"""
     const float4* __restrict__ p = reinterpret_cast<const float4*>(x + (u64)row * L);
     float4* __restrict__ q = reinterpret_cast<float4*>(out + (u64)row * L);
     const u32 nv = L >> 2;
     float m = NEG_FLT_MAX;
-    for (u32 v = {tid}; v < nv; v += {T}) {{ const float4 t = p[v]; m = fmaxf(fmaxf(m, fmaxf(t.x, t.y)), fmaxf(t.z, t.w)); }}
+    for (u32 c = {tid}; c < nv; c += {T}) {{ const float4 t = p[c]; m = fmaxf(fmaxf(m, fmaxf(t.x, t.y)), fmaxf(t.z, t.w)); }}
     m = {red_max};
     float s = 0.0f;
-    for (u32 v = {tid}; v < nv; v += {T}) {{ const float4 t = p[v]; s += (expf(t.x - m) + expf(t.y - m)) + (expf(t.z - m) + expf(t.w - m)); }}
+    for (u32 c = {tid}; c < nv; c += {T}) {{ const float4 t = p[c]; s += (expf(t.x - m) + expf(t.y - m)) + (expf(t.z - m) + expf(t.w - m)); }}
     s = {red_sum};
     const float ls = logf(s); (void)ls;
-    for (u32 v = {tid}; v < nv; v += {T}) {{
-        const float4 t = p[v]; float4 o;
-        #define V t.x
-        o.x = {outexpr};
-        #undef V
-        #define V t.y
-        o.y = {outexpr};
-        #undef V
-        #define V t.z
-        o.z = {outexpr};
-        #undef V
-        #define V t.w
-        o.w = {outexpr};
-        #undef V
-        q[v] = o;
+    for (u32 c = {tid}; c < nv; c += {T}) {{
+        const float4 t = p[c]; float4 o;
+{''.join(f"        o.{c} = {outexpr(f't.{c}')};{chr(10)}" for c in comps)}        q[c] = o;
     }}
 """
     else:
@@ -723,18 +768,20 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool) -> tuple[str, str,
     const float* __restrict__ p = x + (u64)row * L;
     float* __restrict__ q = out + (u64)row * L;
     float m = NEG_FLT_MAX;
-    for (u32 i = {tid}; i < L; i += {T}) m = fmaxf(m, p[i]);
+    for (u32 c = {tid}; c < L; c += {T}) m = fmaxf(m, p[c]);
     m = {red_max};
     float s = 0.0f;
-    for (u32 i = {tid}; i < L; i += {T}) s += expf(p[i] - m);
+    for (u32 c = {tid}; c < L; c += {T}) s += expf(p[c] - m);
     s = {red_sum};
     const float ls = logf(s); (void)ls;
-    for (u32 i = {tid}; i < L; i += {T}) {{
-        #define V p[i]
-        q[i] = {outexpr};
-        #undef V
-    }}
+    for (u32 c = {tid}; c < L; c += {T}) q[c] = {outexpr('p[c]')};
 """
+    if gather:
+        assert log
+        body += f"""
+    if ({tid} == 0) {{ const float* __restrict__ xr = x + (u64)row * L; picked[row] = (xr[(int)target[row]] - m) - ls; }}
+"""
+    extra_params = ", const float* __restrict__ target, float* __restrict__ picked" if gather else ""
     src = f"""{PRELUDE}
 static __device__ __forceinline__ float block_max(float v, float* sm) {{
     v = wave_max(v);
@@ -753,14 +800,25 @@ static __device__ __forceinline__ float block_sum(float v, float* sm) {{
     return v;
 }}
 extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
-        float* __restrict__ out, u32 R, u32 L) {{
+        float* __restrict__ out, u32 R, u32 L{extra_params}) {{
     __shared__ float sm[4];
     const u32 row = {row};
     {'' if per_block else 'if (row >= R) return;'}
 {body}
 }}
 """
-    return src, name, _fmt("P", "P", "I", "I")
+    return src, name, _fmt("P", "P", "I", "I", *(("P", "P") if gather else ()))
+
+
+def softmax_plan(L: int, vec: int) -> tuple[bool, int]:
+    """(per_block, nval) for a row of L floats: the smallest register-resident variant that
+    holds the row, wavefront-per-row first; (True, 0) streams."""
+    items = (L + vec - 1) // vec
+    for per_block, threads in ((False, 64), (True, 256)):
+        for nval in (1, 2, 4, 8, 16) if not per_block else (4, 8, 16, 32, 50) if vec == 4 else (8, 16, 32, 64):
+            if items <= threads * nval:
+                return per_block, nval
+    return True, 0
 
 
 # =====================================================================================

@@ -65,6 +65,8 @@ class CustomOps(Enum):
     # from max/sub/exp/sum/div: tensor.py:634-669, ops.py:337-370)
     SOFTMAX = auto()
     LOG_SOFTMAX = auto()
+    LOG_SOFTMAX_GATHER = auto()     # log-softmax rows + the ce_forward gather, one kernel
+    CE_GRAD = auto()                # ((exp(lsm) - onehot) * upstream) / N, one kernel
 
 
 def prod_(x: Iterable) -> int:

@@ -335,16 +335,19 @@ class CrossEntropy(OP):
         (ops.py:338-357); backward nevertheless scales by 1/N (ops.py:359-370)."""
         assert logits.shape[0] == target.shape[0]
         self.target = target
-        if FUSED and logits.device is Device.HIP and dim == logits.ndim - 1:
-            self.log_softmax = logits.log_softmax(dim)
+        self.N = float(logits.shape[0])
+        self.fused = FUSED and logits.device is Device.HIP and logits.ndim == 2 and dim == 1
+        if self.fused:
+            self.log_softmax, picked = logits.log_softmax_gather(target)
         else:
             shifted = logits - logits.max(dim=dim, keepdim=True)
             self.log_softmax = shifted - shifted.exp().sum(dim=dim, keepdim=True).log()
-        picked = Buffer.ce_forward(self.log_softmax, self.target)
-        self.N = float(logits.shape[0])
+            picked = Buffer.ce_forward(self.log_softmax, self.target)
         return -picked.sum()
 
     def backward(self, upstream_grad: Buffer) -> tuple:
+        if self.fused:
+            return (self.log_softmax.ce_grad(self.target, upstream_grad, self.N),)
         probs = self.log_softmax.exp()
         Buffer.ce_backward(op=CustomOps.CE_BACKWARD, device=probs.device, x=probs, target=self.target)   # p - onehot
         return ((probs * upstream_grad) / self.N,)

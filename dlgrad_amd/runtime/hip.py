@@ -612,9 +612,9 @@ class HIP:
         rows = x.shape[0]
         launch(kernel(K.ce_kernel, True), (rows + 255) // 256, 256, _addr(x), _addr(target), rows, x.stride[0])
 
-    # ---- fused row softmax ---------------------------------------------------------------------------------------------
+    # ---- fused row softmax / cross-entropy ------------------------------------------------------------------------------
     @staticmethod
-    def _softmax(x: Buffer, dim: int, log: bool) -> DevicePtr:
+    def _softmax(x: Buffer, dim: int, log: bool, target: Buffer | None = None):
         if dim < 0:
             dim += x.ndim
         if dim != x.ndim - 1:
@@ -622,13 +622,18 @@ class HIP:
         L = x.shape[-1]
         R = x.numel // max(L, 1)
         out = alloc(x.numel)
+        picked = alloc(R) if target is not None else None
         if x.numel == 0:
-            return out
+            return out if target is None else (out, picked)
         vec = 4 if (L % 4 == 0 and _addr(x) % 16 == 0 and out.addr % 16 == 0) else 1
-        blk = L > 2048
-        launch(kernel(K.softmax_rows_kernel, log, vec, blk), R if blk else (R + 3) // 4, 256,
-               _addr(x), out.addr, R, L)
-        return out
+        blk, nval = K.softmax_plan(L, vec)
+        k = kernel(K.softmax_rows_kernel, log, vec, blk, nval, target is not None)
+        grid = R if blk else (R + 3) // 4
+        if target is None:
+            launch(k, grid, 256, _addr(x), out.addr, R, L)
+            return out
+        launch(k, grid, 256, _addr(x), out.addr, R, L, _addr(target), picked.addr)
+        return out, picked
 
     @staticmethod
     @dispatcher.register(CustomOps.SOFTMAX, Device.HIP)
@@ -639,6 +644,26 @@ class HIP:
     @dispatcher.register(CustomOps.LOG_SOFTMAX, Device.HIP)
     def log_softmax(x: Buffer, dim: int) -> DevicePtr:
         return HIP._softmax(x, dim, True)
+
+    @staticmethod
+    @dispatcher.register(CustomOps.LOG_SOFTMAX_GATHER, Device.HIP)
+    def log_softmax_gather(x: Buffer, target: Buffer) -> tuple[DevicePtr, DevicePtr]:
+        """log-softmax over the rows of a 2-D x and, in the same kernel, the ce_forward
+        gather picked[i] = lsm[i, (int)target[i]] (cpu.py:961-981)."""
+        return HIP._softmax(x, x.ndim - 1, True, target)
+
+    @staticmethod
+    @dispatcher.register(CustomOps.CE_GRAD, Device.HIP)
+    def ce_grad(lsm: Buffer, target: Buffer, upstream: Buffer, n: float) -> DevicePtr:
+        """((exp(lsm) - onehot(target)) * upstream) / n in one pass: the four kernels of
+        CrossEntropy.backward (exp, in-place ce_backward, mul, div; ops.py:359-370) fused.
+        Same operation order, so it differs from them only through expf."""
+        rows = Buffer(target.ptr, (lsm.shape[0], 1), Device.HIP)
+        expr = "((expf(x0) - (((i % C) == (u32)(int)x1) ? 1.0f : 0.0f)) * {g}) / s0"
+        if upstream.is_host_scalar:
+            return _map("cegrad_v", expr.format(g="s1"), [lsm, rows], lsm.shape,
+                        (n, float(upstream.ptr.value)))
+        return _map("cegrad_p", expr.format(g="x2"), [lsm, rows, upstream], lsm.shape, (n,))
 
     # ---- matmul ----------------------------------------------------------------------------------------------------------
     MATMUL_FORCE = os.environ.get("DLGRAD_HIP_MATMUL_TILE")      # e.g. "128x128": benchmarking aid
