@@ -17,8 +17,6 @@ buffer.py:86-90).  Buffers are always contiguous: `stride` is derived from
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
-
 import numpy as np
 
 from dlgrad_amd.device import Device, as_device
@@ -52,15 +50,14 @@ class HostScalar:
         return f"HostScalar({float(self.value)!r})"
 
 
-@dataclass
 class BufferMetadata:
-    shape: tuple
-    numel: int
-    stride: tuple
-    ndim: int
-    dtype: DType
-    device: Device
-    nbytes: int
+    """shape / numel / stride / ndim / dtype / device / nbytes of a Buffer (buffer.py:24-32)."""
+    __slots__ = ("shape", "numel", "stride", "ndim", "dtype", "device", "nbytes")
+
+    def __init__(self, shape: tuple, numel: int, stride: tuple, ndim: int, dtype: DType, device: Device,
+                 nbytes: int) -> None:
+        self.shape, self.numel, self.stride, self.ndim = shape, numel, stride, ndim
+        self.dtype, self.device, self.nbytes = dtype, device, nbytes
 
 
 def _is_scalar(v) -> bool:
@@ -93,12 +90,16 @@ class Buffer:
                  dtype: str | DType | None = None, **kwargs) -> None:
         self.ptr = data
         shape = tuple(shape)
-        dtype = DType.from_str(dtype) if isinstance(dtype, str) else (dtype or DType.FLOAT32)
+        if dtype is None or dtype.__class__ is str:
+            dtype = DType.from_str(dtype) if dtype else DType.FLOAT32
+        if device.__class__ is not Device:
+            device = as_device(device)
         n = prod_(shape)
-        self.metadata = BufferMetadata(
-            shape=shape, numel=n, stride=kwargs.get("stride", calculate_stride(shape)),
-            ndim=kwargs.get("ndim", len(shape)), dtype=dtype, device=as_device(device),
-            nbytes=n * DType.get_n_bytes(dtype))
+        if kwargs:
+            stride, ndim = kwargs.get("stride", calculate_stride(shape)), kwargs.get("ndim", len(shape))
+        else:
+            stride, ndim = calculate_stride(shape), len(shape)
+        self.metadata = BufferMetadata(shape, n, stride, ndim, dtype, device, n * 4)
 
     # ---- plumbing -------------------------------------------------------------------
     def _dispatch(self, op, **kw):
@@ -330,6 +331,11 @@ class Buffer:
         out_shape = idx.shape + (self.shape[-1],)
         return self._like(self._dispatch(CustomOps.EMBEDDING, x=self, idx=idx, out_numel=prod_(out_shape)),
                           out_shape)
+
+    def adam_step(self, g: "Buffer", m: "Buffer", v: "Buffer", consts: tuple) -> tuple["Buffer", "Buffer", "Buffer"]:
+        """One fused Adam update of the parameter `self`; returns new (p, m, v) Buffers."""
+        ptrs = self._dispatch(CustomOps.ADAM_STEP, p=self, g=g, m=m, v=v, consts=consts)
+        return tuple(self._like(q) for q in ptrs)
 
     # ---- binary -----------------------------------------------------------------------------------------
     def _binary_op(self, other: "Buffer", op: BinaryOps) -> "Buffer":

@@ -1017,3 +1017,70 @@ MATMUL_CONFIGS = {
     "64x64": (2, 2, 1, 1, 16),
     "32x32": (1, 1, 1, 1, 16),
 }
+
+
+# =====================================================================================
+# optimizer
+# =====================================================================================
+
+@cache
+def adam_kernel(vec: int) -> tuple[str, str, str]:
+    """One Adam update of one parameter tensor: the fourteen element-wise kernels of
+    dlgrad/nn/optim.py:59-70 in a single pass, writing new p, m and v buffers.
+
+    Every operation is the same fp32 operation, in the same order, as in the unfused
+    expression, and fp contraction is switched off so that no a*b+c becomes an fma: the
+    result is bit-identical to the op-by-op path:
+        m' = m*b1 + g*(1-b1);  v' = v*b2 + (g*g)*(1-b2)
+        p' = p - ((m'/c1) / (sqrt(v'/c2) + eps)) * lr        (c1 = 1-b1^t, c2 = 1-b2^t)"""
+    name = f"adam_step_v{vec}"
+    step = """
+static __device__ __forceinline__ void adam1(float p, float g, float m, float v, const AdamArgs& a,
+                                             float& po, float& mo, float& vo) {
+    #pragma clang fp contract(off)
+    const float t1 = m * a.b1, t2 = g * a.omb1;
+    mo = t1 + t2;
+    const float gg = g * g;
+    const float t3 = v * a.b2, t4 = gg * a.omb2;
+    vo = t3 + t4;
+    const float mh = mo / a.c1, vh = vo / a.c2;
+    const float den = sqrtf(vh) + a.eps;
+    const float q = mh / den;
+    po = p - q * a.lr;
+}
+"""
+    if vec == 4:
+        body = """
+    const u32 nv = n >> 2;
+    const u32 i = blockIdx.x * 256u + threadIdx.x;
+    if (i < nv) {
+        const float4 p4 = reinterpret_cast<const float4*>(p)[i], g4 = reinterpret_cast<const float4*>(g)[i];
+        const float4 m4 = reinterpret_cast<const float4*>(m)[i], v4 = reinterpret_cast<const float4*>(v)[i];
+        float4 po, mo, vo;
+        adam1(p4.x, g4.x, m4.x, v4.x, a, po.x, mo.x, vo.x);
+        adam1(p4.y, g4.y, m4.y, v4.y, a, po.y, mo.y, vo.y);
+        adam1(p4.z, g4.z, m4.z, v4.z, a, po.z, mo.z, vo.z);
+        adam1(p4.w, g4.w, m4.w, v4.w, a, po.w, mo.w, vo.w);
+        reinterpret_cast<float4*>(p_out)[i] = po;
+        reinterpret_cast<float4*>(m_out)[i] = mo;
+        reinterpret_cast<float4*>(v_out)[i] = vo;
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {
+        const u32 j = (nv << 2) + threadIdx.x;
+        adam1(p[j], g[j], m[j], v[j], a, p_out[j], m_out[j], v_out[j]);
+    }
+"""
+    else:
+        body = """
+    const u32 j = blockIdx.x * 256u + threadIdx.x;
+    if (j < n) adam1(p[j], g[j], m[j], v[j], a, p_out[j], m_out[j], v_out[j]);
+"""
+    src = f"""{PRELUDE}
+struct AdamArgs {{ float b1, omb1, b2, omb2, c1, c2, eps, lr; }};
+{step}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ p,
+        const float* __restrict__ g, const float* __restrict__ m, const float* __restrict__ v,
+        float* __restrict__ p_out, float* __restrict__ m_out, float* __restrict__ v_out, u32 n, AdamArgs a) {{
+{body}}}
+"""
+    return src, name, _fmt("P", "P", "P", "P", "P", "P", "P", "I", "8f")

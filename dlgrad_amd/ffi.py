@@ -88,6 +88,9 @@ class HipLib:
             for name, (res, args) in _SIGS.items():
                 fn = getattr(self._lib, name)
                 fn.restype, fn.argtypes = res, args
+            self._alloc_box = ctypes.c_void_p()
+            self._alloc_ref = ctypes.byref(self._alloc_box)
+            self.raw_launch = self._lib.dlg_hip_launch      # (handle, gx,gy,gz, bx,by,bz, shmem, args, size)
 
     # -- cffi binding: same calls, the header text is the cdef ------------------------
     def _load_cffi(self, path: str) -> None:
@@ -102,6 +105,7 @@ class HipLib:
         ffi.cdef(text)
         self._cffi = ffi
         self._lib = ffi.dlopen(path)
+        self.raw_launch = self._lib.dlg_hip_launch
 
     # -- helpers -----------------------------------------------------------------------
     def last_error(self) -> str:
@@ -152,13 +156,18 @@ class HipLib:
 
     # -- memory --------------------------------------------------------------------------
     def alloc(self, nbytes: int, zero: bool = False) -> int:
-        ref, get = self._out(ctypes.c_void_p, "void *")
         fn = self._lib.dlg_hip_alloc_zero if zero else self._lib.dlg_hip_alloc
-        self._check(fn(nbytes, ref), MemoryError)
-        return get()
+        if self._cffi is not None:
+            ref, get = self._out(ctypes.c_void_p, "void *")
+            self._check(fn(nbytes, ref), MemoryError)
+            return get()
+        box = self._alloc_box                     # one reusable out-parameter: this runs per op
+        if fn(nbytes, self._alloc_ref) != 0:
+            self._check(-1, MemoryError)
+        return box.value or 0
 
     def free(self, ptr: int) -> None:
-        self._lib.dlg_hip_free(self._vp(ptr))
+        self._lib.dlg_hip_free(self._vp(ptr) if self._cffi is not None else ptr)
 
     def fill_f32(self, ptr: int, value: float, count: int) -> None:
         self._check(self._lib.dlg_hip_fill_f32(self._vp(ptr), value, count))

@@ -13,6 +13,7 @@ import itertools
 import os
 from collections.abc import Iterable
 from enum import Enum, auto
+from functools import lru_cache
 from math import prod
 
 
@@ -67,19 +68,25 @@ class CustomOps(Enum):
     LOG_SOFTMAX = auto()
     LOG_SOFTMAX_GATHER = auto()     # log-softmax rows + the ce_forward gather, one kernel
     CE_GRAD = auto()                # ((exp(lsm) - onehot) * upstream) / N, one kernel
+    ADAM_STEP = auto()              # the 14 element-wise kernels of one Adam update, one kernel
 
 
 def prod_(x: Iterable) -> int:
     return prod(x) if x else 1
 
 
-def calculate_stride(shape: tuple | list) -> tuple:
-    """Row-major element strides; () for a 0-d shape (helpers.py:176-187)."""
+@lru_cache(maxsize=4096)
+def _stride_of(shape: tuple) -> tuple:
     out, acc = [], 1
-    for d in reversed(tuple(shape)):
+    for d in reversed(shape):
         out.append(acc)
         acc *= d
     return tuple(reversed(out))
+
+
+def calculate_stride(shape: tuple | list) -> tuple:
+    """Row-major element strides; () for a 0-d shape (helpers.py:176-187)."""
+    return _stride_of(tuple(shape))
 
 
 def check_broadcast(x_shape: tuple, y_shape: tuple) -> bool:

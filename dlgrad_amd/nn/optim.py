@@ -1,5 +1,7 @@
 """Optimizers as Tensor expressions (dlgrad/nn/optim.py:4-70): every update is a handful
 of element-wise kernels per parameter and rebinds `param.data` to the new buffer."""
+from dlgrad_amd import ops
+from dlgrad_amd.device import Device
 from dlgrad_amd.tensor import Tensor
 
 
@@ -50,8 +52,14 @@ class Adam(Optimizer):
     def step(self) -> None:
         self.t += 1
         c1, c2 = 1.0 - self.beta1 ** self.t, 1.0 - self.beta2 ** self.t
+        consts = (self.beta1, 1.0 - self.beta1, self.beta2, 1.0 - self.beta2, c1, c2, self.eps, self.lr)
         for p in self.params:
             k, g = id(p), p.grad
+            if ops.FUSED and p.device is Device.HIP:
+                # same fp32 operations in the same order as below, in one kernel (bit-identical)
+                pb, mb, vb = p.data.adam_step(g.data, self.m[k].data, self.v[k].data, consts)
+                p.data, self.m[k], self.v[k] = pb, Tensor(mb), Tensor(vb)
+                continue
             self.m[k] = ((self.m[k] * self.beta1) + (g * (1.0 - self.beta1))).detach()
             self.v[k] = ((self.v[k] * self.beta2) + ((g ** 2.0) * (1.0 - self.beta2))).detach()
             m_hat, v_hat = self.m[k] / c1, self.v[k] / c2

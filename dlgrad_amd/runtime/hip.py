@@ -163,8 +163,9 @@ class DevicePtr:
 
 
 def alloc(numel: int, zero: bool = False) -> DevicePtr:
-    nbytes = 4 * max(int(numel), 1)
-    return DevicePtr(lib().alloc(nbytes, zero), nbytes)
+    nbytes = 4 * numel if numel > 0 else 4
+    l = _state["lib"] or lib()
+    return DevicePtr(l.alloc(nbytes, zero), nbytes)
 
 
 # ---- kernel cache -----------------------------------------------------------------------
@@ -201,12 +202,23 @@ def kernel(gen, *params):
 
 
 def launch(k, grid, block, *args) -> None:
+    """grid / block: an int (x extent) or a 3-tuple."""
     global launch_count
     launch_count += 1
     handle, st = k
-    g = grid if isinstance(grid, tuple) else (grid, 1, 1)
-    b = block if isinstance(block, tuple) else (block, 1, 1)
-    _state["lib"].launch(handle, g + (1,) * (3 - len(g)), b + (1,) * (3 - len(b)), st.pack(*args))
+    packed = st.pack(*args)
+    if grid.__class__ is int:
+        gx, gy, gz = grid, 1, 1
+    else:
+        gx, gy, gz = grid if len(grid) == 3 else (tuple(grid) + (1, 1))[:3]
+    if block.__class__ is int:
+        bx, by, bz = block, 1, 1
+    else:
+        bx, by, bz = block if len(block) == 3 else (tuple(block) + (1, 1))[:3]
+    l = _state["lib"]
+    rc = l.raw_launch(handle, gx, gy, gz, bx, by, bz, 0, packed, len(packed))
+    if rc:
+        l._check(rc)
 
 
 def _addr(b: Buffer) -> int:
@@ -219,61 +231,90 @@ def _pad4(t: tuple, fill: int) -> tuple:
 
 # ---- element-wise launcher ------------------------------------------------------------------
 
+class _MapPlan:
+    """Everything about one (op, operand shapes) combination that does not depend on the
+    addresses: element count, operand modes, the kernel variants and their trailing
+    arguments.  Built once, then each call only packs pointers and launches."""
+    __slots__ = ("n", "is_scalar", "wide", "narrow")
+
+    def __init__(self, tag: str, expr: str, operands: list, out_shape: tuple, n_svals: int) -> None:
+        if len(out_shape) > 4:
+            raise ValueError("dlgrad only supports upto 4D tensors")
+        n = self.n = prod_(out_shape)
+        if n >= 2 ** 31:
+            raise ValueError(f"{n} elements exceed the 32-bit index range of the kernels")
+        self.is_scalar = tuple(b.is_host_scalar for b in operands)
+        self.wide = self.narrow = None
+        if n == 0:
+            return
+        tens = [b for b in operands if not b.is_host_scalar]
+        t_strides = [get_broadcast_strides_2(out_shape, b.shape, b.stride) for b in tens]
+        cshape, cstr = collapse_dims(out_shape, calculate_stride(out_shape), *t_strides)
+        modes: list | None = None
+        C = cshape[-1] if len(cshape) == 2 else 1
+        if len(cshape) <= 2:
+            full = (C, 1) if len(cshape) == 2 else (1,)
+            kinds = {full: "vec", (1, 0): "row", (0, 1): "col"}
+            it = iter(cstr[1:])
+            modes = []
+            for sc in self.is_scalar:
+                if sc:
+                    modes.append("sval")
+                    continue
+                st = next(it)
+                m = "sptr" if not any(st) else kinds.get(st)
+                if m is None:
+                    modes = None
+                    break
+                modes.append(m)
+        if modes is not None:
+            # (generator params, grid, trailing args); the kernel itself is loaded on first use
+            if C % 4 == 0 or not any(m in ("row", "col") for m in modes):
+                self.wide = [(K.map_kernel, tag, expr, tuple(modes), 4, n_svals), K.map_grid(n, 4), (n, C), None,
+                             tuple(m in ("vec", "col") for m in modes)]
+            self.narrow = [(K.map_kernel, tag, expr, tuple(modes), 1, n_svals), K.map_grid(n, 1), (n, C), None, None]
+        else:
+            tail = (n, *_pad4(out_shape, 1), *[x for st in t_strides for x in _pad4(st, 0)])
+            self.narrow = [(K.strided_map_kernel, tag, expr, len(operands), self.is_scalar, n_svals),
+                           (n + 1023) // 1024, tail, None, None]
+
+
+_map_plans: dict = {}
+
+
 def _map(tag: str, expr: str, operands: list[Buffer], out_shape: tuple, svals: tuple = (),
          out: DevicePtr | None = None) -> DevicePtr:
     """Runs `expr` over `operands` broadcast to `out_shape`.
 
-    Collapses the iteration space jointly over all operands; if what is left is a
+    The iteration space is collapsed jointly over all operands; if what is left is a
     row-major (R, C) grid on which each operand is whole, one-per-row, one-row or a
-    single value, the vectorised `map_kernel` runs, otherwise the strided one."""
-    if len(out_shape) > 4:
-        raise ValueError("dlgrad only supports upto 4D tensors")
-    n = prod_(out_shape)
-    if n >= 2 ** 31:
-        raise ValueError(f"{n} elements exceed the 32-bit index range of the kernels")
-    out = out or alloc(n)
-    if n == 0:
+    single value, the vectorised `map_kernel` runs (16-byte accesses when every pointer
+    is 16-byte aligned), otherwise the strided one.  `tag` names `expr` uniquely."""
+    key = (tag, out_shape, tuple([None if b.ptr.__class__ is HostScalar else b.metadata.shape for b in operands]),
+           len(svals))
+    plan = _map_plans.get(key)
+    if plan is None:
+        plan = _map_plans[key] = _MapPlan(tag, expr, operands, out_shape, len(svals))
+    if out is None:
+        out = alloc(plan.n)
+    if plan.n == 0:
         return out
-    tens = [b for b in operands if not b.is_host_scalar]
-    t_strides = [get_broadcast_strides_2(out_shape, b.shape, b.stride) for b in tens]
-    cshape, cstr = collapse_dims(out_shape, calculate_stride(out_shape), *t_strides)
-    modes: list | None = []
-    C = cshape[-1] if len(cshape) == 2 else 1
-    it = iter(cstr[1:])
-    if len(cshape) <= 2:
-        full = (C, 1) if len(cshape) == 2 else (1,)
-        for b in operands:
-            if b.is_host_scalar:
-                modes.append("sval")
-                continue
-            st = next(it)
-            if st == full:
-                modes.append("vec")
-            elif not any(st):
-                modes.append("sptr")
-            elif st == (1, 0):
-                modes.append("row")
-            elif st == (0, 1):
-                modes.append("col")
-            else:
-                modes = None
-                break
+    args = [float(b.ptr.value) if sc else b.ptr.addr for b, sc in zip(operands, plan.is_scalar)]
+    var = plan.wide
+    if var is not None:
+        if out.addr & 15:
+            var = plan.narrow
+        else:
+            for a, needs in zip(args, var[4]):
+                if needs and a & 15:
+                    var = plan.narrow
+                    break
     else:
-        modes = None
-    vals = tuple(float(s) for s in svals)
-    if modes is not None:
-        wide = all(_addr(b) % 16 == 0 for b, m in zip(operands, modes) if m in ("vec", "col")) \
-            and out.addr % 16 == 0 and (C % 4 == 0 or not any(m in ("row", "col") for m in modes))
-        vec = 4 if wide else 1
-        k = kernel(K.map_kernel, tag, expr, tuple(modes), vec, len(vals))
-        args = [float(b.ptr.value) if b.is_host_scalar else _addr(b) for b in operands]
-        launch(k, K.map_grid(n, vec), 256, *args, *vals, out.addr, n, C)
-    else:
-        sval = tuple(b.is_host_scalar for b in operands)
-        k = kernel(K.strided_map_kernel, tag, expr, len(operands), sval, len(vals))
-        args = [float(b.ptr.value) if b.is_host_scalar else _addr(b) for b in operands]
-        st_args = [x for st in t_strides for x in _pad4(st, 0)]
-        launch(k, (n + 1023) // 1024, 256, *args, *vals, out.addr, n, *_pad4(out_shape, 1), *st_args)
+        var = plan.narrow
+    k = var[3]
+    if k is None:
+        k = var[3] = kernel(*var[0])
+    launch(k, var[1], 256, *args, *[float(v) for v in svals], out.addr, *var[2])
     return out
 
 
@@ -664,6 +705,22 @@ class HIP:
             return _map("cegrad_v", expr.format(g="s1"), [lsm, rows], lsm.shape,
                         (n, float(upstream.ptr.value)))
         return _map("cegrad_p", expr.format(g="x2"), [lsm, rows, upstream], lsm.shape, (n,))
+
+    # ---- fused optimizer step -----------------------------------------------------------------------------------------------
+    @staticmethod
+    @dispatcher.register(CustomOps.ADAM_STEP, Device.HIP)
+    def adam_step(p: Buffer, g: Buffer, m: Buffer, v: Buffer, consts: tuple) -> tuple[DevicePtr, DevicePtr, DevicePtr]:
+        """consts = (b1, 1-b1, b2, 1-b2, 1-b1^t, 1-b2^t, eps, lr), each rounded to fp32 exactly
+        where the op-by-op path rounds it (a Python float entering a kernel by value)."""
+        n = p.numel
+        outs = (alloc(n), alloc(n), alloc(n))
+        if n == 0:
+            return outs
+        addrs = [_addr(b) for b in (p, g, m, v)] + [o.addr for o in outs]
+        vec = 4 if not any(a & 15 for a in addrs) else 1
+        launch(kernel(K.adam_kernel, vec), max(1, ((n + vec - 1) // vec + 255) // 256), 256,
+               *addrs, n, *[float(c) for c in consts])
+        return outs
 
     # ---- matmul ----------------------------------------------------------------------------------------------------------
     MATMUL_FORCE = os.environ.get("DLGRAD_HIP_MATMUL_TILE")      # e.g. "128x128": benchmarking aid

@@ -217,3 +217,26 @@ def test_gpt_greedy_decode_hip_vs_cpu_oracle():
         outs[dev] = model.generate_greedy(0, 48)     # runs past block_size: exercises the crop
     if not hip.COMPILE_ONLY:
         assert outs["hip"] == outs["cpu"]
+
+
+@pytest.mark.gpu
+def test_fused_adam_kernel_is_bit_identical_to_the_fourteen_kernel_expression(monkeypatch):
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    from dlgrad_amd import ops
+    rng = np.random.default_rng(9)
+    results = {}
+    for fused in (True, False):
+        monkeypatch.setattr(ops, "FUSED", fused)
+        ps = [Tensor((rng2 := np.random.default_rng(10 + i)).standard_normal(shape).astype(np.float32),
+                     requires_grad=True, device="hip") for i, shape in enumerate([(65, 128), (1, 128), (7,), (513, 3)])]
+        opt = nn.optim.Adam(ps, lr=1e-3)
+        for step in range(3):
+            for i, p in enumerate(ps):
+                p.grad = Tensor(np.random.default_rng(100 * step + i).standard_normal(p.shape).astype(np.float32),
+                                device="hip")
+            opt.step()
+        results[fused] = [p.numpy() for p in ps] + [opt.m[id(p)].numpy() for p in ps] + [opt.v[id(p)].numpy() for p in ps]
+    if not hip.COMPILE_ONLY:
+        for a, b in zip(results[True], results[False]):
+            np.testing.assert_array_equal(a, b)
