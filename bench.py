@@ -196,6 +196,27 @@ def run_matmul(M: int, N: int, K: int, steps: int, warmup: int, seed: int = 3) -
             "bytes": 4.0 * (M * K + K * N + M * N)}
 
 
+def run_matmul_transposed(n: int) -> dict:
+    """The backward shapes A^T.G and G.B^T: as in the reference they are a materialised
+    transpose (permute kernel) followed by a plain GEMM; both launches are timed together."""
+    _, _, Buffer, Device, hip = _imports()
+    lib = hip.lib()
+    rng = np.random.default_rng(4)
+    a = Buffer.from_numpy(rng.standard_normal((n, n), dtype=np.float32) * np.float32(n ** -0.5), Device.HIP)
+    g = Buffer.from_numpy(rng.standard_normal((n, n), dtype=np.float32) * np.float32(n ** -0.5), Device.HIP)
+    out = {}
+    for name, f in ((f"{n}_TN_At.G", lambda: a.T @ g), (f"{n}_NT_G.Bt", lambda: g @ a.T)):
+        for _ in range(2):
+            f()
+        timer = EventTimer(lib)
+        for _ in range(5):
+            timer.run("mm", f)
+        lib.sync()
+        ms = float(np.mean(timer.collect()["mm"]))
+        out[name] = {"TFLOPs": round(2.0 * n ** 3 / ms / 1e9, 2), "ms_permute_plus_gemm": round(ms, 4)}
+    return out
+
+
 def cpu_matmul(n: int = 512) -> dict:
     from oracle import cref
     rng = np.random.default_rng(3)
@@ -296,6 +317,66 @@ def run_gpt(steps: int, warmup: int, cfg: dict = GPT_C4) -> dict:
     return {"ms_per_step": wall / steps * 1e3, "tokens_per_s": tokens * steps / wall,
             "launches_per_step": (hip.launch_count - n0) / steps, "loss_sum": float(loss.numpy()),
             "loss_per_token": float(loss.numpy()) / tokens}
+
+
+GPT_C5 = dict(vocab_size=50304, block_size=1024, n_layer=12, n_head=12, n_embd=768, batch_size=8)
+
+
+def run_gpt_large(steps: int = 2) -> dict:
+    """Scaled GPT (C5): one inference pass and `steps` training steps with Zipf(1.1) token ids.
+    There is no CPU figure beside it: the naive single-thread loops need ~7 TFLOP per step."""
+    Tensor, nn, _, _, hip = _imports()
+    from examples import gpt as G
+    lib = hip.lib()
+    c = G.GPTConfig(device="hip", **GPT_C5)
+    model = G.GPT(c)
+    G.init_weights_(model, 0)
+    rng = np.random.default_rng(7)
+    ids = np.minimum(rng.zipf(1.1, (2, c.batch_size, c.block_size)) - 1, c.vocab_size - 1).astype(np.float32)
+    idx, tgt = Tensor(ids[0], device="hip"), Tensor(ids[1], device="hip")
+    params = nn.utils.get_parameters(model)
+    opt = nn.optim.Adam(params, lr=c.learning_rate)
+    tokens = c.batch_size * c.block_size
+    model(idx)                                                    # warm-up, loads kernels
+    lib.sync()
+    t0 = time.perf_counter()
+    logits, _ = model(idx)
+    lib.sync()
+    t_inf = time.perf_counter() - t0
+    del logits
+    times, loss = [], None
+    for _ in range(steps + 1):
+        t0 = time.perf_counter()
+        opt.zero_grad()
+        _, loss = model(idx, tgt)
+        loss.backward()
+        opt.step()
+        lib.sync()
+        times.append(time.perf_counter() - t0)
+    n_params = sum(p.numel for p in params)
+    in_use, cached, _ = lib.pool_stats()
+    return {"params_M": round(n_params / 1e6, 1), "inference_ms": round(t_inf * 1e3, 2),
+            "inference_tokens_per_s": round(tokens / t_inf, 1),
+            "train_step_ms": round(min(times[1:]) * 1e3, 2), "train_tokens_per_s": round(tokens / min(times[1:]), 1),
+            "train_TFLOPs_est": round(6 * (n_params - c.vocab_size * c.n_embd - c.block_size * c.n_embd) * tokens
+                                      / min(times[1:]) / 1e12, 2),
+            "loss_per_token": round(float(loss.numpy()) / tokens, 4),
+            "pool_GiB": round((in_use + cached) / 2 ** 30, 1)}
+
+
+def run_decode(n_tokens: int = 256) -> dict:
+    """Greedy decode of the char-GPT from a 1-token prompt: full-context recompute per token."""
+    *_, hip = _imports()
+    from examples import gpt as G
+    model = G.GPT(G.GPTConfig(device="hip", **GPT_C4))
+    G.init_weights_(model, 0)
+    model.generate_greedy(0, 4)
+    hip.lib().sync()
+    t0 = time.perf_counter()
+    ids = model.generate_greedy(0, n_tokens)
+    dt = time.perf_counter() - t0
+    return {"tokens": n_tokens, "ms_per_token": round(dt / n_tokens * 1e3, 3), "tokens_per_s": round(n_tokens / dt, 1),
+            "first_ids": ids[:8]}
 
 
 def cpu_gpt(cfg: dict = GPT_C4) -> dict:
@@ -401,10 +482,14 @@ def main() -> None:
             for name, (M_, K_, N_) in (("16384x128.128x512", (16384, 128, 512)), ("2048x128.128x128", (2048, 128, 128))):
                 m = run_matmul(M_, N_, K_, 10, 2)
                 sweep[name] = {"TFLOPs": round(m["TFLOPs"], 2), "kernel_ms": round(m["kernel_ms"], 4)}
+            sweep.update(run_matmul_transposed(4096))
             extra["matmul_fp32_TFLOPs"] = sweep
             g = run_gpt(max(3, min(args.steps, 10)), 2)
             extra["gpt_char_fwd_bwd_adam"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in g.items()}
+            extra["gpt_char_greedy_decode_256"] = run_decode(256)
+            extra["mlp_784_64_10_step"] = {k: round(v, 3) for k, v in run_mlp(50, 5).items()}
             extra["c5_components"] = run_c5(max(3, min(args.steps, 10)), 2)
+            extra["gpt_scaled_c5"] = run_gpt_large(2)
             out["extra"] = extra
     elif args.workload == "matmul":
         n = 4096

@@ -270,7 +270,9 @@ class _MapPlan:
         if modes is not None:
             # (generator params, grid, trailing args); the kernel itself is loaded on first use
             if C % 4 == 0 or not any(m in ("row", "col") for m in modes):
-                self.wide = [(K.map_kernel, tag, expr, tuple(modes), 4, n_svals), K.map_grid(n, 4), (n, C), None,
+                # outputs too large to be re-read from cache are written with nontemporal stores
+                nt = n >= NT_STORE_MIN_ELEMENTS
+                self.wide = [(K.map_kernel, tag, expr, tuple(modes), 4, n_svals, 4, nt), K.map_grid(n, 4), (n, C), None,
                              tuple(m in ("vec", "col") for m in modes)]
             self.narrow = [(K.map_kernel, tag, expr, tuple(modes), 1, n_svals), K.map_grid(n, 1), (n, C), None, None]
         else:
@@ -280,6 +282,7 @@ class _MapPlan:
 
 
 _map_plans: dict = {}
+NT_STORE_MIN_ELEMENTS = int(os.environ.get("DLGRAD_HIP_NT_MIN", str(1 << 25)))   # 128 MiB of fp32
 
 
 def _map(tag: str, expr: str, operands: list[Buffer], out_shape: tuple, svals: tuple = (),
@@ -493,20 +496,28 @@ class HIP:
     # ---- reductions ------------------------------------------------------------------------------------
     @staticmethod
     def _reduce_full_into(kop: str, x_addr: int, n: int, divisor: float, out_addr: int) -> None:
+        """Two launches: blocks of 2048 vector items (32 KiB) -> partials -> one block."""
         vec = 4 if x_addr % 16 == 0 else 1
-        G = max(1, min(2048, n // (256 * 4 * 4)))
+        items = (n + vec - 1) // vec
+        G = (items + 2047) // 2048
         if G == 1:
-            launch(kernel(K.reduce_full_kernel, kop, vec), 1, 256, x_addr, out_addr, n, float(divisor))
+            launch(kernel(K.reduce_full_kernel, kop, vec), 1, 256, x_addr, out_addr, n, float(divisor), items)
             return
         part = alloc(G)
-        launch(kernel(K.reduce_full_kernel, kop, vec), G, 256, x_addr, part.addr, n, 1.0)
-        launch(kernel(K.reduce_full_kernel, kop, 4), 1, 256, part.addr, out_addr, G, float(divisor))
+        launch(kernel(K.reduce_full_kernel, kop, vec), G, 256, x_addr, part.addr, n, 1.0, 2048)
+        if G > 65536:                                    # > 537 M elements: fold the partials recursively
+            HIP._reduce_full_into(kop, part.addr, G, divisor, out_addr)
+            return
+        launch(kernel(K.reduce_full_kernel, kop, 4), 1, 256, part.addr, out_addr, G, float(divisor), (G + 3) // 4)
 
     @staticmethod
     def _reduce_cols(kop: str, x_addr: int, O: int, L: int, I: int, divisor: float, out_addr: int) -> None:
+        """Rows are split into chunks so that about 16 K blocks exist (measured optimum for a
+        512 MiB input) while a chunk keeps >= 32 rows, which bounds the partials at ~3 % of
+        the input; the partials are reduced by the same kernel."""
         vec = 4 if (I % 4 == 0 and x_addr % 16 == 0 and out_addr % 16 == 0) else 1
         bx = (I + 64 * vec - 1) // (64 * vec)
-        chunks = max(1, min(2048 // max(1, bx * O), L // 32))
+        chunks = max(1, min(16384 // max(1, bx * O), L // 32))
         chunk = (L + chunks - 1) // chunks
         chunk = (chunk + 3) // 4 * 4
         chunks = (L + chunk - 1) // chunk
@@ -667,13 +678,13 @@ class HIP:
         if x.numel == 0:
             return out if target is None else (out, picked)
         vec = 4 if (L % 4 == 0 and _addr(x) % 16 == 0 and out.addr % 16 == 0) else 1
-        blk, nval = K.softmax_plan(L, vec)
-        k = kernel(K.softmax_rows_kernel, log, vec, blk, nval, target is not None)
+        blk, nval, threads = K.softmax_plan(L, vec)
+        k = kernel(K.softmax_rows_kernel, log, vec, blk, nval, target is not None, threads)
         grid = R if blk else (R + 3) // 4
         if target is None:
-            launch(k, grid, 256, _addr(x), out.addr, R, L)
+            launch(k, grid, threads, _addr(x), out.addr, R, L)
             return out
-        launch(k, grid, 256, _addr(x), out.addr, R, L, _addr(target), picked.addr)
+        launch(k, grid, threads, _addr(x), out.addr, R, L, _addr(target), picked.addr)
         return out, picked
 
     @staticmethod
