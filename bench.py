@@ -14,6 +14,8 @@ seeded input that is already resident in HBM when the timed region starts.
   gpt                char-GPT (vocab 65, block 128, 6 layers, 4 heads, n_embd 128, batch 16):
                      forward + backward + Adam step.  value = tokens/s.
   mlp                784-64-10 MLP, batch 128: forward + backward + SGD step.  value = samples/s.
+  gpt-large          scaled GPT (vocab 50304, block 1024, 12 layers, 12 heads, n_embd 768, batch 8),
+                     Zipf(1.1) ids: forward + backward + Adam step.  value = tokens/s.
 
 Unless --no-extra is given, the default run also reports the matmul sweep, the GPT step and
 the 4096^2 / 1024^2 suites under "extra", so one run carries every headline figure.
@@ -426,7 +428,7 @@ def main() -> None:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=["c2", "matmul", "gpt", "mlp"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "matmul", "gpt", "mlp", "gpt-large"])
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
@@ -512,6 +514,13 @@ def main() -> None:
                "roofline": None}
         if not args.no_cpu:
             out["cpu_baseline"] = cpu_gpt()
+    elif args.workload == "gpt-large":
+        g = run_gpt_large(max(1, min(args.steps, 5)))
+        out = {"metric": "scaled GPT fwd+bwd tokens/s (1 GPU)", "value": g["train_tokens_per_s"], "unit": "tokens/s",
+               **base, "ms_per_step": g["train_step_ms"],
+               "config": {"workload": "C5 scaled GPT vocab 50304, block 1024, 12 layers, 12 heads, n_embd 768, batch 8; "
+                                      "Zipf(1.1) token ids; forward + backward + Adam step", **g},
+               "roofline": None}
     else:
         r = run_mlp(args.steps, args.warmup)
         out = {"metric": "MLP 784-64-10 step samples/s (1 GPU)", "value": r["samples_per_s"], "unit": "samples/s",

@@ -1025,13 +1025,24 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
     return src, name, _fmt("P", "P", "P", "8I")
 
 
-# name -> (WM, WN, MI, NJ, BK): block tile = (32*MI*WM) x (32*NJ*WN), 64*WM*WN threads
+# name -> (WM, WN, MI, NJ, BK): block tile = (32*MI*WM) x (32*NJ*WN), 64*WM*WN threads.
+# Chosen from a sweep on MI355X (TFLOP/s at 4096^3 / 8192x3072x768 / 2048^3):
+#   256x256 (8 waves, 128 acc regs)   136 / 100 / 34     largest problems, one block per CU
+#   256x128 (4 waves, 128 acc regs)   135 /  92 / 58
+#   128x256 (8 waves,  64 acc regs)   129 / 124 / 64     mid-size N
+#   128x128 (4 waves of 64x64)        128 / 122 / 104    default below ~512 tiles
 MATMUL_CONFIGS = {
-    "128x128": (4, 1, 1, 4, 32),
-    "128x256": (2, 2, 2, 4, 16),
-    "64x128": (2, 1, 1, 4, 32),
+    "256x256": (4, 2, 2, 4, 16),
+    "256x128": (4, 1, 2, 4, 16),
+    "128x256": (4, 2, 1, 4, 32),
+    "128x128": (2, 2, 2, 2, 32),
     "64x64": (2, 2, 1, 1, 16),
     "32x32": (1, 1, 1, 1, 16),
+}
+# (relative per-CU throughput when the chip is full, resident blocks per CU)
+MATMUL_TILE_MODEL = {
+    "256x256": (1.00, 1), "256x128": (0.99, 2), "128x256": (0.95, 1), "128x128": (0.94, 2),
+    "64x64": (0.79, 8), "32x32": (0.65, 8),
 }
 
 

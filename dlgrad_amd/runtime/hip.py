@@ -736,21 +736,21 @@ class HIP:
     # ---- matmul ----------------------------------------------------------------------------------------------------------
     MATMUL_FORCE = os.environ.get("DLGRAD_HIP_MATMUL_TILE")      # e.g. "128x128": benchmarking aid
 
-    # relative per-CU throughput of each tile shape, measured on 4096^3 (larger = faster)
-    _TILE_RATE = {"128x256": 0.95, "128x128": 1.0, "64x128": 0.67, "64x64": 0.83, "32x32": 0.68}
-
     @staticmethod
     def _pick_tile(M: int, N: int, batch: int) -> str:
         """Largest expected throughput = tile rate x fraction of the tile grid that is real
-        output x fraction of the 256 CUs that get a block."""
+        output x how well the block count fills 256 CUs (one block per CU already runs a CU
+        near its rate; beyond the resident capacity, whole rounds of blocks are paid for)."""
         if HIP.MATMUL_FORCE:
             return HIP.MATMUL_FORCE
         best, best_score = "64x64", -1.0
-        for name, rate in HIP._TILE_RATE.items():
+        for name, (rate, per_cu) in K.MATMUL_TILE_MODEL.items():
             bm, bn = (int(v) for v in name.split("x"))
             tm, tn = (M + bm - 1) // bm, (N + bn - 1) // bn
-            eff = (M * N) / float(tm * bm * tn * bn)
-            score = rate * eff * min(1.0, tm * tn * batch / 256.0)
+            nblk = tm * tn * batch
+            slots = 256 * per_cu
+            fill = min(1.0, nblk / 256.0) if nblk <= slots else nblk / float(-(-nblk // slots) * slots)
+            score = rate * (M * N) / float(tm * bm * tn * bn) * fill
             if score > best_score * 1.0001:
                 best, best_score = name, score
         return best

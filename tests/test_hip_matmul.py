@@ -79,7 +79,7 @@ def test_matmul_lower_rank_right_operand_is_padded():
     check_mm(dev(x).matmul(dev(w)).numpy(), x.astype(np.float64) @ w, "3d @ 2d")
 
 
-@pytest.mark.parametrize("tile", ["32x32", "64x64", "64x128", "128x128", "128x256"])
+@pytest.mark.parametrize("tile", list(__import__("dlgrad_amd.codegen.hip_kernel", fromlist=["x"]).MATMUL_CONFIGS))
 @pytest.mark.parametrize("mnk", [(256, 256, 256), (130, 70, 50), (512, 384, 1000)])
 def test_every_tile_configuration(tile, mnk, monkeypatch):
     require_gpu()
