@@ -425,16 +425,16 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 
 
 @cache
-def reduce_cols_kernel(op: str, vec: int) -> tuple[str, str, str]:
+def reduce_cols_kernel(op: str, vec: int, ty: int = 4) -> tuple[str, str, str]:
     """out[o, c, i] = reduce over l in chunk c of x[o, l, i] for an (O, L, I) view, / divisor
     (the non-last-axis case of cpu_kernel.py:68-148, e.g. axis 0 of a matrix).
 
-    The reference walks each column with stride I.  Here a 64x4 block owns 64*vec
-    adjacent columns: lanes read consecutive addresses of one row (coalesced), the
-    four thread rows take every fourth row of the chunk, and LDS joins them.  L is
+    The reference walks each column with stride I.  Here a 64 x ty block (ty = 4 or 16)
+    owns 64*vec adjacent columns: lanes read consecutive addresses of one row (coalesced),
+    the ty thread rows take every ty-th row of the chunk, and LDS joins them.  L is
     split into `chunks` so that tall, narrow inputs still fill the chip; the launcher
     reduces the (O, chunks, I) partials with a second call."""
-    name = f"reduce_cols_{op}_v{vec}"
+    name = f"reduce_cols_{op}_v{vec}_y{ty}"
     if vec == 4:
         defs = """#define VT float4
 #define LD(l) (reinterpret_cast<const float4*>(xp + (u64)(l) * I)[0])
@@ -450,9 +450,9 @@ def reduce_cols_kernel(op: str, vec: int) -> tuple[str, str, str]:
 #define STORE(p, r) { (p)[0] = r / divisor; }
 """
     src = f"""{PRELUDE}{_red_defs(op)}{defs}
-extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+extern "C" __global__ __launch_bounds__({64 * ty}) void {name}(const float* __restrict__ x,
         float* __restrict__ out, u32 L, u32 I, u32 chunk, float divisor) {{
-    __shared__ VT sm[4][64];
+    __shared__ VT sm[{ty}][64];
     const u32 tx = threadIdx.x, ty = threadIdx.y, o = blockIdx.z;
     const u32 col = (blockIdx.x * 64u + tx) * {vec}u;
     const u32 l0 = blockIdx.y * chunk, l1 = min(L, l0 + chunk);
@@ -460,11 +460,11 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
     if (col < I) {{
         const float* __restrict__ xp = x + (u64)o * L * I + col;
         u32 l = l0 + ty;
-        for (; l + 12u < l1; l += 16u) {{
-            const VT t0 = LD(l), t1 = LD(l + 4u), t2 = LD(l + 8u), t3 = LD(l + 12u);
+        for (; l + {3 * ty}u < l1; l += {4 * ty}u) {{
+            const VT t0 = LD(l), t1 = LD(l + {ty}u), t2 = LD(l + {2 * ty}u), t3 = LD(l + {3 * ty}u);
             ACC(a0, t0) ACC(a1, t1) ACC(a2, t2) ACC(a3, t3)
         }}
-        for (; l < l1; l += 4u) {{ const VT t0 = LD(l); ACC(a0, t0) }}
+        for (; l < l1; l += {ty}u) {{ const VT t0 = LD(l); ACC(a0, t0) }}
         ACC(a0, a1) ACC(a2, a3) ACC(a0, a2)
     }}
     sm[ty][tx] = a0;
@@ -472,7 +472,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
     if (ty == 0 && col < I) {{
         VT r = sm[0][tx];
         #pragma unroll
-        for (int k = 1; k < 4; ++k) {{ const VT t = sm[k][tx]; ACC(r, t) }}
+        for (int k = 1; k < {ty}; ++k) {{ const VT t = sm[k][tx]; ACC(r, t) }}
         STORE(out + ((u64)o * gridDim.y + blockIdx.y) * I + col, r)
     }}
 }}
@@ -651,6 +651,124 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
 }}
 """
     return src, name, _fmt("P", "P", "P", "I", "I")
+
+
+_ORDERED_COMPACT = r"""
+// Appends, in increasing j, the positions of [lo, hi) whose id equals `my` (and, if flags is
+// given, whose flag is set) to list[]; returns the count.  256 threads; thread t owns the
+// contiguous slice [lo + t*len, lo + (t+1)*len), counts its matches, a block-wide exclusive
+// prefix sum (wave scan + LDS) turns the counts into offsets, a second walk writes them.
+static __device__ __forceinline__ u32 collect(const float* __restrict__ idx, const u32* __restrict__ flags,
+                                              int my, u32 lo, u32 hi, u32* list, u32* wcount) {
+    const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    const u32 len = (hi - lo + 255u) >> 8;
+    const u32 a = min(hi, lo + tid * len), b = min(hi, a + len);
+    u32 mine = 0;
+    for (u32 j = a; j < b; ++j) mine += ((int)idx[j] == my && (flags == nullptr || flags[j] != 0u)) ? 1u : 0u;
+    u32 inc = mine;
+    #pragma unroll
+    for (int off = 1; off < 64; off <<= 1) { const u32 v = __shfl_up(inc, off, WAVE); if ((int)lane >= off) inc += v; }
+    __syncthreads();                                  // wcount may still be read by an earlier call
+    if (lane == 63u) wcount[w] = inc;
+    __syncthreads();
+    u32 pos = inc - mine;
+    for (u32 k = 0; k < w; ++k) pos += wcount[k];
+    const u32 total = wcount[0] + wcount[1] + wcount[2] + wcount[3];
+    for (u32 j = a; j < b; ++j)
+        if ((int)idx[j] == my && (flags == nullptr || flags[j] != 0u)) list[pos++] = j;
+    __syncthreads();
+    return total;
+}
+"""
+
+EMB_SEGMENT = 512          # positions per segment of the ordered scatter-add
+EMB_ORDERED_MAX = 32768    # at most 64 segments, so a merge list fits 64 entries
+
+
+@cache
+def embedding_backward_ordered_kernel(merge: bool, vec: int = 1) -> tuple[str, str, str]:
+    """Deterministic scatter-add for up to EMB_ORDERED_MAX indices, without atomics.
+
+    The index array is cut into segments of EMB_SEGMENT positions.  Pass 1 (one block per
+    position i): the block whose position is the first occurrence of its id inside its
+    segment adds the rows of that id's occurrences in the segment, in index order, starting
+    from 0 -- exactly the order of the reference's loop (cpu_kernel.py:231-243).  If the id
+    occurs in no other segment the sum is the final table row; otherwise it goes to
+    partial[i], and the block records itself in segpos[f][segment] where f is the id's first
+    position overall (scratch: flag[n], segpos[n][64], zeroed by the launcher).  Pass 2
+    (merge=True): block f of every id that spans segments adds that id's partial rows in
+    segment order.  Ids confined to one segment are therefore bit-identical to the
+    sequential reference; ids that span segments differ from it only in where the
+    parentheses fall, and every run gives the same bits.  A hot id's work is spread over
+    segments instead of serialising on one address as atomics do.  vec=4 moves rows as
+    float4 (W % 4 == 0, aligned bases)."""
+    name = f"embedding_scatter_{'merge' if merge else 'ordered'}_v{vec}"
+    VT = "float4" if vec == 4 else "float"
+    zero = "make_float4(0.f, 0.f, 0.f, 0.f)" if vec == 4 else "0.0f"
+    add = ("acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;" if vec == 4 else "acc += t;")
+    if not merge:
+        body = f"""
+extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out,
+        float* __restrict__ partial, u32* __restrict__ flag, u32* __restrict__ segpos,
+        const float* __restrict__ g, const float* __restrict__ idx, u32 n, u32 W) {{
+    __shared__ u32 list[{EMB_SEGMENT}];
+    __shared__ u32 wcount[4];
+    __shared__ u32 first;
+    const u32 i = blockIdx.x, tid = threadIdx.x;
+    const int my = (int)idx[i];
+    const u32 seg = i / {EMB_SEGMENT}u, s0 = seg * {EMB_SEGMENT}u, s1 = min(n, s0 + {EMB_SEGMENT}u);
+    int dup = 0;
+    for (u32 j = s0 + tid; j < i; j += 256u) dup |= ((int)idx[j] == my);
+    if (tid == 0) first = 0xFFFFFFFFu;
+    if (__syncthreads_or(dup)) return;                       // not the first of its id in this segment
+    const u32 m = collect(idx, nullptr, my, i, s1, list, wcount);
+    int other = 0;
+    u32 lowest = 0xFFFFFFFFu;
+    for (u32 j = tid; j < n; j += 256u)
+        if ((int)idx[j] == my) {{ lowest = min(lowest, j); other |= (j < s0 || j >= s1); }}
+    if (lowest != 0xFFFFFFFFu) atomicMin(&first, lowest);    // LDS atomic
+    other = __syncthreads_or(other);
+    {VT}* __restrict__ dst = reinterpret_cast<{VT}*>(other ? partial + (u64)i * W : out + (long long)my * W);
+    const u32 Wv = W / {vec}u;
+    for (u32 c = tid; c < Wv; c += 256u) {{
+        {VT} acc = {zero};
+        #pragma unroll 8
+        for (u32 q = 0; q < m; ++q) {{ const {VT} t = reinterpret_cast<const {VT}*>(g + (u64)list[q] * W)[c]; {add} }}
+        dst[c] = acc;
+    }}
+    if (other && tid == 0) {{ segpos[(u64)first * 64u + seg] = i + 1u; flag[first] = 1u; }}
+}}
+"""
+        fmt = _fmt("P", "P", "P", "P", "P", "P", "I", "I")
+    else:
+        body = f"""
+extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out,
+        const float* __restrict__ partial, const u32* __restrict__ flag, const u32* __restrict__ segpos,
+        const float* __restrict__ idx, u32 n, u32 W) {{
+    __shared__ u32 list[64];
+    __shared__ u32 cnt;
+    const u32 i = blockIdx.x, tid = threadIdx.x;
+    if (flag[i] == 0u) return;                               // only the first position of a spanning id works
+    if (tid < 64u) {{
+        const u32 p = segpos[(u64)i * 64u + tid];
+        const u64 bal = __ballot(p != 0u);
+        if (p != 0u) list[__popcll(bal & ((1ull << tid) - 1ull))] = p - 1u;
+        if (tid == 0) cnt = (u32)__popcll(bal);
+    }}
+    __syncthreads();
+    const u32 m = cnt;
+    {VT}* __restrict__ dst = reinterpret_cast<{VT}*>(out + (long long)(int)idx[i] * W);
+    const u32 Wv = W / {vec}u;
+    for (u32 c = tid; c < Wv; c += 256u) {{
+        {VT} acc = reinterpret_cast<const {VT}*>(partial + (u64)list[0] * W)[c];
+        #pragma unroll 8
+        for (u32 q = 1; q < m; ++q) {{ const {VT} t = reinterpret_cast<const {VT}*>(partial + (u64)list[q] * W)[c]; {add} }}
+        dst[c] = acc;
+    }}
+}}
+"""
+        fmt = _fmt("P", "P", "P", "P", "P", "I", "I")
+    return f"{PRELUDE}{_ORDERED_COMPACT}{body}", name, fmt
 
 
 @cache

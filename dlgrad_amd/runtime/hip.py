@@ -282,6 +282,7 @@ class _MapPlan:
 
 
 _map_plans: dict = {}
+EMB_ORDERED = os.environ.get("DLGRAD_HIP_EMB_ORDERED", "1") != "0"     # 0: fp32 atomics for every size
 NT_STORE_MIN_ELEMENTS = int(os.environ.get("DLGRAD_HIP_NT_MIN", str(1 << 25)))   # 128 MiB of fp32
 
 
@@ -512,21 +513,22 @@ class HIP:
 
     @staticmethod
     def _reduce_cols(kop: str, x_addr: int, O: int, L: int, I: int, divisor: float, out_addr: int) -> None:
-        """Rows are split into chunks so that about 16 K blocks exist (measured optimum for a
-        512 MiB input) while a chunk keeps >= 32 rows, which bounds the partials at ~3 % of
-        the input; the partials are reduced by the same kernel."""
+        """Up to 512 rows are folded by one launch of 64x16 blocks.  Taller inputs are split
+        into chunks of >= 64 rows (4 loads per thread) sized so that about 8 M threads exist
+        (the measured optimum on a 512 MiB input), which bounds the partials at 1.6 % of the input; the same kernel then folds the
+        (O, chunks, I) partials."""
         vec = 4 if (I % 4 == 0 and x_addr % 16 == 0 and out_addr % 16 == 0) else 1
         bx = (I + 64 * vec - 1) // (64 * vec)
-        chunks = max(1, min(16384 // max(1, bx * O), L // 32))
-        chunk = (L + chunks - 1) // chunks
-        chunk = (chunk + 3) // 4 * 4
-        chunks = (L + chunk - 1) // chunk
-        k = kernel(K.reduce_cols_kernel, kop, vec)
+        ty = 16 if L > 64 else 4
+        k = kernel(K.reduce_cols_kernel, kop, vec, ty)
+        chunks = 1 if L <= 512 else max(1, min(8192 // max(1, bx * O), L // 64))
         if chunks == 1:
-            launch(k, (bx, 1, O), (64, 4, 1), x_addr, out_addr, L, I, L, float(divisor))
+            launch(k, (bx, 1, O), (64, ty, 1), x_addr, out_addr, L, I, L, float(divisor))
             return
+        chunk = ((L + chunks - 1) // chunks + 15) // 16 * 16
+        chunks = (L + chunk - 1) // chunk
         part = alloc(O * chunks * I)
-        launch(k, (bx, chunks, O), (64, 4, 1), x_addr, part.addr, L, I, chunk, 1.0)
+        launch(k, (bx, chunks, O), (64, ty, 1), x_addr, part.addr, L, I, chunk, 1.0)
         HIP._reduce_cols(kop, part.addr, O, chunks, I, divisor, out_addr)
 
     @staticmethod
@@ -638,9 +640,21 @@ class HIP:
         W, n_idx = x.shape[-1], idx.numel
         if backward:
             out = alloc(x.numel, zero=True)                    # init_with_scalar(0), cpu.py:1031
-            if n_idx:
-                launch(kernel(K.embedding_backward_kernel), (n_idx + 3) // 4, 256,
-                       out.addr, _addr(upstream_grad), _addr(idx), n_idx, W)
+            if not n_idx:
+                return out
+            if n_idx <= K.EMB_ORDERED_MAX and EMB_ORDERED:
+                # ordered, atomic-free: same bits every run (and the reference's bits for ids
+                # that stay inside one 512-position segment)
+                partial, scratch = alloc(n_idx * W), alloc(n_idx * 65, zero=True)   # flag[n] then segpos[n][64]
+                flag, segpos = scratch.addr, scratch.addr + 4 * n_idx
+                vec = 4 if (W % 4 == 0 and not (_addr(upstream_grad) | out.addr | partial.addr) & 15) else 1
+                launch(kernel(K.embedding_backward_ordered_kernel, False, vec), n_idx, 256, out.addr, partial.addr,
+                       flag, segpos, _addr(upstream_grad), _addr(idx), n_idx, W)
+                launch(kernel(K.embedding_backward_ordered_kernel, True, vec), n_idx, 256, out.addr, partial.addr,
+                       flag, segpos, _addr(idx), n_idx, W)
+                return out
+            launch(kernel(K.embedding_backward_kernel), (n_idx + 3) // 4, 256,
+                   out.addr, _addr(upstream_grad), _addr(idx), n_idx, W)
             return out
         out = alloc(out_numel)
         if n_idx:
