@@ -337,6 +337,16 @@ class Buffer:
         ptrs = self._dispatch(CustomOps.ADAM_STEP, p=self, g=g, m=m, v=v, consts=consts)
         return tuple(self._like(q) for q in ptrs)
 
+    def adam_step_(self, g: "Buffer", m: "Buffer", v: "Buffer", consts: "Buffer") -> None:
+        """In-place Adam update of self, m and v with the constants held in device memory."""
+        self._dispatch(CustomOps.ADAM_STEP_INPLACE, p=self, g=g, m=m, v=v, consts=consts)
+
+    def upload_(self, arr: np.ndarray) -> None:
+        """Overwrites this Buffer's memory with `arr` (same element count); the address stays."""
+        if arr.size != self.numel:
+            raise ValueError(f"Buffer size mismatch! Expected {self.numel} elements, got {arr.size}")
+        self._dispatch(BufferOps.CREATE, data=arr, into=self)
+
     # ---- binary -----------------------------------------------------------------------------------------
     def _binary_op(self, other: "Buffer", op: BinaryOps) -> "Buffer":
         """x is the operand with more elements and fixes the output shape (buffer.py:402-448).

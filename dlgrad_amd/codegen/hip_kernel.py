@@ -1169,6 +1169,53 @@ MATMUL_TILE_MODEL = {
 # =====================================================================================
 
 @cache
+def adam_inplace_kernel(vec: int) -> tuple[str, str, str]:
+    """adam_kernel's arithmetic applied in place to p, m and v, with the eight constants read
+    from device memory.  This is the form a captured graph can replay: the addresses never
+    change and the step-dependent bias corrections are refreshed by a small upload before
+    each replay instead of being frozen into the kernel arguments."""
+    src, name, _ = adam_kernel(vec)
+    name2 = f"adam_step_inplace_v{vec}"
+    i = src.index('extern "C"')
+    head = src[:i]
+    if vec == 4:
+        body = """
+    const AdamArgs a = *ap;
+    const u32 nv = n >> 2;
+    const u32 i = blockIdx.x * 256u + threadIdx.x;
+    if (i < nv) {
+        const float4 p4 = reinterpret_cast<float4*>(p)[i], g4 = reinterpret_cast<const float4*>(g)[i];
+        const float4 m4 = reinterpret_cast<float4*>(m)[i], v4 = reinterpret_cast<float4*>(v)[i];
+        float4 po, mo, vo;
+        adam1(p4.x, g4.x, m4.x, v4.x, a, po.x, mo.x, vo.x);
+        adam1(p4.y, g4.y, m4.y, v4.y, a, po.y, mo.y, vo.y);
+        adam1(p4.z, g4.z, m4.z, v4.z, a, po.z, mo.z, vo.z);
+        adam1(p4.w, g4.w, m4.w, v4.w, a, po.w, mo.w, vo.w);
+        reinterpret_cast<float4*>(p)[i] = po;
+        reinterpret_cast<float4*>(m)[i] = mo;
+        reinterpret_cast<float4*>(v)[i] = vo;
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {
+        const u32 j = (nv << 2) + threadIdx.x;
+        float po, mo, vo;
+        adam1(p[j], g[j], m[j], v[j], a, po, mo, vo);
+        p[j] = po; m[j] = mo; v[j] = vo;
+    }
+"""
+    else:
+        body = """
+    const AdamArgs a = *ap;
+    const u32 j = blockIdx.x * 256u + threadIdx.x;
+    if (j < n) { float po, mo, vo; adam1(p[j], g[j], m[j], v[j], a, po, mo, vo); p[j] = po; m[j] = mo; v[j] = vo; }
+"""
+    src2 = f"""{head}extern "C" __global__ __launch_bounds__(256) void {name2}(float* p, const float* __restrict__ g,
+        float* m, float* v, u32 n, const AdamArgs* __restrict__ ap) {{
+{body}}}
+"""
+    return src2, name2, _fmt("P", "P", "P", "P", "I", "P")
+
+
+@cache
 def adam_kernel(vec: int) -> tuple[str, str, str]:
     """One Adam update of one parameter tensor: the fourteen element-wise kernels of
     dlgrad/nn/optim.py:59-70 in a single pass, writing new p, m and v buffers.

@@ -43,9 +43,17 @@ std::vector<Kernel> g_kernels;                   // handle = index + 1
 std::vector<hipModule_t> g_modules;
 
 // ---- allocator state --------------------------------------------------------
-std::map<size_t, std::vector<void *>> g_free;    // bucket size -> cached blocks
-std::unordered_map<void *, size_t> g_live;       // block -> bucket size
+// Arena 0 is the ordinary pool.  Other arenas are private pools for captured graphs: a
+// block handed out while an arena is current returns to that arena when freed and is
+// never given to anybody else, because a graph replays writes to its addresses.
+struct Block { size_t bucket; uint64_t arena; };
+std::map<uint64_t, std::map<size_t, std::vector<void *>>> g_free;   // arena -> bucket -> cached blocks
+std::unordered_map<void *, Block> g_live;                            // block -> bucket, arena
+std::map<uint64_t, bool> g_arena_alive;                              // arenas that still exist
+uint64_t g_arena = 0, g_next_arena = 1;
 uint64_t g_bytes_in_use = 0, g_bytes_cached = 0, g_device_allocs = 0;
+bool g_capturing = false;
+std::vector<hipGraphExec_t> g_graphs;                                // handle = index + 1 (null once destroyed)
 
 int fail(const char *what, hipError_t e) {
     char buf[512];
@@ -79,17 +87,26 @@ size_t bucket_of(size_t n) {
     return (n + mib - 1) / mib * mib;
 }
 
-void trim_locked() {
-    for (auto &kv : g_free)
-        for (void *p : kv.second) (void)hipFree(p);
-    g_free.clear();
-    g_bytes_cached = 0;
+void trim_arena_locked(uint64_t arena) {
+    auto it = g_free.find(arena);
+    if (it == g_free.end()) return;
+    for (auto &kv : it->second)
+        for (void *p : kv.second) {
+            (void)hipFree(p);
+            g_bytes_cached -= kv.first;
+        }
+    g_free.erase(it);
+}
+
+void trim_locked() {                              // the ordinary pool only: graph arenas keep their blocks
+    trim_arena_locked(0);
 }
 
 int alloc_locked(size_t nbytes, void **out) {
     size_t b = bucket_of(nbytes);
-    auto it = g_free.find(b);
-    if (it != g_free.end() && !it->second.empty()) {
+    auto &lists = g_free[g_arena];
+    auto it = lists.find(b);
+    if (it != lists.end() && !it->second.empty()) {
         *out = it->second.back();
         it->second.pop_back();
         g_bytes_cached -= b;
@@ -112,7 +129,7 @@ int alloc_locked(size_t nbytes, void **out) {
         ++g_device_allocs;
         *out = p;
     }
-    g_live[*out] = b;
+    g_live[*out] = Block{b, g_arena};
     g_bytes_in_use += b;
     return 0;
 }
@@ -159,7 +176,11 @@ int dlg_hip_shutdown(void) {
     std::lock_guard<std::mutex> lk(g_mu);
     if (!g_inited) return 0;
     (void)hipStreamSynchronize(g_stream);
-    trim_locked();
+    for (hipGraphExec_t ge : g_graphs) if (ge) (void)hipGraphExecDestroy(ge);
+    g_graphs.clear();
+    while (!g_free.empty()) trim_arena_locked(g_free.begin()->first);
+    g_arena = 0;
+    g_capturing = false;
     for (hipModule_t m : g_modules) (void)hipModuleUnload(m);
     g_modules.clear();
     g_kernels.clear();
@@ -206,6 +227,7 @@ int dlg_hip_alloc_zero(size_t nbytes, void **out) {
         int rc = alloc_locked(nbytes, out);
         if (rc) return rc;
     }
+    if (g_capturing) return fail_msg(-9, "dlg_hip_alloc_zero records a memset node; clear with a kernel while capturing");
     if (nbytes) HIP_TRY(hipMemsetAsync(*out, 0, nbytes, g_stream));
     return 0;
 }
@@ -213,6 +235,7 @@ int dlg_hip_alloc_zero(size_t nbytes, void **out) {
 int dlg_hip_fill_f32(void *dst, float value, size_t count) {
     NEED_INIT();
     if (!count) return 0;
+    if (g_capturing) return fail_msg(-9, "dlg_hip_fill_f32 records a memset node; fill with a kernel while capturing");
     uint32_t bits;
     std::memcpy(&bits, &value, 4);
     HIP_TRY(hipMemsetD32Async((hipDeviceptr_t)dst, (int)bits, count, g_stream));
@@ -225,11 +248,15 @@ int dlg_hip_free(void *ptr) {
     if (!g_inited) return 0;                  // after shutdown the driver owns nothing
     auto it = g_live.find(ptr);
     if (it == g_live.end()) return fail_msg(-7, "dlg_hip_free: pointer was not allocated here");
-    size_t b = it->second;
+    Block blk = it->second;
     g_live.erase(it);
-    g_bytes_in_use -= b;
-    g_free[b].push_back(ptr);
-    g_bytes_cached += b;
+    g_bytes_in_use -= blk.bucket;
+    if (blk.arena != 0 && !g_arena_alive[blk.arena]) {      // its graph is gone: give the memory back
+        (void)hipFree(ptr);
+        return 0;
+    }
+    g_free[blk.arena][blk.bucket].push_back(ptr);
+    g_bytes_cached += blk.bucket;
     return 0;
 }
 
@@ -254,6 +281,7 @@ int dlg_hip_pool_trim(void) {
 int dlg_hip_h2d(void *dst, const void *src, size_t n) {
     NEED_INIT();
     if (!n) return 0;
+    if (g_capturing) return fail_msg(-9, "dlg_hip_h2d is a synchronous transfer and cannot be part of a captured graph");
     HIP_TRY(hipMemcpyAsync(dst, src, n, hipMemcpyHostToDevice, g_stream));
     HIP_TRY(hipStreamSynchronize(g_stream));
     return 0;
@@ -262,6 +290,7 @@ int dlg_hip_h2d(void *dst, const void *src, size_t n) {
 int dlg_hip_d2h(void *dst, const void *src, size_t n) {
     NEED_INIT();
     if (!n) return 0;
+    if (g_capturing) return fail_msg(-9, "dlg_hip_d2h is a synchronous transfer and cannot be part of a captured graph");
     HIP_TRY(hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToHost, g_stream));
     HIP_TRY(hipStreamSynchronize(g_stream));
     return 0;
@@ -366,6 +395,83 @@ int dlg_hip_kernel_attrs(uint64_t handle, int32_t *num_regs, int32_t *lds_bytes,
     if (lds_bytes) { HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES, fn)); *lds_bytes = v; }
     if (scratch_bytes) { HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, fn)); *scratch_bytes = v; }
     if (max_threads) { HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_MAX_THREADS_PER_BLOCK, fn)); *max_threads = v; }
+    return 0;
+}
+
+// ---- arenas and graphs ----------------------------------------------------------------
+
+int dlg_hip_arena_create(uint64_t *arena) {
+    NEED_INIT();
+    if (!arena) return fail_msg(-1, "arena is NULL");
+    std::lock_guard<std::mutex> lk(g_mu);
+    *arena = g_next_arena++;
+    g_arena_alive[*arena] = true;
+    return 0;
+}
+
+int dlg_hip_arena_set(uint64_t arena) {
+    NEED_INIT();
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (arena != 0 && !g_arena_alive[arena]) return fail_msg(-30, "no such arena");
+    g_arena = arena;
+    return 0;
+}
+
+int dlg_hip_arena_destroy(uint64_t arena) {
+    NEED_INIT();
+    if (arena == 0) return fail_msg(-30, "the default pool cannot be destroyed");
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_arena == arena) g_arena = 0;
+    g_arena_alive[arena] = false;
+    trim_arena_locked(arena);
+    return 0;
+}
+
+int dlg_hip_graph_begin(void) {
+    NEED_INIT();
+    if (g_capturing) return fail_msg(-31, "a capture is already in progress");
+    HIP_TRY(hipStreamBeginCapture(g_stream, hipStreamCaptureModeRelaxed));
+    g_capturing = true;
+    return 0;
+}
+
+int dlg_hip_graph_end(uint64_t *graph, uint64_t *n_nodes) {
+    NEED_INIT();
+    if (!g_capturing) return fail_msg(-31, "no capture in progress");
+    g_capturing = false;
+    hipGraph_t g = nullptr;
+    HIP_TRY(hipStreamEndCapture(g_stream, &g));
+    if (!graph) {                                  // caller only wants the capture abandoned
+        if (g) (void)hipGraphDestroy(g);
+        return 0;
+    }
+    size_t nodes = 0;
+    (void)hipGraphGetNodes(g, nullptr, &nodes);
+    hipGraphExec_t ge = nullptr;
+    hipError_t e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess) return fail("hipGraphInstantiate", e);
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_graphs.push_back(ge);
+    *graph = (uint64_t)g_graphs.size();
+    if (n_nodes) *n_nodes = nodes;
+    return 0;
+}
+
+int dlg_hip_graph_launch(uint64_t graph) {
+    NEED_INIT();
+    if (graph == 0 || graph > g_graphs.size() || !g_graphs[graph - 1]) return fail_msg(-32, "bad graph handle");
+    HIP_TRY(hipGraphLaunch(g_graphs[graph - 1], g_stream));
+    return 0;
+}
+
+int dlg_hip_graph_destroy(uint64_t graph) {
+    NEED_INIT();
+    if (graph == 0 || graph > g_graphs.size() || !g_graphs[graph - 1]) return fail_msg(-32, "bad graph handle");
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    HIP_TRY(hipGraphExecDestroy(g_graphs[graph - 1]));
+    g_graphs[graph - 1] = nullptr;
     return 0;
 }
 

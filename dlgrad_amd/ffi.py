@@ -41,6 +41,13 @@ _SIGS = {
                                        _c.POINTER(_c.c_uint64)]),
     "dlg_hip_launch": (_c.c_int, [_c.c_uint64] + [_c.c_uint32] * 7 + [_c.c_char_p, _c.c_size_t]),
     "dlg_hip_kernel_attrs": (_c.c_int, [_c.c_uint64] + [_c.POINTER(_c.c_int32)] * 4),
+    "dlg_hip_arena_create": (_c.c_int, [_c.POINTER(_c.c_uint64)]),
+    "dlg_hip_arena_set": (_c.c_int, [_c.c_uint64]),
+    "dlg_hip_arena_destroy": (_c.c_int, [_c.c_uint64]),
+    "dlg_hip_graph_begin": (_c.c_int, []),
+    "dlg_hip_graph_end": (_c.c_int, [_c.POINTER(_c.c_uint64), _c.POINTER(_c.c_uint64)]),
+    "dlg_hip_graph_launch": (_c.c_int, [_c.c_uint64]),
+    "dlg_hip_graph_destroy": (_c.c_int, [_c.c_uint64]),
     "dlg_hip_sync": (_c.c_int, []),
     "dlg_hip_event_create": (_c.c_int, [_c.POINTER(_c.c_uint64)]),
     "dlg_hip_event_record": (_c.c_int, [_c.c_uint64]),
@@ -238,6 +245,37 @@ class HipLib:
         self._check(self._lib.dlg_hip_kernel_attrs(handle, *[o[0] for o in outs]))
         return dict(zip(("num_regs", "lds_bytes", "scratch_bytes", "max_threads"),
                         (int(o[1]()) for o in outs)))
+
+    # -- arenas and graphs ----------------------------------------------------------------
+    def arena_create(self) -> int:
+        ref, get = self._out(ctypes.c_uint64, "uint64_t")
+        self._check(self._lib.dlg_hip_arena_create(ref))
+        return int(get())
+
+    def arena_set(self, arena: int) -> None:
+        self._check(self._lib.dlg_hip_arena_set(arena))
+
+    def arena_destroy(self, arena: int) -> None:
+        self._check(self._lib.dlg_hip_arena_destroy(arena))
+
+    def graph_begin(self) -> None:
+        self._check(self._lib.dlg_hip_graph_begin())
+
+    def graph_end(self) -> tuple[int, int]:
+        g, gget = self._out(ctypes.c_uint64, "uint64_t")
+        n, nget = self._out(ctypes.c_uint64, "uint64_t")
+        self._check(self._lib.dlg_hip_graph_end(g, n))
+        return int(gget()), int(nget())
+
+    def graph_abandon(self) -> None:
+        null = self._cffi.NULL if self._cffi is not None else None
+        self._lib.dlg_hip_graph_end(null, null)
+
+    def graph_launch(self, graph: int) -> None:
+        self._check(self._lib.dlg_hip_graph_launch(graph))
+
+    def graph_destroy(self, graph: int) -> None:
+        self._lib.dlg_hip_graph_destroy(graph)
 
     # -- ordering and timing ---------------------------------------------------------------
     def sync(self) -> None:

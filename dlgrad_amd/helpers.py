@@ -69,6 +69,7 @@ class CustomOps(Enum):
     LOG_SOFTMAX_GATHER = auto()     # log-softmax rows + the ce_forward gather, one kernel
     CE_GRAD = auto()                # ((exp(lsm) - onehot) * upstream) / N, one kernel
     ADAM_STEP = auto()              # the 14 element-wise kernels of one Adam update, one kernel
+    ADAM_STEP_INPLACE = auto()      # the same, in place, constants from device memory (graph replay)
 
 
 def prod_(x: Iterable) -> int:

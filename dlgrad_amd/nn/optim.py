@@ -1,5 +1,7 @@
 """Optimizers as Tensor expressions (dlgrad/nn/optim.py:4-70): every update is a handful
 of element-wise kernels per parameter and rebinds `param.data` to the new buffer."""
+import numpy as np
+
 from dlgrad_amd import ops
 from dlgrad_amd.device import Device
 from dlgrad_amd.tensor import Tensor
@@ -42,17 +44,39 @@ class Adam(Optimizer):
     """m = b1 m + (1-b1) g;  v = b2 v + (1-b2) g^2;  p -= lr * m_hat / (sqrt(v_hat) + eps)."""
 
     def __init__(self, params: list[Tensor], lr: float = 1e-3, betas: tuple[float, float] = (0.9, 0.999),
-                 eps: float = 1e-8) -> None:
+                 eps: float = 1e-8, graph_safe: bool = False) -> None:
+        """graph_safe (hip only): parameters and moments are updated in place and the
+        step-dependent constants live in device memory, so that a captured step can be
+        replayed: call advance() before each replay.  Same arithmetic, same bits."""
         self.params, self.lr, self.eps = params, lr, eps
         self.beta1, self.beta2 = betas
         self.m = {id(p): Tensor.zeros_like(p) for p in params}
         self.v = {id(p): Tensor.zeros_like(p) for p in params}
         self.t = 0
+        self.graph_safe = graph_safe
+        self.consts = Tensor(np.zeros(8, np.float32), device=params[0].device) if graph_safe else None
+
+    def _consts(self) -> tuple:
+        c1, c2 = 1.0 - self.beta1 ** self.t, 1.0 - self.beta2 ** self.t
+        return (self.beta1, 1.0 - self.beta1, self.beta2, 1.0 - self.beta2, c1, c2, self.eps, self.lr)
+
+    def advance(self) -> None:
+        """graph_safe: moves to the next step and uploads its constants (not capturable)."""
+        self.t += 1
+        self.consts.data.upload_(np.asarray(self._consts(), dtype=np.float32))
 
     def step(self) -> None:
+        if self.graph_safe:
+            from dlgrad_amd.runtime import hip
+            if not hip.capturing():
+                self.advance()
+            for p in self.params:
+                k = id(p)
+                p.data.adam_step_(p.grad.data, self.m[k].data, self.v[k].data, self.consts.data)
+            return
         self.t += 1
-        c1, c2 = 1.0 - self.beta1 ** self.t, 1.0 - self.beta2 ** self.t
-        consts = (self.beta1, 1.0 - self.beta1, self.beta2, 1.0 - self.beta2, c1, c2, self.eps, self.lr)
+        consts = self._consts()
+        c1, c2 = consts[4], consts[5]
         for p in self.params:
             k, g = id(p), p.grad
             if ops.FUSED and p.device is Device.HIP:

@@ -165,7 +165,104 @@ class DevicePtr:
 def alloc(numel: int, zero: bool = False) -> DevicePtr:
     nbytes = 4 * numel if numel > 0 else 4
     l = _state["lib"] or lib()
+    if zero and _graph_depth:
+        # a memset node must not enter a captured graph: clear with a kernel instead
+        p = DevicePtr(l.alloc(nbytes, False), nbytes)
+        _map("full", "s0", [], (max(numel, 1),), (0.0,), out=p)
+        return p
     return DevicePtr(l.alloc(nbytes, zero), nbytes)
+
+
+# ---- captured graphs ------------------------------------------------------------------------
+_graph_depth = 0       # > 0 while a Graph's arena is current (warm-up or capture)
+_capturing = False
+
+
+def capturing() -> bool:
+    return _capturing
+
+
+class Graph:
+    """A whole step -- hundreds of launches -- recorded once and replayed as one submission.
+
+        g = Graph()
+        with g.arena():   step()        # eager, inside the graph's private pool: loads every kernel,
+                                        # sizes the pool
+        with g.capture(): out = step()  # recorded, not executed
+        g.replay()                      # runs the recorded launches; `out` is rewritten in place
+
+    What is recorded is the exact launches with their arguments, so the step must keep its
+    state at fixed addresses (in-place optimizer), must not transfer to or from the host,
+    and anything that changes per replay must live in device memory.  Buffers allocated
+    inside arena()/capture() come from a pool nobody else draws from, so replays cannot
+    clobber tensors made elsewhere."""
+
+    def __init__(self) -> None:
+        self._lib = lib()
+        self.arena_id = self._lib.arena_create()
+        self.handle, self.nodes = 0, 0
+
+    def _enter(self) -> None:
+        global _graph_depth
+        if _graph_depth:
+            raise RuntimeError("graph arenas do not nest")
+        self._lib.arena_set(self.arena_id)
+        _graph_depth = 1
+
+    def _leave(self) -> None:
+        global _graph_depth
+        _graph_depth = 0
+        self._lib.arena_set(0)
+
+    def arena(self):
+        import contextlib
+
+        @contextlib.contextmanager
+        def cm():
+            self._enter()
+            try:
+                yield self
+            finally:
+                self._leave()
+        return cm()
+
+    def capture(self):
+        import contextlib
+
+        @contextlib.contextmanager
+        def cm():
+            global _capturing
+            if self.handle:
+                raise RuntimeError("this Graph already holds a capture")
+            self._enter()
+            self._lib.graph_begin()
+            _capturing = True
+            try:
+                yield self
+            except BaseException:
+                _capturing = False
+                self._lib.graph_abandon()
+                self._leave()
+                raise
+            _capturing = False
+            try:
+                self.handle, self.nodes = self._lib.graph_end()
+            finally:
+                self._leave()
+        return cm()
+
+    def replay(self) -> None:
+        global launch_count
+        launch_count += 1
+        self._lib.graph_launch(self.handle)
+
+    def close(self) -> None:
+        if self.handle:
+            self._lib.graph_destroy(self.handle)
+            self.handle = 0
+        if self.arena_id:
+            self._lib.arena_destroy(self.arena_id)
+            self.arena_id = 0
 
 
 # ---- kernel cache -----------------------------------------------------------------------
@@ -328,9 +425,9 @@ class HIP:
     # ---- host boundary ------------------------------------------------------------------------
     @staticmethod
     @dispatcher.register(BufferOps.CREATE, Device.HIP)
-    def create(data: np.ndarray) -> DevicePtr:
+    def create(data: np.ndarray, into: Buffer | None = None) -> DevicePtr:
         a = np.ascontiguousarray(data, dtype=np.float32)
-        p = alloc(a.size)
+        p = into.ptr if into is not None else alloc(a.size)
         if a.size:
             lib().h2d(p.addr, a.ctypes.data, a.nbytes)
         return p
@@ -746,6 +843,19 @@ class HIP:
         launch(kernel(K.adam_kernel, vec), max(1, ((n + vec - 1) // vec + 255) // 256), 256,
                *addrs, n, *[float(c) for c in consts])
         return outs
+
+    @staticmethod
+    @dispatcher.register(CustomOps.ADAM_STEP_INPLACE, Device.HIP)
+    def adam_step_inplace(p: Buffer, g: Buffer, m: Buffer, v: Buffer, consts: Buffer) -> None:
+        """Updates p, m and v where they are; `consts` is a device buffer of the eight values
+        adam_step takes by value."""
+        n = p.numel
+        if n == 0:
+            return
+        addrs = [_addr(b) for b in (p, g, m, v)]
+        vec = 4 if not any(a & 15 for a in addrs) else 1
+        launch(kernel(K.adam_inplace_kernel, vec), max(1, ((n + vec - 1) // vec + 255) // 256), 256,
+               *addrs, n, _addr(consts))
 
     # ---- matmul ----------------------------------------------------------------------------------------------------------
     MATMUL_FORCE = os.environ.get("DLGRAD_HIP_MATMUL_TILE")      # e.g. "128x128": benchmarking aid

@@ -88,7 +88,7 @@ class GPT:
     def __call__(self, idx: Tensor, targets: Tensor | None = None):
         """idx, targets: (B, T) token ids stored as fp32.  Returns (logits, loss)."""
         B, T = idx.shape
-        pos = Tensor(np.arange(T, dtype=np.float32), device=idx.device)
+        pos = Tensor.arange((T,), device=idx.device)            # 0..T-1 made on the device (no upload per step)
         x = self.wte(idx) + self.wpe(pos)
         for block in self.blocks:
             x = block(x)

@@ -107,6 +107,22 @@ int dlg_hip_launch(uint64_t handle,
 int dlg_hip_kernel_attrs(uint64_t handle, int32_t *num_regs, int32_t *lds_bytes,
                          int32_t *scratch_bytes, int32_t *max_threads);
 
+/* ---- arenas and captured graphs ------------------------------------------------
+ * No counterpart in the reference, whose CPU kernels have no launch cost to remove; on a
+ * GPU a char-GPT training step is ~900 tiny launches and is bound by issuing them.
+ * An arena is a private pool: while it is current (dlg_hip_arena_set), dlg_hip_alloc draws
+ * from it and blocks return to it, so a graph captured inside it may replay writes to those
+ * addresses for as long as the arena lives.  dlg_hip_graph_begin/end bracket a capture of
+ * the internal stream (kernel launches only: synchronous transfers and memset-backed
+ * calls fail while capturing); dlg_hip_graph_launch replays it on the same stream.                                                                */
+int dlg_hip_arena_create(uint64_t *arena);
+int dlg_hip_arena_set(uint64_t arena);            /* 0 = the ordinary pool */
+int dlg_hip_arena_destroy(uint64_t arena);
+int dlg_hip_graph_begin(void);
+int dlg_hip_graph_end(uint64_t *graph, uint64_t *n_nodes);   /* graph == NULL abandons the capture */
+int dlg_hip_graph_launch(uint64_t graph);
+int dlg_hip_graph_destroy(uint64_t graph);
+
 /* ---- ordering and timing -----------------------------------------------------
  * The CPU reference is synchronous, so it has no counterpart; the Metal runtime's
  * commit()/waitUntilCompleted() per op (dlgrad/runtime/metal.py:124-128) is the

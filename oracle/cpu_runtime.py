@@ -47,7 +47,10 @@ class CPU:
 
     @staticmethod
     @_reg(BufferOps.CREATE)
-    def create(data: np.ndarray) -> HostPtr:
+    def create(data: np.ndarray, into: Buffer | None = None) -> HostPtr:
+        if into is not None:
+            into.ptr.arr[:data.size] = np.asarray(data, dtype=np.float32).reshape(-1)
+            return into.ptr
         return HostPtr(np.array(data, dtype=np.float32, copy=True))
 
     @staticmethod
