@@ -299,6 +299,18 @@ class Buffer:
         """self is a log-softmax; returns ((exp(self) - onehot(target)) * upstream) / n."""
         return self._like(self._dispatch(CustomOps.CE_GRAD, lsm=self, target=target, upstream=upstream, n=n))
 
+    def rmsnorm(self, weight: "Buffer | None", eps: float) -> tuple["Buffer", "Buffer"]:
+        """Fused RMSNorm over the last axis; returns (y, r) with r = rsqrt(mean(x^2) + eps)
+        per row, kept for the backward pass."""
+        y, r = self._dispatch(CustomOps.RMSNORM, x=self, w=weight, eps=eps)
+        return self._like(y), self._like(r, (self.numel // max(self.shape[-1], 1),))
+
+    def rmsnorm_bwd(self, weight: "Buffer | None", r: "Buffer", dy: "Buffer",
+                    through_mean: bool) -> tuple["Buffer", "Buffer | None"]:
+        """self is the forward input x; returns (dx, dw) with dw shaped like the weight."""
+        dx, dw = self._dispatch(CustomOps.RMSNORM_BWD, x=self, w=weight, r=r, dy=dy, through_mean=through_mean)
+        return self._like(dx), (None if dw is None else self._like(dw, weight.shape))
+
     # ---- selects ----------------------------------------------------------------------------------
     def where(self, inp: "Buffer | Scalar", other: "Buffer | Scalar") -> "Buffer":
         inp = Buffer.from_scalar(inp) if _is_scalar(inp) else inp

@@ -956,6 +956,139 @@ def softmax_plan(L: int, vec: int) -> tuple[bool, int, int]:
 
 
 # =====================================================================================
+# fused RMSNorm
+# =====================================================================================
+
+def rmsnorm_plan(L: int, vec: int) -> int:
+    """Items (float4 or float) each lane of a wavefront keeps for a row of L floats; 0 when
+    a row does not fit 16 items per lane (the caller then composes the op from its parts)."""
+    items = (L + vec - 1) // vec
+    for nval in (1, 2, 3, 4, 6, 8, 12, 16):
+        if items <= 64 * nval:
+            return nval
+    return 0
+
+
+def _rms_lanes(vec: int) -> tuple[str, tuple, str]:
+    """(item type, component suffixes, items-per-row expression) for float4 / float rows."""
+    return ("float4", (".x", ".y", ".z", ".w"), "(L >> 2)") if vec == 4 else ("float", ("",), "L")
+
+
+@cache
+def rmsnorm_fwd_kernel(vec: int, nval: int, affine: bool) -> tuple[str, str, str]:
+    """y = (x * r) * w with r = 1 / sqrt(sum(x^2) / L + eps) per row of the contiguous last
+    axis, and r kept per row for the backward pass: the seven kernels of RMSNorm's
+    composition (pow, mean, add, rsqrt, mul, mul; nn/__init__.py:25-41) in one pass that
+    reads x once.  One wavefront per row, the row held in registers; same operation order
+    per element as the composition, so it differs from it only in the order of the sum."""
+    T, comps, nv = _rms_lanes(vec)
+    name = f"rmsnorm_fwd_v{vec}_r{nval}{'_w' if affine else ''}"
+    sq = " + ".join(f"v[k]{c} * v[k]{c}" for c in comps)
+    outs = "".join(f"            o{c} = (v[k]{c} * r){f' * g{c}' if affine else ''};\n" for c in comps)
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        const float* __restrict__ w, float* __restrict__ y, float* __restrict__ rinv, u32 R, u32 L, float eps) {{
+    const u32 lane = threadIdx.x & 63u;
+    const u32 row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= R) return;
+    const {T}* __restrict__ p = reinterpret_cast<const {T}*>(x + (u64)row * L);
+    {T}* __restrict__ q = reinterpret_cast<{T}*>(y + (u64)row * L);
+    const {T}* __restrict__ wv = reinterpret_cast<const {T}*>(w); (void)wv;
+    const u32 nv = {nv};
+    {T} v[{nval}];
+    float ss = 0.0f;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{
+        const u32 c = lane + k * 64u;
+        if (c < nv) {{ v[k] = p[c]; ss += {sq}; }}
+    }}
+    ss = wave_sum(ss);
+    const float r = 1.0f / sqrtf(ss / (float)L + eps);
+    if (lane == 0) rinv[row] = r;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{
+        const u32 c = lane + k * 64u;
+        if (c < nv) {{
+            {f'const {T} g = wv[c];' if affine else ''}
+            {T} o;
+{outs}            q[c] = o;
+        }}
+    }}
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "P", "I", "I", "f")
+
+
+@cache
+def rmsnorm_bwd_kernel(vec: int, nval: int, affine: bool, through_mean: bool) -> tuple[str, str, str]:
+    """Backward of the fused RMSNorm.  Per row, with dn = dy * w:
+        dx = dn * r                                         (the path through x * r)
+           + (x * 2) * ((1/L) * (sum(dn * x) * (r^3 * -0.5)))   (the path through mean(x^2)),
+    the second term only when through_mean: the reference's Mean.backward scales by
+    full(1/N), whose fill value is truncated to int 0 (ops.py:86-91, cpu.py:252), so its
+    RMSNorm passes no gradient through the normaliser.
+    dw = sum over rows of dy * (x * r): each wavefront walks rows_per_wave consecutive rows
+    with its columns' partial sums in registers and writes one row of `dwpart`; a column
+    reduction over those partial rows finishes it."""
+    T, comps, nv = _rms_lanes(vec)
+    name = f"rmsnorm_bwd_v{vec}_r{nval}{'_w' if affine else ''}{'_m' if through_mean else ''}"
+    dn = lambda c: f"(d[k]{c} * g[k]{c})" if affine else f"d[k]{c}"          # noqa: E731
+    dot = " + ".join(f"{dn(c)} * v[k]{c}" for c in comps)
+    dxs = "".join(
+        f"                o{c} = {dn(c)} * r" + (f" + (v[k]{c} * 2.0f) * coef" if through_mean else "") + ";\n"
+        for c in comps)
+    accs = "".join(f"                acc[k]{c} += d[k]{c} * (v[k]{c} * r);\n" for c in comps) if affine else ""
+    zero = "float4{0.0f, 0.0f, 0.0f, 0.0f}" if vec == 4 else "0.0f"
+    tail = f"""    {T}* __restrict__ pw = reinterpret_cast<{T}*>(dwpart + (u64)wid * L);
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = lane + k * 64u; if (c < nv) pw[c] = acc[k]; }}""" if affine else ""
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        const float* __restrict__ w, const float* __restrict__ rinv, const float* __restrict__ dy,
+        float* __restrict__ dx, float* __restrict__ dwpart, u32 R, u32 L, u32 rows_per_wave) {{
+    const u32 lane = threadIdx.x & 63u;
+    const u32 wid = blockIdx.x * 4u + (threadIdx.x >> 6);
+    const u32 row0 = wid * rows_per_wave;
+    if (row0 >= R) return;
+    const u32 nv = {nv};
+    {T} g[{nval}], acc[{nval}]; (void)g; (void)acc;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{
+        const u32 c = lane + k * 64u;
+        acc[k] = {zero};
+        {f'if (c < nv) g[k] = reinterpret_cast<const {T}*>(w)[c];' if affine else '(void)c;'}
+    }}
+    const u32 row1 = min(row0 + rows_per_wave, R);
+    for (u32 row = row0; row < row1; ++row) {{
+        const {T}* __restrict__ p = reinterpret_cast<const {T}*>(x + (u64)row * L);
+        const {T}* __restrict__ pd = reinterpret_cast<const {T}*>(dy + (u64)row * L);
+        {T}* __restrict__ q = reinterpret_cast<{T}*>(dx + (u64)row * L);
+        const float r = rinv[row];
+        {T} v[{nval}], d[{nval}];
+        float s = 0.0f; (void)s;
+        #pragma unroll
+        for (u32 k = 0; k < {nval}u; ++k) {{
+            const u32 c = lane + k * 64u;
+            if (c < nv) {{ v[k] = p[c]; d[k] = pd[c]; {f's += {dot};' if through_mean else ''} }}
+        }}
+        {'s = wave_sum(s);' if through_mean else ''}
+        const float coef = (1.0f / (float)L) * (s * ((r * r * r) * -0.5f)); (void)coef;
+        #pragma unroll
+        for (u32 k = 0; k < {nval}u; ++k) {{
+            const u32 c = lane + k * 64u;
+            if (c < nv) {{
+                {T} o;
+{dxs}                q[c] = o;
+{accs}            }}
+        }}
+    }}
+{tail}
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "P", "P", "P", "I", "I", "I")
+
+
+# =====================================================================================
 # matmul
 # =====================================================================================
 
@@ -988,16 +1121,18 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     contiguous band of C tiles, walked in groups of 8 tile rows for L2 reuse."""
     BM, BN, T = 32 * MI * WM, 32 * NJ * WN, 64 * WM * WN
     AKQ, BNQ = BK // 4, BN // 4
-    assert T % AKQ == 0 and T % BNQ == 0 and BK % 8 == 0
+    assert T % AKQ == 0 and BK % 8 == 0 and NJ in (1, 2, 3, 4) and T >= BNQ
+    # loader threads walk the A tile in passes of ROWS_A rows and the B tile in passes of
+    # ROWS_B rows; when a tile extent is no multiple of the pass (96- and 192-wide tiles)
+    # the last pass is cut off by a guard, and threads beyond the last whole B row repeat
+    # a neighbour's element (same address, same value)
     ROWS_A, ROWS_B = T // AKQ, T // BNQ
-    PA, PB = max(1, BM // ROWS_A), max(1, BK // ROWS_B)
-    assert BM % ROWS_A == 0 or ROWS_A > BM
-    assert BK % ROWS_B == 0 or ROWS_B > BK
-    guard_a = ROWS_A > BM      # more loader threads than A rows: extra threads idle
-    guard_b = ROWS_B > BK
+    PA, PB = -(-BM // ROWS_A), -(-BK // ROWS_B)
+    guard_a = BM % ROWS_A != 0
+    guard_b = BK % ROWS_B != 0 or T % BNQ != 0
     name = f"matmul_{BM}x{BN}x{BK}_w{WM}x{WN}_{'a4' if veca else 'a1'}{'b4' if vecb else 'b1'}"
     LDA, LDB = BK + 4, BN
-    bvec = {1: "float", 2: "float2", 4: "float4"}[NJ]
+    bvec = {1: "float", 2: "float2", 3: "f3v", 4: "float4"}[NJ]
     comp = ["x", "y", "z", "w"]
 
     if veca:
@@ -1045,6 +1180,7 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
 
     src = f"""{PRELUDE}
 typedef float f16v __attribute__((ext_vector_type(16)));
+struct f3v {{ float x, y, z; }};
 struct MMArgs {{ u32 M, N, K, nbc, sa0, sa1, sb0, sb1; }};
 #define BM {BM}u
 #define BN {BN}u
@@ -1102,10 +1238,10 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
     auto stash_tiles = [&](u32 buf) {{
         #pragma unroll
         for (u32 p = 0; p < {PA}u; ++p)
-            {'if (a_m < BM)' if guard_a else ''} *reinterpret_cast<float4*>(&As[buf][a_m + p * {ROWS_A}u][4u * a_kq]) = ra[p];
+            {f'if (a_m + p * {ROWS_A}u < BM)' if guard_a else ''} *reinterpret_cast<float4*>(&As[buf][a_m + p * {ROWS_A}u][4u * a_kq]) = ra[p];
         #pragma unroll
         for (u32 p = 0; p < {PB}u; ++p)
-            {'if (b_k < BK)' if guard_b else ''} *reinterpret_cast<float4*>(&Bs[buf][b_k + p * {ROWS_B}u][4u * b_nq]) = rb[p];
+            {f'if (b_k + p * {ROWS_B}u < BK)' if guard_b else ''} *reinterpret_cast<float4*>(&Bs[buf][b_k + p * {ROWS_B}u][4u * b_nq]) = rb[p];
     }};
 
     const u32 nk = (g.K + BK - 1u) / BK;
@@ -1144,23 +1280,40 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
 
 
 # name -> (WM, WN, MI, NJ, BK): block tile = (32*MI*WM) x (32*NJ*WN), 64*WM*WN threads.
-# Chosen from a sweep on MI355X (TFLOP/s at 4096^3 / 8192x3072x768 / 2048^3):
-#   256x256 (8 waves, 128 acc regs)   136 / 100 / 34     largest problems, one block per CU
-#   256x128 (4 waves, 128 acc regs)   135 /  92 / 58
-#   128x256 (8 waves,  64 acc regs)   129 / 124 / 64     mid-size N
-#   128x128 (4 waves of 64x64)        128 / 122 / 104    default below ~512 tiles
+# Kept after sweeps on MI355X (TFLOP/s at 4096^3 / 8192x768x768 / batch 8 of 768x3072x1024):
+#   256x256 (8 waves, 128 acc regs)   136 /  .. /  ..    largest problems, one block per CU
+#   256x128 (4 waves, 128 acc regs)   135
+#   128x256 (8 waves,  64 acc regs)   129
+#   128x128 (4 waves of 64x64)        128 /  68 / 107
+#   192x192 (4 waves of 96x96)         .. /  .. / 124    N or M a multiple of 192 (768, 3072)
+#   128x192 (8 waves of 32x96)         .. / 100 / 114    8192x768 as exactly 256 blocks
+#   128x96, 128x64 (4 waves of 32xBN)  .. / 103, 107     narrow outputs: 2-3 resident blocks per CU
+# Every tile accumulates k in the same order, so the choice never changes a result bit.
 MATMUL_CONFIGS = {
     "256x256": (4, 2, 2, 4, 16),
     "256x128": (4, 1, 2, 4, 16),
     "128x256": (4, 2, 1, 4, 32),
+    "192x192": (2, 2, 3, 3, 16),
+    "128x192": (4, 2, 1, 3, 32),
     "128x128": (2, 2, 2, 2, 32),
+    "128x96": (4, 1, 1, 3, 32),
+    "128x64": (4, 1, 1, 2, 32),
     "64x64": (2, 2, 1, 1, 16),
     "32x32": (1, 1, 1, 1, 16),
 }
-# (relative per-CU throughput when the chip is full, resident blocks per CU)
+
+
+def matmul_tile_shape(tile: str) -> tuple[int, int, int]:
+    """(rows, columns, threads) of a block of the named configuration."""
+    wm, wn, mi, nj, _ = MATMUL_CONFIGS[tile]
+    return 32 * mi * wm, 32 * nj * wn, 64 * wm * wn
+
+
+# (relative per-CU throughput when the chip is full, resident blocks per CU): the model that
+# picks a tile for a shape nobody has timed
 MATMUL_TILE_MODEL = {
-    "256x256": (1.00, 1), "256x128": (0.99, 2), "128x256": (0.95, 1), "128x128": (0.94, 2),
-    "64x64": (0.79, 8), "32x32": (0.65, 8),
+    "256x256": (1.00, 1), "256x128": (0.99, 2), "128x256": (0.95, 1), "192x192": (0.93, 2), "128x192": (0.88, 1),
+    "128x128": (0.94, 2), "128x96": (0.86, 3), "128x64": (0.85, 4), "64x64": (0.74, 8), "32x32": (0.60, 8),
 }
 
 

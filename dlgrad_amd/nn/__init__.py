@@ -2,6 +2,7 @@
 dlgrad/nn/__init__.py:8-41."""
 import math
 
+from dlgrad_amd import ops
 from dlgrad_amd.device import Device
 from dlgrad_amd.nn import optim, utils  # noqa: F401
 from dlgrad_amd.tensor import Tensor
@@ -46,5 +47,8 @@ class RMSNorm:
         return x * (ms + self.eps).rsqrt()
 
     def __call__(self, x: Tensor) -> Tensor:
+        if ops.use_fused_rmsnorm(x, self.weight):
+            args = (x,) if self.weight is None else (x, self.weight)
+            return ops.RMSNorm.execute(*args, eps=self.eps)
         y = self._norm(x)
         return y if self.weight is None else y * self.weight

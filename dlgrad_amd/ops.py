@@ -15,7 +15,7 @@ import os
 from dlgrad_amd.buffer import Buffer
 from dlgrad_amd.device import Device
 from dlgrad_amd.dtype import Scalar
-from dlgrad_amd.helpers import CustomOps, broadcast_shapes, check_broadcast
+from dlgrad_amd.helpers import STRICT_REFERENCE, CustomOps, broadcast_shapes, check_broadcast
 from dlgrad_amd.tensor import OP
 
 # Fused row kernels (softmax, log-softmax inside cross-entropy) on the hip device.
@@ -327,6 +327,29 @@ class Softmax(OP):
     def backward(self, upstream_grad: Buffer) -> tuple:
         gy = upstream_grad * self.out
         return (gy - self.out * gy.sum(dim=self.out.ndim - 1, keepdim=True),)
+
+
+def use_fused_rmsnorm(x, weight) -> bool:
+    if not (FUSED and x.device is Device.HIP):
+        return False
+    from dlgrad_amd.runtime.hip import HIP
+    return HIP.rmsnorm_fits(x.data, None if weight is None else weight.data)
+
+
+class RMSNorm(OP):
+    """(x * rsqrt(mean(x^2, last) + eps)) * weight as one forward and one backward kernel
+    (plus the column sum that finishes dw).  The gradient through mean(x^2) is dropped when
+    reference-strict, as the reference's Mean.backward drops it (ops.py:86-91 with the
+    int-truncated fill of cpu.py:252)."""
+
+    def forward(self, x: Buffer, weight: Buffer | None = None, eps: float = 1e-6) -> Buffer:
+        self.x, self.weight = x, weight
+        y, self.r = x.rmsnorm(weight, eps)
+        return y
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        dx, dw = self.x.rmsnorm_bwd(self.weight, self.r, upstream_grad, through_mean=not STRICT_REFERENCE)
+        return (dx,) if self.weight is None else (dx, dw)
 
 
 class CrossEntropy(OP):

@@ -18,6 +18,7 @@ Nothing here falls back to another device: a missing library or GPU raises.
 from __future__ import annotations
 
 import hashlib
+import json
 import os
 import struct
 
@@ -828,6 +829,64 @@ class HIP:
                         (n, float(upstream.ptr.value)))
         return _map("cegrad_p", expr.format(g="x2"), [lsm, rows, upstream], lsm.shape, (n,))
 
+    # ---- fused RMSNorm ------------------------------------------------------------------------------------------------------
+    @staticmethod
+    def rmsnorm_fits(x: Buffer, w: Buffer | None) -> bool:
+        """Whether the fused kernels apply: rows of the last axis fit a wavefront's registers
+        and the weight, if any, is one row of that length."""
+        L = x.shape[-1] if x.ndim else 0
+        if x.ndim < 1 or L == 0 or x.numel >= 2 ** 31 or (w is not None and w.numel != L):
+            return False
+        return K.rmsnorm_plan(L, HIP._rms_vec(L, _addr(x), _addr(w) if w is not None else 0)) > 0
+
+    @staticmethod
+    def _rms_vec(L: int, *addrs: int) -> int:
+        return 4 if (L % 4 == 0 and all(a % 16 == 0 for a in addrs)) else 1
+
+    @staticmethod
+    @dispatcher.register(CustomOps.RMSNORM, Device.HIP)
+    def rmsnorm(x: Buffer, w: Buffer | None, eps: float) -> tuple[DevicePtr, DevicePtr]:
+        L = x.shape[-1]
+        R = x.numel // L
+        y, r = alloc(x.numel), alloc(R)
+        if not HIP.rmsnorm_fits(x, w):
+            raise ValueError(f"fused RMSNorm does not take rows of {L} floats with this weight")
+        vec = HIP._rms_vec(L, _addr(x), y.addr, _addr(w) if w is not None else 0)
+        nval = K.rmsnorm_plan(L, vec)
+        if nval == 0:
+            raise ValueError(f"fused RMSNorm: a row of {L} unaligned floats does not fit a wavefront's registers")
+        k = kernel(K.rmsnorm_fwd_kernel, vec, nval, w is not None)
+        launch(k, (R + 3) // 4, 256, _addr(x), _addr(w) if w is not None else 0, y.addr, r.addr, R, L, float(eps))
+        return y, r
+
+    @staticmethod
+    @dispatcher.register(CustomOps.RMSNORM_BWD, Device.HIP)
+    def rmsnorm_bwd(x: Buffer, w: Buffer | None, r: Buffer, dy: Buffer,
+                    through_mean: bool) -> tuple[DevicePtr, DevicePtr | None]:
+        L = x.shape[-1]
+        R = x.numel // L
+        if dy.numel != x.numel or r.numel != R:
+            raise ValueError(f"rmsnorm_bwd: x {x.shape}, dy {dy.shape}, r {r.shape} do not agree")
+        if _addr(dy) % 16 and L % 4 == 0:                          # a gradient view at an odd offset: realign it
+            dy = Buffer(_map("copy", "x0", [dy], dy.shape), dy.shape, Device.HIP)
+        dx = alloc(x.numel)
+        rows_per_wave = max(1, (R + 2047) // 2048)
+        P = (R + rows_per_wave - 1) // rows_per_wave            # partial rows of dw, one per wavefront
+        part = alloc(P * L) if w is not None else None
+        vec = HIP._rms_vec(L, _addr(x), _addr(dy), dx.addr, _addr(w) if w is not None else 0,
+                           part.addr if part is not None else 0)
+        nval = K.rmsnorm_plan(L, vec)
+        if nval == 0:
+            raise ValueError(f"fused RMSNorm: a row of {L} unaligned floats does not fit a wavefront's registers")
+        k = kernel(K.rmsnorm_bwd_kernel, vec, nval, w is not None, bool(through_mean))
+        launch(k, (P + 3) // 4, 256, _addr(x), _addr(w) if w is not None else 0, _addr(r), _addr(dy), dx.addr,
+               part.addr if part is not None else 0, R, L, rows_per_wave)
+        if w is None:
+            return dx, None
+        dw = alloc(L)
+        HIP._reduce_cols("sum", part.addr, 1, P, L, 1.0, dw.addr)
+        return dx, dw
+
     # ---- fused optimizer step -----------------------------------------------------------------------------------------------
     @staticmethod
     @dispatcher.register(CustomOps.ADAM_STEP, Device.HIP)
@@ -859,25 +918,132 @@ class HIP:
 
     # ---- matmul ----------------------------------------------------------------------------------------------------------
     MATMUL_FORCE = os.environ.get("DLGRAD_HIP_MATMUL_TILE")      # e.g. "128x128": benchmarking aid
+    # "1": a shape met for the first time (and large enough to matter) is timed once with every
+    # plausible tile and the fastest is remembered; "0": shipped table, then the model
+    MATMUL_TUNE = os.environ.get("DLGRAD_HIP_MATMUL_TUNE", "1") != "0"
+    MATMUL_TUNE_MIN_FLOP = 1 << 24
+    _tuned: dict | None = None
+    _tuned_new: dict = {}
+
+    MATMUL_TUNED_FILE = os.path.join(CACHE_DIR, "matmul_tuned.json")
 
     @staticmethod
-    def _pick_tile(M: int, N: int, batch: int) -> str:
+    def _tuned_path() -> str:
+        return HIP.MATMUL_TUNED_FILE
+
+    @staticmethod
+    def _tuned_table() -> dict:
+        """"batch,M,N,K" -> tile: the table shipped beside the kernel generators (measured on
+        MI355X) overlaid with what this machine's own tuning runs have stored in the cache."""
+        if HIP._tuned is None:
+            table = {}
+            for path in (os.path.join(os.path.dirname(K.__file__), "matmul_tuned.json"), HIP._tuned_path()):
+                try:
+                    with open(path) as f:
+                        table.update({k: v for k, v in json.load(f).items() if v in K.MATMUL_CONFIGS})
+                except (OSError, ValueError):
+                    pass
+            HIP._tuned = table
+        return HIP._tuned
+
+    @staticmethod
+    def _model_tile(M: int, N: int, batch: int) -> str:
         """Largest expected throughput = tile rate x fraction of the tile grid that is real
-        output x how well the block count fills 256 CUs (one block per CU already runs a CU
-        near its rate; beyond the resident capacity, whole rounds of blocks are paid for)."""
-        if HIP.MATMUL_FORCE:
-            return HIP.MATMUL_FORCE
+        output x how evenly the blocks load 256 CUs: the busiest CU runs ceil(blocks / 256) of
+        them, and a CU that holds one block of a tile meant to be co-resident is given 85 %."""
         best, best_score = "64x64", -1.0
         for name, (rate, per_cu) in K.MATMUL_TILE_MODEL.items():
-            bm, bn = (int(v) for v in name.split("x"))
+            bm, bn, _ = K.matmul_tile_shape(name)
             tm, tn = (M + bm - 1) // bm, (N + bn - 1) // bn
             nblk = tm * tn * batch
-            slots = 256 * per_cu
-            fill = min(1.0, nblk / 256.0) if nblk <= slots else nblk / float(-(-nblk // slots) * slots)
+            rounds = -(-nblk // 256)
+            fill = nblk / (256.0 * rounds)
+            if rounds == 1 and per_cu > 1:
+                fill *= 0.85
             score = rate * (M * N) / float(tm * bm * tn * bn) * fill
             if score > best_score * 1.0001:
                 best, best_score = name, score
         return best
+
+    @staticmethod
+    def _tile_candidates(M: int, N: int, batch: int) -> list[str]:
+        """Tiles worth timing: none much larger than the output, and the two smallest only
+        where the output is small enough for them to have a chance."""
+        out = []
+        for name in K.MATMUL_CONFIGS:
+            bm, bn, _ = K.matmul_tile_shape(name)
+            if bm > max(32, 2 * M) or bn > max(32, 2 * N):
+                continue
+            if M * N * batch > (1 << 22 if name == "32x32" else 1 << 27 if name == "64x64" else 1 << 62):
+                continue
+            out.append(name)
+        return out
+
+    @staticmethod
+    def _launch_matmul(tile: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple) -> None:
+        bm, bn, threads = K.matmul_tile_shape(tile)
+        k = kernel(K.matmul_kernel, *K.MATMUL_CONFIGS[tile], veca, vecb)
+        launch(k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch), threads, *args)
+
+    @staticmethod
+    def _tune_tile(key: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple) -> str:
+        """Times every plausible tile on the real operands (the output is simply rewritten:
+        all tiles produce the same bits) and stores the winner in the cache directory."""
+        global launch_count
+        l = lib()
+        count0 = launch_count
+        best, best_ms = None, float("inf")
+        e0, e1 = l.event_create(), l.event_create()
+        for tile in HIP._tile_candidates(M, N, batch):
+            HIP._launch_matmul(tile, veca, vecb, M, N, batch, args)                  # loads the code object
+            if COMPILE_ONLY:
+                continue
+            ms, reps = 0.0, 3
+            while True:
+                l.event_record(e0)
+                for _ in range(reps):
+                    HIP._launch_matmul(tile, veca, vecb, M, N, batch, args)
+                l.event_record(e1)
+                l.event_sync(e1)
+                ms = l.event_elapsed_ms(e0, e1) / reps
+                if reps > 3 or ms > 0.1:                             # short kernels: a longer second sample
+                    break
+                reps = 20
+            if ms < best_ms:
+                best, best_ms = tile, ms
+        l.event_destroy(e0)
+        l.event_destroy(e1)
+        launch_count = count0
+        if best is None:
+            return HIP._model_tile(M, N, batch)
+        HIP._tuned_table()[key] = best
+        HIP._tuned_new[key] = best
+        try:
+            os.makedirs(os.path.dirname(HIP._tuned_path()), exist_ok=True)
+            stored = {}
+            if os.path.exists(HIP._tuned_path()):
+                with open(HIP._tuned_path()) as f:
+                    stored = json.load(f)
+            stored.update(HIP._tuned_new)
+            tmp = HIP._tuned_path() + f".{os.getpid()}.tmp"
+            with open(tmp, "w") as f:
+                json.dump(dict(sorted(stored.items())), f, indent=0)
+            os.replace(tmp, HIP._tuned_path())
+        except (OSError, ValueError):
+            pass                                                     # a read-only tree: the choice lives for this process
+        return best
+
+    @staticmethod
+    def _pick_tile(M: int, N: int, Kd: int, batch: int, veca: bool, vecb: bool, args: tuple) -> str:
+        if HIP.MATMUL_FORCE:
+            return HIP.MATMUL_FORCE
+        key = f"{batch},{M},{N},{Kd}"
+        tile = HIP._tuned_table().get(key)
+        if tile is not None:
+            return tile
+        if HIP.MATMUL_TUNE and not capturing() and 2 * M * N * Kd * batch >= HIP.MATMUL_TUNE_MIN_FLOP:
+            return HIP._tune_tile(key, veca, vecb, M, N, batch, args)
+        return HIP._model_tile(M, N, batch)
 
     @staticmethod
     @dispatcher.register(BinaryOps.MATMUL, Device.HIP)
@@ -911,10 +1077,7 @@ class HIP:
             raise ValueError("matrix too large for 32-bit indexing")
         veca = Kd % 4 == 0 and _addr(x) % 16 == 0
         vecb = N % 4 == 0 and _addr(y) % 16 == 0 and out.addr % 16 == 0
-        tile = HIP._pick_tile(M, N, batch)
-        bm, bn = (int(v) for v in tile.split("x"))
-        k = kernel(K.matmul_kernel, *K.MATMUL_CONFIGS[tile], veca, vecb)
-        wm, wn = K.MATMUL_CONFIGS[tile][:2]
-        grid = (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch)
-        launch(k, grid, 64 * wm * wn, _addr(x), _addr(y), out.addr, M, N, Kd, nbc, *sa, *sb)
+        args = (_addr(x), _addr(y), out.addr, M, N, Kd, nbc, *sa, *sb)
+        tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, args)
+        HIP._launch_matmul(tile, veca, vecb, M, N, batch, args)
         return out

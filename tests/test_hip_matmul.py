@@ -10,7 +10,7 @@ import pytest
 
 from dlgrad_amd.runtime import hip
 from oracle import cref
-from tests.hip_util import dev, require_gpu
+from tests.hip_util import check, dev, require_gpu
 
 pytestmark = pytest.mark.gpu
 RNG = np.random.default_rng(3)
@@ -103,3 +103,45 @@ def test_tall_skinny():
     require_gpu()
     x, y = f32(16384, 128), f32(128, 512, scale=128 ** -0.5)
     check_mm((dev(x) @ dev(y)).numpy(), x.astype(np.float64) @ y, "tall-skinny")
+
+
+def test_every_tile_gives_the_same_bits(monkeypatch):
+    """All tiles add the k terms of an output element in the same order, which is what lets
+    the tile be chosen by timing without touching results."""
+    require_gpu()
+    from dlgrad_amd.codegen import hip_kernel as K
+    from dlgrad_amd.runtime.hip import HIP
+    x, y = f32(3, 200, 328), f32(3, 328, 196, scale=328 ** -0.5)
+    xd, yd = dev(x), dev(y)
+    outs = {}
+    for tile in K.MATMUL_CONFIGS:
+        monkeypatch.setattr(HIP, "MATMUL_FORCE", tile)
+        outs[tile] = xd.matmul(yd).numpy()
+    first = outs["64x64"]
+    for tile, got in outs.items():
+        check(got, first, 0, f"{tile} vs 64x64")
+
+
+def test_first_use_of_a_large_shape_times_the_tiles_and_remembers_the_winner(monkeypatch, tmp_path):
+    require_gpu()
+    from dlgrad_amd.runtime import hip as H
+    from dlgrad_amd.runtime.hip import HIP
+    monkeypatch.setattr(HIP, "MATMUL_TUNED_FILE", str(tmp_path / "matmul_tuned.json"))
+    monkeypatch.setattr(HIP, "MATMUL_FORCE", None)
+    monkeypatch.setattr(HIP, "MATMUL_TUNE", True)
+    monkeypatch.setattr(HIP, "_tuned", {})
+    monkeypatch.setattr(HIP, "_tuned_new", {})
+    M, Kd, N = 1000, 520, 776
+    x, y = f32(M, Kd), f32(Kd, N, scale=Kd ** -0.5)
+    n0 = H.launch_count
+    got = (dev(x) @ dev(y)).numpy()
+    assert H.launch_count == n0 + 1                     # the timing launches are not counted as work
+    check_mm(got, x.astype(np.float64) @ y, "tuned shape")
+    if H.COMPILE_ONLY:
+        return
+    key = f"1,{M},{N},{Kd}"
+    assert HIP._tuned[key] in __import__("dlgrad_amd.codegen.hip_kernel", fromlist=["x"]).MATMUL_CONFIGS
+    import json
+    assert json.load(open(tmp_path / "matmul_tuned.json"))[key] == HIP._tuned[key]
+    small = (dev(f32(64, 64)) @ dev(f32(64, 64))).numpy()         # below the threshold: the model picks, nothing is stored
+    assert small.shape == (64, 64) and len(HIP._tuned) == 1
