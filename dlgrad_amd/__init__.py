@@ -6,5 +6,5 @@ from dlgrad_amd import nn  # noqa: F401
 
 
 def manual_seed(seed: int) -> None:
-    """Seeds the host generator behind `uniform` on the hip device."""
+    """Seeds the PCG32 streams behind `uniform` (and so dropout and layer init) on the hip device."""
     _hip_runtime.HIP.manual_seed(seed)

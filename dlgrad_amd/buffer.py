@@ -128,6 +128,16 @@ class Buffer:
         return Buffer(data=dispatcher.dispatch(op=BufferOps.CREATE, device=device, data=arr),
                       shape=arr.shape, device=device, dtype=DType.FLOAT32, ndim=arr.ndim)
 
+    @staticmethod
+    def from_u8(arr: np.ndarray, device: Device) -> "Buffer":
+        """fp32 Buffer holding (float)arr[i] for a uint8 host array: the bytes are uploaded as
+        they are and widened where the Buffer lives."""
+        device = as_device(device)
+        if arr.dtype != np.uint8:
+            raise TypeError(f"from_u8 takes uint8 data, got {arr.dtype}")
+        return Buffer(data=dispatcher.dispatch(op=CustomOps.FROM_U8, device=device, data=arr),
+                      shape=arr.shape, device=device, dtype=DType.FLOAT32, ndim=arr.ndim)
+
     def numpy(self) -> np.ndarray:
         """D2H copy with this Buffer's shape (buffer.py:67-84 returns a host view)."""
         if self.is_host_scalar:
@@ -358,6 +368,13 @@ class Buffer:
         if arr.size != self.numel:
             raise ValueError(f"Buffer size mismatch! Expected {self.numel} elements, got {arr.size}")
         self._dispatch(BufferOps.CREATE, data=arr, into=self)
+
+    def copy_(self, src: "Buffer") -> None:
+        """Overwrites this Buffer's memory with the elements of `src` (same count, same
+        device) without leaving the device; the address stays."""
+        if src.numel != self.numel or src.device is not self.device:
+            raise ValueError(f"copy_: {src.shape} on {src.device} into {self.shape} on {self.device}")
+        self._dispatch(CustomOps.COPY_INTO, dst=self, src=src)
 
     # ---- binary -----------------------------------------------------------------------------------------
     def _binary_op(self, other: "Buffer", op: BinaryOps) -> "Buffer":

@@ -956,6 +956,77 @@ def softmax_plan(L: int, vec: int) -> tuple[bool, int, int]:
 
 
 # =====================================================================================
+# random fill
+# =====================================================================================
+
+PCG32_MULT = 6364136223846793005
+
+
+@cache
+def uniform_pcg32_kernel() -> tuple[str, str, str]:
+    """out[i] = low + (high - low) * f_i (just f_i for low 0, high 1) with f_i = (float)(u_i * 2^-32)
+    and u_i the i-th output of PCG32 (XSH-RR 64/32, the generator of cpu_kernel.py:774-874)
+    started from `state0` on stream increment `inc`.
+
+    The reference walks the generator sequentially.  Here thread t jumps straight to element
+    t (the LCG's state after t steps is state0 * a^t + c * (a^t - 1) / (a - 1), built in
+    O(log t) multiplies), emits it, and then strides through the sequence with the
+    pre-multiplied step (mstride, pstride) = the LCG advanced by the total thread count.
+    Element i therefore holds exactly the value the sequential loop would have written."""
+    name = "uniform_pcg32"
+    src = f"""{PRELUDE}
+static __device__ __forceinline__ u32 pcg_output(u64 s) {{
+    const u32 xorshifted = (u32)(((s >> 18u) ^ s) >> 27u);
+    const u32 rot = (u32)(s >> 59u);
+    return (xorshifted >> rot) | (xorshifted << ((0u - rot) & 31u));
+}}
+extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out, u32 n, u64 state0, u64 inc,
+        u64 mstride, u64 pstride, float low, float high, u32 affine) {{
+    const u32 gid = blockIdx.x * 256u + threadIdx.x;
+    const u32 stride = gridDim.x * 256u;
+    // jump ahead by gid steps
+    u64 acc_mult = 1ull, acc_plus = 0ull, cur_mult = {PCG32_MULT}ull, cur_plus = inc;
+    for (u32 d = gid; d != 0u; d >>= 1) {{
+        if (d & 1u) {{ acc_mult *= cur_mult; acc_plus = acc_plus * cur_mult + cur_plus; }}
+        cur_plus = (cur_mult + 1ull) * cur_plus;
+        cur_mult *= cur_mult;
+    }}
+    u64 s = acc_mult * state0 + acc_plus;
+    const float span = high - low;
+    for (u64 i = gid; i < n; i += stride) {{
+        const float f = (float)pcg_output(s) * 2.3283064365386963e-10f;      // exact: a power of two
+        out[i] = affine ? low + span * f : f;
+        s = s * mstride + pstride;
+    }}
+}}
+"""
+    return src, name, _fmt("P", "I", "Q", "Q", "Q", "Q", "f", "f", "I")
+
+
+@cache
+def u8_to_f32_kernel() -> tuple[str, str, str]:
+    """out[i] = (float)bytes[i]: the cast loop of the MNIST idx loaders (cpu_kernel.py:876-1010),
+    run after the raw bytes have crossed PCIe (a quarter of the fp32 volume).  Four bytes per
+    thread as one 32-bit load and one 16-byte store; `bytes` is 4-byte aligned."""
+    name = "u8_to_f32"
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const unsigned char* __restrict__ bytes,
+        float* __restrict__ out, u32 n) {{
+    const u32 v = blockIdx.x * 256u + threadIdx.x;
+    const u32 i = v * 4u;
+    if (i + 3u < n) {{
+        const u32 w = reinterpret_cast<const u32*>(bytes)[v];
+        reinterpret_cast<float4*>(out)[v] = make_float4((float)(w & 255u), (float)((w >> 8) & 255u),
+                                                        (float)((w >> 16) & 255u), (float)(w >> 24));
+    }} else {{
+        for (u32 j = i; j < n; ++j) out[j] = (float)bytes[j];
+    }}
+}}
+"""
+    return src, name, _fmt("P", "P", "I")
+
+
+# =====================================================================================
 # fused RMSNorm
 # =====================================================================================
 

@@ -6,6 +6,7 @@ from dlgrad_amd import ops
 from dlgrad_amd.device import Device
 from dlgrad_amd.nn import optim, utils  # noqa: F401
 from dlgrad_amd.tensor import Tensor
+from dlgrad_amd.nn import datasets  # noqa: E402,F401  (uses Tensor)
 
 
 class Linear:

@@ -420,6 +420,9 @@ def _map(tag: str, expr: str, operands: list[Buffer], out_shape: tuple, svals: t
     return out
 
 
+_U64 = (1 << 64) - 1
+
+
 class HIP:
     """Dispatch-table entries for Device.HIP."""
 
@@ -432,6 +435,27 @@ class HIP:
         if a.size:
             lib().h2d(p.addr, a.ctypes.data, a.nbytes)
         return p
+
+    @staticmethod
+    @dispatcher.register(CustomOps.FROM_U8, Device.HIP)
+    def from_u8(data: np.ndarray) -> DevicePtr:
+        a = np.ascontiguousarray(data, dtype=np.uint8)
+        n = a.size
+        if n >= 2 ** 32:
+            raise ValueError("array too large for 32-bit indexing")
+        out = alloc(n)
+        if n == 0:
+            return out
+        raw = alloc((n + 3) // 4)                                # staging for the bytes; freed in stream order
+        lib().h2d(raw.addr, a.ctypes.data, n)
+        launch(kernel(K.u8_to_f32_kernel), ((n + 3) // 4 + 255) // 256, 256, raw.addr, out.addr, n)
+        return out
+
+    @staticmethod
+    @dispatcher.register(CustomOps.COPY_INTO, Device.HIP)
+    def copy_into(dst: Buffer, src: Buffer) -> None:
+        if dst.numel:
+            lib().d2d(_addr(dst), _addr(src), 4 * dst.numel)
 
     @staticmethod
     @dispatcher.register(CustomOps.TO_HOST, Device.HIP)
@@ -447,20 +471,60 @@ class HIP:
         print(HIP.to_host(x))
 
     # ---- creation -------------------------------------------------------------------------------
-    _rng = np.random.default_rng()
+    _seed = int.from_bytes(os.urandom(8), "little")        # the reference reads /dev/random per call
+    _stream = 0                                            # one PCG32 stream per uniform() call
 
     @staticmethod
     def manual_seed(seed: int) -> None:
-        HIP._rng = np.random.default_rng(seed)
+        """Makes every later uniform() repeatable: call k after this draws PCG32 stream k of `seed`."""
+        HIP._seed, HIP._stream = int(seed) & _U64, 0
+
+    @staticmethod
+    def _pcg_start(seed: int, seq: int) -> tuple[int, int]:
+        """(state, inc) after pcg32_srandom_r(seed, seq) (cpu_kernel.py:829-836)."""
+        inc = ((seq << 1) | 1) & _U64
+        state = inc                                        # (0 * a + inc)
+        state = (state + seed) & _U64
+        state = (state * K.PCG32_MULT + inc) & _U64
+        return state, inc
+
+    @staticmethod
+    def _lcg_jump(delta: int, inc: int) -> tuple[int, int]:
+        """(m, p) with state_after_delta_steps = state * m + p  (mod 2^64)."""
+        acc_m, acc_p, cur_m, cur_p = 1, 0, K.PCG32_MULT, inc
+        while delta:
+            if delta & 1:
+                acc_m = (acc_m * cur_m) & _U64
+                acc_p = (acc_p * cur_m + cur_p) & _U64
+            cur_p = ((cur_m + 1) * cur_p) & _U64
+            cur_m = (cur_m * cur_m) & _U64
+            delta >>= 1
+        return acc_m, acc_p
 
     @staticmethod
     @dispatcher.register(BufferOps.UNIFORM, Device.HIP)
     def uniform(shape: tuple, low: float = 0.0, high: float = 1.0) -> DevicePtr:
-        """U[low, high) drawn on the host and uploaded.  The reference's generator
-        (PCG32 reseeded from /dev/random per call, cpu_kernel.py:774-874) cannot be
-        reproduced value for value; only range and moments are comparable."""
-        u = HIP._rng.random(shape, dtype=np.float32)
-        return HIP.create(np.float32(low) + (np.float32(high) - np.float32(low)) * u)
+        """U[low, high) generated on the device: PCG32 as in cpu_kernel.py:774-874, element i
+        being the i-th output of the stream, (float)ldexp(u32, -32), then low + (high-low)*f.
+        The reference reseeds from /dev/random on every call; here the seed is the process's
+        (random unless manual_seed was called) and each call takes the next stream, so a
+        seeded run repeats and successive tensors differ."""
+        n = prod_(shape)
+        if n >= 2 ** 32:
+            raise ValueError("tensor too large for 32-bit indexing")
+        if capturing():
+            raise RuntimeError("uniform() inside a captured graph would replay the same numbers on every launch")
+        out = alloc(n)
+        if n == 0:
+            return out
+        state0, inc = HIP._pcg_start(HIP._seed, HIP._stream)
+        HIP._stream += 1
+        blocks = min((n + 255) // 256, 4096)
+        m, p = HIP._lcg_jump(blocks * 256, inc)
+        affine = not (float(low) == 0.0 and float(high) == 1.0)
+        launch(kernel(K.uniform_pcg32_kernel), blocks, 256, out.addr, n, state0, inc, m, p, float(low), float(high),
+               int(affine))
+        return out
 
     @staticmethod
     @dispatcher.register(BufferOps.FULL, Device.HIP)

@@ -4,13 +4,16 @@ RMSNorm (not LayerNorm), ReLU MLP, no biases, no dropout, untied lm_head, learne
 positional embedding -- what that file builds, not what its config comment suggests.
 Differences that do not change values: the causal mask (seven small kernels,
 examples/gpt.py:52-53) is built once per (T, device) instead of once per block per step,
-and every parameter is created on the model's device.
+every parameter is created on the model's device, and the key/value cache of incremental
+decoding stays on the device (the reference concatenates it in numpy on the host,
+examples/gpt.py:57-60).
 """
 from __future__ import annotations
 
 import numpy as np
 
 from dlgrad_amd import Tensor, nn
+from dlgrad_amd.helpers import STRICT_REFERENCE
 
 
 class GPTConfig:
@@ -42,17 +45,57 @@ class CausalSelfAttention:
         self.v_proj = nn.Linear(c.n_embd, c.n_embd, bias=False, device=c.device)
         self.c_proj = nn.Linear(c.n_embd, c.n_embd, bias=False, device=c.device)
 
-    def __call__(self, x: Tensor) -> Tensor:
+    def __call__(self, x: Tensor, cache: "KVCache | None" = None, layer: int = 0) -> Tensor:
+        """Without a cache, or with an empty one: causal attention over the T positions of x
+        (whose k/v projections are stored if a cache is given).  With a filled cache and
+        T == 1: the new position attends to everything cached plus itself, no mask
+        (examples/gpt.py:44-66)."""
         B, T, C = x.shape
         split = (B, T, self.n_head, self.head_dim)
         q = self.q_proj(x).reshape(split).transpose(1, 2)            # (B, h, T, d)
-        k = self.k_proj(x).reshape(split).transpose(1, 2)
-        v = self.v_proj(x).reshape(split).transpose(1, 2)
-        att = (q @ k.transpose(2, 3)) * self.scale                   # (B, h, T, T)
-        att = att.masked_fill(causal_mask(T, x.device), float("-inf"))
-        att = att.softmax(dim=3)
+        k_lin, v_lin = self.k_proj(x), self.v_proj(x)                # (B, T, C)
+        if cache is not None and cache.length > 0:
+            assert T == 1, "incremental attention takes one new position"
+            cache.write(layer, k_lin, v_lin, cache.length)
+            k, v = cache.view(layer, cache.length + 1, self.n_head)  # (B, h, n, d)
+            att = ((q @ k.transpose(2, 3)) * self.scale).softmax(dim=3)
+        else:
+            if cache is not None:
+                cache.write(layer, k_lin, v_lin, 0)
+            k = k_lin.reshape(split).transpose(1, 2)
+            v = v_lin.reshape(split).transpose(1, 2)
+            att = (q @ k.transpose(2, 3)) * self.scale               # (B, h, T, T)
+            att = att.masked_fill(causal_mask(T, x.device), float("-inf"))
+            att = att.softmax(dim=3)
         y = (att @ v).transpose(1, 2).reshape((B, T, C))
         return self.c_proj(y)
+
+
+class KVCache:
+    """The k and v projections of every position so far, per layer, on the model's device.
+
+    Stored as (block_size, B, C): the first n positions are then one contiguous view, and
+    appending a position is a single device-to-device copy of B*C floats.  `view` hands
+    attention the same (B, h, n, d) values the reference gets by concatenating on the host."""
+
+    def __init__(self, c: GPTConfig, batch: int) -> None:
+        shape = (c.block_size, batch, c.n_embd)
+        self.k = [Tensor.full(shape, 0.0, device=c.device) for _ in range(c.n_layer)]
+        self.v = [Tensor.full(shape, 0.0, device=c.device) for _ in range(c.n_layer)]
+        self.batch, self.length = batch, 0
+
+    def write(self, layer: int, k: Tensor, v: Tensor, at: int) -> None:
+        """k, v: (B, T, C) projections of positions at .. at+T-1."""
+        B, T, C = k.shape
+        for store, new in ((self.k[layer], k), (self.v[layer], v)):
+            rows = new if (B == 1 or T == 1) else new.transpose(0, 1)          # (T, B, C) order
+            store[at:at + T].data.copy_(rows.data)
+
+    def view(self, layer: int, n: int, n_head: int) -> tuple[Tensor, Tensor]:
+        C = self.k[layer].shape[2]
+        split = (n, self.batch, n_head, C // n_head)
+        return (self.k[layer][0:n].reshape(split).permute((1, 2, 0, 3)),
+                self.v[layer][0:n].reshape(split).permute((1, 2, 0, 3)))
 
 
 class MLP:
@@ -71,8 +114,8 @@ class Block:
         self.ln2 = nn.RMSNorm(c.n_embd, device=c.device)
         self.mlp = MLP(c)
 
-    def __call__(self, x: Tensor) -> Tensor:
-        x = x + self.attn(self.ln1(x))
+    def __call__(self, x: Tensor, cache: KVCache | None = None, layer: int = 0) -> Tensor:
+        x = x + self.attn(self.ln1(x), cache, layer)
         return x + self.mlp(self.ln2(x))
 
 
@@ -98,6 +141,59 @@ class GPT:
         V = self.config.vocab_size
         loss = logits.reshape((B * T, V)).cross_entropy_loss(targets.reshape((B * T, 1)))
         return logits, loss
+
+    # ---- incremental decoding with a device-resident key/value cache -----------------------------
+    def _hidden(self, idx: Tensor, pos: Tensor, cache: KVCache) -> Tensor:
+        x = self.wte(idx) + self.wpe(pos)
+        for i, block in enumerate(self.blocks):
+            x = block(x, cache, i)
+        return self.ln_f(x)
+
+    def prefill(self, idx: Tensor) -> tuple[Tensor, KVCache]:
+        """Full forward over idx (B, T) that also fills a fresh cache; returns the logits of
+        the last position as (B, 1, V) and the cache (the inference branch of
+        examples/gpt.py:103-112, which slices the last position out on the host)."""
+        B, T = idx.shape
+        cache = KVCache(self.config, B)
+        x = self._hidden(idx, Tensor.arange((T,), device=idx.device), cache)
+        cache.length = T
+        C = x.shape[2]
+        last = x.reshape((T, C))[T - 1:T] if B == 1 else x.transpose(0, 1)[T - 1:T]
+        return self.lm_head(last.reshape((B, 1, C))), cache
+
+    def forward_incremental(self, new_idx: Tensor, pos: Tensor, cache: KVCache) -> Tensor:
+        """One new token per sequence: new_idx (B, 1), pos (1, 1) its position id; appends to
+        the cache and returns logits (B, 1, V) (examples/gpt.py:114-136)."""
+        assert new_idx.shape[1] == 1, "incremental forward expects a single token"
+        x = self._hidden(new_idx, pos, cache)
+        cache.length += 1
+        return self.lm_head(x)
+
+    def generate_greedy_cached(self, first_token: int, max_new_tokens: int,
+                               reference_positions: bool = STRICT_REFERENCE) -> list[int]:
+        """The control flow of the reference's generate (examples/gpt.py:169-226) with argmax in
+        place of sampling: a full forward when there is no cache, one-token steps after it,
+        and -- as there -- no sliding: once the sequence has reached block_size the cache is
+        dropped and every further token is a full forward over the last block_size tokens.
+        reference_positions reproduces its position id for an incremental token, the sequence
+        length *including* that token (one more than the token's index, examples/gpt.py:199).
+        Tokens, cache and argmax stay on the device; the ids come back in one download."""
+        c = self.config
+        seq = Tensor.full((max_new_tokens + 1, 1), float(int(first_token)), device=c.device)
+        n, start, cache = 1, 0, None                       # tokens so far; first token of the context window
+        for _ in range(max_new_tokens):
+            if n - start >= c.block_size:
+                start, cache = n - c.block_size, None
+            if cache is None:
+                logits, cache = self.prefill(seq[start:n].reshape((1, n - start)))
+            else:
+                length = n - start
+                pos = Tensor.full((1, 1), float(length if reference_positions else length - 1), device=c.device)
+                logits = self.forward_incremental(seq[n - 1:n], pos, cache)
+            nxt = logits.reshape((1, c.vocab_size)).argmax(1)                           # (1, 1), on the device
+            seq[n:n + 1].data.copy_(nxt.data)
+            n += 1
+        return [int(v) for v in seq.numpy().reshape(-1)]
 
     def generate_greedy(self, first_token: int, max_new_tokens: int) -> list[int]:
         """Greedy decode with full-context recompute per token, context cropped to

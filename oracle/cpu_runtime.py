@@ -39,11 +39,13 @@ def _reg(op):
 
 
 class CPU:
-    _rng = np.random.default_rng()
+    _seed = int.from_bytes(__import__("os").urandom(8), "little")
+    _stream = 0
 
     @staticmethod
     def manual_seed(seed: int) -> None:
-        CPU._rng = np.random.default_rng(seed)
+        """Same convention as the hip runtime: call k after this draws PCG32 stream k of `seed`."""
+        CPU._seed, CPU._stream = int(seed) & ((1 << 64) - 1), 0
 
     @staticmethod
     @_reg(BufferOps.CREATE)
@@ -52,6 +54,16 @@ class CPU:
             into.ptr.arr[:data.size] = np.asarray(data, dtype=np.float32).reshape(-1)
             return into.ptr
         return HostPtr(np.array(data, dtype=np.float32, copy=True))
+
+    @staticmethod
+    @_reg(CustomOps.FROM_U8)
+    def from_u8(data: np.ndarray) -> HostPtr:
+        return HostPtr(np.asarray(data, dtype=np.uint8).astype(np.float32))
+
+    @staticmethod
+    @_reg(CustomOps.COPY_INTO)
+    def copy_into(dst: Buffer, src: Buffer) -> None:
+        dst.ptr.arr[:dst.numel] = src.ptr.arr[:src.numel]
 
     @staticmethod
     @_reg(CustomOps.TO_HOST)
@@ -66,8 +78,8 @@ class CPU:
     @staticmethod
     @_reg(BufferOps.UNIFORM)
     def uniform(shape: tuple, low: float = 0.0, high: float = 1.0) -> HostPtr:
-        u = CPU._rng.random(shape, dtype=np.float32)
-        return HostPtr(np.float32(low) + (np.float32(high) - np.float32(low)) * u)
+        seq, CPU._stream = CPU._stream, CPU._stream + 1
+        return HostPtr(cref.uniform(shape, low, high, seed=CPU._seed, seq=seq))
 
     @staticmethod
     @_reg(BufferOps.FULL)

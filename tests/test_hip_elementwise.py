@@ -9,6 +9,7 @@ import pytest
 from dlgrad_amd.buffer import Buffer
 from dlgrad_amd.device import Device
 from oracle import cref
+from dlgrad_amd.runtime import hip
 from tests.hip_util import check, dev, require_gpu
 
 pytestmark = pytest.mark.gpu
@@ -139,3 +140,64 @@ def test_fills():
     u = Buffer.uniform((100000,), Device.HIP, "float32", low=-2.0, high=2.0).numpy()
     if u.any():
         assert u.min() >= -2 and u.max() < 2 and abs(u.mean()) < 0.05
+
+
+@pytest.mark.parametrize("n", [1, 6, 255, 256, 257, 100003, 4096 * 256 + 77, 3_000_001])
+def test_uniform_is_the_sequential_pcg32_stream(n):
+    """Element i is the i-th output of PCG32 (seed, stream), however many threads shared the
+    work: bit-exact in the [0, 1) form, where no arithmetic follows the conversion; the affine
+    form may differ from the oracle by the rounding of one fused multiply-add (the reference's
+    -ffast-math leaves that contraction to its compiler)."""
+    require_gpu()
+    import dlgrad_amd
+    from dlgrad_amd.runtime.hip import HIP
+    dlgrad_amd.manual_seed(42)
+    HIP._stream = 54
+    got = Buffer.uniform((n,), Device.HIP, "float32").numpy()
+    assert HIP._stream == 55
+    check(got, cref.uniform((n,), 0.0, 1.0, seed=42, seq=54), 0, f"U[0,1) n={n}")
+    if n >= 6 and not hip.COMPILE_ONLY:       # the published pcg32 demo vector (seed 42, sequence 54)
+        want = np.array([0xa15c02b7, 0x7b47f409, 0xba1d3330, 0x83d2f293, 0xbfa4784b, 0xcbed606e], np.float64)
+        np.testing.assert_array_equal(got[:6], (want / 2 ** 32).astype(np.float32))
+    HIP._stream = 7
+    got = Buffer.uniform((n,), Device.HIP, "float32", low=-0.0357, high=0.0357).numpy()
+    want = cref.uniform((n,), -0.0357, 0.0357, seed=42, seq=7)
+    if not hip.COMPILE_ONLY:
+        assert np.abs(got - want).max() <= np.spacing(np.float32(0.0357))
+        assert got.min() >= np.float32(-0.0357) and got.max() <= np.float32(0.0357)
+
+
+def test_seeded_layers_start_equal_on_both_devices():
+    """manual_seed + the per-call streams give the hip device and the oracle's cpu device the
+    same initial weights."""
+    require_gpu()
+    import dlgrad_amd
+    import oracle.cpu_runtime as ocpu
+    from dlgrad_amd import nn
+    dlgrad_amd.manual_seed(5)
+    ocpu.CPU.manual_seed(5)
+    a, b = nn.Linear(33, 17, device="hip"), nn.Linear(33, 17, device="cpu")
+    if not hip.COMPILE_ONLY:
+        assert np.abs(a.weight.numpy() - b.weight.numpy()).max() <= np.spacing(np.float32(33 ** -0.5))
+        assert np.abs(a.bias.numpy() - b.bias.numpy()).max() <= np.spacing(np.float32(33 ** -0.5))
+        assert not np.array_equal(a.weight.numpy().ravel()[:17], a.bias.numpy().ravel())     # different streams
+
+
+def test_dropout_mask_comes_from_the_seeded_stream():
+    """dropout(p) keeps x / (1 - p) where the stream's U[0,1) value is >= p and zeroes the rest
+    (ops.py:442-462); the gradient passes through the same mask."""
+    require_gpu()
+    import dlgrad_amd
+    from dlgrad_amd import Tensor
+    x = f32(64, 100)
+    dlgrad_amd.manual_seed(9)
+    t = Tensor(x, device="hip", requires_grad=True)
+    y = t.dropout(0.3)
+    y.sum().backward()
+    if hip.COMPILE_ONLY:
+        return
+    keep = cref.uniform((64, 100), 0.0, 1.0, seed=9, seq=0) >= np.float32(0.3)
+    scale = np.float32(1.0 / (1.0 - 0.3))
+    check(y.numpy(), np.where(keep, x, np.float32(0)) * scale, 0, "dropout forward")
+    check(t.grad.numpy(), np.where(keep, np.float32(1), np.float32(0)) * scale, 0, "dropout backward")
+    assert 0.6 < keep.mean() < 0.8

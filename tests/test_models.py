@@ -219,6 +219,59 @@ def test_gpt_greedy_decode_hip_vs_cpu_oracle():
         assert outs["hip"] == outs["cpu"]
 
 
+def test_cached_decode_reproduces_full_recompute_on_the_cpu_oracle():
+    """With each incremental token at its own position the key/value cache changes nothing but
+    the amount of work: same ids as recomputing the whole context, before and after the
+    window fills up.  With the reference's position ids (one too many) the ids differ."""
+    model = G.GPT(G.GPTConfig(device="cpu", **dict(TINY, n_embd=32, block_size=12)))
+    G.init_weights_(model, 3, std=0.5)
+    full = model.generate_greedy(3, 30)
+    assert model.generate_greedy_cached(3, 30, reference_positions=False) == full
+    shifted = model.generate_greedy_cached(3, 30, reference_positions=True)
+    assert len(shifted) == 31 and shifted[:2] == full[:2] and shifted != full
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("reference_positions", [True, False])
+def test_gpt_cached_decode_hip_vs_cpu_oracle(reference_positions):
+    """Device-resident cache (hip) against the same loop on the C oracle's cpu device: equal
+    ids through prefill, incremental steps and the window-full regime; logits of one
+    incremental step within 1e-4 of the largest."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    outs, logits = {}, {}
+    for dev in ("cpu", "hip"):
+        model = G.GPT(G.GPTConfig(device=dev, **dict(TINY, n_embd=64, block_size=32)))
+        G.init_weights_(model, 3, std=0.2)
+        outs[dev] = model.generate_greedy_cached(0, 48, reference_positions=reference_positions)
+        idx = Tensor(np.array([[5, 1, 4, 2, 2, 7]], np.float32), device=dev)
+        _, cache = model.prefill(idx)
+        step = model.forward_incremental(Tensor(np.array([[3]], np.float32), device=dev),
+                                         Tensor(np.array([[6]], np.float32), device=dev), cache)
+        assert cache.length == 7 and step.shape == (1, 1, model.config.vocab_size)
+        logits[dev] = step.numpy()
+    if not hip.COMPILE_ONLY:
+        assert outs["hip"] == outs["cpu"]
+        tensors_close(logits["hip"], logits["cpu"], "incremental logits", 1e-4)
+
+
+@pytest.mark.gpu
+def test_cached_decode_with_a_batch_keeps_sequences_apart():
+    """B = 3: prefill + two incremental steps equal the last-position logits of full forwards."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    model = G.GPT(G.GPTConfig(device="hip", **dict(TINY, n_embd=64, block_size=32)))
+    G.init_weights_(model, 4, std=0.2)
+    ids = np.random.default_rng(1).integers(0, model.config.vocab_size, (3, 9)).astype(np.float32)
+    _, cache = model.prefill(Tensor(ids[:, :7], device="hip"))
+    for t in (7, 8):
+        inc = model.forward_incremental(Tensor(ids[:, t:t + 1], device="hip"),
+                                        Tensor(np.array([[t]], np.float32), device="hip"), cache).numpy()
+        full, _ = model(Tensor(ids[:, :t + 1], device="hip"))
+        if not hip.COMPILE_ONLY:
+            tensors_close(inc[:, 0], full.numpy()[:, t], f"position {t}", 1e-4)
+
+
 @pytest.mark.gpu
 def test_fused_adam_kernel_is_bit_identical_to_the_fourteen_kernel_expression(monkeypatch):
     if not (hip.available() or hip.COMPILE_ONLY):
