@@ -240,6 +240,24 @@ class Buffer:
         y = other if other.shape == p2 else other._like(other.ptr, p2)
         return self._like(self._dispatch(BinaryOps.MATMUL, x=x, y=y), out_shape)
 
+    def matmul_nt(self, other: "Buffer") -> "Buffer":
+        """self (.., M, K) @ other(.., N, K)^T without materialising the transpose."""
+        swapped = other.shape[:-2] + (other.shape[-1], other.shape[-2])
+        p1, p2, out_shape = broadcast_shapes(self.shape, swapped)
+        p2 = p2[:-2] + (p2[-1], p2[-2])
+        x = self if self.shape == p1 else self._like(self.ptr, p1)
+        y = other if other.shape == p2 else other._like(other.ptr, p2)
+        return self._like(self._dispatch(CustomOps.MATMUL_NT, x=x, y=y), out_shape)
+
+    def matmul_tn(self, other: "Buffer") -> "Buffer":
+        """self(.., K, M)^T @ other (.., K, N) without materialising the transpose."""
+        swapped = self.shape[:-2] + (self.shape[-1], self.shape[-2])
+        p1, p2, out_shape = broadcast_shapes(swapped, other.shape)
+        p1 = p1[:-2] + (p1[-1], p1[-2])
+        x = self if self.shape == p1 else self._like(self.ptr, p1)
+        y = other if other.shape == p2 else other._like(other.ptr, p2)
+        return self._like(self._dispatch(CustomOps.MATMUL_TN, x=x, y=y), out_shape)
+
     def permute(self, order: tuple) -> "Buffer":
         order = tuple(order)
         return self._like(self._dispatch(UnaryOps.PERMUTE, x=self, order=order),

@@ -1163,91 +1163,159 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 # matmul
 # =====================================================================================
 
+MATMUL_LDS_LIMIT = 160 * 1024          # LDS per CU on gfx950, all of it available to one block
+
+
+def matmul_lds_bytes(WM: int, WN: int, MI: int, NJ: int, BK: int, ta: bool = False, tb: bool = False) -> int:
+    """Static LDS of one block (both operands, double-buffered)."""
+    BM, BN = 32 * MI * WM, 32 * NJ * WN
+    a = BK * BM if ta else BM * (BK + 4)
+    b = BN * (BK + 4) if tb else BK * BN
+    return 2 * 4 * (a + b)
+
+
 @cache
-def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb: bool) -> tuple[str, str, str]:
-    """C[z] = A[z] . B[z], fp32, row-major, on the matrix cores (v_mfma_f32_32x32x2_f32).
+def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb: bool,
+                  ta: bool = False, tb: bool = False) -> tuple[str, str, str]:
+    """C[z] = op(A[z]) . op(B[z]), fp32, row-major, on the matrix cores (v_mfma_f32_32x32x2_f32).
 
     Replaces the i-k-j loops of cpu_kernel.py:351-428.  Batched over blockIdx.z with two
     batch extents (z = zb * nbc + zc) whose operand strides may be 0, which is how the
     reference broadcasts a batch or channel dim (cpu.py:519-532, :553-559).
+    ta: A is given transposed, as a (K, M) row-major array; tb: B is given transposed, as
+    (N, K).  These read in place what MatMul.backward and Linear otherwise materialise with a
+    permute kernel (ops.py:308-335, tensor.py:549-563); the k terms of every output element
+    are added in the same order in all variants, so the results are bit-identical.
 
     Tiling.  A block of WM x WN wavefronts owns a (32*MI*WM) x (32*NJ*WN) tile of C; each
     wavefront owns MI x NJ MFMA tiles of 32x32, i.e. 16*MI*NJ accumulator registers.  The
     K loop advances BK at a time through double-buffered LDS (one barrier per step; the
     next A/B tiles are in flight in registers while the current ones are multiplied).
 
-    Operand layout chosen for 16-byte LDS traffic:
-      * A sits in LDS as [m][k] with a 4-float pad per row.  One 32x32x2 MFMA consumes,
-        per lane, A[m = lane%32][k = lane/32].  The k order inside a group of 8 is
-        permuted (lane half h takes k = 8*blk + 4*h + s at step s, for A and B alike), so
-        one ds_read_b128 per lane feeds four MFMA steps.
-      * the NJ column tiles of a wavefront interleave: lane c of column tile j owns
-        column NJ*c + j.  One read of NJ consecutive floats of B[k][...] then feeds NJ
-        MFMAs, and in the epilogue each lane holds NJ adjacent columns of a row: one
-        dwordx4 store for NJ = 4, a fully coalesced 512-byte row segment per half wave.
-    veca / vecb: 16-byte global loads of A (needs K % 4 == 0) and of B plus 16-byte
-    stores of C (needs N % 4 == 0); bases and batch strides are then 16-byte aligned.
-    Out-of-range rows, columns and k are read as zero and never written.
+    An operand whose global rows run along k (A, or B when tb) sits in LDS as [row][k] with a
+    4-float pad; one 32x32x2 MFMA consumes, per lane, X[row = lane%32][k = lane/32], and the
+    k order inside a group of 8 is permuted (lane half h takes k = 8*blk + 4*h + s at step s,
+    for both operands alike), so one ds_read_b128 per lane feeds four MFMA steps.
+    An operand whose global rows run along the output dim (B, or A when ta) sits in LDS as
+    [k][col]; the tiles a wavefront owns along that dim interleave (lane c of tile j owns
+    col NJ*c + j), so one read of NJ consecutive floats feeds NJ MFMAs, and for B the
+    epilogue then holds NJ adjacent columns of a row per lane: one dwordx4 store for NJ = 4,
+    a coalesced 512-byte row segment per half wave.
+    veca / vecb: 16-byte global loads of A / of B (the contiguous extent is a multiple of 4
+    and bases and batch strides are 16-byte aligned); vecb and not tb also means 16-byte
+    stores of C.  Out-of-range rows, columns and k are read as zero and never written.
     Blocks are renumbered so that the eight XCDs (round-robin dispatch) each work on a
     contiguous band of C tiles, walked in groups of 8 tile rows for L2 reuse."""
     BM, BN, T = 32 * MI * WM, 32 * NJ * WN, 64 * WM * WN
-    AKQ, BNQ = BK // 4, BN // 4
-    assert T % AKQ == 0 and BK % 8 == 0 and NJ in (1, 2, 3, 4) and T >= BNQ
-    # loader threads walk the A tile in passes of ROWS_A rows and the B tile in passes of
-    # ROWS_B rows; when a tile extent is no multiple of the pass (96- and 192-wide tiles)
-    # the last pass is cut off by a guard, and threads beyond the last whole B row repeat
-    # a neighbour's element (same address, same value)
-    ROWS_A, ROWS_B = T // AKQ, T // BNQ
-    PA, PB = -(-BM // ROWS_A), -(-BK // ROWS_B)
-    guard_a = BM % ROWS_A != 0
-    guard_b = BK % ROWS_B != 0 or T % BNQ != 0
-    name = f"matmul_{BM}x{BN}x{BK}_w{WM}x{WN}_{'a4' if veca else 'a1'}{'b4' if vecb else 'b1'}"
-    LDA, LDB = BK + 4, BN
-    bvec = {1: "float", 2: "float2", 3: "f3v", 4: "float4"}[NJ]
+    assert BK % 8 == 0 and MI in (1, 2, 3, 4) and NJ in (1, 2, 3, 4)
+    assert matmul_lds_bytes(WM, WN, MI, NJ, BK, ta, tb) <= MATMUL_LDS_LIMIT
+    name = (f"matmul_{BM}x{BN}x{BK}_w{WM}x{WN}_{'a4' if veca else 'a1'}{'b4' if vecb else 'b1'}"
+            f"{'_tn' if ta else ''}{'_nt' if tb else ''}")
     comp = ["x", "y", "z", "w"]
+    vtype = {1: "float", 2: "float2", 3: "f3v", 4: "float4"}
 
-    if veca:
-        load_a = """            ra[p] = (m < g.M && k < g.K) ? *reinterpret_cast<const float4*>(A + (u64)m * g.K + k)
-                                         : make_float4(0.f, 0.f, 0.f, 0.f);"""
-    else:
-        load_a = """            const float* __restrict__ s = A + (u64)m * g.K + k;
-            const bool okm = m < g.M;
-            ra[p].x = (okm && k + 0u < g.K) ? s[0] : 0.f;
-            ra[p].y = (okm && k + 1u < g.K) ? s[1] : 0.f;
-            ra[p].z = (okm && k + 2u < g.K) ? s[2] : 0.f;
-            ra[p].w = (okm && k + 3u < g.K) ? s[3] : 0.f;"""
-    if vecb:
-        load_b = """            rb[p] = (k < g.K && n < g.N) ? *reinterpret_cast<const float4*>(B + (u64)k * g.N + n)
-                                         : make_float4(0.f, 0.f, 0.f, 0.f);"""
-    else:
-        load_b = """            const float* __restrict__ s = B + (u64)k * g.N + n;
-            const bool okk = k < g.K;
-            rb[p].x = (okk && n + 0u < g.N) ? s[0] : 0.f;
-            rb[p].y = (okk && n + 1u < g.N) ? s[1] : 0.f;
-            rb[p].z = (okk && n + 2u < g.N) ? s[2] : 0.f;
-            rb[p].w = (okk && n + 3u < g.N) ? s[3] : 0.f;"""
+    def loader(X: str, along_k: bool, rows_name: str, R: int, ld: str, ext: str, base: str, vec: bool):
+        """Global -> registers -> LDS for operand X (A or B).
+        along_k: global rows run along k: element (row, k) at X[row * K + k]; LDS [row][k].
+        else:    global rows run along the output dim: element (k, col) at X[k * ld + col]; LDS [k][col].
+        Loader threads walk the tile in passes; a tile extent that is no multiple of the pass
+        is cut off by a guard, and threads beyond the last whole row repeat a neighbour's
+        element (same address, same value)."""
+        x = X.lower()
+        if along_k:
+            Q = BK // 4
+            assert T % Q == 0
+            rpp = T // Q                                   # tile rows per pass
+            P = -(-R // rpp)
+            guard = f"if ({x}_r + p * {rpp}u < {R}u) " if R % rpp else ""
+            idx = f"const u32 {x}_q = tid % {Q}u, {x}_r = tid / {Q}u;"
+            where = f"const u32 row = {base} + {x}_r + p * {rpp}u, k = k0 + 4u * {x}_q;"
+            if vec:
+                ld_code = (f"r{x}[p] = (row < g.{ext} && k < g.K) ? *reinterpret_cast<const float4*>({X} + (u64)row * g.K + k)\n"
+                           f"                                         : make_float4(0.f, 0.f, 0.f, 0.f);")
+            else:
+                ld_code = (f"const float* __restrict__ s = {X} + (u64)row * g.K + k;\n"
+                           f"            const bool ok = row < g.{ext};\n" +
+                           "".join(f"            r{x}[p].{c} = (ok && k + {n}u < g.K) ? s[{n}] : 0.f;\n" for n, c in enumerate(comp)))
+            st = f"{guard}*reinterpret_cast<float4*>(&{X}s[buf][{x}_r + p * {rpp}u][4u * {x}_q]) = r{x}[p];"
+            decl = f"__shared__ __attribute__((aligned(16))) float {X}s[2][{R}][{BK + 4}];"
+        else:
+            Q = R // 4
+            assert T >= Q
+            rpp = T // Q                                   # k rows per pass
+            P = -(-BK // rpp)
+            guard = f"if ({x}_r + p * {rpp}u < BK) " if (BK % rpp or T % Q) else ""
+            idx = f"const u32 {x}_q = tid % {Q}u, {x}_r = tid / {Q}u;"
+            where = f"const u32 k = k0 + {x}_r + p * {rpp}u, col = {base} + 4u * {x}_q;"
+            if vec:
+                ld_code = (f"r{x}[p] = (k < g.K && col < g.{ext}) ? *reinterpret_cast<const float4*>({X} + (u64)k * g.{ext} + col)\n"
+                           f"                                         : make_float4(0.f, 0.f, 0.f, 0.f);")
+            else:
+                ld_code = (f"const float* __restrict__ s = {X} + (u64)k * g.{ext} + col;\n"
+                           f"            const bool ok = k < g.K;\n" +
+                           "".join(f"            r{x}[p].{c} = (ok && col + {n}u < g.{ext}) ? s[{n}] : 0.f;\n" for n, c in enumerate(comp)))
+            st = f"{guard}*reinterpret_cast<float4*>(&{X}s[buf][{x}_r + p * {rpp}u][4u * {x}_q]) = r{x}[p];"
+            decl = f"__shared__ __attribute__((aligned(16))) float {X}s[2][{BK}][{R}];"
+        load = f"""        #pragma unroll
+        for (u32 p = 0; p < {P}u; ++p) {{
+            {where}
+            {ld_code}
+        }}
+"""
+        stash = f"""        #pragma unroll
+        for (u32 p = 0; p < {P}u; ++p)
+            {st}
+"""
+        return decl, idx, P, load, stash
 
-    mfma = ""
-    for s in range(4):
-        mfma += f"            {{ const {bvec} b = *reinterpret_cast<const {bvec}*>(&Bs[buf][kb + 4u * h + {s}u][wn0 + {NJ}u * r]);\n"
-        for i in range(MI):
-            for j in range(NJ):
-                bj = "b" if NJ == 1 else f"b.{comp[j]}"
-                mfma += (f"              acc[{i}][{j}] = __builtin_amdgcn_mfma_f32_32x32x2f32("
-                         f"a[{i}].{comp[s]}, {bj}, acc[{i}][{j}], 0, 0, 0);\n")
+    decl_a, idx_a, PA, load_a, stash_a = loader("A", not ta, "M", BM, "M", "M", "m0", veca)
+    decl_b, idx_b, PB, load_b, stash_b = loader("B", tb, "N", BN, "N", "N", "n0", vecb)
+
+    # ---- the multiply: one group of 8 k per iteration, four MFMA steps
+    pre = ""
+    if not ta:
+        pre += (f"            float4 a[MI];\n            #pragma unroll\n            for (int i = 0; i < MI; ++i)\n"
+                f"                a[i] = *reinterpret_cast<const float4*>(&As[buf][wm0 + 32u * i + r][kb + 4u * h]);\n")
+    if tb:
+        pre += (f"            float4 b[NJ];\n            #pragma unroll\n            for (int j = 0; j < NJ; ++j)\n"
+                f"                b[j] = *reinterpret_cast<const float4*>(&Bs[buf][wn0 + 32u * j + r][kb + 4u * h]);\n")
+    mfma = pre
+    for st_ in range(4):
+        mfma += "            {\n"
+        if ta:
+            mfma += (f"              const {vtype[MI]} av = *reinterpret_cast<const {vtype[MI]}*>"
+                     f"(&As[buf][kb + 4u * h + {st_}u][wm0 + {MI}u * r]);\n")
+        if not tb:
+            mfma += (f"              const {vtype[NJ]} bv = *reinterpret_cast<const {vtype[NJ]}*>"
+                     f"(&Bs[buf][kb + 4u * h + {st_}u][wn0 + {NJ}u * r]);\n")
+        for i_ in range(MI):
+            ai = (("av" if MI == 1 else f"av.{comp[i_]}") if ta else f"a[{i_}].{comp[st_]}")
+            for j_ in range(NJ):
+                bj = (f"b[{j_}].{comp[st_]}" if tb else ("bv" if NJ == 1 else f"bv.{comp[j_]}"))
+                mfma += (f"              acc[{i_}][{j_}] = __builtin_amdgcn_mfma_f32_32x32x2f32("
+                         f"{ai}, {bj}, acc[{i_}][{j_}], 0, 0, 0);\n")
         mfma += "            }\n"
 
-    if vecb and NJ == 4:
-        store = """                    if (col + 3u < g.N) {
-                        *reinterpret_cast<float4*>(crow + col) =
-                            make_float4(acc[i][0][e], acc[i][1][e], acc[i][2][e], acc[i][3][e]);
-                    } else {
-                        #pragma unroll
-                        for (int j = 0; j < NJ; ++j) if (col + j < g.N) crow[col + j] = acc[i][j][e];
-                    }"""
+    # ---- epilogue: accumulator e of tile (i, j) belongs to operand-row index 8*(e/4) + 4*h + e%4
+    # of A's tile i and operand-row index lane%32 of B's tile j
+    row_expr = (f"m0 + wm0 + {MI}u * (8u * (e >> 2) + 4u * h + (e & 3)) + i" if ta
+                else "m0 + wm0 + 32u * i + 8u * (e >> 2) + 4u * h + (e & 3)")
+    if tb:
+        store = """                #pragma unroll
+                for (int j = 0; j < NJ; ++j) { const u32 col = n0 + wn0 + 32u * j + r; if (col < g.N) crow[col] = acc[i][j][e]; }"""
+    elif vecb and NJ == 4:
+        store = f"""                const u32 col = n0 + wn0 + {NJ}u * r;
+                if (col + 3u < g.N) {{
+                    *reinterpret_cast<float4*>(crow + col) =
+                        make_float4(acc[i][0][e], acc[i][1][e], acc[i][2][e], acc[i][3][e]);
+                }} else {{
+                    #pragma unroll
+                    for (int j = 0; j < NJ; ++j) if (col + j < g.N) crow[col + j] = acc[i][j][e];
+                }}"""
     else:
-        store = """                    #pragma unroll
-                    for (int j = 0; j < NJ; ++j) if (col + j < g.N) crow[col + j] = acc[i][j][e];"""
+        store = f"""                const u32 col = n0 + wn0 + {NJ}u * r;
+                #pragma unroll
+                for (int j = 0; j < NJ; ++j) if (col + j < g.N) crow[col + j] = acc[i][j][e];"""
 
     src = f"""{PRELUDE}
 typedef float f16v __attribute__((ext_vector_type(16)));
@@ -1260,8 +1328,8 @@ struct MMArgs {{ u32 M, N, K, nbc, sa0, sa1, sb0, sb1; }};
 #define NJ {NJ}
 extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict__ A,
         const float* __restrict__ B, float* __restrict__ C, MMArgs g) {{
-    __shared__ __attribute__((aligned(16))) float As[2][{BM}][{LDA}];
-    __shared__ __attribute__((aligned(16))) float Bs[2][{BK}][{LDB}];
+    {decl_a}
+    {decl_b}
 
     // ---- which C tile: XCD-contiguous renumbering, then groups of 8 tile rows
     const u32 tiles_m = (g.M + BM - 1u) / BM, tiles_n = (g.N + BN - 1u) / BN;
@@ -1282,8 +1350,8 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
     const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const u32 r = lane & 31u, h = lane >> 5;
     const u32 wm0 = (wave / {WN}u) * {32 * MI}u, wn0 = (wave % {WN}u) * {32 * NJ}u;
-    const u32 a_kq = tid % {AKQ}u, a_m = tid / {AKQ}u;
-    const u32 b_nq = tid % {BNQ}u, b_k = tid / {BNQ}u;
+    {idx_a}
+    {idx_b}
 
     f16v acc[MI][NJ];
     #pragma unroll
@@ -1295,25 +1363,9 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
 
     float4 ra[{PA}], rb[{PB}];
     auto load_tiles = [&](u32 k0) {{
-        #pragma unroll
-        for (u32 p = 0; p < {PA}u; ++p) {{
-            const u32 m = m0 + a_m + p * {ROWS_A}u, k = k0 + 4u * a_kq;
-{load_a}
-        }}
-        #pragma unroll
-        for (u32 p = 0; p < {PB}u; ++p) {{
-            const u32 k = k0 + b_k + p * {ROWS_B}u, n = n0 + 4u * b_nq;
-{load_b}
-        }}
-    }};
+{load_a}{load_b}    }};
     auto stash_tiles = [&](u32 buf) {{
-        #pragma unroll
-        for (u32 p = 0; p < {PA}u; ++p)
-            {f'if (a_m + p * {ROWS_A}u < BM)' if guard_a else ''} *reinterpret_cast<float4*>(&As[buf][a_m + p * {ROWS_A}u][4u * a_kq]) = ra[p];
-        #pragma unroll
-        for (u32 p = 0; p < {PB}u; ++p)
-            {f'if (b_k + p * {ROWS_B}u < BK)' if guard_b else ''} *reinterpret_cast<float4*>(&Bs[buf][b_k + p * {ROWS_B}u][4u * b_nq]) = rb[p];
-    }};
+{stash_a}{stash_b}    }};
 
     const u32 nk = (g.K + BK - 1u) / BK;
     load_tiles(0u);
@@ -1324,24 +1376,18 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
         if (kt + 1u < nk) load_tiles((kt + 1u) * BK);
         #pragma unroll
         for (u32 kb = 0; kb < BK; kb += 8u) {{
-            float4 a[MI];
-            #pragma unroll
-            for (int i = 0; i < MI; ++i)
-                a[i] = *reinterpret_cast<const float4*>(&As[buf][wm0 + 32u * i + r][kb + 4u * h]);
 {mfma}        }}
         if (kt + 1u < nk) stash_tiles(buf ^ 1u);
         __syncthreads();
     }}
 
-    // ---- epilogue: accumulator e of tile (i, j) is C[8*(e/4) + 4*h + e%4][lane%32]
     #pragma unroll
     for (int i = 0; i < MI; ++i)
         #pragma unroll
         for (int e = 0; e < 16; ++e) {{
-            const u32 row = m0 + wm0 + 32u * i + 8u * (e >> 2) + 4u * h + (e & 3);
+            const u32 row = {row_expr};
             if (row < g.M) {{
                 float* __restrict__ crow = C + (u64)row * g.N;
-                const u32 col = n0 + wn0 + {NJ}u * r;
 {store}
             }}
         }}

@@ -70,6 +70,8 @@ class CustomOps(Enum):
     CE_GRAD = auto()                # ((exp(lsm) - onehot) * upstream) / N, one kernel
     ADAM_STEP = auto()              # the 14 element-wise kernels of one Adam update, one kernel
     ADAM_STEP_INPLACE = auto()      # the same, in place, constants from device memory (graph replay)
+    MATMUL_NT = auto()              # x @ y^T with y read in place (no materialised transpose)
+    MATMUL_TN = auto()              # x^T @ y with x read in place
     FROM_U8 = auto()                # host uint8 array -> device fp32 buffer, cast on the device
     COPY_INTO = auto()              # device-to-device copy into an existing buffer (a KV-cache row)
     RMSNORM = auto()                # (x * rsqrt(mean(x^2) + eps)) * w over the last axis, one kernel

@@ -312,9 +312,32 @@ class MatMul(OP):
             upstream_grad = upstream_grad.reshape(self.out_shape)
         xr, yr = self.x.reshape(self.p1), self.y.reshape(self.p2)
         nd = xr.ndim
-        grad_x = upstream_grad @ yr.transpose(nd - 2, nd - 1)
-        grad_y = xr.transpose(nd - 2, nd - 1) @ upstream_grad
+        if FUSED and upstream_grad.device is Device.HIP:
+            # the same two products with the transposed operand read in place: same bits, two
+            # permute kernels and two temporaries fewer
+            grad_x = upstream_grad.matmul_nt(yr)
+            grad_y = xr.matmul_tn(upstream_grad)
+        else:
+            grad_x = upstream_grad @ yr.transpose(nd - 2, nd - 1)
+            grad_y = xr.transpose(nd - 2, nd - 1) @ upstream_grad
         return unbroadcast(grad_x, self.x.shape), unbroadcast(grad_y, self.y.shape)
+
+
+class LinearNT(OP):
+    """x @ W^T for W stored (out, in), the product inside Tensor.linear (tensor.py:549-563),
+    with W read in place.  The reference builds it as Transpose -> MatMul, i.e. one permute
+    forward and three backward (Y^T, X^T, and the transpose of dW^T back); here
+    dX = G @ W and dW = sum over the batch of G^T @ X need none.  Same products, same order
+    of additions: bit-identical to that composition."""
+
+    def forward(self, x: Buffer, w: Buffer) -> Buffer:
+        self.x, self.w = x, w
+        return x.matmul_nt(w)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        grad_x = upstream_grad @ self.w
+        grad_w = upstream_grad.matmul_tn(self.x)
+        return unbroadcast(grad_x, self.x.shape), unbroadcast(grad_w, self.w.shape)
 
 
 class Softmax(OP):

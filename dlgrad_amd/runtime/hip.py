@@ -421,6 +421,7 @@ def _map(tag: str, expr: str, operands: list[Buffer], out_shape: tuple, svals: t
 
 
 _U64 = (1 << 64) - 1
+_permute_plans: dict = {}
 
 
 class HIP:
@@ -765,22 +766,33 @@ class HIP:
         """Materialised permutation (cpu.py:333-368).  After merging dims that stay
         adjacent, either the innermost dim is still innermost (strided row copy) or
         another dim became innermost (LDS-tiled transpose of that pair of dims)."""
-        out_shape = tuple(x.shape[i] for i in order)
-        in_str = tuple(x.stride[i] for i in order)
         n = x.numel
         out = alloc(n)
         if n == 0:
             return out
-        cshape, (cout, cin) = collapse_dims(out_shape, calculate_stride(out_shape), in_str)
-        if n == 1 or cin[-1] == 1:
-            wide = (cshape[-1] % 4 == 0 and all(s % 4 == 0 for s in cin[:-1])
-                    and _addr(x) % 16 == 0 and out.addr % 16 == 0)
-            vec = 4 if wide else 1
-            shape4 = list(_pad4(cshape, 1))
-            shape4[3] //= vec
+        key = (x.shape, x.stride, tuple(order))
+        plan = _permute_plans.get(key)
+        if plan is None:
+            plan = _permute_plans[key] = HIP._permute_plan(x.shape, x.stride, order)
+        if plan[0] == "gather":
+            _, wide_ok, cshape, cin = plan
+            vec = 4 if (wide_ok and _addr(x) % 16 == 0 and out.addr % 16 == 0) else 1
             launch(kernel(K.permute_gather_kernel, vec), (n // vec + 1023) // 1024, 256,
-                   _addr(x), out.addr, n // vec, *shape4, *_pad4(cin, 0))
+                   _addr(x), out.addr, n // vec, *cshape[:3], cshape[3] // vec, *cin)
             return out
+        _, grid, args = plan
+        launch(kernel(K.permute_tiled_kernel), grid, 256, _addr(x), out.addr, *args)
+        return out
+
+    @staticmethod
+    def _permute_plan(shape: tuple, stride: tuple, order: tuple) -> tuple:
+        """Everything about a permutation that depends only on shape, strides and order."""
+        out_shape = tuple(shape[i] for i in order)
+        in_str = tuple(stride[i] for i in order)
+        cshape, (cout, cin) = collapse_dims(out_shape, calculate_stride(out_shape), in_str)
+        if prod_(shape) == 1 or cin[-1] == 1:
+            wide_ok = cshape[-1] % 4 == 0 and all(s % 4 == 0 for s in cin[:-1])
+            return "gather", wide_ok, _pad4(cshape, 1), _pad4(cin, 0)
         t = cin.index(1)
         others = [d for d in range(len(cshape) - 1) if d != t]
         ext = [cshape[d] for d in others]
@@ -790,9 +802,7 @@ class HIP:
             ext.insert(0, 1), i_st.insert(0, 0), o_st.insert(0, 0)
         nt, nb = cshape[t], cshape[-1]
         grid = ((nb + 31) // 32) * ((nt + 31) // 32) * ext[0] * ext[1]
-        launch(kernel(K.permute_tiled_kernel), grid, 256, _addr(x), out.addr,
-               ext[0], ext[1], nt, nb, i_st[0], i_st[1], cin[-1], o_st[0], o_st[1], cout[t])
-        return out
+        return "tiled", grid, (ext[0], ext[1], nt, nb, i_st[0], i_st[1], cin[-1], o_st[0], o_st[1], cout[t])
 
     # ---- embedding and cross-entropy helpers ----------------------------------------------------------------------
     @staticmethod
@@ -1044,13 +1054,15 @@ class HIP:
         return out
 
     @staticmethod
-    def _launch_matmul(tile: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple) -> None:
+    def _launch_matmul(tile: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple,
+                       ta: bool = False, tb: bool = False) -> None:
         bm, bn, threads = K.matmul_tile_shape(tile)
-        k = kernel(K.matmul_kernel, *K.MATMUL_CONFIGS[tile], veca, vecb)
+        k = kernel(K.matmul_kernel, *K.MATMUL_CONFIGS[tile], veca, vecb, ta, tb)
         launch(k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch), threads, *args)
 
     @staticmethod
-    def _tune_tile(key: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple) -> str:
+    def _tune_tile(key: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple,
+                   ta: bool, tb: bool) -> str:
         """Times every plausible tile on the real operands (the output is simply rewritten:
         all tiles produce the same bits) and stores the winner in the cache directory."""
         global launch_count
@@ -1059,14 +1071,14 @@ class HIP:
         best, best_ms = None, float("inf")
         e0, e1 = l.event_create(), l.event_create()
         for tile in HIP._tile_candidates(M, N, batch):
-            HIP._launch_matmul(tile, veca, vecb, M, N, batch, args)                  # loads the code object
+            HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb)          # loads the code object
             if COMPILE_ONLY:
                 continue
             ms, reps = 0.0, 3
             while True:
                 l.event_record(e0)
                 for _ in range(reps):
-                    HIP._launch_matmul(tile, veca, vecb, M, N, batch, args)
+                    HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb)
                 l.event_record(e1)
                 l.event_sync(e1)
                 ms = l.event_elapsed_ms(e0, e1) / reps
@@ -1098,27 +1110,30 @@ class HIP:
         return best
 
     @staticmethod
-    def _pick_tile(M: int, N: int, Kd: int, batch: int, veca: bool, vecb: bool, args: tuple) -> str:
+    def _pick_tile(M: int, N: int, Kd: int, batch: int, veca: bool, vecb: bool, args: tuple,
+                   ta: bool = False, tb: bool = False) -> str:
         if HIP.MATMUL_FORCE:
             return HIP.MATMUL_FORCE
-        key = f"{batch},{M},{N},{Kd}"
+        key = f"{batch},{M},{N},{Kd}" + (",tn" if ta else ",nt" if tb else "")
         tile = HIP._tuned_table().get(key)
         if tile is not None:
             return tile
         if HIP.MATMUL_TUNE and not capturing() and 2 * M * N * Kd * batch >= HIP.MATMUL_TUNE_MIN_FLOP:
-            return HIP._tune_tile(key, veca, vecb, M, N, batch, args)
+            return HIP._tune_tile(key, veca, vecb, M, N, batch, args, ta, tb)
         return HIP._model_tile(M, N, batch)
 
     @staticmethod
     @dispatcher.register(BinaryOps.MATMUL, Device.HIP)
-    def matmul(x: Buffer, y: Buffer) -> DevicePtr:
+    def matmul(x: Buffer, y: Buffer, ta: bool = False, tb: bool = False) -> DevicePtr:
         """x (.., M, K) @ y (.., K, N) for operands already padded to the same rank 2..4
         (buffer.py:231-243); batch dims of extent 1 broadcast through a zero stride as in
         cpu.py:519-532 and :553-559.  When y carries no batch at all the batch of x is
-        folded into M: one tall GEMM instead of many small ones."""
-        assert x.ndim == y.ndim and 2 <= x.ndim <= 4
-        M, Kd, N = x.shape[-2], x.shape[-1], y.shape[-1]
-        assert y.shape[-2] == Kd
+        folded into M: one tall GEMM instead of many small ones.
+        ta: x is stored as (.., K, M) and used transposed; tb: y is stored as (.., N, K)."""
+        assert x.ndim == y.ndim and 2 <= x.ndim <= 4 and not (ta and tb)
+        (Kd, M) = x.shape[-2:] if ta else x.shape[-2:][::-1]
+        (N, Ky) = y.shape[-2:] if tb else y.shape[-2:][::-1]
+        assert Ky == Kd, f"inner dims differ: {x.shape} {y.shape} ta={ta} tb={tb}"
         xb = (1,) * (4 - x.ndim) + tuple(x.shape[:-2])
         yb = (1,) * (4 - y.ndim) + tuple(y.shape[:-2])
         B0, B1 = max(xb[0], yb[0]), max(xb[1], yb[1])
@@ -1128,7 +1143,7 @@ class HIP:
         if Kd == 0:
             lib().fill_f32(out.addr, 0.0, B0 * B1 * M * N)
             return out
-        if yb == (1, 1):
+        if yb == (1, 1) and not ta:
             M, nbc, batch = xb[0] * xb[1] * M, 1, 1
             sa = sb = (0, 0)
         else:
@@ -1139,9 +1154,21 @@ class HIP:
             raise ValueError(f"{batch} batches exceed the grid limit")
         if max(M * Kd, Kd * N, M * N) >= 2 ** 31:
             raise ValueError("matrix too large for 32-bit indexing")
-        veca = Kd % 4 == 0 and _addr(x) % 16 == 0
-        vecb = N % 4 == 0 and _addr(y) % 16 == 0 and out.addr % 16 == 0
+        veca = (M if ta else Kd) % 4 == 0 and _addr(x) % 16 == 0
+        vecb = (Kd if tb else N) % 4 == 0 and _addr(y) % 16 == 0 and out.addr % 16 == 0
         args = (_addr(x), _addr(y), out.addr, M, N, Kd, nbc, *sa, *sb)
-        tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, args)
-        HIP._launch_matmul(tile, veca, vecb, M, N, batch, args)
+        tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, args, ta, tb)
+        HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb)
         return out
+
+    @staticmethod
+    @dispatcher.register(CustomOps.MATMUL_NT, Device.HIP)
+    def matmul_nt(x: Buffer, y: Buffer) -> DevicePtr:
+        """x (.., M, K) times the transpose of y (.., N, K), read in place."""
+        return HIP.matmul(x, y, tb=True)
+
+    @staticmethod
+    @dispatcher.register(CustomOps.MATMUL_TN, Device.HIP)
+    def matmul_tn(x: Buffer, y: Buffer) -> DevicePtr:
+        """The transpose of x (.., K, M), read in place, times y (.., K, N)."""
+        return HIP.matmul(x, y, ta=True)

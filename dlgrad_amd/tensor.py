@@ -241,7 +241,10 @@ class Tensor:
     def linear(self, weight: "Tensor", bias: "Tensor | None") -> "Tensor":
         """self @ weight.T + bias (tensor.py:549-563); weight is (out, in), so every call
         materialises the transpose, as there."""
-        out = self @ weight.T
+        if ops.FUSED and self.device is Device.HIP and weight.ndim == 2 and self.ndim >= 2:
+            out = ops.LinearNT.execute(self, weight)
+        else:
+            out = self @ weight.T
         return out + bias if bias is not None else out
 
     def softmax(self, dim: int = -1) -> "Tensor":

@@ -145,3 +145,46 @@ def test_first_use_of_a_large_shape_times_the_tiles_and_remembers_the_winner(mon
     assert json.load(open(tmp_path / "matmul_tuned.json"))[key] == HIP._tuned[key]
     small = (dev(f32(64, 64)) @ dev(f32(64, 64))).numpy()         # below the threshold: the model picks, nothing is stored
     assert small.shape == (64, 64) and len(HIP._tuned) == 1
+
+
+TRANSPOSED_CASES = [((64, 48), (40, 48)), ((130, 70), (50, 70)), ((200, 328), (196, 328)), ((97, 33), (45, 33)),
+                    ((3, 200, 72), (3, 196, 72)), ((4, 50, 36), (1, 44, 36)), ((16, 128, 128), (128, 128)),
+                    ((2, 3, 64, 32), (2, 3, 80, 32)), ((2, 3, 64, 32), (2, 1, 80, 32)), ((2048, 128), (512, 128))]
+
+
+@pytest.mark.parametrize("xs,ys", TRANSPOSED_CASES)
+def test_nt_product_reads_the_transposed_operand_in_place(xs, ys):
+    """x @ y^T with y stored (.., N, K): the same bits as permute + matmul, and 1e-4 of float64."""
+    require_gpu()
+    x, y = f32(*xs), f32(*ys, scale=xs[-1] ** -0.5)
+    xd, yd = dev(x), dev(y)
+    got = xd.matmul_nt(yd).numpy()
+    nd = yd.ndim
+    check(got, xd.matmul(yd.transpose(nd - 2, nd - 1)).numpy(), 0, f"NT {xs} {ys} vs permute + NN")
+    check_mm(got, x.astype(np.float64) @ np.swapaxes(y.astype(np.float64), -1, -2), f"NT {xs} {ys}")
+
+
+@pytest.mark.parametrize("xs,ys", TRANSPOSED_CASES)
+def test_tn_product_reads_the_transposed_operand_in_place(xs, ys):
+    """x^T @ y with x stored (.., K, M); shapes are the NT cases with both operands swapped around."""
+    require_gpu()
+    xs, ys = xs[:-2] + (xs[-1], xs[-2]), ys[:-2] + (ys[-1], ys[-2])          # (.., K, M), (.., K, N)
+    x, y = f32(*xs), f32(*ys, scale=xs[-2] ** -0.5)
+    xd, yd = dev(x), dev(y)
+    got = xd.matmul_tn(yd).numpy()
+    nd = xd.ndim
+    check(got, xd.transpose(nd - 2, nd - 1).matmul(yd).numpy(), 0, f"TN {xs} {ys} vs permute + NN")
+    check_mm(got, np.swapaxes(x.astype(np.float64), -1, -2) @ y.astype(np.float64), f"TN {xs} {ys}")
+
+
+@pytest.mark.parametrize("tile", list(__import__("dlgrad_amd.codegen.hip_kernel", fromlist=["x"]).MATMUL_CONFIGS))
+def test_every_tile_configuration_transposed(tile, monkeypatch):
+    require_gpu()
+    from dlgrad_amd.runtime.hip import HIP
+    x, y, z = f32(2, 260, 72), f32(2, 388, 72, scale=72 ** -0.5), f32(2, 260, 100)
+    xd, yd, zd = dev(x), dev(y), dev(z)
+    monkeypatch.setattr(HIP, "MATMUL_FORCE", "64x64")
+    want_nt, want_tn = xd.matmul(yd.transpose(1, 2)).numpy(), xd.transpose(1, 2).matmul(zd).numpy()
+    monkeypatch.setattr(HIP, "MATMUL_FORCE", tile)
+    check(xd.matmul_nt(yd).numpy(), want_nt, 0, f"NT {tile}")
+    check(xd.matmul_tn(zd).numpy(), want_tn, 0, f"TN {tile}")
