@@ -518,7 +518,7 @@ def main() -> None:
                                       "exp relu log sqrt; sum/max x axis0,axis1,all)"},
                "roofline": {"bound": "hbm", "achieved": add["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                             "frac": add["GBps"] / HBM_PEAK_GBS, "traffic": C2_ADD_TRAFFIC_BYTES,
-                            "kernel": "map_add_vec_vec_v4u4" + ("nt" if R * C >= hip.NT_STORE_MIN_ELEMENTS else ""),
+                            "kernel": "map_add_vec_vec_v4u1nt" if R * C >= hip.NT_STORE_MIN_ELEMENTS else "map_add_vec_vec_v4u4",
                             "bytes_per_launch": 12 * R * C,
                             "avg_launch_ms": add["ms"]},
                "per_op": {k: {"GBps": round(v["GBps"], 1), "frac_hbm": round(v["frac_hbm"], 3),

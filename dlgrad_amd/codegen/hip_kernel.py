@@ -43,6 +43,11 @@ typedef unsigned long long u64;
 typedef float v4f __attribute__((ext_vector_type(4)));
 #define WAVE 64
 #define NEG_FLT_MAX (-3.402823466e+38f)
+// 16-byte load that does not displace cached data (inputs streamed once)
+static __device__ __forceinline__ float4 ld4_stream(const float4* p) {
+    const v4f t = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(p));
+    return make_float4(t.x, t.y, t.z, t.w);
+}
 
 // ---- wavefront-64 reductions: DPP inside each row of 16 lanes, then two
 // cross-row exchanges.  After the call every lane holds the result.
@@ -139,6 +144,10 @@ def map_kernel(tag: str, expr: str, modes: tuple[str, ...], vec: int, n_sval_ext
     vec=4 uses 16-byte accesses (dwordx4): the launcher guarantees 16-byte aligned
     pointers and, for row/col operands, C % 4 == 0.  The n % 4 tail is done by the
     first threads of block 0 with scalar accesses.
+    nt_store: the streaming form for tensors far larger than the caches -- same-shape operands
+    are read with nontemporal loads and the output is written with nontemporal stores, so
+    neither evicts what the next kernel is about to read (broadcast operands, which are
+    reused, keep ordinary loads).
     """
     assert vec in (1, 4) and all(m in MODES for m in modes)
     name = f"map_{tag}_{'_'.join(modes) if modes else 'gen'}_v{vec}u{unroll}{'nt' if nt_store else ''}"
@@ -173,7 +182,9 @@ def map_kernel(tag: str, expr: str, modes: tuple[str, ...], vec: int, n_sval_ext
         loads = ""
         for k in range(nx):
             if modes[k] == "vec":
-                loads += f"            r{k}[u] = reinterpret_cast<const float4*>(a{k})[v];\n"
+                loads += (f"            {{ const v4f t = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(a{k}) + v); "
+                          f"r{k}[u] = make_float4(t.x, t.y, t.z, t.w); }}\n" if nt_store else
+                          f"            r{k}[u] = reinterpret_cast<const float4*>(a{k})[v];\n")
             elif modes[k] == "col":
                 loads += f"            r{k}[u] = reinterpret_cast<const float4*>(a{k})[((v << 2) % C) >> 2];\n"
             elif modes[k] == "row":
@@ -317,6 +328,12 @@ static __device__ __forceinline__ float block_reduce(float v, float* sm) {
 """
 
 
+def _ld4_define(nt: bool) -> str:
+    """LD4(p): how a reduction reads 16 bytes -- streaming (nontemporal) for inputs far larger
+    than the caches, ordinary otherwise."""
+    return "\n#define LD4(p) ld4_stream(p)\n" if nt else "\n#define LD4(p) (*(p))\n"
+
+
 def _red_defs(op: str) -> str:
     ident, comb, wred = _RED[op]
     return (f"#define IDENT {ident}\n#define COMB(a, b) {comb.format(a='(a)', b='(b)')}\n"
@@ -324,7 +341,7 @@ def _red_defs(op: str) -> str:
 
 
 @cache
-def reduce_full_kernel(op: str, vec: int) -> tuple[str, str, str]:
+def reduce_full_kernel(op: str, vec: int, nt: bool = False) -> tuple[str, str, str]:
     """Stage kernel of the full reduction (cpu_kernel.py:150-177): block b folds the
     contiguous slice [b*chunk, (b+1)*chunk) of x (in units of `vec` floats) into one
     value, out[b] = value / divisor.  Contiguous slices (32 KiB per block, walked 16 KiB
@@ -332,23 +349,23 @@ def reduce_full_kernel(op: str, vec: int) -> tuple[str, str, str]:
     pages; a grid-strided walk of the same data measured ~10 % slower.  The launcher runs
     it once over x and once more, with one block, over the partials; `divisor` is 1
     except in the last stage of a mean."""
-    name = f"reduce_full_{op}_v{vec}"
+    name = f"reduce_full_{op}_v{vec}{'nt' if nt else ''}"
     if vec == 4:
-        loop = r"""
+        loop = _ld4_define(nt) + r"""
     const u32 nv = n >> 2;
     const float4* __restrict__ x4 = reinterpret_cast<const float4*>(x);
     float a0 = IDENT, a1 = IDENT, a2 = IDENT, a3 = IDENT;
     const u32 end = min(nv, (blockIdx.x + 1u) * chunk);
     u32 v = blockIdx.x * chunk + threadIdx.x;
     for (; v + 768u < end; v += 1024u) {
-        const float4 p = x4[v], q = x4[v + 256u], r = x4[v + 512u], s = x4[v + 768u];
+        const float4 p = LD4(x4 + v), q = LD4(x4 + v + 256u), r = LD4(x4 + v + 512u), s = LD4(x4 + v + 768u);
         a0 = COMB(a0, COMB(COMB(p.x, p.y), COMB(p.z, p.w)));
         a1 = COMB(a1, COMB(COMB(q.x, q.y), COMB(q.z, q.w)));
         a2 = COMB(a2, COMB(COMB(r.x, r.y), COMB(r.z, r.w)));
         a3 = COMB(a3, COMB(COMB(s.x, s.y), COMB(s.z, s.w)));
     }
     for (; v < end; v += 256u) {
-        const float4 p = x4[v];
+        const float4 p = LD4(x4 + v);
         a0 = COMB(a0, COMB(COMB(p.x, p.y), COMB(p.z, p.w)));
     }
     float acc = COMB(COMB(a0, a1), COMB(a2, a3));
@@ -376,11 +393,11 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 
 
 @cache
-def reduce_rows_kernel(op: str, vec: int, per_block: bool) -> tuple[str, str, str]:
+def reduce_rows_kernel(op: str, vec: int, per_block: bool, nt: bool = False) -> tuple[str, str, str]:
     """out[r] = reduce over the contiguous row r of an (R, L) view, / divisor
     (the last-axis case of cpu_kernel.py:68-148).  Either one wavefront per row
     (four rows per 256-thread block) or, for long rows, one block per row."""
-    name = f"reduce_rows_{op}_v{vec}_{'blk' if per_block else 'wav'}"
+    name = f"reduce_rows_{op}_v{vec}_{'blk' if per_block else 'wav'}{'nt' if nt else ''}"
     T = "256u" if per_block else "64u"
     tid = "threadIdx.x" if per_block else "(threadIdx.x & 63u)"
     row = "blockIdx.x" if per_block else "(blockIdx.x * 4u + (threadIdx.x >> 6))"
@@ -391,13 +408,14 @@ def reduce_rows_kernel(op: str, vec: int, per_block: bool) -> tuple[str, str, st
     float a0 = IDENT, a1 = IDENT;
     u32 v = {tid};
     for (; v + {T} < nv; v += 2u * {T}) {{
-        const float4 s = p[v], t = p[v + {T}];
+        const float4 s = LD4(p + v), t = LD4(p + v + {T});
         a0 = COMB(a0, COMB(COMB(s.x, s.y), COMB(s.z, s.w)));
         a1 = COMB(a1, COMB(COMB(t.x, t.y), COMB(t.z, t.w)));
     }}
-    if (v < nv) {{ const float4 s = p[v]; a0 = COMB(a0, COMB(COMB(s.x, s.y), COMB(s.z, s.w))); }}
+    if (v < nv) {{ const float4 s = LD4(p + v); a0 = COMB(a0, COMB(COMB(s.x, s.y), COMB(s.z, s.w))); }}
     float acc = COMB(a0, a1);
 """
+        loop = _ld4_define(nt) + loop
     else:
         loop = f"""
     const float* __restrict__ p = x + (u64)row * L;
@@ -425,7 +443,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 
 
 @cache
-def reduce_cols_kernel(op: str, vec: int, ty: int = 4) -> tuple[str, str, str]:
+def reduce_cols_kernel(op: str, vec: int, ty: int = 4, nt: bool = False) -> tuple[str, str, str]:
     """out[o, c, i] = reduce over l in chunk c of x[o, l, i] for an (O, L, I) view, / divisor
     (the non-last-axis case of cpu_kernel.py:68-148, e.g. axis 0 of a matrix).
 
@@ -434,10 +452,10 @@ def reduce_cols_kernel(op: str, vec: int, ty: int = 4) -> tuple[str, str, str]:
     the ty thread rows take every ty-th row of the chunk, and LDS joins them.  L is
     split into `chunks` so that tall, narrow inputs still fill the chip; the launcher
     reduces the (O, chunks, I) partials with a second call."""
-    name = f"reduce_cols_{op}_v{vec}_y{ty}"
+    name = f"reduce_cols_{op}_v{vec}_y{ty}{'nt' if nt else ''}"
     if vec == 4:
-        defs = """#define VT float4
-#define LD(l) (reinterpret_cast<const float4*>(xp + (u64)(l) * I)[0])
+        defs = _ld4_define(nt) + """#define VT float4
+#define LD(l) LD4(reinterpret_cast<const float4*>(xp + (u64)(l) * I))
 #define ACC(a, t) { a.x = COMB(a.x, t.x); a.y = COMB(a.y, t.y); a.z = COMB(a.z, t.z); a.w = COMB(a.w, t.w); }
 #define VINIT make_float4(IDENT, IDENT, IDENT, IDENT)
 #define STORE(p, r) { r.x /= divisor; r.y /= divisor; r.z /= divisor; r.w /= divisor; reinterpret_cast<float4*>(p)[0] = r; }
@@ -798,7 +816,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 
 @cache
 def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gather: bool = False,
-                        threads: int = 256) -> tuple[str, str, str]:
+                        threads: int = 256, nt: bool = False) -> tuple[str, str, str]:
     """Row softmax / log-softmax over the contiguous last axis of an (R, L) view, replacing
     the reference's five kernels and four temporaries (tensor.py:634-669).  Same formula:
     e = exp(x - max); e / sum(e)   (or (x - max) - log(sum)).
@@ -812,8 +830,9 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     ce_forward gather of cpu_kernel.py:430-441, fused."""
     if not per_block:
         threads = 256
+    nt = nt and bool(nval) and vec == 4                   # streaming loads/stores: register-resident float4 form only
     name = (f"{'log_' if log else ''}softmax_rows_v{vec}_{f'blk{threads}' if per_block else 'wav'}"
-            f"{f'_r{nval}' if nval else ''}{'_g' if gather else ''}")
+            f"{f'_r{nval}' if nval else ''}{'_g' if gather else ''}{'nt' if nt else ''}")
     T = f"{threads}u" if per_block else "64u"
     NW = threads // 64
     tid = "threadIdx.x" if per_block else "(threadIdx.x & 63u)"
@@ -831,7 +850,7 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     const u32 nv = L >> 2;
     float4 v[{nval}];
     #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < nv) v[k] = p[c]; }}
+    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < nv) v[k] = {'ld4_stream(p + c)' if nt else 'p[c]'}; }}
     float m = NEG_FLT_MAX;
     #pragma unroll
     for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < nv)
@@ -848,7 +867,7 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
         const u32 c = {tid} + k * {T};
         if (c < nv) {{
             float4 o;
-{''.join(f"            o.{c} = {outexpr(f'v[k].{c}')};{chr(10)}" for c in comps)}            q[c] = o;
+{''.join(f"            o.{c} = {outexpr(f'v[k].{c}')};{chr(10)}" for c in comps)}            {'{ const v4f ov = {o.x, o.y, o.z, o.w}; __builtin_nontemporal_store(ov, reinterpret_cast<v4f*>(q) + c); }' if nt else 'q[c] = o;'}
         }}
     }}
 """

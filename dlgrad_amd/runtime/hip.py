@@ -369,8 +369,10 @@ class _MapPlan:
             # (generator params, grid, trailing args); the kernel itself is loaded on first use
             if C % 4 == 0 or not any(m in ("row", "col") for m in modes):
                 # outputs too large to be re-read from cache are written with nontemporal stores
+                # (streaming form: one float4 per thread, which measures 5-8 % above four)
                 nt = n >= NT_STORE_MIN_ELEMENTS
-                self.wide = [(K.map_kernel, tag, expr, tuple(modes), 4, n_svals, 4, nt), K.map_grid(n, 4), (n, C), None,
+                unroll = 1 if nt else 4
+                self.wide = [(K.map_kernel, tag, expr, tuple(modes), 4, n_svals, unroll, nt), K.map_grid(n, 4, unroll), (n, C), None,
                              tuple(m in ("vec", "col") for m in modes)]
             self.narrow = [(K.map_kernel, tag, expr, tuple(modes), 1, n_svals), K.map_grid(n, 1), (n, C), None, None]
         else:
@@ -649,6 +651,10 @@ class HIP:
     @dispatcher.register(UnaryOps.WHERE, Device.HIP)
     def where(cond: Buffer, x: Buffer, y: Buffer) -> DevicePtr:
         out_shape = broadcast_shapes_2(broadcast_shapes_2(x.shape, y.shape), cond.shape)
+        if (cond.ptr.__class__ is DevicePtr and x.ptr.__class__ is DevicePtr and cond.ptr.addr == x.ptr.addr
+                and cond.shape == x.shape):
+            # relu / leaky_relu call where(t, t, other): read t once
+            return _map("where_self", "(x0 > 0.0f) ? x0 : x1", [x, y], out_shape)
         return _map("where", "(x0 > 0.0f) ? x1 : x2", [cond, x, y], out_shape)
 
     @staticmethod
@@ -668,7 +674,8 @@ class HIP:
             launch(kernel(K.reduce_full_kernel, kop, vec), 1, 256, x_addr, out_addr, n, float(divisor), items)
             return
         part = alloc(G)
-        launch(kernel(K.reduce_full_kernel, kop, vec), G, 256, x_addr, part.addr, n, 1.0, 2048)
+        nt = vec == 4 and n >= NT_STORE_MIN_ELEMENTS                # streamed once: keep it out of the caches
+        launch(kernel(K.reduce_full_kernel, kop, vec, nt), G, 256, x_addr, part.addr, n, 1.0, 2048)
         if G > 65536:                                    # > 537 M elements: fold the partials recursively
             HIP._reduce_full_into(kop, part.addr, G, divisor, out_addr)
             return
@@ -683,7 +690,8 @@ class HIP:
         vec = 4 if (I % 4 == 0 and x_addr % 16 == 0 and out_addr % 16 == 0) else 1
         bx = (I + 64 * vec - 1) // (64 * vec)
         ty = 16 if L > 64 else 4
-        k = kernel(K.reduce_cols_kernel, kop, vec, ty)
+        nt = vec == 4 and O * L * I >= NT_STORE_MIN_ELEMENTS
+        k = kernel(K.reduce_cols_kernel, kop, vec, ty, nt)
         chunks = 1 if L <= 512 else max(1, min(8192 // max(1, bx * O), L // 64))
         if chunks == 1:
             launch(k, (bx, 1, O), (64, ty, 1), x_addr, out_addr, L, I, L, float(divisor))
@@ -720,7 +728,8 @@ class HIP:
                 return out
             vec = 4 if (L % 4 == 0 and _addr(x) % 16 == 0) else 1
             blk = L >= 2048
-            launch(kernel(K.reduce_rows_kernel, kop, vec, blk), O if blk else (O + 3) // 4, 256,
+            nt = vec == 4 and O * L >= NT_STORE_MIN_ELEMENTS
+            launch(kernel(K.reduce_rows_kernel, kop, vec, blk, nt), O if blk else (O + 3) // 4, 256,
                    _addr(x), out.addr, O, L, divisor)
         else:
             if O > 65535:
@@ -865,7 +874,8 @@ class HIP:
             return out if target is None else (out, picked)
         vec = 4 if (L % 4 == 0 and _addr(x) % 16 == 0 and out.addr % 16 == 0) else 1
         blk, nval, threads = K.softmax_plan(L, vec)
-        k = kernel(K.softmax_rows_kernel, log, vec, blk, nval, target is not None, threads)
+        k = kernel(K.softmax_rows_kernel, log, vec, blk, nval, target is not None, threads,
+                   x.numel >= NT_STORE_MIN_ELEMENTS)
         grid = R if blk else (R + 3) // 4
         if target is None:
             launch(k, grid, threads, _addr(x), out.addr, R, L)
