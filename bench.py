@@ -199,15 +199,19 @@ def run_matmul(M: int, N: int, K: int, steps: int, warmup: int, seed: int = 3) -
 
 
 def run_matmul_transposed(n: int) -> dict:
-    """The backward shapes A^T.G and G.B^T: as in the reference they are a materialised
-    transpose (permute kernel) followed by a plain GEMM; both launches are timed together."""
+    """The backward shapes A^T.G and G.B^T, two ways: as the reference issues them (a
+    materialised transpose -- a permute kernel -- followed by a plain GEMM, both launches
+    timed together) and with the transposed operand read in place by the TN / NT kernels."""
     _, _, Buffer, Device, hip = _imports()
     lib = hip.lib()
     rng = np.random.default_rng(4)
     a = Buffer.from_numpy(rng.standard_normal((n, n), dtype=np.float32) * np.float32(n ** -0.5), Device.HIP)
     g = Buffer.from_numpy(rng.standard_normal((n, n), dtype=np.float32) * np.float32(n ** -0.5), Device.HIP)
     out = {}
-    for name, f in ((f"{n}_TN_At.G", lambda: a.T @ g), (f"{n}_NT_G.Bt", lambda: g @ a.T)):
+    for name, f, key in ((f"{n}_TN_At.G", lambda: a.T @ g, "ms_permute_plus_gemm"),
+                         (f"{n}_NT_G.Bt", lambda: g @ a.T, "ms_permute_plus_gemm"),
+                         (f"{n}_TN_At.G_in_place", lambda: a.matmul_tn(g), "kernel_ms"),
+                         (f"{n}_NT_G.Bt_in_place", lambda: g.matmul_nt(a), "kernel_ms")):
         for _ in range(2):
             f()
         timer = EventTimer(lib)
@@ -215,7 +219,7 @@ def run_matmul_transposed(n: int) -> dict:
             timer.run("mm", f)
         lib.sync()
         ms = float(np.mean(timer.collect()["mm"]))
-        out[name] = {"TFLOPs": round(2.0 * n ** 3 / ms / 1e9, 2), "ms_permute_plus_gemm": round(ms, 4)}
+        out[name] = {"TFLOPs": round(2.0 * n ** 3 / ms / 1e9, 2), key: round(ms, 4)}
     return out
 
 
@@ -403,11 +407,12 @@ def run_gpt_large(steps: int = 2) -> dict:
         times.append(time.perf_counter() - t0)
     n_params = sum(p.numel for p in params)
     in_use, cached, _ = lib.pool_stats()
+    step_s = sum(times[1:]) / steps                               # the first step (kernel loading, tile timing) is warm-up
     return {"params_M": round(n_params / 1e6, 1), "inference_ms": round(t_inf * 1e3, 2),
             "inference_tokens_per_s": round(tokens / t_inf, 1),
-            "train_step_ms": round(min(times[1:]) * 1e3, 2), "train_tokens_per_s": round(tokens / min(times[1:]), 1),
+            "train_step_ms": round(step_s * 1e3, 2), "train_tokens_per_s": round(tokens / step_s, 1),
             "train_TFLOPs_est": round(6 * (n_params - c.vocab_size * c.n_embd - c.block_size * c.n_embd) * tokens
-                                      / min(times[1:]) / 1e12, 2),
+                                      / step_s / 1e12, 2),
             "loss_per_token": round(float(loss.numpy()) / tokens, 4),
             "pool_GiB": round((in_use + cached) / 2 ** 30, 1)}
 
@@ -475,6 +480,12 @@ def run_mlp(steps: int, warmup: int) -> dict:
     wall = time.perf_counter() - t0
     return {"ms_per_step": wall / steps * 1e3, "samples_per_s": 128 * steps / wall,
             "launches_per_step": (hip.launch_count - n0) / steps}
+
+
+def step_roofline(flops: float, ms: float, note: str) -> dict:
+    achieved = flops / (ms * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": achieved, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": achieved / MFMA_FP32_PEAK_TFLOPS, "traffic": None, "note": note}
 
 
 # ---------------------------------------------------------------------------------------------
@@ -569,7 +580,9 @@ def main() -> None:
                "config": {"workload": "C4 char-GPT vocab 65, block 128, 6 layers, 4 heads, n_embd 128, batch 16; "
                                       "forward + backward + Adam step (RMSNorm, ReLU MLP, no bias, as examples/gpt.py)",
                           "launches_per_step": g["launches_per_step"], "loss_per_token": g["loss_per_token"]},
-               "roofline": None}
+               "roofline": step_roofline(6 * 1_187_968 * 2048, g["ms_per_step"],
+                                         "whole eager step against the fp32 MFMA peak; 6 x 1.19 M matmul parameters x 2048 "
+                                         "tokens; the step is bound by Python-issued launches, not by the GPU")}
         if not args.no_cpu:
             out["cpu_baseline"] = cpu_gpt()
     elif args.workload == "gpt-large":
@@ -578,7 +591,9 @@ def main() -> None:
                **base, "ms_per_step": g["train_step_ms"],
                "config": {"workload": "C5 scaled GPT vocab 50304, block 1024, 12 layers, 12 heads, n_embd 768, batch 8; "
                                       "Zipf(1.1) token ids; forward + backward + Adam step", **g},
-               "roofline": None}
+               "roofline": step_roofline(g["train_TFLOPs_est"] * 1e12 * g["train_step_ms"] * 1e-3, g["train_step_ms"],
+                                         "whole step against the fp32 MFMA peak; 6 x 124 M matmul parameters x 8192 tokens "
+                                         "(attention products not counted)")}
     else:
         r = run_mlp(args.steps, args.warmup)
         out = {"metric": "MLP 784-64-10 step samples/s (1 GPU)", "value": r["samples_per_s"], "unit": "samples/s",

@@ -1435,7 +1435,8 @@ MATMUL_CONFIGS = {
     "128x96": (4, 1, 1, 3, 32),
     "128x64": (4, 1, 1, 2, 32),
     "64x64": (2, 2, 1, 1, 16),
-    "32x32": (1, 1, 1, 1, 16),
+    "64x64k64": (2, 2, 1, 1, 64),       # same tile, K walked 64 at a time: fewer barriers when one block per CU
+    "32x32": (1, 1, 1, 1, 16),          # has nobody to overlap with (1024^3: 73 against 62 TFLOP/s)
 }
 
 

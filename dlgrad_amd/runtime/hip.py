@@ -1031,7 +1031,7 @@ class HIP:
         return HIP._tuned
 
     @staticmethod
-    def _model_tile(M: int, N: int, batch: int) -> str:
+    def _model_tile(M: int, N: int, batch: int, Kd: int = 0) -> str:
         """Largest expected throughput = tile rate x fraction of the tile grid that is real
         output x how evenly the blocks load 256 CUs: the busiest CU runs ceil(blocks / 256) of
         them, and a CU that holds one block of a tile meant to be co-resident is given 85 %."""
@@ -1047,6 +1047,8 @@ class HIP:
             score = rate * (M * N) / float(tm * bm * tn * bn) * fill
             if score > best_score * 1.0001:
                 best, best_score = name, score
+        if best == "64x64" and Kd >= 512 and -(-M // 64) * -(-N // 64) * batch <= 512:
+            best = "64x64k64"                       # few blocks, long K: the deep-K form of the same tile
         return best
 
     @staticmethod
@@ -1058,7 +1060,7 @@ class HIP:
             bm, bn, _ = K.matmul_tile_shape(name)
             if bm > max(32, 2 * M) or bn > max(32, 2 * N):
                 continue
-            if M * N * batch > (1 << 22 if name == "32x32" else 1 << 27 if name == "64x64" else 1 << 62):
+            if M * N * batch > (1 << 22 if name == "32x32" else 1 << 27 if name.startswith("64x64") else 1 << 62):
                 continue
             out.append(name)
         return out
@@ -1130,7 +1132,7 @@ class HIP:
             return tile
         if HIP.MATMUL_TUNE and not capturing() and 2 * M * N * Kd * batch >= HIP.MATMUL_TUNE_MIN_FLOP:
             return HIP._tune_tile(key, veca, vecb, M, N, batch, args, ta, tb)
-        return HIP._model_tile(M, N, batch)
+        return HIP._model_tile(M, N, batch, Kd)
 
     @staticmethod
     @dispatcher.register(BinaryOps.MATMUL, Device.HIP)
