@@ -279,6 +279,48 @@ def run_c5(steps: int, warmup: int) -> dict:
             for name, _, b in work}
 
 
+def run_layout_and_select(steps: int, warmup: int) -> dict:
+    """The kernel classes the C2 suite does not touch, at sizes beyond the caches: transposes
+    and head permutes (8 B/elt), argmax (4 B/elt + 4 B/output), comparisons, clamp, pow,
+    masked_fill with the causal mask broadcast over (8, 12, 1024, 1024) (8 B/elt), where with
+    three tensor operands (16 B/elt)."""
+    _, _, Buffer, Device, hip = _imports()
+    lib = hip.lib()
+    rng = np.random.default_rng(6)
+    sq = Buffer.from_numpy(rng.standard_normal((8192, 8192), dtype=np.float32), Device.HIP)
+    heads = Buffer.from_numpy(rng.standard_normal((64, 1024, 12, 64), dtype=np.float32), Device.HIP)
+    att = Buffer.from_numpy(rng.standard_normal((8, 12, 1024, 1024), dtype=np.float32), Device.HIP)
+    mask = Buffer.from_numpy(np.triu(np.ones((1024, 1024), np.float32), 1), Device.HIP)
+    logits = Buffer.from_numpy(rng.standard_normal((8192, 50304), dtype=np.float32), Device.HIP)
+    tall = Buffer.from_numpy(rng.standard_normal((1000000, 10), dtype=np.float32), Device.HIP)
+    n2, nh, na = sq.numel, heads.numel, att.numel
+    cond, other = Buffer(logits.ptr, sq.shape, Device.HIP), Buffer(logits.ptr + n2, sq.shape, Device.HIP)   # views into logits
+    work = [("transpose_8192x8192", lambda: sq.transpose(0, 1), 8 * n2),
+            ("permute_heads_(64,1024,12,64)->(64,12,1024,64)", lambda: heads.permute((0, 2, 1, 3)), 8 * nh),
+            ("transpose_last_two_(64,12,1024,64)", lambda: heads.reshape((64, 12, 1024, 64)).permute((0, 1, 3, 2)), 8 * nh),
+            ("argmax_rows_8192x50304", lambda: logits.argmax(1), 4 * logits.numel + 4 * 8192),
+            ("argmax_rows_1000000x10", lambda: tall.argmax(1), 4 * tall.numel + 4 * 1000000),
+            ("argmax_cols_8192x8192", lambda: sq.argmax(0), 4 * n2 + 4 * 8192),
+            ("gt_scalar_(8,12,1024,1024)", lambda: att > 0.0, 8 * na),
+            ("clamp_(8,12,1024,1024)", lambda: att.clamp(-0.5, 0.5), 8 * na),
+            ("pow3_(8,12,1024,1024)", lambda: att ** 3, 8 * na),
+            ("masked_fill_causal_(8,12,1024,1024)", lambda: Buffer.masked_fill(att, mask, float("-inf")), 8 * na + 4 * mask.numel),
+            ("where_3_tensors_8192x8192", lambda: cond.where(sq, other), 16 * n2)]
+    timer = EventTimer(lib)
+    for _ in range(warmup):
+        for _, f, _ in work:
+            f()
+    for _ in range(steps):
+        for name, f, _ in work:
+            timer.run(name, f)
+    lib.sync()
+    per = timer.collect()
+    return {name: {"ms": round(float(np.mean(per[name])), 4),
+                   "GBps": round(b / float(np.mean(per[name])) / 1e6, 1),
+                   "frac_hbm": round(b / float(np.mean(per[name])) / 1e6 / HBM_PEAK_GBS, 3)}
+            for name, _, b in work}
+
+
 # ---------------------------------------------------------------------------------------------
 # GPT / MLP steps
 # ---------------------------------------------------------------------------------------------
@@ -560,6 +602,7 @@ def main() -> None:
             extra["gpt_char_greedy_decode_256"] = run_decode(256)
             extra["mlp_784_64_10_step"] = {k: round(v, 3) for k, v in run_mlp(50, 5).items()}
             extra["c5_components"] = run_c5(max(3, min(args.steps, 10)), 2)
+            extra["layout_and_select"] = run_layout_and_select(max(3, min(args.steps, 10)), 2)
             extra["gpt_scaled_c5"] = run_gpt_large(2)
             out["extra"] = extra
     elif args.workload == "matmul":

@@ -95,6 +95,9 @@ class Buffer:
         if device.__class__ is not Device:
             device = as_device(device)
         n = prod_(shape)
+        room = getattr(data, "nbytes", None)               # device pointers know how much of their block is left
+        if room is not None and n * 4 > room:
+            raise ValueError(f"a Buffer of shape {shape} needs {n * 4} bytes, the pointer has {room}")
         if kwargs:
             stride, ndim = kwargs.get("stride", calculate_stride(shape)), kwargs.get("ndim", len(shape))
         else:

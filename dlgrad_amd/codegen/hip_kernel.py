@@ -498,46 +498,154 @@ extern "C" __global__ __launch_bounds__({64 * ty}) void {name}(const float* __re
     return src, name, _fmt("P", "P", "I", "I", "I", "f")
 
 
+_ARGMAX_PAIR = r"""
+// (value, index) pairs: the larger value wins, equal values keep the lower index, which is
+// the index the reference's sequential `if (v > best)` scan ends with.  A scan starts from
+// (-FLT_MAX, 0), so a row that never exceeds -FLT_MAX (all -inf, or NaN) answers 0, as there.
+#define TAKE(bv, bi, ov, oi) if ((ov) > (bv) || ((ov) == (bv) && (oi) < (bi))) { bv = (ov); bi = (oi); }
+static __device__ __forceinline__ void wave_argmax(float& best, u32& bi) {
+    #pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off, WAVE);
+        const u32 oi = __shfl_xor(bi, off, WAVE);
+        TAKE(best, bi, ov, oi)
+    }
+}
+"""
+
+
 @cache
-def argmax_kernel(rows: bool) -> tuple[str, str, str]:
+def argmax_kernel(mode: str, vec: int = 1) -> tuple[str, str, str]:
     """Index (as float) of the first maximum along L of an (O, L, I) view
     (cpu_kernel.py:459-517: strict '>', start value -FLT_MAX at index 0).
-    rows=True handles I == 1 with one wavefront per row; otherwise one thread per
-    output column walks L.  Ties resolve to the lowest index in both."""
-    if rows:
-        name = "argmax_rows"
+      rows_thread  I == 1, short rows (the (N, 10) class scores): one thread per row
+      rows_wave    I == 1: one wavefront per row
+      rows_block   I == 1, long rows (50304-wide logits): one block per row
+      cols_part    I > 1: a 64 x 16 block owns 64 columns of one chunk of L; thread rows take
+                   every 16th row, LDS joins them; writes the chunk's (value, index) per column,
+                   or, when there is one chunk, the answer
+      cols_fin     folds the chunks of cols_part in order
+    vec = 4: 16-byte loads along the row (rows_wave / rows_block)."""
+    name = f"argmax_{mode}" + (f"_v{vec}" if mode in ("rows_wave", "rows_block") else "")
+    if mode == "rows_thread":
         src = f"""{PRELUDE}
 extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
         float* __restrict__ out, u32 R, u32 L) {{
-    const u32 row = blockIdx.x * 4u + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    const u32 row = blockIdx.x * 256u + threadIdx.x;
     if (row >= R) return;
     const float* __restrict__ p = x + (u64)row * L;
     float best = NEG_FLT_MAX; u32 bi = 0;
-    for (u32 i = lane; i < L; i += 64u) {{ const float v = p[i]; if (v > best) {{ best = v; bi = i; }} }}
-    #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {{
-        const float ov = __shfl_xor(best, off, WAVE);
-        const u32 oi = __shfl_xor(bi, off, WAVE);
-        if (ov > best || (ov == best && oi < bi)) {{ best = ov; bi = oi; }}
-    }}
-    if (lane == 0) out[row] = (float)bi;
+    for (u32 i = 0; i < L; ++i) {{ const float v = p[i]; if (v > best) {{ best = v; bi = i; }} }}
+    out[row] = (float)bi;
 }}
 """
         return src, name, _fmt("P", "P", "I", "I")
-    name = "argmax_cols"
-    src = f"""{PRELUDE}
+    if mode in ("rows_wave", "rows_block"):
+        blk = mode == "rows_block"
+        T = "256u" if blk else "64u"
+        tid = "threadIdx.x" if blk else "(threadIdx.x & 63u)"
+        row = "blockIdx.x" if blk else "(blockIdx.x * 4u + (threadIdx.x >> 6))"
+        if vec == 4:
+            scan = f"""
+    const float4* __restrict__ p4 = reinterpret_cast<const float4*>(p);
+    for (u32 v = {tid}; v < (L >> 2); v += {T}) {{
+        const float4 t = p4[v]; const u32 i = v << 2;
+        if (t.x > best) {{ best = t.x; bi = i; }}
+        if (t.y > best) {{ best = t.y; bi = i + 1u; }}
+        if (t.z > best) {{ best = t.z; bi = i + 2u; }}
+        if (t.w > best) {{ best = t.w; bi = i + 3u; }}
+    }}
+    if ({tid} < (L & 3u)) {{ const u32 i = (L & ~3u) + {tid}; const float v = p[i]; TAKE(best, bi, v, i) }}
+"""
+        else:
+            scan = f"""
+    for (u32 i = {tid}; i < L; i += {T}) {{ const float v = p[i]; if (v > best) {{ best = v; bi = i; }} }}
+"""
+        if blk:
+            fin = """    wave_argmax(best, bi);
+    __shared__ float sv[4]; __shared__ u32 si[4];
+    if ((threadIdx.x & 63u) == 0) { sv[threadIdx.x >> 6] = best; si[threadIdx.x >> 6] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        #pragma unroll
+        for (int w = 1; w < 4; ++w) TAKE(best, bi, sv[w], si[w])
+        out[row] = (float)bi;
+    }"""
+        else:
+            fin = """    wave_argmax(best, bi);
+    if ((threadIdx.x & 63u) == 0) out[row] = (float)bi;"""
+        src = f"""{PRELUDE}{_ARGMAX_PAIR}
 extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
-        float* __restrict__ out, u32 O, u32 L, u32 I) {{
+        float* __restrict__ out, u32 R, u32 L) {{
+    const u32 row = {row};
+    {'' if blk else 'if (row >= R) return;'}
+    const float* __restrict__ p = x + (u64)row * L;
+    float best = NEG_FLT_MAX; u32 bi = 0;
+{scan}
+{fin}
+}}
+"""
+        return src, name, _fmt("P", "P", "I", "I")
+    if mode == "cols_part":
+        name += f"_v{vec}"
+        if vec == 4:
+            scan = """
+        for (u32 l = l0 + ty; l < l1; l += 16u) {
+            const float4 v = *reinterpret_cast<const float4*>(xp + (u64)l * I);
+            if (v.x > best[0]) { best[0] = v.x; bi[0] = l; }
+            if (v.y > best[1]) { best[1] = v.y; bi[1] = l; }
+            if (v.z > best[2]) { best[2] = v.z; bi[2] = l; }
+            if (v.w > best[3]) { best[3] = v.w; bi[3] = l; }
+        }"""
+        else:
+            scan = """
+        for (u32 l = l0 + ty; l < l1; l += 16u) { const float v = xp[(u64)l * I]; if (v > best[0]) { best[0] = v; bi[0] = l; } }"""
+        src = f"""{PRELUDE}{_ARGMAX_PAIR}
+#define VEC {vec}
+extern "C" __global__ __launch_bounds__(1024) void {name}(const float* __restrict__ x,
+        float* __restrict__ out, float* __restrict__ pv, u32* __restrict__ pi, u32 L, u32 I, u32 chunk, u32 final) {{
+    __shared__ float sv[16][64 * VEC + 1]; __shared__ u32 si[16][64 * VEC + 1];
+    const u32 tx = threadIdx.x, ty = threadIdx.y, o = blockIdx.z;
+    const u32 col = (blockIdx.x * 64u + tx) * VEC;
+    const u32 l0 = blockIdx.y * chunk, l1 = min(L, l0 + chunk);
+    float best[VEC]; u32 bi[VEC];
+    #pragma unroll
+    for (int c = 0; c < VEC; ++c) {{ best[c] = NEG_FLT_MAX; bi[c] = 0; }}
+    if (col < I) {{
+        const float* __restrict__ xp = x + (u64)o * L * I + col;{scan}
+    }}
+    #pragma unroll
+    for (int c = 0; c < VEC; ++c) {{ sv[ty][tx * VEC + c] = best[c]; si[ty][tx * VEC + c] = bi[c]; }}
+    __syncthreads();
+    if (ty == 0 && col < I) {{
+        #pragma unroll
+        for (int c = 0; c < VEC; ++c) {{
+            #pragma unroll
+            for (int k = 1; k < 16; ++k) TAKE(best[c], bi[c], sv[k][tx * VEC + c], si[k][tx * VEC + c])
+            if (final) out[(u64)o * I + col + c] = (float)bi[c];
+            else {{ const u64 at = ((u64)o * gridDim.y + blockIdx.y) * I + col + c; pv[at] = best[c]; pi[at] = bi[c]; }}
+        }}
+    }}
+}}
+"""
+        return src, name, _fmt("P", "P", "P", "P", "I", "I", "I", "I")
+    assert mode == "cols_fin"
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ pv,
+        const u32* __restrict__ pi, float* __restrict__ out, u32 O, u32 chunks, u32 I) {{
     const u32 t = blockIdx.x * 256u + threadIdx.x;
     if (t >= O * I) return;
     const u32 o = t / I, i = t % I;
-    const float* __restrict__ p = x + (u64)o * L * I + i;
     float best = NEG_FLT_MAX; u32 bi = 0;
-    for (u32 l = 0; l < L; ++l) {{ const float v = p[(u64)l * I]; if (v > best) {{ best = v; bi = l; }} }}
+    for (u32 c = 0; c < chunks; ++c) {{
+        const u64 at = ((u64)o * chunks + c) * I + i;
+        const float v = pv[at];
+        if (v > best) {{ best = v; bi = pi[at]; }}
+    }}
     out[t] = (float)bi;
 }}
 """
-    return src, name, _fmt("P", "P", "I", "I", "I")
+    return src, name, _fmt("P", "P", "P", "I", "I", "I")
 
 
 # =====================================================================================
@@ -582,19 +690,57 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 
 
 @cache
-def permute_tiled_kernel() -> tuple[str, str, str]:
+def permute_tiled_kernel(vec: int = 1) -> tuple[str, str, str]:
     """Permutations that move another dim into the innermost position, e.g. (.., a, b) ->
     (.., b, a) or (B,T,h,d) -> (B,h,d,T).  Out dims are (p, q, t, b) after padding where
-    b is the out-innermost dim and t is the out dim whose *input* stride is 1.  A 32x32
-    tile of the (t, b) plane goes through LDS (33-float rows, no bank conflicts) so that
+    b is the out-innermost dim and t is the out dim whose *input* stride is 1.  A tile of
+    the (t, b) plane goes through LDS (rows padded by one float, no bank conflicts) so that
     reads run along t and writes along b, both coalesced; p and q only offset the tile.
+    vec = 1: 32 x 32 tile, 4-byte accesses.  vec = 4: 64 x 64 tile, 16-byte loads along t and
+    16-byte stores along b (256-byte row segments); needs extents and strides that are
+    multiples of 4 and 16-byte aligned bases.
     The reference reads with the large stride directly (cpu_kernel.py:207-212)."""
-    name = "permute_tiled"
-    src = f"""{PRELUDE}
+    name = "permute_tiled" + ("_v4" if vec == 4 else "")
+    head = f"""{PRELUDE}
 struct PArgs {{ u32 np, nq, nt, nb;        // extents: two carried dims, tile dims t and b
                u32 ip, iq, ib;            // input strides of p, q, b (t has input stride 1)
                u32 op, oq, ot; }};        // output strides of p, q, t (b has output stride 1)
-extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+"""
+    if vec == 4:
+        src = head + f"""extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        float* __restrict__ out, PArgs a) {{
+    __shared__ float tile[64][65];          // [b][t]
+    const u32 tb = (a.nb + 63u) >> 6, tt = (a.nt + 63u) >> 6;
+    u32 r = blockIdx.x;
+    const u32 bb = r % tb; r /= tb;
+    const u32 bt = r % tt; r /= tt;
+    const u32 q = r % a.nq, p = r / a.nq;
+    const float* __restrict__ xi = x + (u64)p * a.ip + (u64)q * a.iq;
+    float* __restrict__ oo = out + (u64)p * a.op + (u64)q * a.oq;
+    const u32 c4 = threadIdx.x & 15u, r16 = threadIdx.x >> 4;
+    #pragma unroll
+    for (u32 k = 0; k < 64u; k += 16u) {{
+        const u32 t = bt * 64u + 4u * c4, b = bb * 64u + r16 + k;
+        if (t < a.nt && b < a.nb) {{
+            const float4 v = *reinterpret_cast<const float4*>(xi + (u64)b * a.ib + t);
+            float* __restrict__ d = &tile[r16 + k][4u * c4];
+            d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+        }}
+    }}
+    __syncthreads();
+    #pragma unroll
+    for (u32 k = 0; k < 64u; k += 16u) {{
+        const u32 t = bt * 64u + r16 + k, b = bb * 64u + 4u * c4;
+        if (t < a.nt && b < a.nb) {{
+            const u32 lt = r16 + k, lb = 4u * c4;
+            *reinterpret_cast<float4*>(oo + (u64)t * a.ot + b) =
+                make_float4(tile[lb][lt], tile[lb + 1u][lt], tile[lb + 2u][lt], tile[lb + 3u][lt]);
+        }}
+    }}
+}}
+"""
+        return src, name, _fmt("P", "P", "10I")
+    src = head + f"""extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
         float* __restrict__ out, PArgs a) {{
     __shared__ float tile[32][33];
     const u32 tb = (a.nb + 31u) >> 5, tt = (a.nt + 31u) >> 5;

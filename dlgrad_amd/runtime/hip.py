@@ -762,10 +762,34 @@ class HIP:
                 dim += x.ndim
             O, L, I = prod_(x.shape[:dim]), x.shape[dim], prod_(x.shape[dim + 1:])
         out = alloc(O * I)
+        if O * I == 0:
+            return out
+        if L >= 2 ** 31 or O * L * I >= 2 ** 32:
+            raise ValueError("tensor too large for 32-bit indexing")
         if I == 1:
-            launch(kernel(K.argmax_kernel, True), (O + 3) // 4, 256, _addr(x), out.addr, O, L)
-        else:
-            launch(kernel(K.argmax_kernel, False), (O * I + 255) // 256, 256, _addr(x), out.addr, O, L, I)
+            vec = 4 if (L % 4 == 0 and _addr(x) % 16 == 0) else 1
+            if L <= 32:
+                launch(kernel(K.argmax_kernel, "rows_thread"), (O + 255) // 256, 256, _addr(x), out.addr, O, L)
+            elif L < 2048:
+                launch(kernel(K.argmax_kernel, "rows_wave", vec), (O + 3) // 4, 256, _addr(x), out.addr, O, L)
+            else:
+                launch(kernel(K.argmax_kernel, "rows_block", vec), O, 256, _addr(x), out.addr, O, L)
+            return out
+        if O > 65535:
+            raise ValueError("outer extent too large for the column argmax grid")
+        vec = 4 if (I % 4 == 0 and _addr(x) % 16 == 0) else 1
+        bx = (I + 64 * vec - 1) // (64 * vec)
+        # about a thousand blocks fill the chip; more chunks only lengthen the fold over them
+        chunks = 1 if L <= 256 else max(1, min(1024 // max(1, bx * O), L // 64, 65535))
+        chunk = (L + chunks - 1) // chunks
+        chunks = (L + chunk - 1) // chunk
+        k = kernel(K.argmax_kernel, "cols_part", vec)
+        if chunks == 1:
+            launch(k, (bx, 1, O), (64, 16, 1), _addr(x), out.addr, 0, 0, L, I, L, 1)
+            return out
+        pv, pi = alloc(O * chunks * I), alloc(O * chunks * I)
+        launch(k, (bx, chunks, O), (64, 16, 1), _addr(x), out.addr, pv.addr, pi.addr, L, I, chunk, 0)
+        launch(kernel(K.argmax_kernel, "cols_fin"), (O * I + 255) // 256, 256, pv.addr, pi.addr, out.addr, O, chunks, I)
         return out
 
     # ---- permute ---------------------------------------------------------------------------------------------
@@ -789,8 +813,11 @@ class HIP:
             launch(kernel(K.permute_gather_kernel, vec), (n // vec + 1023) // 1024, 256,
                    _addr(x), out.addr, n // vec, *cshape[:3], cshape[3] // vec, *cin)
             return out
-        _, grid, args = plan
-        launch(kernel(K.permute_tiled_kernel), grid, 256, _addr(x), out.addr, *args)
+        _, grid, args, grid4 = plan
+        if grid4 and _addr(x) % 16 == 0 and out.addr % 16 == 0:
+            launch(kernel(K.permute_tiled_kernel, 4), grid4, 256, _addr(x), out.addr, *args)
+        else:
+            launch(kernel(K.permute_tiled_kernel, 1), grid, 256, _addr(x), out.addr, *args)
         return out
 
     @staticmethod
@@ -811,7 +838,11 @@ class HIP:
             ext.insert(0, 1), i_st.insert(0, 0), o_st.insert(0, 0)
         nt, nb = cshape[t], cshape[-1]
         grid = ((nb + 31) // 32) * ((nt + 31) // 32) * ext[0] * ext[1]
-        return "tiled", grid, (ext[0], ext[1], nt, nb, i_st[0], i_st[1], cin[-1], o_st[0], o_st[1], cout[t])
+        args = (ext[0], ext[1], nt, nb, i_st[0], i_st[1], cin[-1], o_st[0], o_st[1], cout[t])
+        # 64 x 64 tiles with 16-byte accesses when every extent and stride is a multiple of 4
+        wide = all(v % 4 == 0 for v in (nt, nb, i_st[0], i_st[1], cin[-1], o_st[0], o_st[1], cout[t]))
+        grid4 = ((nb + 63) // 64) * ((nt + 63) // 64) * ext[0] * ext[1] if wide else 0
+        return "tiled", grid, args, grid4
 
     # ---- embedding and cross-entropy helpers ----------------------------------------------------------------------
     @staticmethod

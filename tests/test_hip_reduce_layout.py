@@ -79,7 +79,8 @@ def test_max_of_minus_inf_rows_matches_reference_start_value():
     check(dev(x[:2]).max().numpy(), cref.reduce("max", x[:2]), 0, "max all -inf")
 
 
-@pytest.mark.parametrize("shape", [(128, 10), (10000, 10), (1, 65), (1, 50304), (7, 1000), (300, 257)])
+@pytest.mark.parametrize("shape", [(128, 10), (10000, 10), (1, 65), (1, 50304), (7, 1000), (300, 257), (5, 50304), (3, 5003),
+                                   (5000, 300), (70000, 33), (9, 2048), (257, 32)])
 def test_argmax_bit_exact_with_ties(shape):
     require_gpu()
     x = RNG.integers(0, 5, shape).astype(np.float32)         # few distinct values: many ties
@@ -90,7 +91,23 @@ def test_argmax_bit_exact_with_ties(shape):
     check(dev(y).argmax(1).numpy(), y.argmax(1).astype(np.float32).reshape(-1, 1), 0, "argmax random")
 
 
-PERMS = [((4, 7), (1, 0)), ((64, 784), (1, 0)), ((10, 64), (1, 0)), ((128, 128), (1, 0)), ((512, 128), (1, 0)),
+def test_argmax_never_selects_minus_inf():
+    """The scan starts at (-FLT_MAX, index 0) and moves on `v > best` only (cpu_kernel.py:497-499):
+    rows of -inf answer 0; every kernel variant must agree.  (NaN is left out: the reference
+    compiles that comparison under -ffinite-math-only, which leaves its outcome to the compiler.)"""
+    require_gpu()
+    for shape in ((6, 10), (6, 300), (6, 4096), (600, 70)):
+        x = np.full(shape, -np.inf, np.float32)
+        x[1, shape[1] - 1] = -1e30
+        x[2, 5] = 7.0
+        x[4, 2] = x[4, shape[1] - 2] = 9.0
+        for d in (0, 1):
+            want = cref.argmax(x, d).reshape((1, shape[1]) if d == 0 else (shape[0], 1))
+            check(dev(x).argmax(d).numpy(), want, 0, f"argmax {shape} dim {d} with -inf")
+
+
+PERMS = [((256, 512), (1, 0)), ((8, 12, 64, 128), (0, 1, 3, 2)), ((4, 128, 8, 64), (0, 2, 3, 1)), ((132, 260), (1, 0)),
+         ((2048, 768), (1, 0)), ((4, 7), (1, 0)), ((64, 784), (1, 0)), ((10, 64), (1, 0)), ((128, 128), (1, 0)), ((512, 128), (1, 0)),
          ((2, 3, 4), (0, 2, 1)), ((2, 3, 4), (2, 0, 1)), ((2, 3, 4), (1, 0, 2)), ((2, 3, 4, 5), (0, 2, 1, 3)),
          ((2, 3, 4, 5), (0, 1, 3, 2)), ((2, 3, 4, 5), (3, 2, 1, 0)), ((2, 3, 4, 5), (1, 3, 0, 2)),
          ((16, 128, 4, 32), (0, 2, 1, 3)), ((16, 4, 128, 32), (0, 1, 3, 2)), ((16, 4, 128, 32), (0, 2, 1, 3)),
@@ -102,6 +119,14 @@ def test_permute_bit_exact(shape, order):
     require_gpu()
     x = f32(*shape)
     check(dev(x).permute(order).numpy(), cref.permute(x, order), 0, f"permute {shape} {order}")
+
+
+def test_transpose_at_bench_size_is_exact_and_its_own_inverse():
+    require_gpu()
+    x = f32(8192, 4096)
+    t = dev(x).transpose(0, 1)
+    check(t.numpy(), x.T, 0, "8192 x 4096 transpose")
+    check(t.transpose(0, 1).numpy(), x, 0, "transposed twice")
 
 
 def test_transpose_helpers():
