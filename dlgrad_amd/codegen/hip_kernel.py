@@ -653,13 +653,18 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 # =====================================================================================
 
 @cache
-def permute_gather_kernel(vec: int) -> tuple[str, str, str]:
+def permute_gather_kernel(vec: int, nt: bool = False) -> tuple[str, str, str]:
     """out (contiguous, <=4-D, padded on the left) <- x read through permuted strides
     (cpu_kernel.py:179-215), for permutations that keep the innermost dim innermost:
     both sides are then contiguous along that dim and each thread moves `vec` floats.
     vec=4 needs the inner extent, every input stride and both bases to be multiples of 4."""
-    name = f"permute_gather_v{vec}"
-    if vec == 4:
+    nt = nt and vec == 4                                  # streaming form for tensors far larger than the caches
+    name = f"permute_gather_v{vec}{'nt' if nt else ''}"
+    if nt:
+        move = ("{ const v4f t = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(x + off)); "
+                "__builtin_nontemporal_store(t, reinterpret_cast<v4f*>(out) + i); }")
+        scale = "const u32 c3 = (r % shape.d[3]) << 2; r /= shape.d[3];"
+    elif vec == 4:
         move = ("reinterpret_cast<float4*>(out)[i] = "
                 "reinterpret_cast<const float4*>(x + off)[0];")
         scale = "const u32 c3 = (r % shape.d[3]) << 2; r /= shape.d[3];"   # shape.d[3] is in float4 units

@@ -810,7 +810,7 @@ class HIP:
         if plan[0] == "gather":
             _, wide_ok, cshape, cin = plan
             vec = 4 if (wide_ok and _addr(x) % 16 == 0 and out.addr % 16 == 0) else 1
-            launch(kernel(K.permute_gather_kernel, vec), (n // vec + 1023) // 1024, 256,
+            launch(kernel(K.permute_gather_kernel, vec, n >= NT_STORE_MIN_ELEMENTS), (n // vec + 1023) // 1024, 256,
                    _addr(x), out.addr, n // vec, *cshape[:3], cshape[3] // vec, *cin)
             return out
         _, grid, args, grid4 = plan
