@@ -384,6 +384,10 @@ class Buffer:
         """In-place Adam update of self, m and v with the constants held in device memory."""
         self._dispatch(CustomOps.ADAM_STEP_INPLACE, p=self, g=g, m=m, v=v, consts=consts)
 
+    def sgd_step_(self, g: "Buffer", v: "Buffer | None", lr: float, momentum: float) -> None:
+        """In-place SGD update of self (and of the velocity v when momentum is used)."""
+        self._dispatch(CustomOps.SGD_STEP_INPLACE, p=self, g=g, v=v, lr=lr, momentum=momentum)
+
     def upload_(self, arr: np.ndarray) -> None:
         """Overwrites this Buffer's memory with `arr` (same element count); the address stays."""
         if arr.size != self.numel:

@@ -1610,6 +1610,28 @@ MATMUL_TILE_MODEL = {
 # =====================================================================================
 
 @cache
+def sgd_inplace_kernel(momentum: bool) -> tuple[str, str, str]:
+    """p -= (momentum ? (v = v * mu + g) : g) * lr, in place (dlgrad/nn/optim.py:22-45): the
+    form a captured graph can replay, since no buffer changes its address.  fp contraction is
+    off, so the two or four roundings are those of the op-by-op expression."""
+    name = f"sgd_step_inplace{'_mom' if momentum else ''}"
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(float* p, const float* __restrict__ g, float* v,
+        u32 n, float lr, float mu) {{
+    #pragma clang fp contract(off)
+    const u32 j = blockIdx.x * 256u + threadIdx.x;
+    if (j < n) {{
+        float upd = g[j];
+        {'{ const float t = v[j] * mu; upd = t + upd; v[j] = upd; }' if momentum else '(void)v; (void)mu;'}
+        const float t2 = upd * lr;
+        p[j] = p[j] - t2;
+    }}
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "I", "f", "f")
+
+
+@cache
 def adam_inplace_kernel(vec: int) -> tuple[str, str, str]:
     """adam_kernel's arithmetic applied in place to p, m and v, with the eight constants read
     from device memory.  This is the form a captured graph can replay: the addresses never

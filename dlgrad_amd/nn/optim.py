@@ -23,9 +23,13 @@ class Optimizer:
 
 
 class SGD(Optimizer):
-    def __init__(self, params: list[Tensor], lr: float = 1e-3, momentum: float = 0.0) -> None:
+    def __init__(self, params: list[Tensor], lr: float = 1e-3, momentum: float = 0.0,
+                 graph_safe: bool = False) -> None:
+        """graph_safe (hip only): parameters and velocities are updated in place, so a captured
+        step can be replayed.  Same arithmetic, same bits."""
         super().__init__(params, lr)
         self.momentum = momentum
+        self.graph_safe = graph_safe
         self.velocities = {id(p): Tensor.zeros_like(p) for p in params} if momentum else {}
 
     def step(self) -> None:
@@ -33,6 +37,10 @@ class SGD(Optimizer):
             if p.grad is None:
                 continue
             assert p.shape == p.grad.shape, f"The shape of the parameter {p.shape} and its grad {p.grad.shape} do not match"
+            if self.graph_safe:
+                v = self.velocities[id(p)].data if self.momentum != 0 else None
+                p.data.sgd_step_(p.grad.data, v, self.lr, self.momentum)
+                continue
             upd = p.grad
             if self.momentum != 0:
                 upd = self.velocities[id(p)] * self.momentum + p.grad          # v = mu * v + g

@@ -94,6 +94,12 @@ class _CompileOnlyLib:
     def pool_stats(self) -> tuple:
         return (0, 0, 0)
 
+    def arena_create(self) -> int:
+        return 1
+
+    def graph_end(self) -> tuple:
+        return (1, 0)
+
     def __getattr__(self, name: str):           # free, h2d, launch, sync, fill_f32, events ...
         return lambda *a, **k: None
 
@@ -1030,6 +1036,17 @@ class HIP:
         vec = 4 if not any(a & 15 for a in addrs) else 1
         launch(kernel(K.adam_inplace_kernel, vec), max(1, ((n + vec - 1) // vec + 255) // 256), 256,
                *addrs, n, _addr(consts))
+
+    @staticmethod
+    @dispatcher.register(CustomOps.SGD_STEP_INPLACE, Device.HIP)
+    def sgd_step_inplace(p: Buffer, g: Buffer, v: Buffer | None, lr: float, momentum: float) -> None:
+        n = p.numel
+        if n == 0:
+            return
+        if g.numel != n or (v is not None and v.numel != n):
+            raise ValueError(f"sgd_step_: parameter {p.shape}, gradient {g.shape}")
+        launch(kernel(K.sgd_inplace_kernel, v is not None), (n + 255) // 256, 256,
+               _addr(p), _addr(g), _addr(v) if v is not None else 0, n, float(lr), float(momentum))
 
     # ---- matmul ----------------------------------------------------------------------------------------------------------
     MATMUL_FORCE = os.environ.get("DLGRAD_HIP_MATMUL_TILE")      # e.g. "128x128": benchmarking aid

@@ -347,3 +347,53 @@ def test_captured_graph_replays_match_eager_steps_bit_for_bit():
         for name, p in nn.utils.get_state_dict(model).items():
             np.testing.assert_array_equal(p.numpy(), eager[k][1][name], err_msg=f"{name} after replay {k}")
     g.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("momentum", [0.0, 0.9])
+def test_captured_mlp_step_with_in_place_sgd_matches_eager_steps_bit_for_bit(momentum):
+    """The 784-64-10 MLP step (test/test_forward_backward.py's shape) as a replayed graph with a new
+    batch uploaded into the same buffers before every replay, against eager steps with the
+    reference's out-of-place SGD expression: same losses and parameters, bit for bit."""
+    if not hip.available():
+        pytest.skip("no HIP device (graph capture needs one)")
+    batches = [M.synthetic_batch(s) for s in range(5)]
+
+    def build(graph_safe):
+        model = M.MLP(device="hip")
+        M.init_weights_(model, 0)
+        params = [model.fc1.weight, model.fc1.bias, model.fc2.weight, model.fc2.bias]
+        opt = nn.optim.SGD(params, lr=1e-2, momentum=momentum, graph_safe=graph_safe)
+        xt, yt = Tensor(batches[0][0], device="hip"), Tensor(batches[0][1], device="hip")
+
+        def step():
+            opt.zero_grad()
+            loss = model(xt).cross_entropy_loss(yt)
+            loss.backward()
+            opt.step()
+            return loss
+        return params, xt, yt, step
+
+    params, xt, yt, step = build(False)
+    eager = []
+    for x, y in batches:
+        xt.data.upload_(x)
+        yt.data.upload_(y)
+        loss = step()
+        eager.append((float(loss.numpy()), [p.numpy() for p in params]))
+
+    params, xt, yt, step = build(True)
+    g = hip.Graph()
+    with g.arena():
+        loss = step()                                    # batch 0, eager inside the arena
+    assert float(loss.numpy()) == eager[0][0]
+    with g.capture():
+        loss = step()
+    for k in range(1, len(batches)):
+        xt.data.upload_(batches[k][0])                   # same addresses, new contents
+        yt.data.upload_(batches[k][1])
+        g.replay()
+        assert float(loss.numpy()) == eager[k][0], f"loss after replay {k}"
+        for p, want in zip(params, eager[k][1]):
+            np.testing.assert_array_equal(p.numpy(), want, err_msg=f"replay {k}")
+    g.close()
