@@ -222,12 +222,12 @@ int dlg_hip_alloc(size_t nbytes, void **out) {
 int dlg_hip_alloc_zero(size_t nbytes, void **out) {
     NEED_INIT();
     if (!out) return fail_msg(-1, "out is NULL");
+    if (g_capturing) return fail_msg(-9, "dlg_hip_alloc_zero records a memset node; clear with a kernel while capturing");
     {
         std::lock_guard<std::mutex> lk(g_mu);
         int rc = alloc_locked(nbytes, out);
         if (rc) return rc;
     }
-    if (g_capturing) return fail_msg(-9, "dlg_hip_alloc_zero records a memset node; clear with a kernel while capturing");
     if (nbytes) HIP_TRY(hipMemsetAsync(*out, 0, nbytes, g_stream));
     return 0;
 }
@@ -375,21 +375,30 @@ int dlg_hip_launch(uint64_t handle, uint32_t gx, uint32_t gy, uint32_t gz, uint3
                    uint32_t by, uint32_t bz, uint32_t shared_bytes, const void *args,
                    size_t args_size) {
     NEED_INIT();
-    if (handle == 0 || handle > g_kernels.size()) return fail_msg(-20, "bad kernel handle");
+    hipFunction_t fn;
+    {                                             // module_load on another thread may grow the table
+        std::lock_guard<std::mutex> lk(g_mu);
+        if (handle == 0 || handle > g_kernels.size()) return fail_msg(-20, "bad kernel handle");
+        fn = g_kernels[handle - 1].fn;
+    }
     if (!gx || !gy || !gz || !bx || !by || !bz) return fail_msg(-21, "empty grid or block");
     if ((uint64_t)bx * by * bz > 1024) return fail_msg(-22, "block larger than 1024 threads");
+    if (!args && args_size) return fail_msg(-23, "argument block is NULL");
     void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void *>(args),
                       HIP_LAUNCH_PARAM_BUFFER_SIZE, &args_size, HIP_LAUNCH_PARAM_END};
-    HIP_TRY(hipModuleLaunchKernel(g_kernels[handle - 1].fn, gx, gy, gz, bx, by, bz, shared_bytes,
-                                  g_stream, nullptr, config));
+    HIP_TRY(hipModuleLaunchKernel(fn, gx, gy, gz, bx, by, bz, shared_bytes, g_stream, nullptr, config));
     return 0;
 }
 
 int dlg_hip_kernel_attrs(uint64_t handle, int32_t *num_regs, int32_t *lds_bytes,
                          int32_t *scratch_bytes, int32_t *max_threads) {
     NEED_INIT();
-    if (handle == 0 || handle > g_kernels.size()) return fail_msg(-20, "bad kernel handle");
-    hipFunction_t fn = g_kernels[handle - 1].fn;
+    hipFunction_t fn;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        if (handle == 0 || handle > g_kernels.size()) return fail_msg(-20, "bad kernel handle");
+        fn = g_kernels[handle - 1].fn;
+    }
     int v = 0;
     if (num_regs) { HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_NUM_REGS, fn)); *num_regs = v; }
     if (lds_bytes) { HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES, fn)); *lds_bytes = v; }

@@ -17,6 +17,14 @@
  * calls back into the host language.  All work is issued on one internal,
  * default-priority stream; calls are asynchronous with respect to the host
  * unless stated otherwise.
+ *
+ * Threads: the allocator, the kernel table and the graph table are guarded by a
+ * mutex, so allocation, free, module load and launch may come from any thread.
+ * The stream is shared: work is ordered as issued, and the "current arena" and
+ * "capture in progress" states are per process, so a capture (graph_begin ..
+ * graph_end) and everything issued during it must come from one thread while
+ * no other thread issues work.  The reference is single-threaded throughout
+ * (dlgrad/runtime/cpu.py holds no lock).
  */
 #ifndef DLGRAD_HIP_H
 #define DLGRAD_HIP_H

@@ -145,3 +145,69 @@ def test_pow_expression_is_repeated_multiplication():
         return eval(K.pow_expr(n).replace("1.0f", "1.0").replace("powf", "pow"), {"x0": x0})
     for n in (0, 1, 2, 3, 5, 8, -1, -2):
         assert abs(ev(n) - x0 ** n) < 1e-12
+
+
+# ---- failure handling on a device: every condition is forced from the host, every kernel exits normally
+@pytest.mark.gpu
+def test_failures_surface_as_python_exceptions_and_leave_the_device_usable():
+    """The error contract of dlgrad/runtime/cpu.py:104,132,189 (MemoryError on a failed
+    allocation) and :61-62 (RuntimeError on a failed compile), plus the host-side checks that
+    stop a bad launch before it reaches the GPU."""
+    from dlgrad_amd.runtime import hip
+    if not hip.available():
+        pytest.skip("no HIP device")
+    import numpy as np
+    from dlgrad_amd.buffer import Buffer
+    from dlgrad_amd.device import Device
+    lib = hip.lib()
+    in_use0, _, _ = lib.pool_stats()
+    with pytest.raises(MemoryError, match="Failed to allocate"):
+        hip.alloc(80 * 2 ** 30)                                   # 320 GiB of fp32 on a 288 GB card
+    assert lib.pool_stats()[0] == in_use0                         # nothing is left registered by the failure
+    with pytest.raises(RuntimeError, match="Compilation failed"):
+        hip.code_object('extern "C" __global__ void broken(float* p) { p[0] = undefined_name; }', "broken")
+    k = hip.kernel(K.map_kernel, "copy", "x0", ("vec",), 4)
+    with pytest.raises(RuntimeError, match="empty grid"):
+        hip.launch(k, 0, 256, 0, 0, 0, 1)
+    with pytest.raises(RuntimeError, match="1024"):
+        hip.launch(k, 1, 2048, 0, 0, 0, 1)
+    with pytest.raises(RuntimeError, match="bad kernel handle"):
+        hip.launch((10 ** 9, k[1]), 1, 64, 0, 0, 0, 1)
+    with pytest.raises(ValueError, match="needs"):
+        Buffer(hip.alloc(16), (5, 5), Device.HIP)                 # a view larger than its block
+    with pytest.raises(ValueError, match="32-bit"):
+        Buffer.uniform((2 ** 16, 2 ** 16), Device.HIP, "float32")
+    x = Buffer.from_numpy(np.arange(12, dtype=np.float32).reshape(3, 4), Device.HIP)
+    np.testing.assert_array_equal((x + x).numpy(), 2 * np.arange(12, dtype=np.float32).reshape(3, 4))
+
+
+@pytest.mark.gpu
+def test_capture_refuses_what_a_graph_cannot_replay():
+    from dlgrad_amd.runtime import hip
+    if not hip.available():
+        pytest.skip("no HIP device")
+    import numpy as np
+    from dlgrad_amd.buffer import Buffer
+    from dlgrad_amd.device import Device
+    lib = hip.lib()
+    x = Buffer.from_numpy(np.ones((8, 8), np.float32), Device.HIP)
+    g = hip.Graph()
+    with g.arena():
+        y = x + x
+    in_use = lib.pool_stats()[0]
+    with pytest.raises(RuntimeError):
+        with g.capture():
+            y = x + x
+            y.numpy()                                             # a download inside a capture
+    assert not hip.capturing()                                    # the failed capture was closed
+    with pytest.raises(RuntimeError, match="replay the same numbers"):
+        with g.capture():
+            Buffer.uniform((4,), Device.HIP, "float32")
+    assert not hip.capturing()
+    with g.capture():
+        y = x + x
+    g.replay()
+    np.testing.assert_array_equal(y.numpy(), np.full((8, 8), 2, np.float32))
+    g.close()
+    del y
+    assert lib.pool_stats()[0] <= in_use
