@@ -480,6 +480,20 @@ def run_decode(n_tokens: int = 256) -> dict:
     model.generate_greedy_cached(0, 120)
     dt = time.perf_counter() - t0
     out["kv_cached_120_tokens"] = {"ms_per_token": round(dt / 120 * 1e3, 3), "tokens_per_s": round(120 / dt, 1)}
+    # the same decoding as one fixed-shape step (whole cache attended, unwritten rows masked),
+    # captured as a HIP graph and replayed per token: no Python between tokens
+    dec = G.StaticDecoder(model)
+    if not hip.COMPILE_ONLY:
+        dec.capture()
+    dec.generate(0, 8)
+    hip.lib().sync()
+    t0 = time.perf_counter()
+    ids2 = dec.generate(0, 120)
+    dt = time.perf_counter() - t0
+    out["fixed_shape_step_hipgraph_120_tokens"] = {
+        "ms_per_token": round(dt / 120 * 1e3, 3), "tokens_per_s": round(120 / dt, 1),
+        "graph_nodes": dec.graph.nodes if dec.graph else 0, "same_ids_as_cached_loop": ids2 == model.generate_greedy_cached(0, 120)}
+    dec.close()
     return out
 
 

@@ -384,6 +384,15 @@ class Buffer:
         """In-place Adam update of self, m and v with the constants held in device memory."""
         self._dispatch(CustomOps.ADAM_STEP_INPLACE, p=self, g=g, m=m, v=v, consts=consts)
 
+    def row_store_(self, src: "Buffer", idx: "Buffer") -> None:
+        """self[(int)idx, :] = src, rows being the leading dim of self; idx is a one-element
+        Buffer on the same device, read where the kernel runs."""
+        rows = self.shape[0]
+        width = self.numel // max(rows, 1)
+        if src.numel != width or idx.numel != 1 or idx.is_host_scalar:
+            raise ValueError(f"row_store_: row of {src.numel} into {self.shape}, index {idx.shape}")
+        self._dispatch(CustomOps.ROW_STORE, dst=self, src=src, idx=idx, rows=rows, width=width)
+
     def sgd_step_(self, g: "Buffer", v: "Buffer | None", lr: float, momentum: float) -> None:
         """In-place SGD update of self (and of the velocity v when momentum is used)."""
         self._dispatch(CustomOps.SGD_STEP_INPLACE, p=self, g=g, v=v, lr=lr, momentum=momentum)

@@ -1196,6 +1196,25 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const unsigned char* __
     return src, name, _fmt("P", "P", "I")
 
 
+@cache
+def row_store_kernel() -> tuple[str, str, str]:
+    """dst[(int)idx[0], :] = src[:] for a (R, W) dst: a row written at a position that is itself
+    device data, which is what lets one captured decoding step append to the key/value cache
+    at a different place on every replay.  A row index outside [0, R) writes nothing."""
+    name = "row_store"
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ dst, const float* __restrict__ src,
+        const float* __restrict__ idx, u32 R, u32 W) {{
+    const float fi = idx[0];
+    if (!(fi >= 0.0f) || fi >= (float)R) return;
+    const u32 row = (u32)fi;
+    const u32 j = blockIdx.x * 256u + threadIdx.x;
+    if (j < W) dst[(u64)row * W + j] = src[j];
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "I", "I")
+
+
 # =====================================================================================
 # fused RMSNorm
 # =====================================================================================

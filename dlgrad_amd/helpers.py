@@ -73,6 +73,7 @@ class CustomOps(Enum):
     MATMUL_NT = auto()              # x @ y^T with y read in place (no materialised transpose)
     MATMUL_TN = auto()              # x^T @ y with x read in place
     FROM_U8 = auto()                # host uint8 array -> device fp32 buffer, cast on the device
+    ROW_STORE = auto()              # dst[(int)idx, :] = src with idx read on the device (KV cache inside a graph)
     COPY_INTO = auto()              # device-to-device copy into an existing buffer (a KV-cache row)
     SGD_STEP_INPLACE = auto()       # p -= (momentum-filtered) g * lr where p is (graph replay)
     RMSNORM = auto()                # (x * rsqrt(mean(x^2) + eps)) * w over the last axis, one kernel

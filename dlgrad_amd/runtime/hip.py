@@ -461,6 +461,12 @@ class HIP:
         return out
 
     @staticmethod
+    @dispatcher.register(CustomOps.ROW_STORE, Device.HIP)
+    def row_store(dst: Buffer, src: Buffer, idx: Buffer, rows: int, width: int) -> None:
+        if rows and width:
+            launch(kernel(K.row_store_kernel), (width + 255) // 256, 256, _addr(dst), _addr(src), _addr(idx), rows, width)
+
+    @staticmethod
     @dispatcher.register(CustomOps.COPY_INTO, Device.HIP)
     def copy_into(dst: Buffer, src: Buffer) -> None:
         if dst.numel:

@@ -209,6 +209,92 @@ class GPT:
         return ids
 
 
+class StaticDecoder:
+    """Greedy decoding inside the context window as one step of fixed shape.
+
+    forward_incremental attends to a cache that grows by one row per token, so every token has
+    new tensor shapes and must be issued launch by launch from Python (~170 launches per token
+    for the char model, which is what bounds its speed).  Here the step always attends to all
+    block_size cache rows and masks the ones not written yet (-inf before the softmax, so they
+    weigh exactly 0), and everything that changes from token to token -- the token, the cache
+    row to write, the position id, the mask -- is device data updated by the step itself.  The
+    step therefore has no host input at all and can be captured once as a HIP graph and
+    replayed per token.  Same tokens as generate_greedy_cached (the probabilities differ only
+    in the order of the softmax sums)."""
+
+    def __init__(self, model: GPT, reference_positions: bool = STRICT_REFERENCE) -> None:
+        c = model.config
+        self.model, self.reference_positions = model, reference_positions
+        self.cache = KVCache(c, 1)
+        self.tok = Tensor.full((1, 1), 0.0, device=c.device)          # token to feed
+        self.slot = Tensor.full((1, 1), 0.0, device=c.device)         # its index = cache row to write
+        self.seq = Tensor.full((c.block_size + 1, 1), 0.0, device=c.device)
+        self.graph = None
+
+    def reset(self, first_token: int) -> None:
+        self.tok.data.upload_(np.array([[first_token]], np.float32))
+        self.slot.data.upload_(np.zeros((1, 1), np.float32))
+        first = np.zeros(self.seq.shape, np.float32)
+        first[0, 0] = first_token
+        self.seq.data.upload_(first)
+
+    def _attend(self, attn: CausalSelfAttention, x: Tensor, layer: int, hidden: Tensor) -> Tensor:
+        C = x.shape[2]
+        T = self.model.config.block_size
+        q = attn.q_proj(x).reshape((1, 1, attn.n_head, attn.head_dim)).transpose(1, 2)      # (1, h, 1, d)
+        self.cache.k[layer].data.row_store_(attn.k_proj(x).data, self.slot.data)
+        self.cache.v[layer].data.row_store_(attn.v_proj(x).data, self.slot.data)
+        k, v = self.cache.view(layer, T, attn.n_head)                                       # (1, h, T, d)
+        att = (q @ k.transpose(2, 3)) * attn.scale                                          # (1, h, 1, T)
+        att = att.masked_fill(hidden, float("-inf")).softmax(dim=3)
+        return attn.c_proj((att @ v).transpose(1, 2).reshape((1, 1, C)))
+
+    def step(self) -> None:
+        """Feeds self.tok at index self.slot; leaves the argmax in seq[slot + 1] and as the next
+        token, and advances slot.  Reads and writes device memory only."""
+        m, c = self.model, self.model.config
+        slot = self.slot
+        # the reference numbers an incremental token one too high (examples/gpt.py:199); token 0 is a full forward there
+        pos = slot + slot.clamp(min=0, max=1) if self.reference_positions else slot
+        hidden = Tensor.arange((1, c.block_size), device=c.device) > slot                   # cache rows not written yet
+        x = m.wte(self.tok) + m.wpe(pos)
+        for i, block in enumerate(m.blocks):
+            x = x + self._attend(block.attn, block.ln1(x), i, hidden)
+            x = x + block.mlp(block.ln2(x))
+        nxt = m.lm_head(m.ln_f(x)).reshape((1, c.vocab_size)).argmax(1)                     # (1, 1)
+        nslot = slot + 1.0
+        self.seq.data.row_store_(nxt.data, nslot.data)
+        self.tok.data.copy_(nxt.data)
+        self.slot.data.copy_(nslot.data)
+
+    def capture(self) -> None:
+        """hip only: records step() into a graph (one warm-up step fixes every address first)."""
+        from dlgrad_amd.runtime import hip
+        self.graph = hip.Graph()
+        self.reset(0)
+        with self.graph.arena():
+            self.step()
+        with self.graph.capture():
+            self.step()
+
+    def generate(self, first_token: int, max_new_tokens: int) -> list[int]:
+        c = self.model.config
+        if not 0 <= max_new_tokens <= c.block_size - 1:
+            raise ValueError(f"the static step decodes inside the window: at most {c.block_size - 1} new tokens")
+        self.reset(first_token)
+        for _ in range(max_new_tokens):
+            if self.graph is not None:
+                self.graph.replay()
+            else:
+                self.step()
+        return [int(v) for v in self.seq.numpy().reshape(-1)[:max_new_tokens + 1]]
+
+    def close(self) -> None:
+        if self.graph is not None:
+            self.graph.close()
+            self.graph = None
+
+
 def init_weights_(model: GPT, seed: int, std: float = 0.02) -> None:
     """Overwrites every parameter with seeded numpy values: N(0, std) for matrices and
     embeddings, ones for the RMSNorm gains -- the same values on any device."""

@@ -61,6 +61,13 @@ class CPU:
         return HostPtr(np.asarray(data, dtype=np.uint8).astype(np.float32))
 
     @staticmethod
+    @_reg(CustomOps.ROW_STORE)
+    def row_store(dst: Buffer, src: Buffer, idx: Buffer, rows: int, width: int) -> None:
+        i = float(idx.ptr.arr[0])
+        if 0 <= i < rows:
+            dst.ptr.arr[int(i) * width:(int(i) + 1) * width] = src.ptr.arr[:width]
+
+    @staticmethod
     @_reg(CustomOps.COPY_INTO)
     def copy_into(dst: Buffer, src: Buffer) -> None:
         dst.ptr.arr[:dst.numel] = src.ptr.arr[:src.numel]

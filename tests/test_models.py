@@ -231,6 +231,46 @@ def test_cached_decode_reproduces_full_recompute_on_the_cpu_oracle():
     assert len(shifted) == 31 and shifted[:2] == full[:2] and shifted != full
 
 
+@pytest.mark.parametrize("reference_positions", [True, False])
+def test_fixed_shape_decoding_step_reproduces_cached_decoding_on_the_cpu_oracle(reference_positions):
+    """Attending to the whole (masked) cache instead of its filled part changes no token."""
+    model = G.GPT(G.GPTConfig(device="cpu", **dict(TINY, n_embd=32, block_size=12)))
+    G.init_weights_(model, 3, std=0.5)
+    want = model.generate_greedy_cached(3, 11, reference_positions=reference_positions)
+    dec = G.StaticDecoder(model, reference_positions=reference_positions)
+    assert dec.generate(3, 11) == want
+    assert dec.generate(7, 5) == model.generate_greedy_cached(7, 5, reference_positions=reference_positions)
+    with pytest.raises(ValueError):
+        dec.generate(3, 12)                              # would leave the window (and the position table)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("reference_positions", [True, False])
+def test_decoding_step_replayed_as_a_graph_gives_the_eager_tokens(reference_positions):
+    """hip: the fixed-shape step eager, the same step captured once and replayed per token,
+    and the growing-cache loop on the C oracle's cpu device all produce the same ids; the
+    captured step is reused for a second sequence."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    cfg = dict(TINY, n_embd=64, block_size=32)
+    models = {}
+    for dev in ("cpu", "hip"):
+        models[dev] = G.GPT(G.GPTConfig(device=dev, **cfg))
+        G.init_weights_(models[dev], 3, std=0.2)
+    want = {t: models["cpu"].generate_greedy_cached(t, 31, reference_positions=reference_positions) for t in (0, 9)}
+    dec = G.StaticDecoder(models["hip"], reference_positions=reference_positions)
+    eager = dec.generate(0, 31)
+    if hip.COMPILE_ONLY:
+        return
+    assert eager == want[0]
+    dec.capture()
+    assert dec.graph.nodes > 50
+    assert dec.generate(0, 31) == want[0]
+    assert dec.generate(9, 31) == want[9]
+    assert dec.generate(0, 4) == want[0][:5]
+    dec.close()
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("reference_positions", [True, False])
 def test_gpt_cached_decode_hip_vs_cpu_oracle(reference_positions):
