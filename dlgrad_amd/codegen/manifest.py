@@ -43,22 +43,23 @@ def merge(entries) -> None:
         f.write("[\n" + ",\n".join(json.dumps(r) for r in rows) + "\n]\n")
 
 
-def _compile_one(entry) -> str:
+def _compile_one(job) -> str:
     from dlgrad_amd.codegen import hip_kernel as K
     from dlgrad_amd.runtime import hip
-    gen, params = entry
+    (gen, params), force = job
     src, name, _ = getattr(K, gen)(*params)
-    hip.code_object(src, name)
+    hip.code_object(src, name, force=force)
     return name
 
 
-def compile_all(jobs: int = 8) -> int:
+def compile_all(jobs: int = 8, force: bool = False) -> int:
+    """Compiles every listed kernel; force=True recompiles the ones already in the cache."""
     entries = load()
     if not entries:
         return 0
     from concurrent.futures import ProcessPoolExecutor
     with ProcessPoolExecutor(max_workers=jobs) as ex:
-        names = list(ex.map(_compile_one, entries, chunksize=4))
+        names = list(ex.map(_compile_one, [(e, force) for e in entries], chunksize=4))
     return len(names)
 
 
@@ -82,4 +83,4 @@ if __name__ == "__main__":
     if "--record" in sys.argv:
         record()
     if "--compile" in sys.argv or "--record" not in sys.argv:
-        print(compile_all(), "kernels compiled or found in the cache")
+        print(compile_all(force="--force" in sys.argv), "kernels compiled or found in the cache")

@@ -274,16 +274,18 @@ class Graph:
 
 # ---- kernel cache -----------------------------------------------------------------------
 
-def code_object(src: str, name: str, l: _ffi.HipLib | None = None) -> bytes:
-    """Code object for `src`: from the on-disk cache, else hiprtc.  Needs no GPU."""
+def code_object(src: str, name: str, l: _ffi.HipLib | None = None, force: bool = False) -> bytes:
+    """Code object for `src`: from the on-disk cache, else hiprtc (always hiprtc when `force`,
+    which is how the build step recompiles everything).  Needs no GPU."""
     opts = list(K.COMPILE_OPTIONS)
     key = hashlib.sha256((src + "\0" + " ".join(opts)).encode()).hexdigest()[:20]
     path = os.path.join(CACHE_DIR, f"{name}_{key}.hsaco")
-    try:
-        with open(path, "rb") as f:
-            return f.read()
-    except FileNotFoundError:
-        pass
+    if not force:
+        try:
+            with open(path, "rb") as f:
+                return f.read()
+        except FileNotFoundError:
+            pass
     code = (l or _ffi.get_lib()).compile(src, name + ".hip", opts)
     compiled_now.append(name)
     os.makedirs(CACHE_DIR, exist_ok=True)
