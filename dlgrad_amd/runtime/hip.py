@@ -733,8 +733,12 @@ class HIP:
         O, L, I = prod_(x.shape[:dim]), x.shape[dim], prod_(x.shape[dim + 1:])
         divisor = float(L) if op == "mean" else 1.0
         out = alloc(O * I)
-        if O * I == 0 or L == 0:
+        if O * I == 0:
             return out
+        if L == 0:
+            # nothing to fold: the reference's loops leave the start value (0, or -FLT_MAX for max), and mean divides it by 0
+            start = {"sum": 0.0, "max": -3.4028234663852886e38, "mean": float("nan")}[op]
+            return _map("full", "s0", [], (O * I,), (start,), out=out)
         if I == 1:
             if O < 64 and L >= (1 << 16):                  # a few very long rows: full reduction each
                 for r in range(O):

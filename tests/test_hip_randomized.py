@@ -1,0 +1,137 @@
+"""GPU parity on seeded random shapes: the launcher's classification of an op (vectorised
+row/column/scalar broadcast, strided fallback, 16-byte or 4-byte accesses, tile and block
+choices) depends on shape, strides and alignment, so the shape space is sampled rather than
+listed.  Every case is compared with the C oracle or a float64 closed form at the bars of the
+fixed-shape tests: bit-exact for + - * selects comparisons permutes max argmax, 1e-6 for
+division and transcendental maps, 1e-5 for sums (or at least as close to float64 as the CPU
+path), 1e-4 for matmul.  Inputs include zero-sized dims, size-1 dims in every position,
+extents that are no multiple of 4, and views that start at odd offsets."""
+import numpy as np
+import pytest
+
+from dlgrad_amd.buffer import Buffer
+from dlgrad_amd.device import Device
+from dlgrad_amd.runtime import hip
+from oracle import cref
+from tests.hip_util import check, dev, require_gpu
+
+pytestmark = pytest.mark.gpu
+DIMS = [1, 1, 2, 3, 4, 5, 7, 8, 12, 16, 31, 33, 64, 100]
+
+
+def shape_of(rng, rank, big=False):
+    return tuple(int(rng.choice(DIMS if not big else DIMS + [128, 257])) for _ in range(rank))
+
+
+def misaligned(a):
+    """The same values as a device view that starts 4 bytes into its block."""
+    flat = np.concatenate([np.zeros(1, np.float32), a.reshape(-1)])
+    base = Buffer.from_numpy(flat, Device.HIP)
+    return Buffer(base.ptr + 1, a.shape, Device.HIP)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_broadcast_binary_ops(seed):
+    require_gpu()
+    rng = np.random.default_rng(1000 + seed)
+    for _ in range(12):
+        rank = int(rng.integers(1, 5))
+        xs = shape_of(rng, rank, big=rank <= 2)
+        ys = tuple(1 if rng.random() < 0.4 else d for d in xs)
+        if rng.random() < 0.25:
+            ys = ys[int(rng.integers(0, rank)):] or (1,)              # lower-rank right operand
+        x = rng.standard_normal(xs, dtype=np.float32)
+        y = (rng.standard_normal(ys, dtype=np.float32) + np.float32(3.0)) * np.float32(rng.choice([-1, 1]))
+        xd = misaligned(x) if rng.random() < 0.3 else dev(x)
+        yd = misaligned(y) if rng.random() < 0.3 else dev(y)
+        for op, tol in (("add", 0), ("sub", 0), ("mul", 0), ("div", 1e-6)):
+            got = getattr(xd, f"__{op if op != 'div' else 'truediv'}__")(yd).numpy()
+            check(got, cref.binary(op, x, y), tol, f"{op} {xs} {ys}")
+        check((xd > yd).numpy(), (x > np.broadcast_to(y, xs)).astype(np.float32), 0, f"gt {xs} {ys}")
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_unary_select_and_fill_ops(seed):
+    require_gpu()
+    rng = np.random.default_rng(2000 + seed)
+    for _ in range(10):
+        xs = shape_of(rng, int(rng.integers(1, 5)), big=True)
+        x = rng.standard_normal(xs, dtype=np.float32)
+        xd = misaligned(x) if rng.random() < 0.3 else dev(x)
+        check(xd.exp().numpy(), cref.unary("exp", x), 1e-6, f"exp {xs}")
+        check((-xd).numpy(), -x, 0, f"neg {xs}")
+        check((xd ** 2).numpy(), x * x, 0, f"pow2 {xs}")
+        check(xd.relu().numpy(), np.where(x > 0, x, np.float32(0)), 0, f"relu {xs}")
+        check(xd.clamp(-1, 1).numpy(), cref.clamp(x, -1, 1), 0, f"clamp {xs}")
+        pos = np.abs(x) + np.float32(1e-3)
+        check(dev(pos).log().numpy(), cref.unary("log", pos), 1e-6, f"log {xs}")
+        check(dev(pos).sqrt().numpy(), np.sqrt(pos), 1e-6, f"sqrt {xs}")
+        ms = tuple(1 if rng.random() < 0.5 else d for d in xs)
+        mask = (rng.random(ms) < 0.5).astype(np.float32)
+        check(Buffer.masked_fill(xd, dev(mask), -np.inf).numpy(), cref.masked_fill(x, mask, -np.inf), 0, f"masked_fill {xs} {ms}")
+        other = rng.standard_normal(xs, dtype=np.float32)
+        check(dev(np.broadcast_to(mask, xs).copy()).where(xd, dev(other)).numpy(),
+              np.where(np.broadcast_to(mask, xs) > 0, x, other), 0, f"where {xs}")
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_reductions_argmax_and_permutes(seed):
+    require_gpu()
+    rng = np.random.default_rng(3000 + seed)
+    for _ in range(10):
+        rank = int(rng.integers(1, 5))
+        xs = shape_of(rng, rank, big=rank <= 2)
+        x = rng.standard_normal(xs, dtype=np.float32)
+        xd = misaligned(x) if rng.random() < 0.3 else dev(x)
+        x64 = x.astype(np.float64)
+        for d in [-1] + list(range(rank)):
+            want = x64.sum() if d == -1 else x64.sum(d)
+            got = xd.sum(d).numpy().reshape(np.shape(want))
+            if not hip.COMPILE_ONLY:
+                ref = cref.reduce("sum", x, d).reshape(np.shape(want)).astype(np.float64)
+                scale = np.abs(x64).sum() if d == -1 else np.abs(x64).sum(d)
+                err_gpu, err_cpu = np.abs(got - want), np.abs(ref - want)
+                assert (err_gpu <= 1e-5 * np.abs(want) + 1e-7 * scale).all() or (err_gpu <= err_cpu + 1e-12).all(), \
+                    f"sum {xs} dim {d}"
+            check(xd.max(d).numpy().reshape(np.shape(want)), x.max() if d == -1 else x.max(d), 0, f"max {xs} dim {d}")
+        order = tuple(int(v) for v in rng.permutation(rank))
+        check(xd.permute(order).numpy(), np.transpose(x, order), 0, f"permute {xs} {order}")
+        if rank == 2:
+            t = rng.integers(0, 4, xs).astype(np.float32)                # ties everywhere
+            for d in (0, 1):
+                want = cref.argmax(t, d).reshape((1, xs[1]) if d == 0 else (xs[0], 1))
+                check(dev(t).argmax(d).numpy(), want, 0, f"argmax {xs} dim {d}")
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_matmuls_plain_and_transposed(seed):
+    require_gpu()
+    rng = np.random.default_rng(4000 + seed)
+    for _ in range(8):
+        M, Kd, N = (int(rng.choice([1, 3, 4, 7, 16, 33, 64, 100, 130])) for _ in range(3))
+        batch = tuple(int(rng.choice([1, 2, 3])) for _ in range(int(rng.integers(0, 3))))
+        yb = tuple(1 if rng.random() < 0.4 else b for b in batch)
+        x = rng.standard_normal(batch + (M, Kd), dtype=np.float32)
+        y = rng.standard_normal(yb + (Kd, N), dtype=np.float32) * np.float32(Kd ** -0.5)
+        want = x.astype(np.float64) @ y.astype(np.float64)
+        xd, yd = dev(x), dev(y)
+        scale = float(np.abs(want).max()) + 1e-30
+        nn_ = xd.matmul(yd).numpy()
+        if not hip.COMPILE_ONLY:
+            assert np.abs(nn_ - want).max() <= 1e-4 * scale, f"matmul {x.shape} {y.shape}"
+        yt = np.ascontiguousarray(np.swapaxes(y, -1, -2))
+        xt = np.ascontiguousarray(np.swapaxes(x, -1, -2))
+        check(xd.matmul_nt(dev(yt)).numpy(), nn_, 0, f"NT {x.shape} {yt.shape}")          # same bits as the plain product
+        check(dev(xt).matmul_tn(yd).numpy(), nn_, 0, f"TN {xt.shape} {y.shape}")
+
+
+def test_zero_sized_tensors_go_through_every_op_family():
+    require_gpu()
+    z = dev(np.zeros((0, 5), np.float32))
+    assert (z + z).numpy().shape == (0, 5) and z.exp().numpy().shape == (0, 5)
+    assert z.permute((1, 0)).numpy().shape == (5, 0)
+    assert z.sum(0).numpy().shape == (5,) and not z.sum(0).numpy().any()
+    w = dev(np.ones((5, 3), np.float32))
+    assert z.matmul(w).numpy().shape == (0, 3)
+    e = dev(np.ones((4, 0), np.float32)).matmul(dev(np.ones((0, 6), np.float32))).numpy()     # empty inner dim: zeros
+    assert e.shape == (4, 6) and not e.any()
