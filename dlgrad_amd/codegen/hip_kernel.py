@@ -1629,6 +1629,51 @@ MATMUL_TILE_MODEL = {
 # =====================================================================================
 
 @cache
+def adam_multi_inplace_kernel() -> tuple[str, str, str]:
+    """adam_inplace_kernel for a whole parameter list in one launch.  `ptrs` holds four rows of
+    addresses (p, g, m, v) per tensor, `sizes` the element counts, `first` the first block of each
+    tensor and `owner` the tensor of every block; a block updates 1024 consecutive elements of its
+    tensor (16-byte accesses: every address is 16-byte aligned, the n % 4 tail is done by the
+    tensor's first block).  Same arithmetic as the per-tensor kernel, so the same bits."""
+    src, _, _ = adam_kernel(4)
+    head = src[:src.index('extern "C"')]
+    name = "adam_multi_inplace"
+    src2 = f"""{head}extern "C" __global__ __launch_bounds__(256) void {name}(const u64* __restrict__ ptrs,
+        const u32* __restrict__ sizes, const u32* __restrict__ first, const u32* __restrict__ owner,
+        u32 n_tensors, const AdamArgs* __restrict__ ap) {{
+    const AdamArgs a = *ap;
+    const u32 t = owner[blockIdx.x];
+    const u32 lb = blockIdx.x - first[t];
+    float* p = reinterpret_cast<float*>(ptrs[t]);
+    const float* __restrict__ g = reinterpret_cast<const float*>(ptrs[n_tensors + t]);
+    float* m = reinterpret_cast<float*>(ptrs[2u * n_tensors + t]);
+    float* v = reinterpret_cast<float*>(ptrs[3u * n_tensors + t]);
+    const u32 n = sizes[t], nv = n >> 2;
+    const u32 i = lb * 256u + threadIdx.x;
+    if (i < nv) {{
+        const float4 p4 = reinterpret_cast<float4*>(p)[i], g4 = reinterpret_cast<const float4*>(g)[i];
+        const float4 m4 = reinterpret_cast<float4*>(m)[i], v4 = reinterpret_cast<float4*>(v)[i];
+        float4 po, mo, vo;
+        adam1(p4.x, g4.x, m4.x, v4.x, a, po.x, mo.x, vo.x);
+        adam1(p4.y, g4.y, m4.y, v4.y, a, po.y, mo.y, vo.y);
+        adam1(p4.z, g4.z, m4.z, v4.z, a, po.z, mo.z, vo.z);
+        adam1(p4.w, g4.w, m4.w, v4.w, a, po.w, mo.w, vo.w);
+        reinterpret_cast<float4*>(p)[i] = po;
+        reinterpret_cast<float4*>(m)[i] = mo;
+        reinterpret_cast<float4*>(v)[i] = vo;
+    }}
+    if (lb == 0 && threadIdx.x < (n & 3u)) {{
+        const u32 j = (nv << 2) + threadIdx.x;
+        float po, mo, vo;
+        adam1(p[j], g[j], m[j], v[j], a, po, mo, vo);
+        p[j] = po; m[j] = mo; v[j] = vo;
+    }}
+}}
+"""
+    return src2, name, _fmt("P", "P", "P", "P", "I", "P")
+
+
+@cache
 def sgd_inplace_kernel(momentum: bool) -> tuple[str, str, str]:
     """p -= (momentum ? (v = v * mu + g) : g) * lr, in place (dlgrad/nn/optim.py:22-45): the
     form a captured graph can replay, since no buffer changes its address.  fp contraction is

@@ -75,6 +75,7 @@ class CustomOps(Enum):
     FROM_U8 = auto()                # host uint8 array -> device fp32 buffer, cast on the device
     ROW_STORE = auto()              # dst[(int)idx, :] = src with idx read on the device (KV cache inside a graph)
     COPY_INTO = auto()              # device-to-device copy into an existing buffer (a KV-cache row)
+    ADAM_MULTI_INPLACE = auto()     # one launch for a whole parameter list (addresses in a device table)
     SGD_STEP_INPLACE = auto()       # p -= (momentum-filtered) g * lr where p is (graph replay)
     RMSNORM = auto()                # (x * rsqrt(mean(x^2) + eps)) * w over the last axis, one kernel
     RMSNORM_BWD = auto()            # its backward: dx in one kernel, dw by partial rows + a column sum

@@ -63,6 +63,8 @@ class Adam(Optimizer):
         self.t = 0
         self.graph_safe = graph_safe
         self.consts = Tensor(np.zeros(8, np.float32), device=params[0].device) if graph_safe else None
+        self._table = None                 # device-side address table of the one-launch update
+        self._graph_tables: list = []
 
     def _consts(self) -> tuple:
         c1, c2 = 1.0 - self.beta1 ** self.t, 1.0 - self.beta2 ** self.t
@@ -78,9 +80,19 @@ class Adam(Optimizer):
             from dlgrad_amd.runtime import hip
             if not hip.capturing():
                 self.advance()
-            for p in self.params:
-                k = id(p)
-                p.data.adam_step_(p.grad.data, self.m[k].data, self.v[k].data, self.consts.data)
+            quads = [(p.data, p.grad.data, self.m[id(p)].data, self.v[id(p)].data) for p in self.params
+                     if p.grad is not None and p.numel]
+            if all(not (b.ptr.addr & 15) for q in quads for b in q):
+                # every parameter in one launch; the address table is uploaded on the first step only
+                from dlgrad_amd.dispatch import dispatcher
+                from dlgrad_amd.helpers import CustomOps
+                self._table = dispatcher.dispatch(CustomOps.ADAM_MULTI_INPLACE, Device.HIP, tensors=quads,
+                                                  consts=self.consts.data, table=self._table)
+                if self._table["frozen"] and self._table not in self._graph_tables:
+                    self._graph_tables.append(self._table)         # a captured graph reads it on every replay
+                return
+            for pb, gb, mb, vb in quads:
+                pb.adam_step_(gb, mb, vb, self.consts.data)
             return
         self.t += 1
         consts = self._consts()

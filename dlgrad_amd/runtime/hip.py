@@ -182,6 +182,7 @@ def alloc(numel: int, zero: bool = False) -> DevicePtr:
 
 # ---- captured graphs ------------------------------------------------------------------------
 _graph_depth = 0       # > 0 while a Graph's arena is current (warm-up or capture)
+_after_capture: list = []   # host work a captured step deferred until its capture has ended (table uploads)
 _capturing = False
 
 
@@ -248,13 +249,17 @@ class Graph:
                 yield self
             except BaseException:
                 _capturing = False
+                _after_capture.clear()
                 self._lib.graph_abandon()
                 self._leave()
                 raise
             _capturing = False
             try:
                 self.handle, self.nodes = self._lib.graph_end()
+                for job in _after_capture:
+                    job()
             finally:
+                _after_capture.clear()
                 self._leave()
         return cm()
 
@@ -1048,6 +1053,45 @@ class HIP:
         vec = 4 if not any(a & 15 for a in addrs) else 1
         launch(kernel(K.adam_inplace_kernel, vec), max(1, ((n + vec - 1) // vec + 255) // 256), 256,
                *addrs, n, _addr(consts))
+
+    @staticmethod
+    @dispatcher.register(CustomOps.ADAM_MULTI_INPLACE, Device.HIP)
+    def adam_multi_inplace(tensors: list, consts: Buffer, table: dict | None) -> dict:
+        """tensors: (p, g, m, v) Buffers per parameter.  `table` is what the previous call
+        returned: the device-side address table is rewritten (a host-to-device upload) only when
+        some address differs from it.  A table written for a captured step is never touched
+        again (the caller keeps it alive as long as the graph); later eager steps get their own."""
+        addrs = tuple(_addr(b) for quad in tensors for b in quad)
+        if any(a & 15 for a in addrs):
+            raise ValueError("adam_multi_inplace needs 16-byte aligned tensors")
+        if table is None or table["addrs"] != addrs:
+            nt = len(tensors)
+            sizes = np.array([q[0].numel for q in tensors], dtype=np.uint32)
+            nblk = np.maximum(1, (sizes.astype(np.int64) // 4 + 255) // 256)
+            first = np.concatenate([[0], np.cumsum(nblk)[:-1]]).astype(np.uint32)
+            owner = np.repeat(np.arange(nt, dtype=np.uint32), nblk)
+            ptrs = np.array([[_addr(q[k]) for q in tensors] for k in range(4)], dtype=np.uint64).reshape(-1)
+            arrays = [np.ascontiguousarray(a).view(np.float32) for a in (ptrs, sizes, first, owner)]     # raw bits
+            reuse = (table is not None and not table["frozen"]
+                     and [a.size for a in arrays] == [b.nbytes // 4 for b in table["bufs"]])
+            bufs = table["bufs"] if reuse else [alloc(a.size) for a in arrays]
+
+            def upload(bufs=bufs, arrays=arrays):
+                for b, a in zip(bufs, arrays):
+                    if a.size:
+                        lib().h2d(b.addr, a.ctypes.data, a.nbytes)
+            if capturing():
+                # a captured launch only records where the table is; its contents are written once the
+                # capture has ended, and never again: the graph replays with exactly these addresses
+                _after_capture.append(upload)
+            else:
+                upload()
+            table = {"addrs": addrs, "grid": int(nblk.sum()), "nt": nt, "bufs": bufs, "frozen": capturing()}
+        if table["nt"]:
+            b = table["bufs"]
+            launch(kernel(K.adam_multi_inplace_kernel), table["grid"], 256, b[0].addr, b[1].addr, b[2].addr, b[3].addr,
+                   table["nt"], _addr(consts))
+        return table
 
     @staticmethod
     @dispatcher.register(CustomOps.SGD_STEP_INPLACE, Device.HIP)

@@ -437,3 +437,29 @@ def test_captured_mlp_step_with_in_place_sgd_matches_eager_steps_bit_for_bit(mom
         for p, want in zip(params, eager[k][1]):
             np.testing.assert_array_equal(p.numpy(), want, err_msg=f"replay {k}")
     g.close()
+
+
+@pytest.mark.gpu
+def test_one_launch_adam_over_a_parameter_list_is_bit_identical_to_the_per_tensor_update():
+    """graph_safe Adam updates every parameter in one launch through a device-side address
+    table; sizes with an n % 4 tail and tiny tensors included, three steps, against the
+    out-of-place per-tensor kernel."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    shapes = [(65, 128), (1, 128), (7,), (513, 3), (2,), (1024, 1024), (3, 1, 5)]
+    results = {}
+    for graph_safe in (False, True):
+        ps = [Tensor(np.random.default_rng(10 + i).standard_normal(shape).astype(np.float32), requires_grad=True, device="hip")
+              for i, shape in enumerate(shapes)]
+        opt = nn.optim.Adam(ps, lr=1e-3, graph_safe=graph_safe)
+        n0 = hip.launch_count
+        for step in range(3):
+            for i, p in enumerate(ps):
+                p.grad = Tensor(np.random.default_rng(100 * step + i).standard_normal(p.shape).astype(np.float32), device="hip")
+            opt.step()
+        launches = hip.launch_count - n0
+        results[graph_safe] = [p.numpy() for p in ps] + [opt.m[id(p)].numpy() for p in ps] + [opt.v[id(p)].numpy() for p in ps]
+        assert launches == (3 if graph_safe else 3 * len(shapes)), launches
+    if not hip.COMPILE_ONLY:
+        for a, b in zip(results[True], results[False]):
+            np.testing.assert_array_equal(a, b)
