@@ -318,6 +318,10 @@ class Buffer:
         """Fused row softmax (one kernel instead of max, sub, exp, sum, div)."""
         return self._unary(CustomOps.SOFTMAX, dim=dim)
 
+    def softmax_bwd(self, upstream: "Buffer") -> "Buffer":
+        """self is a softmax output over the last axis; returns self * (upstream - sum(upstream * self))."""
+        return self._like(self._dispatch(CustomOps.SOFTMAX_BWD, y=self, g=upstream))
+
     def log_softmax(self, dim: int) -> "Buffer":
         return self._unary(CustomOps.LOG_SOFTMAX, dim=dim)
 

@@ -1125,6 +1125,51 @@ def softmax_plan(L: int, vec: int) -> tuple[bool, int, int]:
     return True, 0, 256
 
 
+@cache
+def softmax_bwd_rows_kernel(vec: int, nval: int, nt: bool = False) -> tuple[str, str, str]:
+    """dx = y * (g - sum(g * y)) along the contiguous last axis: the backward of a row softmax
+    with output y and upstream gradient g, one wavefront per row, both rows held in registers
+    (12 B per element instead of the ~36 of the four element-wise and one reduction kernels the
+    expression otherwise takes).  Rows of up to 64 * nval items (float4 or float)."""
+    T, comps, nvx = _rms_lanes(vec)
+    nt = nt and vec == 4
+    name = f"softmax_bwd_rows_v{vec}_r{nval}{'nt' if nt else ''}"
+    ld = (lambda p: f"ld4_stream({p} + c)") if nt else (lambda p: f"{p}[c]")
+    dot = " + ".join(f"g[k]{c} * y[k]{c}" for c in comps)
+    outs = "".join(f"            o{c} = y[k]{c} * (g[k]{c} - s);\n" for c in comps)
+    st = ("{ const v4f ov = {o.x, o.y, o.z, o.w}; __builtin_nontemporal_store(ov, reinterpret_cast<v4f*>(q) + c); }" if nt
+          else "q[c] = o;")
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ yp,
+        const float* __restrict__ gp, float* __restrict__ dx, u32 R, u32 L) {{
+    const u32 lane = threadIdx.x & 63u;
+    const u32 row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= R) return;
+    const {T}* __restrict__ py = reinterpret_cast<const {T}*>(yp + (u64)row * L);
+    const {T}* __restrict__ pg = reinterpret_cast<const {T}*>(gp + (u64)row * L);
+    {T}* __restrict__ q = reinterpret_cast<{T}*>(dx + (u64)row * L);
+    const u32 nv = {nvx};
+    {T} y[{nval}], g[{nval}];
+    float s = 0.0f;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{
+        const u32 c = lane + k * 64u;
+        if (c < nv) {{ y[k] = {ld('py')}; g[k] = {ld('pg')}; s += {dot}; }}
+    }}
+    s = wave_sum(s);
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{
+        const u32 c = lane + k * 64u;
+        if (c < nv) {{
+            {T} o;
+{outs}            {st}
+        }}
+    }}
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "I", "I")
+
+
 # =====================================================================================
 # random fill
 # =====================================================================================

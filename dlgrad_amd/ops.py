@@ -348,6 +348,9 @@ class Softmax(OP):
         return self.out
 
     def backward(self, upstream_grad: Buffer) -> tuple:
+        from dlgrad_amd.runtime.hip import HIP
+        if FUSED and self.out.device is Device.HIP and HIP.softmax_bwd_fits(self.out, upstream_grad):
+            return (self.out.softmax_bwd(upstream_grad),)
         gy = upstream_grad * self.out
         return (gy - self.out * gy.sum(dim=self.out.ndim - 1, keepdim=True),)
 

@@ -943,6 +943,27 @@ class HIP:
         return HIP._softmax(x, dim, False)
 
     @staticmethod
+    def softmax_bwd_fits(y: Buffer, g: Buffer) -> bool:
+        L = y.shape[-1] if y.ndim else 0
+        if not L or g.numel != y.numel or g.is_host_scalar:
+            return False
+        return K.rmsnorm_plan(L, HIP._rms_vec(L, _addr(y), _addr(g))) > 0
+
+    @staticmethod
+    @dispatcher.register(CustomOps.SOFTMAX_BWD, Device.HIP)
+    def softmax_bwd(y: Buffer, g: Buffer) -> DevicePtr:
+        L = y.shape[-1]
+        R = y.numel // L
+        dx = alloc(y.numel)
+        vec = HIP._rms_vec(L, _addr(y), _addr(g), dx.addr)
+        nval = K.rmsnorm_plan(L, vec)
+        if nval == 0 or g.numel != y.numel:
+            raise ValueError(f"fused softmax backward does not take rows of {L} floats here")
+        launch(kernel(K.softmax_bwd_rows_kernel, vec, nval, y.numel >= NT_STORE_MIN_ELEMENTS), (R + 3) // 4, 256,
+               _addr(y), _addr(g), dx.addr, R, L)
+        return dx
+
+    @staticmethod
     @dispatcher.register(CustomOps.LOG_SOFTMAX, Device.HIP)
     def log_softmax(x: Buffer, dim: int) -> DevicePtr:
         return HIP._softmax(x, dim, True)

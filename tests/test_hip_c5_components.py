@@ -96,3 +96,27 @@ def test_cross_entropy_forward_backward_on_8192x50304():
     want = sm / NTOK
     assert np.abs(grad[sub] - want).max() <= 1e-4 * np.abs(want).max()
     assert np.abs(grad.sum(1, dtype=np.float64)).max() <= 1e-6   # each row of softmax - onehot sums to 0
+
+
+@pytest.mark.parametrize("R,L", [(8 * 12 * 1024, 1024), (8192, 128), (300, 130), (64, 4096)])
+def test_fused_softmax_backward_rows(R, L):
+    """dx = y (g - sum(g y)): against float64 on a slice, the op-by-op expression on the C oracle's
+    kernels on the same slice (1e-5 of the largest entry), and the identity sum(dx) = 0 per row
+    (softmax rows sum to 1) over the whole tensor."""
+    require_gpu()
+    rng = np.random.default_rng(53)
+    x = rng.standard_normal((R, L), dtype=np.float32) * 2
+    g = rng.standard_normal((R, L), dtype=np.float32)
+    y = dev(x).softmax(1)
+    dx = y.softmax_bwd(dev(g)).numpy()
+    if hip.COMPILE_ONLY:
+        return
+    yh = y.numpy()
+    assert np.abs(dx.sum(1, dtype=np.float64)).max() <= 2e-5
+    sl = slice(0, 256)
+    y64, g64 = yh[sl].astype(np.float64), g[sl].astype(np.float64)
+    want = y64 * (g64 - (g64 * y64).sum(1, keepdims=True))
+    assert np.abs(dx[sl] - want).max() <= 2e-6 * np.abs(want).max() + 1e-9
+    gy = cref.binary("mul", g[sl], yh[sl])                         # the four-kernel form of ops.Softmax.backward
+    ref = cref.binary("sub", gy, cref.binary("mul", yh[sl], cref.reduce("sum", gy, 1)[:, None]))
+    assert np.abs(dx[sl] - ref).max() <= 1e-5 * np.abs(ref).max()
