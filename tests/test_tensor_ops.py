@@ -226,6 +226,21 @@ def test_cross_entropy_sum_forward_mean_backward(shape, device):
     close(a.grad.numpy(), ta.grad, atol=1e-6, rtol=1e-4)
 
 
+@pytest.mark.parametrize("shape", [(4, 7), (1000, 1000)])
+def test_bce_with_logits_forward_backward(shape, device):
+    """test/test_loss.py:39-65: mean of the numerically stable BCE-with-logits and its
+    gradient (sigmoid(x) - t) / N, against torch."""
+    x = RNG.uniform(-1.0, 1.0, shape).astype(np.float32)
+    t = RNG.integers(0, 2, shape).astype(np.float32)
+    (a,), (ta,) = both((x,), device)
+    loss = a.bcewithlogitsloss(Tensor(t, device=device))
+    tl = torch.nn.BCEWithLogitsLoss()(ta, torch.tensor(t))
+    close(loss.numpy().reshape(()), tl.detach(), atol=1e-6, rtol=1e-4)
+    loss.backward()
+    tl.backward()
+    close(a.grad.numpy(), ta.grad, atol=1e-5, rtol=1e-4)
+
+
 def test_rmsnorm_forward(device):
     x = f32(4, 128, 256)
     norm = nn.RMSNorm(256, device=device)
