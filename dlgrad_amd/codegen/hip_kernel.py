@@ -723,14 +723,17 @@ struct PArgs {{ u32 np, nq, nt, nb;        // extents: two carried dims, tile di
     const float* __restrict__ xi = x + (u64)p * a.ip + (u64)q * a.iq;
     float* __restrict__ oo = out + (u64)p * a.op + (u64)q * a.oq;
     const u32 c4 = threadIdx.x & 15u, r16 = threadIdx.x >> 4;
+    float4 v[4];
     #pragma unroll
-    for (u32 k = 0; k < 64u; k += 16u) {{
-        const u32 t = bt * 64u + 4u * c4, b = bb * 64u + r16 + k;
-        if (t < a.nt && b < a.nb) {{
-            const float4 v = *reinterpret_cast<const float4*>(xi + (u64)b * a.ib + t);
-            float* __restrict__ d = &tile[r16 + k][4u * c4];
-            d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
-        }}
+    for (u32 k = 0; k < 4u; ++k) {{                   // all four loads in flight before the first LDS write
+        const u32 t = bt * 64u + 4u * c4, b = bb * 64u + r16 + 16u * k;
+        v[k] = (t < a.nt && b < a.nb) ? *reinterpret_cast<const float4*>(xi + (u64)b * a.ib + t)
+                                      : make_float4(0.f, 0.f, 0.f, 0.f);
+    }}
+    #pragma unroll
+    for (u32 k = 0; k < 4u; ++k) {{
+        float* __restrict__ d = &tile[r16 + 16u * k][4u * c4];
+        d[0] = v[k].x; d[1] = v[k].y; d[2] = v[k].z; d[3] = v[k].w;
     }}
     __syncthreads();
     #pragma unroll
