@@ -53,6 +53,7 @@ std::map<uint64_t, bool> g_arena_alive;                              // arenas t
 uint64_t g_arena = 0, g_next_arena = 1;
 uint64_t g_bytes_in_use = 0, g_bytes_cached = 0, g_device_allocs = 0;
 bool g_capturing = false;
+std::map<void *, size_t> g_pinned;                                   // page-locked host blocks handed out
 std::vector<hipGraphExec_t> g_graphs;                                // handle = index + 1 (null once destroyed)
 
 int fail(const char *what, hipError_t e) {
@@ -181,6 +182,8 @@ int dlg_hip_shutdown(void) {
     while (!g_free.empty()) trim_arena_locked(g_free.begin()->first);
     g_arena = 0;
     g_capturing = false;
+    for (auto &kv : g_pinned) (void)hipHostFree(kv.first);
+    g_pinned.clear();
     for (hipModule_t m : g_modules) (void)hipModuleUnload(m);
     g_modules.clear();
     g_kernels.clear();
@@ -300,6 +303,56 @@ int dlg_hip_d2d(void *dst, const void *src, size_t n) {
     NEED_INIT();
     if (!n) return 0;
     HIP_TRY(hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToDevice, g_stream));
+    return 0;
+}
+
+// ---- pinned staging ---------------------------------------------------------------
+
+int dlg_hip_host_alloc(size_t nbytes, void **out) {
+    NEED_INIT();
+    if (!out) return fail_msg(-1, "out is NULL");
+    *out = nullptr;
+    void *p = nullptr;
+    hipError_t e = hipHostMalloc(&p, nbytes ? nbytes : 1, hipHostMallocDefault);
+    if (e != hipSuccess || !p) {
+        (void)hipGetLastError();
+        char buf[160];
+        std::snprintf(buf, sizeof buf, "Failed to allocate %zu bytes of pinned host memory", nbytes);
+        return fail_msg(-3, buf);
+    }
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_pinned[p] = nbytes;
+    *out = p;
+    return 0;
+}
+
+int dlg_hip_host_free(void *ptr) {
+    if (!ptr) return 0;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        if (!g_inited) return 0;
+        auto it = g_pinned.find(ptr);
+        if (it == g_pinned.end()) return fail_msg(-7, "dlg_hip_host_free: pointer was not allocated here");
+        g_pinned.erase(it);
+    }
+    (void)hipStreamSynchronize(g_stream);        // a copy out of it may still be queued
+    HIP_TRY(hipHostFree(ptr));
+    return 0;
+}
+
+int dlg_hip_h2d_async(void *dst, const void *src, size_t n) {
+    NEED_INIT();
+    if (!n) return 0;
+    {                                            // pageable memory would make this copy synchronous or unsafe
+        std::lock_guard<std::mutex> lk(g_mu);
+        bool ok = false;
+        for (const auto &kv : g_pinned) {
+            const char *b = (const char *)kv.first;
+            if ((const char *)src >= b && (const char *)src + n <= b + kv.second) { ok = true; break; }
+        }
+        if (!ok) return fail_msg(-8, "dlg_hip_h2d_async: the source is not inside a dlg_hip_host_alloc block");
+    }
+    HIP_TRY(hipMemcpyAsync(dst, src, n, hipMemcpyHostToDevice, g_stream));
     return 0;
 }
 

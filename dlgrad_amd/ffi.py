@@ -33,6 +33,9 @@ _SIGS = {
     "dlg_hip_h2d": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_size_t]),
     "dlg_hip_d2h": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_size_t]),
     "dlg_hip_d2d": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_size_t]),
+    "dlg_hip_host_alloc": (_c.c_int, [_c.c_size_t, _c.POINTER(_c.c_void_p)]),
+    "dlg_hip_host_free": (_c.c_int, [_c.c_void_p]),
+    "dlg_hip_h2d_async": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_size_t]),
     "dlg_hip_compile": (_c.c_int, [_c.c_char_p, _c.c_char_p, _c.POINTER(_c.c_char_p), _c.c_int,
                                    _c.POINTER(_c.c_void_p), _c.POINTER(_c.c_size_t)]),
     "dlg_hip_code_free": (_c.c_int, [_c.c_void_p]),
@@ -201,6 +204,17 @@ class HipLib:
 
     def d2d(self, dst: int, src: int, nbytes: int) -> None:
         self._check(self._lib.dlg_hip_d2d(self._vp(dst), self._vp(src), nbytes))
+
+    def host_alloc(self, nbytes: int) -> int:
+        ref, get = self._out(ctypes.c_void_p, "void *")
+        self._check(self._lib.dlg_hip_host_alloc(nbytes, ref), MemoryError)
+        return get() or 0
+
+    def host_free(self, ptr: int) -> None:
+        self._check(self._lib.dlg_hip_host_free(self._vp(ptr)))
+
+    def h2d_async(self, dst: int, pinned_addr: int, nbytes: int) -> None:
+        self._check(self._lib.dlg_hip_h2d_async(self._vp(dst), self._vp(pinned_addr), nbytes))
 
     # -- kernels -------------------------------------------------------------------------
     def compile(self, source: str, name: str, options: list[str]) -> bytes:

@@ -28,23 +28,29 @@ MNIST_FILES = (
 )
 
 
-def read_idx(path: str, images: bool, magic_number: int) -> np.ndarray:
-    """uint8 array (count, rows*cols) or (count, 1) from an idx file, plain or gzip."""
+def read_idx(path: str, images: bool, magic_number: int, empty=np.empty) -> np.ndarray:
+    """uint8 array (count, rows*cols) or (count, 1) from an idx file, plain or gzip.  `empty`
+    allocates the result (shape, dtype) -- page-locked memory when the bytes go to a GPU."""
     opener = gzip.open if path.endswith(".gz") else open
-    with opener(path, "rb") as f:
-        raw = f.read()
     nhead = 16 if images else 8
-    if len(raw) < nhead:
-        raise ValueError(f"{path}: shorter than an idx header")
-    fields = struct.unpack(">" + "I" * (nhead // 4), raw[:nhead])
-    if fields[0] != magic_number:
-        raise ValueError(f"{path}: invalid magic number {fields[0]}, expected {magic_number}")
-    count = fields[1]
-    per = fields[2] * fields[3] if images else 1
-    if len(raw) - nhead < count * per:
-        raise ValueError(f"{path}: read error or unexpected EOF ({len(raw) - nhead} data bytes, "
-                         f"{count * per} announced)")
-    return np.frombuffer(raw, dtype=np.uint8, count=count * per, offset=nhead).reshape(count, per)
+    with opener(path, "rb") as f:
+        head = f.read(nhead)
+        if len(head) < nhead:
+            raise ValueError(f"{path}: shorter than an idx header")
+        fields = struct.unpack(">" + "I" * (nhead // 4), head)
+        if fields[0] != magic_number:
+            raise ValueError(f"{path}: invalid magic number {fields[0]}, expected {magic_number}")
+        count = fields[1]
+        per = fields[2] * fields[3] if images else 1
+        out = empty((count, per), np.uint8)
+        view = memoryview(out).cast("B") if out.size else memoryview(b"")
+        got = 0
+        while got < len(view):
+            n = f.readinto(view[got:])
+            if not n:
+                raise ValueError(f"{path}: read error or unexpected EOF ({got} data bytes, {len(view)} announced)")
+            got += n
+    return out
 
 
 def _find(root: str, name: str) -> str:
@@ -58,7 +64,14 @@ def mnist(device: Device = Device.CPU, root: str | None = None) -> list[Tensor]:
     """[train_images, train_labels, test_images, test_labels]."""
     root = root or os.path.join(CACHE_DIR, "downloads")
     out = []
+    from dlgrad_amd.device import as_device
+    on_hip = as_device(device) is Device.HIP
+    if on_hip:
+        from dlgrad_amd.runtime import hip
     for name, images, magic in MNIST_FILES:
-        data = read_idx(_find(root, name), images, magic)
+        # hip: file -> page-locked buffer -> DMA -> widened to fp32 by a kernel; the upload is only enqueued
+        data = read_idx(_find(root, name), images, magic, empty=hip.pinned_empty if on_hip else np.empty)
         out.append(Tensor(Buffer.from_u8(data, device), requires_grad=False, device=device))
+    if on_hip:
+        hip.lib().sync()                   # the staging buffers are released when `data` goes out of scope
     return out

@@ -180,6 +180,53 @@ def alloc(numel: int, zero: bool = False) -> DevicePtr:
     return DevicePtr(l.alloc(nbytes, zero), nbytes)
 
 
+# ---- pinned host staging ------------------------------------------------------------------
+_pinned: dict = {}     # address -> bytes of every live page-locked block
+
+
+def pinned_empty(shape, dtype=np.float32) -> np.ndarray:
+    """A numpy array in page-locked host memory.  Uploads from it (Buffer.from_numpy, upload_,
+    from_u8) are enqueued without waiting for the copy, and may be recorded into a captured
+    graph, which then re-reads the array on every replay.  Do not modify the array between an
+    upload and the next sync().  The memory is released when the array is collected."""
+    import ctypes
+    import weakref
+    shape = tuple(shape) if not isinstance(shape, int) else (shape,)
+    nbytes = int(np.prod(shape, dtype=np.int64)) * np.dtype(dtype).itemsize
+    if COMPILE_ONLY:
+        return np.empty(shape, dtype)
+    l = lib()
+    addr = l.host_alloc(max(nbytes, 1))
+    raw = (ctypes.c_char * max(nbytes, 1)).from_address(addr)
+    _pinned[addr] = max(nbytes, 1)
+
+    def release(addr=addr):
+        _pinned.pop(addr, None)
+        cur = _state["lib"]
+        if cur is not None:
+            try:
+                cur.host_free(addr)
+            except Exception:      # interpreter shutdown
+                pass
+    weakref.finalize(raw, release)
+    return np.frombuffer(raw, dtype=dtype, count=nbytes // np.dtype(dtype).itemsize).reshape(shape)
+
+
+def _is_pinned(a: np.ndarray) -> bool:
+    p, n = a.ctypes.data, a.nbytes
+    return any(b <= p and p + n <= b + size for b, size in _pinned.items())
+
+
+def _upload(dst_addr: int, a: np.ndarray) -> None:
+    """Host array -> device: enqueued without a wait when the array is page-locked."""
+    if not a.nbytes:
+        return
+    if _pinned and _is_pinned(a):
+        lib().h2d_async(dst_addr, a.ctypes.data, a.nbytes)
+    else:
+        lib().h2d(dst_addr, a.ctypes.data, a.nbytes)
+
+
 # ---- captured graphs ------------------------------------------------------------------------
 _graph_depth = 0       # > 0 while a Graph's arena is current (warm-up or capture)
 _after_capture: list = []   # host work a captured step deferred until its capture has ended (table uploads)
@@ -448,8 +495,7 @@ class HIP:
     def create(data: np.ndarray, into: Buffer | None = None) -> DevicePtr:
         a = np.ascontiguousarray(data, dtype=np.float32)
         p = into.ptr if into is not None else alloc(a.size)
-        if a.size:
-            lib().h2d(p.addr, a.ctypes.data, a.nbytes)
+        _upload(p.addr, a)
         return p
 
     @staticmethod
@@ -463,7 +509,7 @@ class HIP:
         if n == 0:
             return out
         raw = alloc((n + 3) // 4)                                # staging for the bytes; freed in stream order
-        lib().h2d(raw.addr, a.ctypes.data, n)
+        _upload(raw.addr, a)
         launch(kernel(K.u8_to_f32_kernel), ((n + 3) // 4 + 255) // 256, 256, raw.addr, out.addr, n)
         return out
 

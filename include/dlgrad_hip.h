@@ -86,6 +86,18 @@ int dlg_hip_h2d(void *dst_dev, const void *src_host, size_t nbytes);
 int dlg_hip_d2h(void *dst_host, const void *src_dev, size_t nbytes);
 int dlg_hip_d2d(void *dst_dev, const void *src_dev, size_t nbytes);
 
+/* ---- pinned staging (the data path of dlgrad/nn/datasets.py:9-39 and of the
+ * per-step batch in examples/mnist_mlp.py, where the reference hands numpy memory
+ * to the kernels directly).  dlg_hip_host_alloc returns page-locked host memory
+ * the GPU reads by DMA; dlg_hip_h2d_async enqueues a copy from such memory on the
+ * stream and returns at once: the source must stay unchanged until a later
+ * dlg_hip_sync (or event) has passed.  Unlike dlg_hip_h2d it may be issued during
+ * a capture: the graph then re-reads the same host buffer on every replay, so a
+ * loop only refills that buffer between replays.                              */
+int dlg_hip_host_alloc(size_t nbytes, void **out);
+int dlg_hip_host_free(void *ptr);
+int dlg_hip_h2d_async(void *dst_dev, const void *src_pinned, size_t nbytes);
+
 /* ---- kernels ---------------------------------------------------------------
  * dlg_hip_compile <- CPU._build_shared_object(source, so_path) cpu.py:52-62
  *      (clang/gcc subprocess).  Here hiprtc compiles HIP source for the given

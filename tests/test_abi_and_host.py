@@ -211,3 +211,39 @@ def test_capture_refuses_what_a_graph_cannot_replay():
     g.close()
     del y
     assert lib.pool_stats()[0] <= in_use
+
+
+@pytest.mark.gpu
+def test_pinned_staging_uploads_without_a_wait_and_inside_a_captured_graph():
+    """A page-locked array is uploaded by an enqueued DMA; recorded into a graph, the copy
+    re-reads the array on every replay, so a loop refills it between replays (after a sync)
+    and nothing else crosses the host boundary."""
+    from dlgrad_amd.runtime import hip
+    if not hip.available():
+        pytest.skip("no HIP device")
+    lib = hip.lib()
+    rng = np.random.default_rng(8)
+    stage = hip.pinned_empty((128, 784))
+    assert stage.dtype == np.float32 and stage.shape == (128, 784) and hip._is_pinned(stage)
+    stage[:] = rng.random((128, 784), dtype=np.float32)
+    want = stage.copy()
+    x = Buffer.from_numpy(stage, Device.HIP)                      # enqueued, not waited for
+    np.testing.assert_array_equal(x.numpy(), want)                # numpy() waits for the stream
+    with pytest.raises(RuntimeError, match="host_alloc block"):
+        lib.h2d_async(x.ptr.addr, want.ctypes.data, want.nbytes)  # pageable memory is refused
+    g = hip.Graph()
+    with g.arena():
+        y = x * 2.0
+    with g.capture():
+        x.upload_(stage)                                          # a memcpy node that reads `stage` at replay time
+        y = x * 2.0
+    for k in range(3):
+        lib.sync()                                                # the previous replay has read the staging array
+        stage[:] = np.float32(k + 1)
+        g.replay()
+        np.testing.assert_array_equal(y.numpy(), np.full((128, 784), 2 * (k + 1), np.float32))
+    g.close()
+    del stage, x, y
+    import gc
+    gc.collect()
+    assert not hip._pinned                                        # the page-locked block went back
