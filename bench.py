@@ -584,6 +584,35 @@ def run_mlp_graph(steps: int, warmup: int) -> dict:
     return res
 
 
+def run_transfers() -> dict:
+    """Host <-> device rates at the boundary (never part of `value`): 256 MiB uploaded from
+    pageable memory (copy + wait, what Tensor(np_array) does), from page-locked staging memory
+    (enqueued DMA), and downloaded."""
+    _, _, Buffer, Device, hip = _imports()
+    lib = hip.lib()
+    n = 64 * 2 ** 20
+    host = np.ones(n, np.float32)
+    stage = hip.pinned_empty((n,))
+    stage[:] = 1.0
+    dst = hip.alloc(n)
+    out = {}
+    for name, src in (("h2d_pageable_GBps", host), ("h2d_page_locked_GBps", stage)):
+        hip._upload(dst.addr, src)
+        lib.sync()
+        t0 = time.perf_counter()
+        for _ in range(3):
+            hip._upload(dst.addr, src)
+        lib.sync()
+        out[name] = round(3 * 4 * n / (time.perf_counter() - t0) / 1e9, 1)
+    back = np.empty(n, np.float32)
+    lib.d2h(back.ctypes.data, dst.addr, 4 * n)
+    t0 = time.perf_counter()
+    for _ in range(3):
+        lib.d2h(back.ctypes.data, dst.addr, 4 * n)
+    out["d2h_pageable_GBps"] = round(3 * 4 * n / (time.perf_counter() - t0) / 1e9, 1)
+    return out
+
+
 def step_roofline(flops: float, ms: float, note: str) -> dict:
     achieved = flops / (ms * 1e-3) / 1e12
     return {"bound": "mfma", "achieved": achieved, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -664,6 +693,7 @@ def main() -> None:
             extra["mlp_784_64_10_step_hipgraph"] = {k: round(v, 3) for k, v in run_mlp_graph(200, 10).items()}
             extra["c5_components"] = run_c5(max(3, min(args.steps, 10)), 2)
             extra["layout_and_select"] = run_layout_and_select(max(3, min(args.steps, 10)), 2)
+            extra["host_device_transfers"] = run_transfers()
             extra["gpt_scaled_c5"] = run_gpt_large(2)
             out["extra"] = extra
     elif args.workload == "matmul":
