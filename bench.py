@@ -708,15 +708,20 @@ def main() -> None:
         if not args.no_cpu:
             out["cpu_baseline"] = cpu_matmul(512)
     elif args.workload == "gpt":
-        g = run_gpt(args.steps, args.warmup)
-        out = {"metric": "GPT fwd+bwd tokens/s (1 GPU)", "value": g["tokens_per_s"], "unit": "tokens/s", **base,
-               "ms_per_step": g["ms_per_step"],
+        gg = run_gpt_graph(args.steps, args.warmup)               # the step as it is meant to be run on this device
+        g = run_gpt(max(3, min(args.steps, 10)), 2)               # the same step issued launch by launch from Python
+        out = {"metric": "GPT fwd+bwd tokens/s (1 GPU)", "value": gg["tokens_per_s"], "unit": "tokens/s", **base,
+               "ms_per_step": gg["ms_per_step"],
                "config": {"workload": "C4 char-GPT vocab 65, block 128, 6 layers, 4 heads, n_embd 128, batch 16; "
-                                      "forward + backward + Adam step (RMSNorm, ReLU MLP, no bias, as examples/gpt.py)",
-                          "launches_per_step": g["launches_per_step"], "loss_per_token": g["loss_per_token"]},
-               "roofline": step_roofline(6 * 1_187_968 * 2048, g["ms_per_step"],
-                                         "whole eager step against the fp32 MFMA peak; 6 x 1.19 M matmul parameters x 2048 "
-                                         "tokens; the step is bound by Python-issued launches, not by the GPU")}
+                                      "forward + backward + Adam step (RMSNorm, ReLU MLP, no bias, as examples/gpt.py), "
+                                      "captured once as a HIP graph and replayed per step (same kernels, bit-identical)",
+                          "graph_nodes": gg["graph_nodes"], "loss_per_token": gg["loss_per_token"],
+                          "eager_ms_per_step": round(g["ms_per_step"], 3), "eager_tokens_per_s": round(g["tokens_per_s"], 1),
+                          "eager_launches_per_step": g["launches_per_step"]},
+               "roofline": step_roofline(6 * 1_187_968 * 2048, gg["ms_per_step"],
+                                         "whole step against the fp32 MFMA peak; 6 x 1.19 M matmul parameters x 2048 tokens; "
+                                         "at this size every kernel is a few microseconds and the step is bound by per-kernel "
+                                         "latency, not by the matrix cores")}
         if not args.no_cpu:
             out["cpu_baseline"] = cpu_gpt()
     elif args.workload == "gpt-large":
