@@ -515,10 +515,11 @@ static __device__ __forceinline__ void wave_argmax(float& best, u32& bi) {
 
 
 @cache
-def argmax_kernel(mode: str, vec: int = 1) -> tuple[str, str, str]:
+def argmax_kernel(mode: str, vec: int = 1, unroll: int = 4, nt: bool = False) -> tuple[str, str, str]:
     """Index (as float) of the first maximum along L of an (O, L, I) view
     (cpu_kernel.py:459-517: strict '>', start value -FLT_MAX at index 0).
-      rows_thread  I == 1, short rows (the (N, 10) class scores): one thread per row
+      rows_thread  I == 1, short rows, few of them: one thread per row
+      rows_staged  I == 1, short rows (the (N, 10) class scores): 256 rows per block through LDS
       rows_wave    I == 1: one wavefront per row
       rows_block   I == 1, long rows (50304-wide logits): one block per row
       cols_part    I > 1: a 64 x 16 block owns 64 columns of one chunk of L; thread rows take
@@ -537,6 +538,52 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
     float best = NEG_FLT_MAX; u32 bi = 0;
     for (u32 i = 0; i < L; ++i) {{ const float v = p[i]; if (v > best) {{ best = v; bi = i; }} }}
     out[row] = (float)bi;
+}}
+"""
+        return src, name, _fmt("P", "P", "I", "I")
+    if mode == "rows_staged":
+        # vec is (cap << 3) | width: rows of at most cap floats, loads of `width` floats
+        cap, width = vec >> 3, vec & 7
+        name = f"argmax_rows_staged_c{cap}_v{width}"
+        if width == 4:
+            fill = """
+    u32 e = threadIdx.x * 4u, r = e / L, c = e % L;
+    const u32 dq = 1024u / L, dr = 1024u % L;
+    for (; e + 3u < n; e += 1024u) {
+        const float4 v = ld4_stream(reinterpret_cast<const float4*>(p + e));
+        u32 rr = r, cc = c;
+        s[rr * Lp + cc] = v.x; if (++cc == L) { cc = 0; ++rr; }
+        s[rr * Lp + cc] = v.y; if (++cc == L) { cc = 0; ++rr; }
+        s[rr * Lp + cc] = v.z; if (++cc == L) { cc = 0; ++rr; }
+        s[rr * Lp + cc] = v.w;
+        c += dr; r += dq; if (c >= L) { c -= L; ++r; }
+    }
+    for (u32 t = (n & ~3u) + threadIdx.x; t < n; t += 256u) s[(t / L) * Lp + t % L] = p[t];"""
+        else:
+            fill = """
+    u32 r = threadIdx.x / L, c = threadIdx.x % L;
+    const u32 dq = 256u / L, dr = 256u % L;
+    for (u32 e = threadIdx.x; e < n; e += 256u) {
+        s[r * Lp + c] = p[e];
+        c += dr; r += dq; if (c >= L) { c -= L; ++r; }
+    }"""
+        src = f"""{PRELUDE}
+// 256 rows of L <= {cap} floats are one contiguous run: it is read with full-width coalesced
+// loads into LDS (row pitch L | 1, so the per-row scans that follow hit distinct banks).
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        float* __restrict__ out, u32 R, u32 L) {{
+    __shared__ float s[256 * {cap | 1}];
+    const u32 row0 = blockIdx.x * 256u;
+    const u32 rows = min(256u, R - row0);
+    const u32 n = rows * L, Lp = L | 1u;
+    const float* __restrict__ p = x + (u64)row0 * L;
+{fill}
+    __syncthreads();
+    if (threadIdx.x >= rows) return;
+    const float* q = s + threadIdx.x * Lp;
+    float best = NEG_FLT_MAX; u32 bi = 0;
+    for (u32 i = 0; i < L; ++i) {{ const float v = q[i]; if (v > best) {{ best = v; bi = i; }} }}
+    out[row0 + threadIdx.x] = (float)bi;
 }}
 """
         return src, name, _fmt("P", "P", "I", "I")
@@ -589,14 +636,20 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
     if mode == "cols_part":
         name += f"_v{vec}"
         if vec == 4:
-            scan = """
-        for (u32 l = l0 + ty; l < l1; l += 16u) {
-            const float4 v = *reinterpret_cast<const float4*>(xp + (u64)l * I);
-            if (v.x > best[0]) { best[0] = v.x; bi[0] = l; }
-            if (v.y > best[1]) { best[1] = v.y; bi[1] = l; }
-            if (v.z > best[2]) { best[2] = v.z; bi[2] = l; }
-            if (v.w > best[3]) { best[3] = v.w; bi[3] = l; }
-        }"""
+            name += f"u{unroll}" + ("nt" if nt else "")
+            ld = "ld4_stream(" if nt else "*("
+            loads = "\n".join(f"            const float4 v{u} = {ld}reinterpret_cast<const float4*>(xp + (u64)(l + {16 * u}u) * I));"
+                              for u in range(unroll))
+            steps = " ".join(f"STEP(v{u}, l + {16 * u}u)" for u in range(unroll))
+            scan = f"""
+        #define STEP(v, l) {{ if (v.x > best[0]) {{ best[0] = v.x; bi[0] = (l); }} if (v.y > best[1]) {{ best[1] = v.y; bi[1] = (l); }} \\
+                             if (v.z > best[2]) {{ best[2] = v.z; bi[2] = (l); }} if (v.w > best[3]) {{ best[3] = v.w; bi[3] = (l); }} }}
+        u32 l = l0 + ty;
+        for (; l + {16 * (unroll - 1)}u < l1; l += {16 * unroll}u) {{                  // {unroll} rows in flight, compared in row order
+{loads}
+            {steps}
+        }}
+        for (; l < l1; l += 16u) {{ const float4 v = {ld}reinterpret_cast<const float4*>(xp + (u64)l * I)); STEP(v, l) }}"""
         else:
             scan = """
         for (u32 l = l0 + ty; l < l1; l += 16u) { const float v = xp[(u64)l * I]; if (v > best[0]) { best[0] = v; bi[0] = l; } }"""
@@ -630,19 +683,27 @@ extern "C" __global__ __launch_bounds__(1024) void {name}(const float* __restric
 """
         return src, name, _fmt("P", "P", "P", "P", "I", "I", "I", "I")
     assert mode == "cols_fin"
-    src = f"""{PRELUDE}
-extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ pv,
+    src = f"""{PRELUDE}{_ARGMAX_PAIR}
+// 64 columns x 16 chunk lanes per block: lane ty folds chunks ty, ty + 16, ..., LDS joins the lanes
+extern "C" __global__ __launch_bounds__(1024) void {name}(const float* __restrict__ pv,
         const u32* __restrict__ pi, float* __restrict__ out, u32 O, u32 chunks, u32 I) {{
-    const u32 t = blockIdx.x * 256u + threadIdx.x;
-    if (t >= O * I) return;
-    const u32 o = t / I, i = t % I;
+    __shared__ float sv[16][65]; __shared__ u32 si[16][65];
+    const u32 tx = threadIdx.x, ty = threadIdx.y, o = blockIdx.y;
+    const u32 col = blockIdx.x * 64u + tx;
     float best = NEG_FLT_MAX; u32 bi = 0;
-    for (u32 c = 0; c < chunks; ++c) {{
-        const u64 at = ((u64)o * chunks + c) * I + i;
-        const float v = pv[at];
-        if (v > best) {{ best = v; bi = pi[at]; }}
+    if (col < I)
+        for (u32 c = ty; c < chunks; c += 16u) {{
+            const u64 at = ((u64)o * chunks + c) * I + col;
+            const float v = pv[at]; const u32 i = pi[at];
+            TAKE(best, bi, v, i)
+        }}
+    sv[ty][tx] = best; si[ty][tx] = bi;
+    __syncthreads();
+    if (ty == 0 && col < I) {{
+        #pragma unroll
+        for (int k = 1; k < 16; ++k) TAKE(best, bi, sv[k][tx], si[k][tx])
+        out[(u64)o * I + col] = (float)bi;
     }}
-    out[t] = (float)bi;
 }}
 """
     return src, name, _fmt("P", "P", "P", "I", "I", "I")
@@ -695,54 +756,70 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 
 
 @cache
-def permute_tiled_kernel(vec: int = 1) -> tuple[str, str, str]:
+def permute_tiled_kernel(vec: int = 1, swz: int = 0, tile: int = 64, nt: bool = False) -> tuple[str, str, str]:
     """Permutations that move another dim into the innermost position, e.g. (.., a, b) ->
     (.., b, a) or (B,T,h,d) -> (B,h,d,T).  Out dims are (p, q, t, b) after padding where
     b is the out-innermost dim and t is the out dim whose *input* stride is 1.  A tile of
-    the (t, b) plane goes through LDS (rows padded by one float, no bank conflicts) so that
-    reads run along t and writes along b, both coalesced; p and q only offset the tile.
-    vec = 1: 32 x 32 tile, 4-byte accesses.  vec = 4: 64 x 64 tile, 16-byte loads along t and
-    16-byte stores along b (256-byte row segments); needs extents and strides that are
-    multiples of 4 and 16-byte aligned bases.
+    the (t, b) plane goes through LDS (rows padded by one float) so that reads run along t
+    and writes along b, both coalesced; p and q only offset the tile.
+    vec = 1: 32 x 32 tile, 4-byte accesses.  vec = 4: tile x tile (64 or 128), 16-byte loads
+    along t and 16-byte stores along b; needs extents and strides that are multiples of 4 and
+    16-byte aligned bases.
+    swz = 1 walks the tiles of one block row diagonally: when the input's row pitch is a large
+    power of two, the tiles that run at the same time otherwise read the same few memory
+    channels.  nt: streaming loads and stores (planes far larger than the caches).
     The reference reads with the large stride directly (cpu_kernel.py:207-212)."""
-    name = "permute_tiled" + ("_v4" if vec == 4 else "")
+    name = "permute_tiled" + ("_v4" if vec == 4 else "") + (f"_t{tile}" if tile != 64 else "") \
+        + (f"_s{swz}" if swz else "") + ("nt" if nt else "")
     head = f"""{PRELUDE}
 struct PArgs {{ u32 np, nq, nt, nb;        // extents: two carried dims, tile dims t and b
                u32 ip, iq, ib;            // input strides of p, q, b (t has input stride 1)
                u32 op, oq, ot; }};        // output strides of p, q, t (b has output stride 1)
 """
     if vec == 4:
+        assert tile in (64, 128)
+        lanes = tile // 4                 # threads across one tile row
+        rows = 256 // lanes               # tile rows per pass of the block
+        passes = tile // rows
+        order = {0: """    const u32 bb = r % tb; r /= tb;
+    const u32 bt = r % tt; r /= tt;""",
+                 1: """    const u32 bb = r % tb; r /= tb;
+    const u32 bt = (r % tt + bb) % tt; r /= tt;"""}[swz]
+        load = "ld4_stream(reinterpret_cast<const float4*>(xi + (u64)b * a.ib + t))" if nt \
+            else "*reinterpret_cast<const float4*>(xi + (u64)b * a.ib + t)"
+        store = ("{ const v4f o = {tile[lb][lt], tile[lb + 1u][lt], tile[lb + 2u][lt], tile[lb + 3u][lt]};\n"
+                 "              __builtin_nontemporal_store(o, reinterpret_cast<v4f*>(oo + (u64)t * a.ot + b)); }") if nt \
+            else ("*reinterpret_cast<float4*>(oo + (u64)t * a.ot + b) =\n"
+                  "                make_float4(tile[lb][lt], tile[lb + 1u][lt], tile[lb + 2u][lt], tile[lb + 3u][lt]);")
         src = head + f"""extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
         float* __restrict__ out, PArgs a) {{
-    __shared__ float tile[64][65];          // [b][t]
-    const u32 tb = (a.nb + 63u) >> 6, tt = (a.nt + 63u) >> 6;
+    __shared__ float tile[{tile}][{tile + 1}];          // [b][t]
+    const u32 tb = (a.nb + {tile - 1}u) / {tile}u, tt = (a.nt + {tile - 1}u) / {tile}u;
     u32 r = blockIdx.x;
-    const u32 bb = r % tb; r /= tb;
-    const u32 bt = r % tt; r /= tt;
+{order}
     const u32 q = r % a.nq, p = r / a.nq;
     const float* __restrict__ xi = x + (u64)p * a.ip + (u64)q * a.iq;
     float* __restrict__ oo = out + (u64)p * a.op + (u64)q * a.oq;
-    const u32 c4 = threadIdx.x & 15u, r16 = threadIdx.x >> 4;
-    float4 v[4];
+    const u32 c4 = threadIdx.x % {lanes}u, rw = threadIdx.x / {lanes}u;
+    float4 v[{passes}];
     #pragma unroll
-    for (u32 k = 0; k < 4u; ++k) {{                   // all four loads in flight before the first LDS write
-        const u32 t = bt * 64u + 4u * c4, b = bb * 64u + r16 + 16u * k;
-        v[k] = (t < a.nt && b < a.nb) ? *reinterpret_cast<const float4*>(xi + (u64)b * a.ib + t)
+    for (u32 k = 0; k < {passes}u; ++k) {{              // every load in flight before the first LDS write
+        const u32 t = bt * {tile}u + 4u * c4, b = bb * {tile}u + rw + {rows}u * k;
+        v[k] = (t < a.nt && b < a.nb) ? {load}
                                       : make_float4(0.f, 0.f, 0.f, 0.f);
     }}
     #pragma unroll
-    for (u32 k = 0; k < 4u; ++k) {{
-        float* __restrict__ d = &tile[r16 + 16u * k][4u * c4];
+    for (u32 k = 0; k < {passes}u; ++k) {{
+        float* __restrict__ d = &tile[rw + {rows}u * k][4u * c4];
         d[0] = v[k].x; d[1] = v[k].y; d[2] = v[k].z; d[3] = v[k].w;
     }}
     __syncthreads();
     #pragma unroll
-    for (u32 k = 0; k < 64u; k += 16u) {{
-        const u32 t = bt * 64u + r16 + k, b = bb * 64u + 4u * c4;
+    for (u32 k = 0; k < {tile}u; k += {rows}u) {{
+        const u32 t = bt * {tile}u + rw + k, b = bb * {tile}u + 4u * c4;
         if (t < a.nt && b < a.nb) {{
-            const u32 lt = r16 + k, lb = 4u * c4;
-            *reinterpret_cast<float4*>(oo + (u64)t * a.ot + b) =
-                make_float4(tile[lb][lt], tile[lb + 1u][lt], tile[lb + 2u][lt], tile[lb + 3u][lt]);
+            const u32 lt = rw + k, lb = 4u * c4;
+            {store}
         }}
     }}
 }}

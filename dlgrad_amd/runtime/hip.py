@@ -483,7 +483,9 @@ def _map(tag: str, expr: str, operands: list[Buffer], out_shape: tuple, svals: t
 
 
 _U64 = (1 << 64) - 1
+ARGMAX_COL_BLOCKS = 512            # blocks of 64 x 16 threads the column argmax aims for; more only lengthen the fold
 _permute_plans: dict = {}
+PERMUTE_DIAG = os.environ.get("DLGRAD_HIP_PERMUTE_DIAG", "1") != "0"     # diagonal tile order for power-of-two pitches
 
 
 class HIP:
@@ -837,7 +839,11 @@ class HIP:
             raise ValueError("tensor too large for 32-bit indexing")
         if I == 1:
             vec = 4 if (L % 4 == 0 and _addr(x) % 16 == 0) else 1
-            if L <= 32:
+            if L <= 32 and O >= 4096:
+                cap = 8 if L <= 8 else 16 if L <= 16 else 32
+                wide = 4 if _addr(x) % 16 == 0 else 1
+                launch(kernel(K.argmax_kernel, "rows_staged", (cap << 3) | wide), (O + 255) // 256, 256, _addr(x), out.addr, O, L)
+            elif L <= 32:
                 launch(kernel(K.argmax_kernel, "rows_thread"), (O + 255) // 256, 256, _addr(x), out.addr, O, L)
             elif L < 2048:
                 launch(kernel(K.argmax_kernel, "rows_wave", vec), (O + 3) // 4, 256, _addr(x), out.addr, O, L)
@@ -848,17 +854,16 @@ class HIP:
             raise ValueError("outer extent too large for the column argmax grid")
         vec = 4 if (I % 4 == 0 and _addr(x) % 16 == 0) else 1
         bx = (I + 64 * vec - 1) // (64 * vec)
-        # about a thousand blocks fill the chip; more chunks only lengthen the fold over them
-        chunks = 1 if L <= 256 else max(1, min(1024 // max(1, bx * O), L // 64, 65535))
+        chunks = 1 if L <= 256 else max(1, min(ARGMAX_COL_BLOCKS // max(1, bx * O), L // 64, 65535))
         chunk = (L + chunks - 1) // chunks
         chunks = (L + chunk - 1) // chunk
-        k = kernel(K.argmax_kernel, "cols_part", vec)
+        k = kernel(K.argmax_kernel, "cols_part", vec, 4, vec == 4 and O * L * I >= NT_STORE_MIN_ELEMENTS)
         if chunks == 1:
             launch(k, (bx, 1, O), (64, 16, 1), _addr(x), out.addr, 0, 0, L, I, L, 1)
             return out
         pv, pi = alloc(O * chunks * I), alloc(O * chunks * I)
         launch(k, (bx, chunks, O), (64, 16, 1), _addr(x), out.addr, pv.addr, pi.addr, L, I, chunk, 0)
-        launch(kernel(K.argmax_kernel, "cols_fin"), (O * I + 255) // 256, 256, pv.addr, pi.addr, out.addr, O, chunks, I)
+        launch(kernel(K.argmax_kernel, "cols_fin"), ((I + 63) // 64, O), (64, 16, 1), pv.addr, pi.addr, out.addr, O, chunks, I)
         return out
 
     # ---- permute ---------------------------------------------------------------------------------------------
@@ -882,9 +887,14 @@ class HIP:
             launch(kernel(K.permute_gather_kernel, vec, n >= NT_STORE_MIN_ELEMENTS), (n // vec + 1023) // 1024, 256,
                    _addr(x), out.addr, n // vec, *cshape[:3], cshape[3] // vec, *cin)
             return out
-        _, grid, args, grid4 = plan
+        _, grid, args, grid4, camped, grid128 = plan
         if grid4 and _addr(x) % 16 == 0 and out.addr % 16 == 0:
-            launch(kernel(K.permute_tiled_kernel, 4), grid4, 256, _addr(x), out.addr, *args)
+            if camped and PERMUTE_DIAG:
+                big = grid128 >= 1024
+                launch(kernel(K.permute_tiled_kernel, 4, 1, 128 if big else 64, n >= NT_STORE_MIN_ELEMENTS),
+                       grid128 if big else grid4, 256, _addr(x), out.addr, *args)
+            else:
+                launch(kernel(K.permute_tiled_kernel, 4), grid4, 256, _addr(x), out.addr, *args)
         else:
             launch(kernel(K.permute_tiled_kernel, 1), grid, 256, _addr(x), out.addr, *args)
         return out
@@ -911,7 +921,11 @@ class HIP:
         # 64 x 64 tiles with 16-byte accesses when every extent and stride is a multiple of 4
         wide = all(v % 4 == 0 for v in (nt, nb, i_st[0], i_st[1], cin[-1], o_st[0], o_st[1], cout[t]))
         grid4 = ((nb + 63) // 64) * ((nt + 63) // 64) * ext[0] * ext[1] if wide else 0
-        return "tiled", grid, args, grid4
+        # an input row pitch that is a multiple of 2 KiB puts the rows of a tile, and the tiles of
+        # one block row, on the same few memory channels: those planes are walked diagonally
+        camped = bool(wide and (cin[-1] * 4) % 2048 == 0 and (nb + 63) // 64 >= 16)
+        grid128 = ((nb + 127) // 128) * ((nt + 127) // 128) * ext[0] * ext[1] if (nt >= 128 and nb >= 128) else 0
+        return "tiled", grid, args, grid4, camped, grid128
 
     # ---- embedding and cross-entropy helpers ----------------------------------------------------------------------
     @staticmethod

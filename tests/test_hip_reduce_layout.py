@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 
 from dlgrad_amd.buffer import Buffer
+from dlgrad_amd.device import Device
 from dlgrad_amd.helpers import CustomOps
 from oracle import cref
 from tests.hip_util import check, dev, rel_err, require_gpu
@@ -91,12 +92,27 @@ def test_argmax_bit_exact_with_ties(shape):
     check(dev(y).argmax(1).numpy(), y.argmax(1).astype(np.float32).reshape(-1, 1), 0, "argmax random")
 
 
+@pytest.mark.parametrize("L", [1, 2, 7, 8, 9, 10, 16, 17, 31, 32])
+def test_argmax_of_many_short_rows(L):
+    """Row counts above 4096 with L <= 32 go through LDS, 256 rows a block; the last block is
+    ragged (row counts that are no multiple of 256, of 4, and an odd total) and a view that
+    starts 4 bytes into its block takes the narrow loads."""
+    require_gpu()
+    for R in (4096, 4099, 10001):
+        x = RNG.integers(0, 4, (R, L)).astype(np.float32)
+        want = cref.argmax(x, 1).reshape(R, 1)
+        check(dev(x).argmax(1).numpy(), want, 0, f"argmax ({R}, {L})")
+        flat = np.concatenate([np.zeros(1, np.float32), x.reshape(-1)])
+        view = Buffer(Buffer.from_numpy(flat, Device.HIP).ptr + 1, x.shape, Device.HIP)
+        check(view.argmax(1).numpy(), want, 0, f"argmax ({R}, {L}) misaligned")
+
+
 def test_argmax_never_selects_minus_inf():
     """The scan starts at (-FLT_MAX, index 0) and moves on `v > best` only (cpu_kernel.py:497-499):
     rows of -inf answer 0; every kernel variant must agree.  (NaN is left out: the reference
     compiles that comparison under -ffinite-math-only, which leaves its outcome to the compiler.)"""
     require_gpu()
-    for shape in ((6, 10), (6, 300), (6, 4096), (600, 70)):
+    for shape in ((6, 10), (6, 300), (6, 4096), (600, 70), (5000, 10)):
         x = np.full(shape, -np.inf, np.float32)
         x[1, shape[1] - 1] = -1e30
         x[2, 5] = 7.0
@@ -111,7 +127,10 @@ PERMS = [((256, 512), (1, 0)), ((8, 12, 64, 128), (0, 1, 3, 2)), ((4, 128, 8, 64
          ((2, 3, 4), (0, 2, 1)), ((2, 3, 4), (2, 0, 1)), ((2, 3, 4), (1, 0, 2)), ((2, 3, 4, 5), (0, 2, 1, 3)),
          ((2, 3, 4, 5), (0, 1, 3, 2)), ((2, 3, 4, 5), (3, 2, 1, 0)), ((2, 3, 4, 5), (1, 3, 0, 2)),
          ((16, 128, 4, 32), (0, 2, 1, 3)), ((16, 4, 128, 32), (0, 1, 3, 2)), ((16, 4, 128, 32), (0, 2, 1, 3)),
-         ((1000, 333), (1, 0)), ((3, 1, 5), (2, 1, 0)), ((5,), (0,)), ((2, 3, 4, 6), (0, 1, 2, 3))]
+         ((1000, 333), (1, 0)), ((3, 1, 5), (2, 1, 0)), ((5,), (0,)), ((2, 3, 4, 6), (0, 1, 2, 3)),
+         # row pitches that are multiples of 2 KiB: diagonal tile order, 64- and 128-wide tiles, ragged last tiles
+         ((1028, 512), (1, 0)), ((3, 1028, 512), (0, 2, 1)), ((1024, 1536), (1, 0)), ((4100, 4096), (1, 0)),
+         ((3, 1156, 4608), (0, 2, 1))]
 
 
 @pytest.mark.parametrize("shape,order", PERMS)
