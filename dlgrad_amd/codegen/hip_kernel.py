@@ -902,113 +902,168 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
     return src, name, _fmt("P", "P", "P", "I", "I")
 
 
-_ORDERED_COMPACT = r"""
-// Appends, in increasing j, the positions of [lo, hi) whose id equals `my` (and, if flags is
-// given, whose flag is set) to list[]; returns the count.  256 threads; thread t owns the
-// contiguous slice [lo + t*len, lo + (t+1)*len), counts its matches, a block-wide exclusive
-// prefix sum (wave scan + LDS) turns the counts into offsets, a second walk writes them.
-static __device__ __forceinline__ u32 collect(const float* __restrict__ idx, const u32* __restrict__ flags,
-                                              int my, u32 lo, u32 hi, u32* list, u32* wcount) {
-    const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
-    const u32 len = (hi - lo + 255u) >> 8;
-    const u32 a = min(hi, lo + tid * len), b = min(hi, a + len);
-    u32 mine = 0;
-    for (u32 j = a; j < b; ++j) mine += ((int)idx[j] == my && (flags == nullptr || flags[j] != 0u)) ? 1u : 0u;
-    u32 inc = mine;
-    #pragma unroll
-    for (int off = 1; off < 64; off <<= 1) { const u32 v = __shfl_up(inc, off, WAVE); if ((int)lane >= off) inc += v; }
-    __syncthreads();                                  // wcount may still be read by an earlier call
-    if (lane == 63u) wcount[w] = inc;
-    __syncthreads();
-    u32 pos = inc - mine;
-    for (u32 k = 0; k < w; ++k) pos += wcount[k];
-    const u32 total = wcount[0] + wcount[1] + wcount[2] + wcount[3];
-    for (u32 j = a; j < b; ++j)
-        if ((int)idx[j] == my && (flags == nullptr || flags[j] != 0u)) list[pos++] = j;
-    __syncthreads();
-    return total;
-}
-"""
-
 EMB_SEGMENT = 512          # positions per segment of the ordered scatter-add
-EMB_ORDERED_MAX = 32768    # at most 64 segments, so a merge list fits 64 entries
+EMB_ORDERED_MAX = 32768    # at most 64 segments: one lane per segment when an id's segments are listed
+
+_ORDERED_COMMON = f"""
+#define EMB_SEG {EMB_SEGMENT}u
+#define EMB_NK {EMB_SEGMENT // 64}
+// Which positions of the segment [s0, s1) hold the id `my`: bit l of hit[k] stands for position
+// s0 + 64 k + l.  All loads are issued before the first comparison; the masks are wave-uniform.
+static __device__ __forceinline__ void segment_hits(const float* __restrict__ idx, int my, u32 s0, u32 s1,
+                                                    u32 n, u32 lane, u64 (&hit)[EMB_NK]) {{
+    float v[EMB_NK];
+    #pragma unroll
+    for (u32 k = 0; k < EMB_NK; ++k) v[k] = idx[min(s0 + 64u * k + lane, n - 1u)];
+    #pragma unroll
+    for (u32 k = 0; k < EMB_NK; ++k) hit[k] = __ballot(s0 + 64u * k + lane < s1 && (int)v[k] == my);
+}}
+// How many hits lie below local position li, and how many there are in all.
+static __device__ __forceinline__ void hit_rank(const u64 (&hit)[EMB_NK], u32 li, u32& below, u32& total) {{
+    below = 0; total = 0;
+    #pragma unroll
+    for (u32 k = 0; k < EMB_NK; ++k) {{
+        total += (u32)__popcll(hit[k]);
+        if (64u * k + 64u <= li) below += (u32)__popcll(hit[k]);
+        else if (64u * k <= li) below += (u32)__popcll(hit[k] & ((1ull << (li - 64u * k)) - 1ull));
+    }}
+}}
+// Lists written by some lanes of a wavefront and read by others of the same wavefront
+static __device__ __forceinline__ void wave_lds_fence() {{
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}}
+"""
 
 
 @cache
-def embedding_backward_ordered_kernel(merge: bool, vec: int = 1) -> tuple[str, str, str]:
+def embedding_backward_ordered_kernel(stage: str, vec: int = 1) -> tuple[str, str, str]:
     """Deterministic scatter-add for up to EMB_ORDERED_MAX indices, without atomics.
 
-    The index array is cut into segments of EMB_SEGMENT positions.  Pass 1 (one block per
-    position i): the block whose position is the first occurrence of its id inside its
-    segment adds the rows of that id's occurrences in the segment, in index order, starting
-    from 0 -- exactly the order of the reference's loop (cpu_kernel.py:231-243).  If the id
-    occurs in no other segment the sum is the final table row; otherwise it goes to
-    partial[i], and the block records itself in segpos[f][segment] where f is the id's first
-    position overall (scratch: flag[n], segpos[n][64], zeroed by the launcher).  Pass 2
-    (merge=True): block f of every id that spans segments adds that id's partial rows in
-    segment order.  Ids confined to one segment are therefore bit-identical to the
-    sequential reference; ids that span segments differ from it only in where the
-    parentheses fall, and every run gives the same bits.  A hot id's work is spread over
-    segments instead of serialising on one address as atomics do.  vec=4 moves rows as
-    float4 (W % 4 == 0, aligned bases)."""
-    name = f"embedding_scatter_{'merge' if merge else 'ordered'}_v{vec}"
+    The index array is cut into segments of EMB_SEGMENT positions; one wavefront works per
+    position.  An id's positions inside one segment are found from the segment's 512 indices
+    (ballots); the lowest of them is the id's owner in that segment.
+      mark     the owner writes owner[id][segment] = position + 1 (zeroed by the launcher), so
+               the row owner[id][*] lists the segments an id occurs in.
+      ordered  the rows of an id's occurrences in a segment are added in index order starting
+               from 0 -- exactly the order of the reference's loop (cpu_kernel.py:231-243).
+               The id's m wavefronts in the segment split the columns between them (each sums
+               all m rows for its slice), so a hot id costs its wavefronts no more than a rare
+               one.  If the id occurs in no other segment the sum is the final table row,
+               otherwise it goes to partial[owner position] and flag[i] = 1 marks the owner.
+      merge    the owners of an id that spans segments add its partial rows in segment order,
+               again each for its slice of the columns.
+    Ids confined to one segment are therefore bit-identical to the sequential reference; ids
+    that span segments differ from it only in where the parentheses fall, and every run
+    gives the same bits.  vec=4 moves rows as float4 (W % 4 == 0, aligned bases)."""
+    assert stage in ("mark", "ordered", "merge")
+    name = f"embedding_scatter_{stage}" + ("" if stage == "mark" else f"_v{vec}")
     VT = "float4" if vec == 4 else "float"
     zero = "make_float4(0.f, 0.f, 0.f, 0.f)" if vec == 4 else "0.0f"
     add = ("acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;" if vec == 4 else "acc += t;")
-    if not merge:
+    add_ = add.replace("t.", "t_.").replace("+= t;", "+= t_;")
+    head = """    const u32 w = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    const u32 i = blockIdx.x * 4u + w;                          // one wavefront per position
+    if (i >= n) return;"""
+    if stage == "mark":
         body = f"""
-extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out,
-        float* __restrict__ partial, u32* __restrict__ flag, u32* __restrict__ segpos,
-        const float* __restrict__ g, const float* __restrict__ idx, u32 n, u32 W) {{
-    __shared__ u32 list[{EMB_SEGMENT}];
-    __shared__ u32 wcount[4];
-    __shared__ u32 first;
-    const u32 i = blockIdx.x, tid = threadIdx.x;
+extern "C" __global__ __launch_bounds__(256) void {name}(u32* __restrict__ owner,
+        const float* __restrict__ idx, u32 n, u32 NS) {{
+{head}
     const int my = (int)idx[i];
-    const u32 seg = i / {EMB_SEGMENT}u, s0 = seg * {EMB_SEGMENT}u, s1 = min(n, s0 + {EMB_SEGMENT}u);
-    int dup = 0;
-    for (u32 j = s0 + tid; j < i; j += 256u) dup |= ((int)idx[j] == my);
-    if (tid == 0) first = 0xFFFFFFFFu;
-    if (__syncthreads_or(dup)) return;                       // not the first of its id in this segment
-    const u32 m = collect(idx, nullptr, my, i, s1, list, wcount);
-    int other = 0;
-    u32 lowest = 0xFFFFFFFFu;
-    for (u32 j = tid; j < n; j += 256u)
-        if ((int)idx[j] == my) {{ lowest = min(lowest, j); other |= (j < s0 || j >= s1); }}
-    if (lowest != 0xFFFFFFFFu) atomicMin(&first, lowest);    // LDS atomic
-    other = __syncthreads_or(other);
-    {VT}* __restrict__ dst = reinterpret_cast<{VT}*>(other ? partial + (u64)i * W : out + (long long)my * W);
-    const u32 Wv = W / {vec}u;
-    for (u32 c = tid; c < Wv; c += 256u) {{
-        {VT} acc = {zero};
-        #pragma unroll 8
-        for (u32 q = 0; q < m; ++q) {{ const {VT} t = reinterpret_cast<const {VT}*>(g + (u64)list[q] * W)[c]; {add} }}
-        dst[c] = acc;
-    }}
-    if (other && tid == 0) {{ segpos[(u64)first * 64u + seg] = i + 1u; flag[first] = 1u; }}
+    const u32 seg = i / EMB_SEG, s0 = seg * EMB_SEG, s1 = min(n, s0 + EMB_SEG);
+    u64 hit[EMB_NK];
+    segment_hits(idx, my, s0, s1, n, lane, hit);
+    u32 below, total;
+    hit_rank(hit, i - s0, below, total);
+    if (below == 0u && lane == 0u) owner[(u64)my * NS + seg] = i + 1u;
 }}
 """
-        fmt = _fmt("P", "P", "P", "P", "P", "P", "I", "I")
+        fmt = _fmt("P", "P", "I", "I")
+    elif stage == "ordered":
+        body = f"""
+extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out,
+        float* __restrict__ partial, u32* __restrict__ flag, const u32* __restrict__ owner,
+        const float* __restrict__ g, const float* __restrict__ idx, u32 n, u32 W, u32 NS) {{
+    __shared__ u32 lists[4][{EMB_SEGMENT}];
+    __shared__ {VT} stage[4][{EMB_SEGMENT}];
+{head}
+    const int my = (int)idx[i];
+    const u32 seg = i / EMB_SEG, s0 = seg * EMB_SEG, s1 = min(n, s0 + EMB_SEG);
+    u64 hit[EMB_NK];
+    segment_hits(idx, my, s0, s1, n, lane, hit);
+    u32 r, m;                                                   // this position is the r-th of the id's m in the segment
+    hit_rank(hit, i - s0, r, m);
+    u32* __restrict__ list = lists[w];                          // the id's positions in the segment, ascending
+    u32 at = 0;
+    #pragma unroll
+    for (u32 k = 0; k < EMB_NK; ++k) {{
+        if ((hit[k] >> lane) & 1ull) list[at + (u32)__popcll(hit[k] & ((1ull << lane) - 1ull))] = s0 + 64u * k + lane;
+        at += (u32)__popcll(hit[k]);
+    }}
+    wave_lds_fence();
+    const u32 mine = lane < NS ? owner[(u64)my * NS + lane] : 0u;
+    const u64 present = __ballot(mine != 0u);                   // the segments the id occurs in (this one among them)
+    const bool other = (present & ~(1ull << seg)) != 0ull;
+    if (lane == 0u) flag[i] = (r == 0u && other) ? 1u : 0u;
+    {VT}* __restrict__ dst = reinterpret_cast<{VT}*>(other ? partial + (u64)list[0] * W : out + (long long)my * W);
+    const u32 Wv = W / {vec}u;
+    const u32 c0 = (u32)((u64)r * Wv / m), c1 = (u32)((u64)(r + 1u) * Wv / m);      // this wavefront's slice of the columns
+    // The (row, column) items of the slice are spread over all 64 lanes, so every load of a pass
+    // is in flight at once whatever m is; they meet in LDS, where each column is added in row order.
+    {VT}* __restrict__ st = stage[w];
+    const u32 cw = max(1u, EMB_SEG / m);                        // columns per pass: m * cw <= EMB_SEG items
+    for (u32 cs = c0; cs < c1; cs += cw) {{
+        const u32 cwn = min(cw, c1 - cs), items = m * cwn;
+        for (u32 t0 = 0; t0 < items; t0 += 256u) {{
+            {VT} v[4];
+            #pragma unroll
+            for (u32 u = 0; u < 4u; ++u) {{                     // loads past the end repeat the last item
+                const u32 t = min(t0 + 64u * u + lane, items - 1u), q = t / cwn, cl = t - q * cwn;
+                v[u] = reinterpret_cast<const {VT}*>(g + (u64)list[q] * W)[cs + cl];
+            }}
+            #pragma unroll
+            for (u32 u = 0; u < 4u; ++u) {{
+                const u32 t = t0 + 64u * u + lane;
+                if (t < items) {{
+                    if (m == 1u) {{ {VT} acc = {zero}; const {VT} t_ = v[u]; {add_} dst[cs + t] = acc; }}     // a single row: 0 + row, no staging
+                    else st[t] = v[u];
+                }}
+            }}
+        }}
+        if (m == 1u) continue;
+        wave_lds_fence();
+        for (u32 cl = lane; cl < cwn; cl += 64u) {{
+            {VT} acc = {zero};
+            #pragma unroll 4
+            for (u32 q = 0; q < m; ++q) {{ const {VT} t = st[q * cwn + cl]; {add} }}
+            dst[cs + cl] = acc;
+        }}
+        wave_lds_fence();                                       // the next pass overwrites the stage
+    }}
+}}
+"""
+        fmt = _fmt("P", "P", "P", "P", "P", "P", "I", "I", "I")
     else:
         body = f"""
 extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out,
-        const float* __restrict__ partial, const u32* __restrict__ flag, const u32* __restrict__ segpos,
-        const float* __restrict__ idx, u32 n, u32 W) {{
-    __shared__ u32 list[64];
-    __shared__ u32 cnt;
-    const u32 i = blockIdx.x, tid = threadIdx.x;
-    if (flag[i] == 0u) return;                               // only the first position of a spanning id works
-    if (tid < 64u) {{
-        const u32 p = segpos[(u64)i * 64u + tid];
-        const u64 bal = __ballot(p != 0u);
-        if (p != 0u) list[__popcll(bal & ((1ull << tid) - 1ull))] = p - 1u;
-        if (tid == 0) cnt = (u32)__popcll(bal);
-    }}
-    __syncthreads();
-    const u32 m = cnt;
-    {VT}* __restrict__ dst = reinterpret_cast<{VT}*>(out + (long long)(int)idx[i] * W);
+        const float* __restrict__ partial, const u32* __restrict__ flag, const u32* __restrict__ owner,
+        const float* __restrict__ idx, u32 n, u32 W, u32 NS) {{
+    __shared__ u32 lists[4][64];
+{head}
+    if (flag[i] == 0u) return;                                  // only the owners of an id that spans segments work
+    const int my = (int)idx[i];
+    const u32 p = lane < NS ? owner[(u64)my * NS + lane] : 0u;
+    const u64 present = __ballot(p != 0u);
+    u32* __restrict__ list = lists[w];                          // the id's owners, in segment order
+    if (p != 0u) list[__popcll(present & ((1ull << lane) - 1ull))] = p - 1u;
+    wave_lds_fence();
+    const u32 m = (u32)__popcll(present);
+    const u32 r = (u32)__popcll(present & ((1ull << (i / EMB_SEG)) - 1ull));        // this owner's rank among them
+    {VT}* __restrict__ dst = reinterpret_cast<{VT}*>(out + (long long)my * W);
     const u32 Wv = W / {vec}u;
-    for (u32 c = tid; c < Wv; c += 256u) {{
+    const u32 c0 = (u32)((u64)r * Wv / m), c1 = (u32)((u64)(r + 1u) * Wv / m);      // the owners split the columns
+    for (u32 c = c0 + lane; c < c1; c += 64u) {{
         {VT} acc = reinterpret_cast<const {VT}*>(partial + (u64)list[0] * W)[c];
         #pragma unroll 8
         for (u32 q = 1; q < m; ++q) {{ const {VT} t = reinterpret_cast<const {VT}*>(partial + (u64)list[q] * W)[c]; {add} }}
@@ -1016,8 +1071,8 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
     }}
 }}
 """
-        fmt = _fmt("P", "P", "P", "P", "P", "I", "I")
-    return f"{PRELUDE}{_ORDERED_COMPACT}{body}", name, fmt
+        fmt = _fmt("P", "P", "P", "P", "P", "I", "I", "I")
+    return f"{PRELUDE}{_ORDERED_COMMON}{body}", name, fmt
 
 
 @cache

@@ -937,16 +937,19 @@ class HIP:
             out = alloc(x.numel, zero=True)                    # init_with_scalar(0), cpu.py:1031
             if not n_idx:
                 return out
-            if n_idx <= K.EMB_ORDERED_MAX and EMB_ORDERED:
+            NS = (n_idx + K.EMB_SEGMENT - 1) // K.EMB_SEGMENT
+            if n_idx <= K.EMB_ORDERED_MAX and NS <= W and EMB_ORDERED:
                 # ordered, atomic-free: same bits every run (and the reference's bits for ids
                 # that stay inside one 512-position segment)
-                partial, scratch = alloc(n_idx * W), alloc(n_idx * 65, zero=True)   # flag[n] then segpos[n][64]
-                flag, segpos = scratch.addr, scratch.addr + 4 * n_idx
+                V = x.numel // W
+                partial, flag, owner = alloc(n_idx * W), alloc(n_idx), alloc(V * NS, zero=True)
                 vec = 4 if (W % 4 == 0 and not (_addr(upstream_grad) | out.addr | partial.addr) & 15) else 1
-                launch(kernel(K.embedding_backward_ordered_kernel, False, vec), n_idx, 256, out.addr, partial.addr,
-                       flag, segpos, _addr(upstream_grad), _addr(idx), n_idx, W)
-                launch(kernel(K.embedding_backward_ordered_kernel, True, vec), n_idx, 256, out.addr, partial.addr,
-                       flag, segpos, _addr(idx), n_idx, W)
+                grid = (n_idx + 3) // 4
+                launch(kernel(K.embedding_backward_ordered_kernel, "mark"), grid, 256, owner.addr, _addr(idx), n_idx, NS)
+                launch(kernel(K.embedding_backward_ordered_kernel, "ordered", vec), grid, 256, out.addr, partial.addr,
+                       flag.addr, owner.addr, _addr(upstream_grad), _addr(idx), n_idx, W, NS)
+                launch(kernel(K.embedding_backward_ordered_kernel, "merge", vec), grid, 256, out.addr, partial.addr,
+                       flag.addr, owner.addr, _addr(idx), n_idx, W, NS)
                 return out
             launch(kernel(K.embedding_backward_kernel), (n_idx + 3) // 4, 256,
                    out.addr, _addr(upstream_grad), _addr(idx), n_idx, W)

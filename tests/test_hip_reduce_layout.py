@@ -193,6 +193,61 @@ def test_embedding_scatter_add_is_deterministic_and_atomics_path_agrees(monkeypa
     np.testing.assert_allclose(atomic, want, rtol=1e-4, atol=1e-4)
 
 
+def ordered_scatter_model(V, idx, g, segment=512):
+    """The summation order of the ordered scatter-add, in float32: inside a segment of 512
+    positions an id's rows are added in index order starting from 0; an id that occurs in
+    several segments then adds those partial sums in segment order, starting from the first."""
+    out = np.zeros((V, g.shape[-1]), np.float32)
+    ids = idx.reshape(-1).astype(np.int64)
+    rows = g.reshape(ids.size, -1)
+    partials = {}
+    for s0 in range(0, ids.size, segment):
+        acc = {}
+        for j in range(s0, min(ids.size, s0 + segment)):
+            acc[ids[j]] = acc.get(ids[j], np.zeros(rows.shape[1], np.float32)) + rows[j]
+        for k, v in acc.items():
+            partials.setdefault(k, []).append(v)
+    for k, parts in partials.items():
+        total = parts[0]
+        for v in parts[1:]:
+            total = total + v
+        out[k] = total
+    return out
+
+
+@pytest.mark.parametrize("W", [4, 7, 96, 2052])
+@pytest.mark.parametrize("pattern", ["same", "pairs", "span", "zipf", "hot"])
+def test_ordered_scatter_add_has_exactly_the_documented_summation_order(pattern, W):
+    """Bit-exact against a float32 model of the order, for id patterns that exercise one id
+    filling whole segments (its 512 wavefronts split the columns, most get none), adjacent
+    pairs, ids that occur once in every segment (merge only), Zipf ids, and one hot id among
+    unique ones; W = 7 takes the 4-byte kernels, W = 2052 needs two passes over a row."""
+    require_gpu()
+    V, n = 3000, 1536 + 77
+    rng = np.random.default_rng(W)
+    ids = {"same": np.full(n, 5), "pairs": np.repeat(rng.permutation(V)[:(n + 1) // 2], 2)[:n],
+           "span": np.tile(rng.permutation(V)[:512], 4)[:n], "zipf": np.minimum(rng.zipf(1.1, n) - 1, V - 1),
+           "hot": np.where(np.arange(n) % 11 == 0, 7, rng.permutation(V)[:n])}[pattern].astype(np.float32)
+    g = rng.standard_normal((n, W), dtype=np.float32)
+    g[3] = -0.0                                                   # 0 + (-0) is +0, as in the reference's `+=`
+    got = dev(f32(V, W)).embedding(dev(ids), backward=True, upstream_grad=dev(g)).numpy()
+    if not hip.COMPILE_ONLY:
+        want = ordered_scatter_model(V, ids, g)
+        np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_scatter_add_with_more_segments_than_columns_takes_the_atomic_path():
+    require_gpu()
+    V, W, n = 40, 2, 2000                                         # 4 segments > 2 columns
+    idx = RNG.integers(0, V, n).astype(np.float32)
+    g = f32(n, W)
+    got = dev(f32(V, W)).embedding(dev(idx), backward=True, upstream_grad=dev(g)).numpy()
+    want = np.zeros((V, W))
+    np.add.at(want, idx.astype(int), g.astype(np.float64))
+    if not hip.COMPILE_ONLY:
+        np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+
+
 def test_embedding_scatter_with_heavy_collisions():
     require_gpu()
     V, W, n = 50, 64, 4096
