@@ -527,7 +527,7 @@ def argmax_kernel(mode: str, vec: int = 1, unroll: int = 4, nt: bool = False) ->
                    or, when there is one chunk, the answer
       cols_fin     folds the chunks of cols_part in order
     vec = 4: 16-byte loads along the row (rows_wave / rows_block)."""
-    name = f"argmax_{mode}" + (f"_v{vec}" if mode in ("rows_wave", "rows_block") else "")
+    name = f"argmax_{mode}" + (f"_v{vec}" + ("nt" if nt and vec == 4 else "") if mode in ("rows_wave", "rows_block") else "")
     if mode == "rows_thread":
         src = f"""{PRELUDE}
 extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
@@ -593,15 +593,17 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
         tid = "threadIdx.x" if blk else "(threadIdx.x & 63u)"
         row = "blockIdx.x" if blk else "(blockIdx.x * 4u + (threadIdx.x >> 6))"
         if vec == 4:
+            ld = "ld4_stream(p4 + " if nt else "*(p4 + "
             scan = f"""
     const float4* __restrict__ p4 = reinterpret_cast<const float4*>(p);
-    for (u32 v = {tid}; v < (L >> 2); v += {T}) {{
-        const float4 t = p4[v]; const u32 i = v << 2;
-        if (t.x > best) {{ best = t.x; bi = i; }}
-        if (t.y > best) {{ best = t.y; bi = i + 1u; }}
-        if (t.z > best) {{ best = t.z; bi = i + 2u; }}
-        if (t.w > best) {{ best = t.w; bi = i + 3u; }}
+    #define STEP4(t, v) {{ const u32 i = (v) << 2; if (t.x > best) {{ best = t.x; bi = i; }} if (t.y > best) {{ best = t.y; bi = i + 1u; }} \\
+                          if (t.z > best) {{ best = t.z; bi = i + 2u; }} if (t.w > best) {{ best = t.w; bi = i + 3u; }} }}
+    u32 v = {tid};
+    for (; v + 3u * {T} < (L >> 2); v += 4u * {T}) {{           // four loads in flight, compared in index order
+        const float4 t0 = {ld}v), t1 = {ld}v + {T}), t2 = {ld}v + 2u * {T}), t3 = {ld}v + 3u * {T});
+        STEP4(t0, v) STEP4(t1, v + {T}) STEP4(t2, v + 2u * {T}) STEP4(t3, v + 3u * {T})
     }}
+    for (; v < (L >> 2); v += {T}) {{ const float4 t = {ld}v); STEP4(t, v) }}
     if ({tid} < (L & 3u)) {{ const u32 i = (L & ~3u) + {tid}; const float v = p[i]; TAKE(best, bi, v, i) }}
 """
         else:

@@ -848,7 +848,8 @@ class HIP:
             elif L < 2048:
                 launch(kernel(K.argmax_kernel, "rows_wave", vec), (O + 3) // 4, 256, _addr(x), out.addr, O, L)
             else:
-                launch(kernel(K.argmax_kernel, "rows_block", vec), O, 256, _addr(x), out.addr, O, L)
+                launch(kernel(K.argmax_kernel, "rows_block", vec, 4, vec == 4 and O * L >= NT_STORE_MIN_ELEMENTS),
+                       O, 256, _addr(x), out.addr, O, L)
             return out
         if O > 65535:
             raise ValueError("outer extent too large for the column argmax grid")
