@@ -322,6 +322,14 @@ class Buffer:
         """self is a softmax output over the last axis; returns self * (upstream - sum(upstream * self))."""
         return self._like(self._dispatch(CustomOps.SOFTMAX_BWD, y=self, g=upstream))
 
+    def masked_softmax(self, mask: "Buffer", scale: float) -> "Buffer":
+        """softmax over the last axis of self * scale with -inf where mask > 0, one kernel."""
+        return self._like(self._dispatch(CustomOps.MASKED_SOFTMAX, x=self, mask=mask, scale=scale))
+
+    def masked_softmax_bwd(self, upstream: "Buffer", mask: "Buffer", scale: float) -> "Buffer":
+        """self is a masked_softmax output; returns the gradient of its input."""
+        return self._like(self._dispatch(CustomOps.MASKED_SOFTMAX_BWD, y=self, g=upstream, mask=mask, scale=scale))
+
     def log_softmax(self, dim: int) -> "Buffer":
         return self._unary(CustomOps.LOG_SOFTMAX, dim=dim)
 

@@ -1104,7 +1104,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 
 @cache
 def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gather: bool = False,
-                        threads: int = 256, nt: bool = False) -> tuple[str, str, str]:
+                        threads: int = 256, nt: bool = False, masked: bool = False) -> tuple[str, str, str]:
     """Row softmax / log-softmax over the contiguous last axis of an (R, L) view, replacing
     the reference's five kernels and four temporaries (tensor.py:634-669).  Same formula:
     e = exp(x - max); e / sum(e)   (or (x - max) - log(sum)).
@@ -1115,12 +1115,16 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     algorithmic minimum); rows of 50304 floats fit in 50 float4 per thread of a block.
     nval = 0 streams the row three times (for rows longer than registers hold).
     gather (log-softmax only): also writes picked[row] = out[row, (int)target[row]], the
-    ce_forward gather of cpu_kernel.py:430-441, fused."""
+    ce_forward gather of cpu_kernel.py:430-441, fused.
+    masked (register-resident forms): the row is x * scale with -inf where mask > 0, the
+    attention chain `(att * scale).masked_fill(mask, -inf).softmax()` of examples/gpt.py:51-54
+    in one pass; the mask has `mrows` rows of L and row r of x uses mask row r % mrows."""
     if not per_block:
         threads = 256
+    assert not masked or (nval and not gather)
     nt = nt and bool(nval) and vec == 4                   # streaming loads/stores: register-resident float4 form only
     name = (f"{'log_' if log else ''}softmax_rows_v{vec}_{f'blk{threads}' if per_block else 'wav'}"
-            f"{f'_r{nval}' if nval else ''}{'_g' if gather else ''}{'nt' if nt else ''}")
+            f"{f'_r{nval}' if nval else ''}{'_g' if gather else ''}{'_m' if masked else ''}{'nt' if nt else ''}")
     T = f"{threads}u" if per_block else "64u"
     NW = threads // 64
     tid = "threadIdx.x" if per_block else "(threadIdx.x & 63u)"
@@ -1131,6 +1135,17 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     def outexpr(v: str) -> str:
         return f"(({v}) - m) - ls" if log else f"expf(({v}) - m) / s"
     comps = ("x", "y", "z", "w")
+    mask4 = mask1 = ""
+    if masked:
+        sel4 = " ".join(f"v[k].{c} = mk.{c} > 0.0f ? -__builtin_inff() : v[k].{c} * scale;" for c in comps)
+        mask4 = f"""    const float4* __restrict__ pm = reinterpret_cast<const float4*>(mask + (u64)(row % mrows) * L);
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < nv) {{ const float4 mk = pm[c]; {sel4} }} }}
+"""
+        mask1 = f"""    const float* __restrict__ pm = mask + (u64)(row % mrows) * L;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < L) v[k] = pm[c] > 0.0f ? -__builtin_inff() : v[k] * scale; }}
+"""
     if nval and vec == 4:
         body = f"""
     const float4* __restrict__ p = reinterpret_cast<const float4*>(x + (u64)row * L);
@@ -1139,7 +1154,7 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     float4 v[{nval}];
     #pragma unroll
     for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < nv) v[k] = {'ld4_stream(p + c)' if nt else 'p[c]'}; }}
-    float m = NEG_FLT_MAX;
+{mask4}    float m = NEG_FLT_MAX;
     #pragma unroll
     for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < nv)
         m = fmaxf(fmaxf(m, fmaxf(v[k].x, v[k].y)), fmaxf(v[k].z, v[k].w));
@@ -1166,7 +1181,7 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     float v[{nval}];
     #pragma unroll
     for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < L) v[k] = p[c]; }}
-    float m = NEG_FLT_MAX;
+{mask1}    float m = NEG_FLT_MAX;
     #pragma unroll
     for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < L) m = fmaxf(m, v[k]);
     m = {red_max};
@@ -1214,6 +1229,8 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     if ({tid} == 0) {{ const float* __restrict__ xr = x + (u64)row * L; picked[row] = (xr[(int)target[row]] - m) - ls; }}
 """
     extra_params = ", const float* __restrict__ target, float* __restrict__ picked" if gather else ""
+    if masked:
+        extra_params = ", const float* __restrict__ mask, u32 mrows, float scale"
     src = f"""{PRELUDE}
 static __device__ __forceinline__ float block_max(float v, float* sm) {{
     v = wave_max(v);
@@ -1243,7 +1260,7 @@ extern "C" __global__ __launch_bounds__({threads}) void {name}(const float* __re
 {body}
 }}
 """
-    return src, name, _fmt("P", "P", "I", "I", *(("P", "P") if gather else ()))
+    return src, name, _fmt("P", "P", "I", "I", *(("P", "P") if gather else ("P", "I", "f") if masked else ()))
 
 
 def softmax_plan(L: int, vec: int) -> tuple[bool, int, int]:
@@ -1263,25 +1280,32 @@ def softmax_plan(L: int, vec: int) -> tuple[bool, int, int]:
 
 
 @cache
-def softmax_bwd_rows_kernel(vec: int, nval: int, nt: bool = False) -> tuple[str, str, str]:
+def softmax_bwd_rows_kernel(vec: int, nval: int, nt: bool = False, masked: bool = False) -> tuple[str, str, str]:
     """dx = y * (g - sum(g * y)) along the contiguous last axis: the backward of a row softmax
     with output y and upstream gradient g, one wavefront per row, both rows held in registers
     (12 B per element instead of the ~36 of the four element-wise and one reduction kernels the
-    expression otherwise takes).  Rows of up to 64 * nval items (float4 or float)."""
+    expression otherwise takes).  Rows of up to 64 * nval items (float4 or float).
+    masked: the backward of the scaled, masked form: dx = (mask > 0 ? 0 : y * (g - s)) * scale,
+    which is what the backward nodes of softmax, masked_fill and the scalar multiply produce."""
     T, comps, nvx = _rms_lanes(vec)
     nt = nt and vec == 4
-    name = f"softmax_bwd_rows_v{vec}_r{nval}{'nt' if nt else ''}"
+    name = f"softmax_bwd_rows_v{vec}_r{nval}{'_m' if masked else ''}{'nt' if nt else ''}"
     ld = (lambda p: f"ld4_stream({p} + c)") if nt else (lambda p: f"{p}[c]")
     dot = " + ".join(f"g[k]{c} * y[k]{c}" for c in comps)
-    outs = "".join(f"            o{c} = y[k]{c} * (g[k]{c} - s);\n" for c in comps)
+    if masked:
+        outs = f"            const {T} mk = pm[c];\n" + "".join(
+            f"            o{c} = (mk{c} > 0.0f ? 0.0f : y[k]{c} * (g[k]{c} - s)) * scale;\n" for c in comps)
+    else:
+        outs = "".join(f"            o{c} = y[k]{c} * (g[k]{c} - s);\n" for c in comps)
     st = ("{ const v4f ov = {o.x, o.y, o.z, o.w}; __builtin_nontemporal_store(ov, reinterpret_cast<v4f*>(q) + c); }" if nt
           else "q[c] = o;")
     src = f"""{PRELUDE}
 extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ yp,
-        const float* __restrict__ gp, float* __restrict__ dx, u32 R, u32 L) {{
+        const float* __restrict__ gp, float* __restrict__ dx, u32 R, u32 L{", const float* __restrict__ mask, u32 mrows, float scale" if masked else ""}) {{
     const u32 lane = threadIdx.x & 63u;
     const u32 row = blockIdx.x * 4u + (threadIdx.x >> 6);
     if (row >= R) return;
+    {f"const {T}* __restrict__ pm = reinterpret_cast<const {T}*>(mask + (u64)(row % mrows) * L);" if masked else ""}
     const {T}* __restrict__ py = reinterpret_cast<const {T}*>(yp + (u64)row * L);
     const {T}* __restrict__ pg = reinterpret_cast<const {T}*>(gp + (u64)row * L);
     {T}* __restrict__ q = reinterpret_cast<{T}*>(dx + (u64)row * L);
@@ -1304,7 +1328,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
     }}
 }}
 """
-    return src, name, _fmt("P", "P", "P", "I", "I")
+    return src, name, _fmt("P", "P", "P", "I", "I", *(("P", "I", "f") if masked else ()))
 
 
 # =====================================================================================

@@ -66,6 +66,8 @@ class CustomOps(Enum):
     # from max/sub/exp/sum/div: tensor.py:634-669, ops.py:337-370)
     SOFTMAX = auto()
     SOFTMAX_BWD = auto()            # y * (g - sum(g * y)) over the last axis, one kernel
+    MASKED_SOFTMAX = auto()         # softmax(masked_fill(x * scale, mask, -inf)) over the last axis, one kernel
+    MASKED_SOFTMAX_BWD = auto()     # its backward, one kernel
     LOG_SOFTMAX = auto()
     LOG_SOFTMAX_GATHER = auto()     # log-softmax rows + the ce_forward gather, one kernel
     CE_GRAD = auto()                # ((exp(lsm) - onehot) * upstream) / N, one kernel

@@ -355,6 +355,31 @@ class Softmax(OP):
         return (gy - self.out * gy.sum(dim=self.out.ndim - 1, keepdim=True),)
 
 
+def use_fused_masked_softmax(x, mask, dim: int) -> bool:
+    if not (use_fused(x, dim) and mask.device is Device.HIP):
+        return False
+    from dlgrad_amd.runtime.hip import HIP
+    return HIP.masked_softmax_fits(x.data, mask.data)
+
+
+class MaskedSoftmax(OP):
+    """softmax(masked_fill(x * scale, mask, -inf)) along the last axis as one forward and one
+    backward kernel; the values and gradients are those of the three-op chain."""
+
+    def forward(self, x: Buffer, mask: Buffer, scale: float) -> Buffer:
+        self.mask, self.scale = mask, scale
+        self.out = x.masked_softmax(mask, scale)
+        return self.out
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        from dlgrad_amd.runtime.hip import HIP
+        if HIP.softmax_bwd_fits(self.out, upstream_grad):
+            return self.out.masked_softmax_bwd(upstream_grad, self.mask, self.scale), None
+        gy = upstream_grad * self.out
+        g = gy - self.out * gy.sum(dim=self.out.ndim - 1, keepdim=True)
+        return Buffer.masked_fill(x=g, mask=self.mask, val=0.0) * self.scale, None
+
+
 def use_fused_rmsnorm(x, weight) -> bool:
     if not (FUSED and x.device is Device.HIP):
         return False

@@ -1028,6 +1028,67 @@ class HIP:
         return dx
 
     @staticmethod
+    def _mask_rows(x: Buffer, mask: Buffer) -> int:
+        """How many rows of x.shape[-1] floats the mask has if it lines up with the trailing dims
+        of a contiguous x (row r of x then uses mask row r % rows), else 0."""
+        if x.ndim == 0 or mask.is_host_scalar or not mask.numel:
+            return 0
+        L = x.shape[-1]
+        mshape = tuple(mask.shape)
+        while len(mshape) > 1 and mshape[0] == 1:
+            mshape = mshape[1:]
+        if len(mshape) > x.ndim or mshape != tuple(x.shape[x.ndim - len(mshape):]):
+            return 0
+        if tuple(mask.stride) != tuple(calculate_stride(mask.shape)):
+            return 0
+        return mask.numel // L
+
+    @staticmethod
+    def masked_softmax_fits(x: Buffer, mask: Buffer) -> bool:
+        """The fused scaled, masked softmax takes rows that the register-resident softmax and its
+        one-wavefront backward hold, and a contiguous mask shaped like the trailing dims of x."""
+        if not x.numel or not HIP._mask_rows(x, mask):
+            return False
+        L = x.shape[-1]
+        vec = HIP._rms_vec(L, _addr(x), _addr(mask))
+        return K.softmax_plan(L, vec)[1] > 0 and K.rmsnorm_plan(L, vec) > 0
+
+    @staticmethod
+    @dispatcher.register(CustomOps.MASKED_SOFTMAX, Device.HIP)
+    def masked_softmax(x: Buffer, mask: Buffer, scale: float) -> DevicePtr:
+        """softmax over the last axis of x * scale with -inf where mask > 0: the three kernels of
+        `(att * scale).masked_fill(mask, -inf).softmax(dim)` (examples/gpt.py:51-54) as one,
+        same arithmetic in the same order."""
+        L = x.shape[-1]
+        R = x.numel // L
+        mrows = HIP._mask_rows(x, mask)
+        out = alloc(x.numel)
+        vec = HIP._rms_vec(L, _addr(x), _addr(mask), out.addr)
+        blk, nval, threads = K.softmax_plan(L, vec)
+        if not mrows or not nval:
+            raise ValueError(f"fused masked softmax does not take x {x.shape} with mask {mask.shape}")
+        k = kernel(K.softmax_rows_kernel, False, vec, blk, nval, False, threads, x.numel >= NT_STORE_MIN_ELEMENTS, True)
+        launch(k, R if blk else (R + 3) // 4, threads, _addr(x), out.addr, R, L, _addr(mask), mrows, float(scale))
+        return out
+
+    @staticmethod
+    @dispatcher.register(CustomOps.MASKED_SOFTMAX_BWD, Device.HIP)
+    def masked_softmax_bwd(y: Buffer, g: Buffer, mask: Buffer, scale: float) -> DevicePtr:
+        """(mask > 0 ? 0 : y * (g - sum(g * y))) * scale: the backward nodes of softmax,
+        masked_fill and the multiplication by a scalar in one kernel."""
+        L = y.shape[-1]
+        R = y.numel // L
+        mrows = HIP._mask_rows(y, mask)
+        dx = alloc(y.numel)
+        vec = HIP._rms_vec(L, _addr(y), _addr(g), _addr(mask), dx.addr)
+        nval = K.rmsnorm_plan(L, vec)
+        if not mrows or nval == 0 or g.numel != y.numel or g.is_host_scalar:
+            raise ValueError(f"fused masked softmax backward does not take y {y.shape} with mask {mask.shape}")
+        launch(kernel(K.softmax_bwd_rows_kernel, vec, nval, y.numel >= NT_STORE_MIN_ELEMENTS, True), (R + 3) // 4, 256,
+               _addr(y), _addr(g), dx.addr, R, L, _addr(mask), mrows, float(scale))
+        return dx
+
+    @staticmethod
     @dispatcher.register(CustomOps.LOG_SOFTMAX, Device.HIP)
     def log_softmax(x: Buffer, dim: int) -> DevicePtr:
         return HIP._softmax(x, dim, True)

@@ -257,6 +257,15 @@ class Tensor:
         e = (self - m).exp()
         return e / e.sum(dim=dim, keepdim=True)
 
+    def masked_softmax(self, mask: "Tensor", scale: float = 1.0, dim: int = -1) -> "Tensor":
+        """`(self * scale).masked_fill(mask, -inf).softmax(dim)`, the attention chain of
+        examples/gpt.py:51-54.  On the hip device, along the last axis, with a mask shaped like
+        the trailing dims, this is one kernel forward and one backward (the scores are read and
+        the probabilities written once); anywhere else it is that chain, op by op."""
+        if ops.use_fused_masked_softmax(self, mask, dim):
+            return ops.MaskedSoftmax.execute(self, mask, scale=scale)
+        return (self * scale).masked_fill(mask, float("-inf")).softmax(dim=dim)
+
     def log_softmax(self, dim: int = 1) -> "Tensor":
         m = self - self.max(dim=dim, keepdim=True)
         return m - m.exp().sum(dim=dim, keepdim=True).log()

@@ -64,9 +64,8 @@ class CausalSelfAttention:
                 cache.write(layer, k_lin, v_lin, 0)
             k = k_lin.reshape(split).transpose(1, 2)
             v = v_lin.reshape(split).transpose(1, 2)
-            att = (q @ k.transpose(2, 3)) * self.scale               # (B, h, T, T)
-            att = att.masked_fill(causal_mask(T, x.device), float("-inf"))
-            att = att.softmax(dim=3)
+            # (att * scale).masked_fill(mask, -inf).softmax(dim=3), one kernel on the hip device
+            att = (q @ k.transpose(2, 3)).masked_softmax(causal_mask(T, x.device), self.scale, dim=3)   # (B, h, T, T)
         y = (att @ v).transpose(1, 2).reshape((B, T, C))
         return self.c_proj(y)
 
@@ -245,8 +244,7 @@ class StaticDecoder:
         self.cache.k[layer].data.row_store_(attn.k_proj(x).data, self.slot.data)
         self.cache.v[layer].data.row_store_(attn.v_proj(x).data, self.slot.data)
         k, v = self.cache.view(layer, T, attn.n_head)                                       # (1, h, T, d)
-        att = (q @ k.transpose(2, 3)) * attn.scale                                          # (1, h, 1, T)
-        att = att.masked_fill(hidden, float("-inf")).softmax(dim=3)
+        att = (q @ k.transpose(2, 3)).masked_softmax(hidden, attn.scale, dim=3)              # (1, h, 1, T)
         return attn.c_proj((att @ v).transpose(1, 2).reshape((1, 1, C)))
 
     def step(self) -> None:

@@ -13,7 +13,7 @@ import pytest
 
 from dlgrad_amd import Tensor
 from dlgrad_amd.runtime import hip
-from oracle import cref
+from oracle import cpu_runtime, cref  # noqa: F401  (registers the CPU device the chain is checked against)
 from tests.hip_util import check, dev, require_gpu
 
 pytestmark = pytest.mark.gpu
@@ -120,3 +120,68 @@ def test_fused_softmax_backward_rows(R, L):
     gy = cref.binary("mul", g[sl], yh[sl])                         # the four-kernel form of ops.Softmax.backward
     ref = cref.binary("sub", gy, cref.binary("mul", yh[sl], cref.reduce("sum", gy, 1)[:, None]))
     assert np.abs(dx[sl] - ref).max() <= 1e-5 * np.abs(ref).max()
+
+
+MASKED_CASES = [((2, 4, 128, 128), (128, 128)), ((8, 12, 1024, 1024), (1024, 1024)), ((3, 5, 100, 100), (100, 100)),
+                ((2, 3, 7, 7), (7, 7)), ((1, 4, 1, 128), (1, 1, 1, 128)), ((6, 130), (6, 130)), ((5, 33), (33,))]
+
+
+@pytest.mark.parametrize("xs,ms", MASKED_CASES)
+def test_fused_masked_softmax_is_the_three_op_chain(xs, ms, monkeypatch):
+    """`(x * scale).masked_fill(mask, -inf).softmax(last)` as one kernel, and its backward as one
+    kernel: values and input gradients bit-identical to the chain of kernels they replace
+    (same arithmetic in the same order), masked probabilities exactly 0 with gradient +0,
+    every row summing to 1; a slice is also held against float64 (2e-6)."""
+    require_gpu()
+    from dlgrad_amd import ops
+    rng = np.random.default_rng(60)
+    x = rng.standard_normal(xs, dtype=np.float32) * 3
+    g = rng.standard_normal(xs, dtype=np.float32)
+    mask = (rng.random(ms) < 0.4).astype(np.float32)
+    mask.reshape(-1, ms[-1])[:, 0] = 0                      # no row is masked entirely
+    scale, dim = 0.125 * 1.37, len(xs) - 1
+
+    def run(fused):
+        monkeypatch.setattr(ops, "use_fused_masked_softmax", (lambda *a: False) if not fused else ops.use_fused_masked_softmax)
+        t = Tensor(x, device="hip", requires_grad=True)
+        y = t.masked_softmax(Tensor(mask, device="hip"), scale, dim=dim)
+        node = type(y._ctx).__name__
+        (y * Tensor(g, device="hip")).sum().backward()
+        return y, t.grad, node
+
+    (y1, g1, n1), (y0, g0, n0) = run(True), run(False)
+    assert n1 == "MaskedSoftmax" and n0 != "MaskedSoftmax"
+    if hip.COMPILE_ONLY:
+        return
+    y1, g1, y0, g0 = y1.numpy(), g1.numpy(), y0.numpy(), g0.numpy()
+    np.testing.assert_array_equal(y1.view(np.uint32), y0.view(np.uint32))
+    np.testing.assert_array_equal(g1.view(np.uint32), g0.view(np.uint32))
+    full = np.broadcast_to(mask.reshape((1,) * (len(xs) - mask.ndim) + mask.shape), xs) > 0
+    assert not y1[full].any() and not g1[full].any() and not np.signbit(g1[full]).any()
+    assert np.abs(y1.sum(-1, dtype=np.float64) - 1).max() <= 1e-5
+    sl = (slice(0, 1),) * (len(xs) - 2) + (slice(0, 64),)
+    z = np.where(full[sl], -np.inf, x[sl].astype(np.float64) * np.float32(scale))
+    e = np.exp(z - z.max(-1, keepdims=True))
+    want = e / e.sum(-1, keepdims=True)
+    assert np.abs(y1[sl] - want).max() <= 2e-6
+    gw = want * (g[sl] - (g[sl] * want).sum(-1, keepdims=True)) * scale
+    assert np.abs(g1[sl] - gw).max() <= 2e-6 * max(1.0, np.abs(gw).max())
+
+
+def test_masked_softmax_falls_back_to_the_chain_where_the_kernel_does_not_fit():
+    """Rows too long for registers, a mask that does not line up with the trailing dims, or
+    another axis: the op-by-op chain runs, with the same result as on the CPU oracle (1e-6)."""
+    require_gpu()
+    from dlgrad_amd import ops
+    rng = np.random.default_rng(61)
+    for xs, ms, dim in (((2, 70000), (70000,), 1), ((4, 6, 8), (4, 1, 8), 2), ((4, 8), (4, 8), 0)):
+        x = rng.standard_normal(xs, dtype=np.float32)
+        mask = (rng.random(ms) < 0.3).astype(np.float32)
+        mask[..., 0] = 0
+        if dim == 0:
+            mask[0] = 0
+        t, m = Tensor(x, device="hip"), Tensor(mask, device="hip")
+        assert not ops.use_fused_masked_softmax(t, m, dim)
+        got = t.masked_softmax(m, 0.5, dim=dim).numpy()
+        want = Tensor(x).masked_softmax(Tensor(mask), 0.5, dim=dim).numpy()
+        check(got, want, 1e-6, f"masked softmax chain {xs} {ms} dim {dim}")
