@@ -666,7 +666,7 @@ def main() -> None:
                "per_op": {k: {"GBps": round(v["GBps"], 1), "frac_hbm": round(v["frac_hbm"], 3),
                               "ms": round(v["ms"], 4)} for k, v in r["per_op"].items()}}
         if not args.no_cpu:
-            out["cpu_baseline"] = cpu_c2(4096, 4096)
+            out["cpu_baseline"] = cpu_c2(8192, 8192, reps=3)
         if not args.no_extra:
             extra = {}
             for (r2, c2) in ((4096, 4096), (1024, 1024)):
