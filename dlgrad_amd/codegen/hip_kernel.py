@@ -515,7 +515,7 @@ static __device__ __forceinline__ void wave_argmax(float& best, u32& bi) {
 
 
 @cache
-def argmax_kernel(mode: str, vec: int = 1, unroll: int = 4, nt: bool = False) -> tuple[str, str, str]:
+def argmax_kernel(mode: str, vec: int = 1, unroll: int = 4, nt: bool = False, cap: int = 32) -> tuple[str, str, str]:
     """Index (as float) of the first maximum along L of an (O, L, I) view
     (cpu_kernel.py:459-517: strict '>', start value -FLT_MAX at index 0).
       rows_thread  I == 1, short rows, few of them: one thread per row
@@ -526,7 +526,8 @@ def argmax_kernel(mode: str, vec: int = 1, unroll: int = 4, nt: bool = False) ->
                    every 16th row, LDS joins them; writes the chunk's (value, index) per column,
                    or, when there is one chunk, the answer
       cols_fin     folds the chunks of cols_part in order
-    vec = 4: 16-byte loads along the row (rows_wave / rows_block)."""
+    vec = 4: 16-byte loads along the row (rows_staged / rows_wave / rows_block) or across four
+    columns (cols_part); unroll: rows in flight per thread (cols_part); nt: streaming loads."""
     name = f"argmax_{mode}" + (f"_v{vec}" + ("nt" if nt and vec == 4 else "") if mode in ("rows_wave", "rows_block") else "")
     if mode == "rows_thread":
         src = f"""{PRELUDE}
@@ -542,8 +543,8 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 """
         return src, name, _fmt("P", "P", "I", "I")
     if mode == "rows_staged":
-        # vec is (cap << 3) | width: rows of at most cap floats, loads of `width` floats
-        cap, width = vec >> 3, vec & 7
+        # rows of at most cap floats (sizes the LDS stage), loads of vec floats
+        width = vec
         name = f"argmax_rows_staged_c{cap}_v{width}"
         if width == 4:
             fill = """

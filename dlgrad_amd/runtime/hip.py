@@ -842,7 +842,7 @@ class HIP:
             if L <= 32 and O >= 4096:
                 cap = 8 if L <= 8 else 16 if L <= 16 else 32
                 wide = 4 if _addr(x) % 16 == 0 else 1
-                launch(kernel(K.argmax_kernel, "rows_staged", (cap << 3) | wide), (O + 255) // 256, 256, _addr(x), out.addr, O, L)
+                launch(kernel(K.argmax_kernel, "rows_staged", wide, 4, False, cap), (O + 255) // 256, 256, _addr(x), out.addr, O, L)
             elif L <= 32:
                 launch(kernel(K.argmax_kernel, "rows_thread"), (O + 255) // 256, 256, _addr(x), out.addr, O, L)
             elif L < 2048:
