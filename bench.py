@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hip kernel backend on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|matmul|gpt|mlp] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|matmul|gpt|mlp|gpt-large|components] [--no-extra]
 
 Prints ONE JSON line.  A "step" is one pass of the workload over one batch of synthetic,
 seeded input that is already resident in HBM when the timed region starts.
@@ -16,6 +16,11 @@ seeded input that is already resident in HBM when the timed region starts.
   mlp                784-64-10 MLP, batch 128: forward + backward + SGD step.  value = samples/s.
   gpt-large          scaled GPT (vocab 50304, block 1024, 12 layers, 12 heads, n_embd 768, batch 8),
                      Zipf(1.1) ids: forward + backward + Adam step.  value = tokens/s.
+
+  components         the kernel classes c2 does not reach, at sizes beyond the caches: transposes, head
+                     permutes, argmax, selects, and the scaled GPT's embedding gather / scatter-add,
+                     softmax and cross-entropy shapes.  value = algorithmic GB/s over all of them;
+                     `roofline` names the one that takes longest.
 
 Unless --no-extra is given, the default run also reports the matmul sweep, the GPT step and
 the 4096^2 / 1024^2 suites under "extra", so one run carries every headline figure.
@@ -625,7 +630,7 @@ def main() -> None:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=["c2", "matmul", "gpt", "mlp", "gpt-large"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "matmul", "gpt", "mlp", "gpt-large", "components"])
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
@@ -733,6 +738,21 @@ def main() -> None:
                "roofline": step_roofline(g["train_TFLOPs_est"] * 1e12 * g["train_step_ms"] * 1e-3, g["train_step_ms"],
                                          "whole step against the fp32 MFMA peak; 6 x 124 M matmul parameters x 8192 tokens "
                                          "(attention products not counted)")}
+    elif args.workload == "components":
+        # the kernel classes C2 does not reach, each at a size beyond the caches: C5's embedding, softmax
+        # and cross-entropy shapes, transposes, permutes, argmax, selects
+        comp = {**run_c5(args.steps, args.warmup), **run_layout_and_select(args.steps, args.warmup)}
+        total_ms = sum(v["ms"] for v in comp.values())
+        total_bytes = sum(v["GBps"] * v["ms"] * 1e6 for v in comp.values())
+        worst = max(comp, key=lambda k: comp[k]["ms"])
+        out = {"metric": "elementwise/reduce HBM GB/s (1 GPU)", "value": total_bytes / total_ms / 1e6, "unit": "GB/s",
+               **base, "ms_per_step": total_ms,
+               "config": {"workload": f"{len(comp)} layout, select, argmax, embedding, softmax and cross-entropy kernels at the "
+                                      "scaled-GPT shapes, one launch each per step; value = algorithmic bytes / summed kernel time"},
+               "roofline": {"bound": "hbm", "achieved": comp[worst]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                            "frac": comp[worst]["GBps"] / HBM_PEAK_GBS, "traffic": None, "kernel": worst,
+                            "avg_launch_ms": comp[worst]["ms"]},
+               "per_op": comp}
     else:
         r = run_mlp(args.steps, args.warmup)
         out = {"metric": "MLP 784-64-10 step samples/s (1 GPU)", "value": r["samples_per_s"], "unit": "samples/s",
