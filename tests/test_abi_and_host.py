@@ -247,3 +247,33 @@ def test_pinned_staging_uploads_without_a_wait_and_inside_a_captured_graph():
     import gc
     gc.collect()
     assert not hip._pinned                                        # the page-locked block went back
+
+
+def _run_bench(*args):
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, DLGRAD_HIP_COMPILE_ONLY="1")
+    return subprocess.run([sys.executable, os.path.join(root, "bench.py"), *args], capture_output=True, text=True,
+                          env=env, cwd=root, timeout=600)
+
+
+def test_bench_refuses_more_than_one_gpu_with_a_message():
+    r = _run_bench("--gpus", "2")
+    assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_bench_prints_one_json_line_with_the_contract_keys():
+    """Compile-only mode runs the whole host side of a workload without a device (timings are
+    placeholders): the line must parse and carry every key the harness reads."""
+    import json
+    r = _run_bench("--workload", "mlp", "--steps", "2", "--warmup", "1", "--no-cpu")
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [ln for ln in r.stdout.splitlines() if ln.startswith("{")]
+    assert len(lines) == 1
+    out = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline"):
+        assert key in out, key
+    assert out["n_gpus"] == 1 and out["steps"] == 2 and out["warmup"] == 1 and out["vs_baseline"] is None
+    assert out["dtype"] == "f32" and out["data"] == "synthetic" and "workload" in out["config"]
