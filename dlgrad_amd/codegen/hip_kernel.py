@@ -1811,6 +1811,9 @@ MATMUL_CONFIGS = {
     "128x128": (2, 2, 2, 2, 32),
     "128x96": (4, 1, 1, 3, 32),
     "128x64": (4, 1, 1, 2, 32),
+    "128x128w16": (4, 4, 1, 1, 32),     # sixteen waves of 32x32: outputs of about 256 tiles (2048^2), where a CU holds
+    "128x64w8": (4, 2, 1, 1, 32),       # one block and only its own waves can overlap loads with MFMA (2048^3: 115
+    "64x128w8": (2, 4, 1, 1, 32),       # against 97 TFLOP/s for four waves of 64x64); the eight-wave halves for narrow outputs
     "64x64": (2, 2, 1, 1, 16),
     "64x64k64": (2, 2, 1, 1, 64),       # same tile, K walked 64 at a time: fewer barriers when one block per CU
     "32x32": (1, 1, 1, 1, 16),          # has nobody to overlap with (1024^3: 73 against 62 TFLOP/s)
@@ -1827,7 +1830,7 @@ def matmul_tile_shape(tile: str) -> tuple[int, int, int]:
 # picks a tile for a shape nobody has timed
 MATMUL_TILE_MODEL = {
     "256x256": (1.00, 1), "256x128": (0.99, 2), "128x256": (0.95, 1), "192x192": (0.93, 2), "128x192": (0.88, 1),
-    "128x128": (0.94, 2), "128x96": (0.86, 3), "128x64": (0.85, 4), "64x64": (0.74, 8), "32x32": (0.60, 8),
+    "128x128": (0.94, 2), "128x128w16": (0.86, 1), "128x96": (0.86, 3), "128x64": (0.85, 4), "64x64": (0.74, 8), "32x32": (0.60, 8),
 }
 
 
