@@ -135,3 +135,72 @@ def test_zero_sized_tensors_go_through_every_op_family():
     assert z.matmul(w).numpy().shape == (0, 3)
     e = dev(np.ones((4, 0), np.float32)).matmul(dev(np.ones((0, 6), np.float32))).numpy()     # empty inner dim: zeros
     assert e.shape == (4, 6) and not e.any()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_embedding_gathers_and_ordered_scatter_adds(seed):
+    """Random table sizes, row widths (4-byte and 16-byte kernels), index counts on either side of
+    the 512-position segment size and id distributions from all-distinct to one id everywhere:
+    the gather is bit-exact, the scatter-add bit-exact against the float32 model of its summation
+    order (or, where it takes the atomic path, 1e-4 against float64)."""
+    require_gpu()
+    from tests.test_hip_reduce_layout import ordered_scatter_model
+    rng = np.random.default_rng(5000 + seed)
+    for _ in range(6):
+        V = int(rng.choice([1, 3, 50, 700, 5000]))
+        W = int(rng.choice([1, 4, 6, 32, 100, 260]))
+        n = int(rng.choice([1, 5, 511, 512, 513, 1300, 2100]))
+        kind = rng.choice(["uniform", "zipf", "same", "few"])
+        ids = {"uniform": rng.integers(0, V, n), "zipf": np.minimum(rng.zipf(1.2, n) - 1, V - 1),
+               "same": np.full(n, V - 1), "few": rng.integers(0, min(V, 3), n)}[kind].astype(np.float32)
+        table = rng.standard_normal((V, W), dtype=np.float32)
+        g = rng.standard_normal((n, W), dtype=np.float32)
+        t = dev(table)
+        check(t.embedding(dev(ids)).numpy(), table[ids.astype(np.int64)], 0, f"gather V{V} W{W} n{n} {kind}")
+        got = t.embedding(dev(ids), backward=True, upstream_grad=dev(g)).numpy()
+        if hip.COMPILE_ONLY:
+            continue
+        segments = (n + 511) // 512
+        if segments <= W:
+            want = ordered_scatter_model(V, ids, g)
+            assert (got.view(np.uint32) == want.view(np.uint32)).all(), f"scatter V{V} W{W} n{n} {kind}"
+        else:
+            want = np.zeros((V, W))
+            np.add.at(want, ids.astype(np.int64), g.astype(np.float64))
+            assert np.abs(got - want).max() <= 1e-4 * max(1.0, np.abs(want).max()), f"atomic scatter V{V} W{W} n{n} {kind}"
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_masked_softmax_equals_its_chain(seed):
+    """Random ranks, row lengths (16-byte and 4-byte kernels, one wavefront or a block per row),
+    mask shapes that cover one row, the trailing two dims or the whole tensor, and scales: the
+    fused forward and backward kernels give the bits of the mul / masked_fill / softmax chain."""
+    require_gpu()
+    from dlgrad_amd import Tensor, ops
+    rng = np.random.default_rng(6000 + seed)
+    for _ in range(6):
+        rank = int(rng.integers(2, 5))
+        L = int(rng.choice([1, 3, 8, 33, 64, 100, 256, 1000, 4096]))     # up to what the one-wavefront backward holds
+        lead = tuple(int(rng.choice([1, 2, 3, 5])) for _ in range(rank - 1))
+        xs = lead + (L,)
+        keep = int(rng.integers(1, rank + 1))                      # the mask spans the last `keep` dims
+        ms = xs[rank - keep:]
+        x = rng.standard_normal(xs, dtype=np.float32) * 4
+        g = rng.standard_normal(xs, dtype=np.float32)
+        mask = (rng.random(ms) < 0.5).astype(np.float32)
+        mask.reshape(-1, L)[:, int(rng.integers(0, L))] = 0       # every row keeps an entry
+        scale = float(rng.choice([1.0, 0.125, 0.3]))
+        outs = []
+        for fused in (True, False):
+            t, m = Tensor(x, device="hip", requires_grad=True), Tensor(mask, device="hip")
+            if fused:
+                assert ops.use_fused_masked_softmax(t, m, rank - 1), (xs, ms)
+                y = t.masked_softmax(m, scale, dim=rank - 1)
+            else:
+                y = (t * scale).masked_fill(m, float("-inf")).softmax(dim=rank - 1)
+            (y * Tensor(g, device="hip")).sum().backward()
+            outs.append((y.numpy(), t.grad.numpy()))
+        if hip.COMPILE_ONLY:
+            continue
+        assert (outs[0][0].view(np.uint32) == outs[1][0].view(np.uint32)).all(), f"forward {xs} {ms} {scale}"
+        assert (outs[0][1].view(np.uint32) == outs[1][1].view(np.uint32)).all(), f"backward {xs} {ms} {scale}"
