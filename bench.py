@@ -249,7 +249,8 @@ def cpu_matmul(n: int = 512) -> dict:
 def run_c5(steps: int, warmup: int) -> dict:
     """Embedding gather / scatter-add on a 50304x768 table with 8192 Zipf(1.1) ids, fused softmax
     on (98304, 1024), fused cross-entropy forward and backward on (8192, 50304).  GB/s are
-    algorithmic: gather 4n + 8nW; scatter 4VW + 4nW + 4n; softmax, CE fwd and CE bwd 8 B/elt."""
+    algorithmic: gather 4n + 8nW; scatter 4VW + 4nW + 4n; softmax, CE fwd and CE bwd 8 B/elt; the scaled,
+    causally masked attention softmax 8 B/elt forward and 12 B/elt backward."""
     Tensor, _, Buffer, Device, hip = _imports()
     lib = hip.lib()
     rng = np.random.default_rng(5)
@@ -263,10 +264,15 @@ def run_c5(steps: int, warmup: int) -> dict:
     tgt = Buffer.from_numpy(ids.reshape(n, 1), Device.HIP)
     one = Buffer.from_scalar(1.0)
     lsm, _ = logits.log_softmax_gather(tgt)
+    att4 = att.reshape((8, 12, 1024, 1024))
+    causal = Buffer.from_numpy(np.triu(np.ones((1024, 1024), np.float32), 1), Device.HIP)
+    probs = att4.masked_softmax(causal, 0.125)
     work = [("embedding_gather", lambda: table.embedding(idx), 4 * n + 8 * n * W),
             ("embedding_scatter_add", lambda: table.embedding(idx, backward=True, upstream_grad=g),
              4 * V * W + 4 * n * W + 4 * n),
             ("softmax_98304x1024", lambda: att.softmax(1), 8 * att.numel),
+            ("scaled_causal_softmax_(8,12,1024,1024)", lambda: att4.masked_softmax(causal, 0.125), 8 * att.numel),
+            ("scaled_causal_softmax_backward", lambda: probs.masked_softmax_bwd(att4, causal, 0.125), 12 * att.numel),
             ("ce_forward_8192x50304", lambda: logits.log_softmax_gather(tgt), 8 * n * V),
             ("ce_backward_8192x50304", lambda: lsm.ce_grad(tgt, one, float(n)), 8 * n * V)]
     timer = EventTimer(lib)
