@@ -1138,31 +1138,48 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     comps = ("x", "y", "z", "w")
     mask4 = mask1 = ""
     if masked:
-        sel4 = " ".join(f"v[k].{c} = mk.{c} > 0.0f ? -__builtin_inff() : v[k].{c} * scale;" for c in comps)
+        sel4 = " ".join(f"v[k].{c} = (mb[k] & {1 << j}u) ? -__builtin_inff() : v[k].{c} * scale;" for j, c in enumerate(comps))
+        ldx = "ld4_stream(p + c)" if nt else "p[c]"
+        # the mask is read first (a few rows, cache resident); items that are masked in all four
+        # lanes are never loaded, which halves the reads of a causal mask
         mask4 = f"""    const float4* __restrict__ pm = reinterpret_cast<const float4*>(mask + (u64)(row % mrows) * L);
+    u32 mb[{nval}];
     #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < nv) {{ const float4 mk = pm[c]; {sel4} }} }}
+    for (u32 k = 0; k < {nval}u; ++k) {{
+        const u32 c = {tid} + k * {T};
+        mb[k] = 15u;
+        if (c < nv) {{ const float4 mk = pm[c]; mb[k] = (mk.x > 0.0f ? 1u : 0u) | (mk.y > 0.0f ? 2u : 0u) | (mk.z > 0.0f ? 4u : 0u) | (mk.w > 0.0f ? 8u : 0u); }}
+    }}
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; v[k] = make_float4(0.f, 0.f, 0.f, 0.f); if (mb[k] != 15u) v[k] = {ldx}; }}
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{ {sel4} }}
 """
         mask1 = f"""    const float* __restrict__ pm = mask + (u64)(row % mrows) * L;
     #pragma unroll
     for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < L) v[k] = pm[c] > 0.0f ? -__builtin_inff() : v[k] * scale; }}
 """
+    load4 = mask4 if masked else (f"    #pragma unroll\n    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; "
+                                  f"if (c < nv) v[k] = {'ld4_stream(p + c)' if nt else 'p[c]'}; }}\n")
     if nval and vec == 4:
+        # with a mask, items masked in all four lanes (mb[k] == 15, also set beyond the row's end) take no
+        # part in the max or the sum and are written as zeros, which is what exp(-inf - m) / s gives
+        live = "mb[k] != 15u" if masked else f"{tid} + k * {T} < nv"
+        zero_dead = "            if (mb[k] == 15u) o = make_float4(0.f, 0.f, 0.f, 0.f); else {\n" if masked else ""
+        close_dead = "            }\n" if masked else ""
         body = f"""
     const float4* __restrict__ p = reinterpret_cast<const float4*>(x + (u64)row * L);
     float4* __restrict__ q = reinterpret_cast<float4*>(out + (u64)row * L);
     const u32 nv = L >> 2;
     float4 v[{nval}];
+{load4}    float m = NEG_FLT_MAX;
     #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < nv) v[k] = {'ld4_stream(p + c)' if nt else 'p[c]'}; }}
-{mask4}    float m = NEG_FLT_MAX;
-    #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < nv)
+    for (u32 k = 0; k < {nval}u; ++k) if ({live})
         m = fmaxf(fmaxf(m, fmaxf(v[k].x, v[k].y)), fmaxf(v[k].z, v[k].w));
     m = {red_max};
     float s = 0.0f;
     #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < nv)
+    for (u32 k = 0; k < {nval}u; ++k) if ({live})
         s += (expf(v[k].x - m) + expf(v[k].y - m)) + (expf(v[k].z - m) + expf(v[k].w - m));
     s = {red_sum};
     const float ls = logf(s); (void)ls;
@@ -1171,7 +1188,7 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
         const u32 c = {tid} + k * {T};
         if (c < nv) {{
             float4 o;
-{''.join(f"            o.{c} = {outexpr(f'v[k].{c}')};{chr(10)}" for c in comps)}            {'{ const v4f ov = {o.x, o.y, o.z, o.w}; __builtin_nontemporal_store(ov, reinterpret_cast<v4f*>(q) + c); }' if nt else 'q[c] = o;'}
+{zero_dead}{''.join(f"            o.{c} = {outexpr(f'v[k].{c}')};{chr(10)}" for c in comps)}{close_dead}            {'{ const v4f ov = {o.x, o.y, o.z, o.w}; __builtin_nontemporal_store(ov, reinterpret_cast<v4f*>(q) + c); }' if nt else 'q[c] = o;'}
         }}
     }}
 """
@@ -1287,17 +1304,50 @@ def softmax_bwd_rows_kernel(vec: int, nval: int, nt: bool = False, masked: bool 
     (12 B per element instead of the ~36 of the four element-wise and one reduction kernels the
     expression otherwise takes).  Rows of up to 64 * nval items (float4 or float).
     masked: the backward of the scaled, masked form: dx = (mask > 0 ? 0 : y * (g - s)) * scale,
-    which is what the backward nodes of softmax, masked_fill and the scalar multiply produce."""
+    which is what the backward nodes of softmax, masked_fill and the scalar multiply produce.
+    With 16-byte items the mask is read first and items masked in all four lanes (y = 0 there,
+    so they add nothing to the sum) are not loaded: a causal mask halves the reads."""
     T, comps, nvx = _rms_lanes(vec)
     nt = nt and vec == 4
     name = f"softmax_bwd_rows_v{vec}_r{nval}{'_m' if masked else ''}{'nt' if nt else ''}"
     ld = (lambda p: f"ld4_stream({p} + c)") if nt else (lambda p: f"{p}[c]")
-    dot = " + ".join(f"g[k]{c} * y[k]{c}" for c in comps)
-    if masked:
-        outs = f"            const {T} mk = pm[c];\n" + "".join(
-            f"            o{c} = (mk{c} > 0.0f ? 0.0f : y[k]{c} * (g[k]{c} - s)) * scale;\n" for c in comps)
+    # the row's dot product, with its roundings spelled out (one product, then fused multiply-adds in
+    # lane order) so that every variant of this kernel adds the same numbers in the same way
+    dot = f"g[k]{comps[0]} * y[k]{comps[0]}"
+    for c in comps[1:]:
+        dot = f"fmaf(g[k]{c}, y[k]{c}, {dot})"
+    skip = masked and vec == 4
+    if skip:
+        outs = "".join(f"            o{c} = ((mb[k] & {1 << j}u) ? 0.0f : y[k]{c} * (g[k]{c} - s)) * scale;\n"
+                       for j, c in enumerate(comps))
+        loads = f"""    u32 mb[{nval}];
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{
+        const u32 c = lane + k * 64u;
+        mb[k] = 15u;
+        if (c < nv) {{ const float4 mk = pm[c]; mb[k] = (mk.x > 0.0f ? 1u : 0u) | (mk.y > 0.0f ? 2u : 0u) | (mk.z > 0.0f ? 4u : 0u) | (mk.w > 0.0f ? 8u : 0u); }}
+    }}
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{
+        const u32 c = lane + k * 64u;
+        y[k] = g[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (mb[k] != 15u) {{ y[k] = {ld('py')}; g[k] = {ld('pg')}; }}
+    }}
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) if (mb[k] != 15u) s += {dot};
+"""
     else:
-        outs = "".join(f"            o{c} = y[k]{c} * (g[k]{c} - s);\n" for c in comps)
+        if masked:
+            outs = f"            const {T} mk = pm[c];\n" + "".join(
+                f"            o{c} = (mk{c} > 0.0f ? 0.0f : y[k]{c} * (g[k]{c} - s)) * scale;\n" for c in comps)
+        else:
+            outs = "".join(f"            o{c} = y[k]{c} * (g[k]{c} - s);\n" for c in comps)
+        loads = f"""    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{
+        const u32 c = lane + k * 64u;
+        if (c < nv) {{ y[k] = {ld('py')}; g[k] = {ld('pg')}; s += {dot}; }}
+    }}
+"""
     st = ("{ const v4f ov = {o.x, o.y, o.z, o.w}; __builtin_nontemporal_store(ov, reinterpret_cast<v4f*>(q) + c); }" if nt
           else "q[c] = o;")
     src = f"""{PRELUDE}
@@ -1313,12 +1363,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
     const u32 nv = {nvx};
     {T} y[{nval}], g[{nval}];
     float s = 0.0f;
-    #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) {{
-        const u32 c = lane + k * 64u;
-        if (c < nv) {{ y[k] = {ld('py')}; g[k] = {ld('pg')}; s += {dot}; }}
-    }}
-    s = wave_sum(s);
+{loads}    s = wave_sum(s);
     #pragma unroll
     for (u32 k = 0; k < {nval}u; ++k) {{
         const u32 c = lane + k * 64u;
