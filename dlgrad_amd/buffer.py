@@ -237,29 +237,34 @@ class Buffer:
         return self._like(self._dispatch(UnaryOps.ARGMAX, x=self, dim=dim), shape)
 
     # ---- matmul / layout ----------------------------------------------------------------------
-    def matmul(self, other: "Buffer") -> "Buffer":
+    def _tri(self, tri: str) -> dict:
+        """A triangular-structure hint for the product kernels (see HIP.matmul); runtimes that
+        do not know it compute the whole product, which gives the same kept values."""
+        return {"tri": tri} if tri and self.device is Device.HIP else {}
+
+    def matmul(self, other: "Buffer", tri: str = "") -> "Buffer":
         p1, p2, out_shape = broadcast_shapes(self.shape, other.shape)
         x = self if self.shape == p1 else self._like(self.ptr, p1)
         y = other if other.shape == p2 else other._like(other.ptr, p2)
-        return self._like(self._dispatch(BinaryOps.MATMUL, x=x, y=y), out_shape)
+        return self._like(self._dispatch(BinaryOps.MATMUL, x=x, y=y, **self._tri(tri)), out_shape)
 
-    def matmul_nt(self, other: "Buffer") -> "Buffer":
+    def matmul_nt(self, other: "Buffer", tri: str = "") -> "Buffer":
         """self (.., M, K) @ other(.., N, K)^T without materialising the transpose."""
         swapped = other.shape[:-2] + (other.shape[-1], other.shape[-2])
         p1, p2, out_shape = broadcast_shapes(self.shape, swapped)
         p2 = p2[:-2] + (p2[-1], p2[-2])
         x = self if self.shape == p1 else self._like(self.ptr, p1)
         y = other if other.shape == p2 else other._like(other.ptr, p2)
-        return self._like(self._dispatch(CustomOps.MATMUL_NT, x=x, y=y), out_shape)
+        return self._like(self._dispatch(CustomOps.MATMUL_NT, x=x, y=y, **self._tri(tri)), out_shape)
 
-    def matmul_tn(self, other: "Buffer") -> "Buffer":
+    def matmul_tn(self, other: "Buffer", tri: str = "") -> "Buffer":
         """self(.., K, M)^T @ other (.., K, N) without materialising the transpose."""
         swapped = self.shape[:-2] + (self.shape[-1], self.shape[-2])
         p1, p2, out_shape = broadcast_shapes(swapped, other.shape)
         p1 = p1[:-2] + (p1[-1], p1[-2])
         x = self if self.shape == p1 else self._like(self.ptr, p1)
         y = other if other.shape == p2 else other._like(other.ptr, p2)
-        return self._like(self._dispatch(CustomOps.MATMUL_TN, x=x, y=y), out_shape)
+        return self._like(self._dispatch(CustomOps.MATMUL_TN, x=x, y=y, **self._tri(tri)), out_shape)
 
     def permute(self, order: tuple) -> "Buffer":
         order = tuple(order)

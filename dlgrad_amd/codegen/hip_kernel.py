@@ -1615,9 +1615,12 @@ def matmul_lds_bytes(WM: int, WN: int, MI: int, NJ: int, BK: int, ta: bool = Fal
     return 2 * 4 * (a + b)
 
 
+MATMUL_TRI = ("", "out_lower", "a_lower", "at_lower")
+
+
 @cache
 def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb: bool,
-                  ta: bool = False, tb: bool = False) -> tuple[str, str, str]:
+                  ta: bool = False, tb: bool = False, tri: str = "") -> tuple[str, str, str]:
     """C[z] = op(A[z]) . op(B[z]), fp32, row-major, on the matrix cores (v_mfma_f32_32x32x2_f32).
 
     Replaces the i-k-j loops of cpu_kernel.py:351-428.  Batched over blockIdx.z with two
@@ -1646,12 +1649,19 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     and bases and batch strides are 16-byte aligned); vecb and not tb also means 16-byte
     stores of C.  Out-of-range rows, columns and k are read as zero and never written.
     Blocks are renumbered so that the eight XCDs (round-robin dispatch) each work on a
-    contiguous band of C tiles, walked in groups of 8 tile rows for L2 reuse."""
+    contiguous band of C tiles, walked in groups of 8 tile rows for L2 reuse.
+    tri: square (T x T) structure the caller vouches for, per batch entry; the skipped work is
+    products with exact zeros or output nobody reads, so the kept results keep their bits:
+      out_lower  only output tiles that touch n <= m are computed (the others are left unwritten)
+      a_lower    op(A) = A is lower triangular (A[m][k] = 0 for k > m): k stops at the tile's last row
+      at_lower   op(A) = A^T with the stored A (K x M) lower triangular: k starts at the tile's first row
+    """
     BM, BN, T = 32 * MI * WM, 32 * NJ * WN, 64 * WM * WN
     assert BK % 8 == 0 and MI in (1, 2, 3, 4) and NJ in (1, 2, 3, 4)
     assert matmul_lds_bytes(WM, WN, MI, NJ, BK, ta, tb) <= MATMUL_LDS_LIMIT
     name = (f"matmul_{BM}x{BN}x{BK}_w{WM}x{WN}_{'a4' if veca else 'a1'}{'b4' if vecb else 'b1'}"
-            f"{'_tn' if ta else ''}{'_nt' if tb else ''}")
+            f"{'_tn' if ta else ''}{'_nt' if tb else ''}{'_' + tri if tri else ''}")
+    assert tri in MATMUL_TRI and not (tri == "a_lower" and ta) and not (tri == "at_lower" and not ta)
     comp = ["x", "y", "z", "w"]
     vtype = {1: "float", 2: "float2", 3: "f3v", 4: "float4"}
 
@@ -1758,6 +1768,28 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
                 #pragma unroll
                 for (int j = 0; j < NJ; ++j) if (col + j < g.N) crow[col + j] = acc[i][j][e];"""
 
+    # a triangular job makes the tile rows unequal (short near one end of the diagonal, long at the other)
+    # and consecutive blocks go to consecutive XCDs: rotating the row by the batch index keeps one XCD
+    # from collecting all the long rows
+    m0n0 = ("    const u32 m0 = ((tm + blockIdx.z) % tiles_m) * BM, n0 = tn * BN;" if tri
+            else "    const u32 m0 = tm * BM, n0 = tn * BN;")
+    skip_tile = "    if (n0 > m0 + BM - 1u) return;                    // the whole tile lies above the diagonal\n" if tri == "out_lower" else ""
+    if tri in ("", "out_lower"):
+        kloop = """    const u32 nk = (g.K + BK - 1u) / BK;
+    load_tiles(0u);
+    stash_tiles(0u);
+    __syncthreads();
+    for (u32 kt = 0; kt < nk; ++kt) {
+        const u32 buf = kt & 1u;"""
+    else:
+        krange = {"a_lower": "const u32 nk = (min(g.K, m0 + BM) + BK - 1u) / BK, kt0 = 0u;       // A is zero right of the diagonal",
+                  "at_lower": "const u32 nk = (g.K + BK - 1u) / BK, kt0 = m0 / BK;                 // the stored A is zero above the diagonal"}[tri]
+        kloop = f"""    {krange}
+    load_tiles(kt0 * BK);
+    stash_tiles(0u);
+    __syncthreads();
+    for (u32 kt = kt0; kt < nk; ++kt) {{
+        const u32 buf = (kt - kt0) & 1u;"""
     src = f"""{PRELUDE}
 typedef float f16v __attribute__((ext_vector_type(16)));
 struct f3v {{ float x, y, z; }};
@@ -1781,8 +1813,8 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
     const u32 first_m = (pid / width) * 8u;
     const u32 gsz = min(tiles_m - first_m, 8u);
     const u32 tm = first_m + (pid % width) % gsz, tn = (pid % width) / gsz;
-    const u32 m0 = tm * BM, n0 = tn * BN;
-
+{m0n0}
+{skip_tile}
     const u32 zb = blockIdx.z / g.nbc, zc = blockIdx.z % g.nbc;
     A += (u64)zb * g.sa0 + (u64)zc * g.sa1;
     B += (u64)zb * g.sb0 + (u64)zc * g.sb1;
@@ -1808,12 +1840,7 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
     auto stash_tiles = [&](u32 buf) {{
 {stash_a}{stash_b}    }};
 
-    const u32 nk = (g.K + BK - 1u) / BK;
-    load_tiles(0u);
-    stash_tiles(0u);
-    __syncthreads();
-    for (u32 kt = 0; kt < nk; ++kt) {{
-        const u32 buf = kt & 1u;
+{kloop}
         if (kt + 1u < nk) load_tiles((kt + 1u) * BK);
         #pragma unroll
         for (u32 kb = 0; kb < BK; kb += 8u) {{

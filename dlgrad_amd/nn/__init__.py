@@ -53,3 +53,16 @@ class RMSNorm:
             return ops.RMSNorm.execute(*args, eps=self.eps)
         y = self._norm(x)
         return y if self.weight is None else y * self.weight
+
+
+def causal_attention(q: Tensor, k: Tensor, v: Tensor, scale: float) -> Tensor:
+    """softmax(causal_mask(q @ k^T * scale)) @ v over the last two dims of q, k (.., T, d) and
+    v (.., T, dv): the no-cache branch of the reference's attention (examples/gpt.py:50-55).
+    On the hip device it is one graph node that runs the chain's kernels with the causal
+    structure known (ops.CausalAttention: same values, about half the work); elsewhere it is
+    the chain itself."""
+    if ops.use_fused_causal_attention(q, k, v):
+        return ops.CausalAttention.execute(q, k, v, scale=scale)
+    nd, T = q.ndim, q.shape[-2]
+    mask = Tensor(ops.causal_mask(T, q.device))
+    return (q @ k.transpose(nd - 2, nd - 1)).masked_softmax(mask, scale, dim=nd - 1) @ v

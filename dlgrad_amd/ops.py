@@ -380,6 +380,53 @@ class MaskedSoftmax(OP):
         return Buffer.masked_fill(x=g, mask=self.mask, val=0.0) * self.scale, None
 
 
+_causal_masks: dict = {}
+
+
+def causal_mask(T: int, device) -> Buffer:
+    """(T, T) of 1.0 where column > row (attention not allowed), else 0.0; built once per size
+    and device: what `Tensor.tril(Tensor.ones((T, T))) == 0` gives (examples/gpt.py:52-53)."""
+    key = (T, device)
+    if key not in _causal_masks:
+        allowed = Buffer.arange((1, T), device) <= Buffer.arange((T, 1), device)
+        _causal_masks[key] = allowed == 0.0
+    return _causal_masks[key]
+
+
+def use_fused_causal_attention(q, k, v) -> bool:
+    if not (FUSED and q.device is Device.HIP and k.device is Device.HIP and v.device is Device.HIP):
+        return False
+    if not (q.ndim == k.ndim == v.ndim and q.ndim >= 2 and q.shape == k.shape and q.shape[:-1] == v.shape[:-1]):
+        return False
+    from dlgrad_amd.runtime.hip import HIP
+    return HIP.causal_softmax_fits(q.shape[-2])
+
+
+class CausalAttention(OP):
+    """softmax(mask(q k^T * scale)) v for q, k (.., T, d) and v (.., T, dv) with the causal mask,
+    built from the same kernels as the op-by-op chain of examples/gpt.py:50-55 (a product, the
+    scaled masked softmax, a product) and giving the same bits, but knowing the structure:
+    k is read in place instead of being transposed first; score tiles that lie entirely
+    above the diagonal are not computed (the softmax never reads them); products with the
+    probabilities, or with their gradient, stop or start at the diagonal, because everything
+    beyond it is an exact zero.  Backward likewise.  Only the probabilities are kept."""
+
+    def forward(self, q: Buffer, k: Buffer, v: Buffer, scale: float) -> Buffer:
+        self.q, self.k, self.v, self.scale = q, k, v, scale
+        self.mask = causal_mask(q.shape[-2], q.device)
+        scores = q.matmul_nt(k, tri="out_lower")
+        self.p = scores.masked_softmax(self.mask, scale)
+        return self.p.matmul(v, tri="a_lower")
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        dp = upstream_grad.matmul_nt(self.v, tri="out_lower")
+        dv = self.p.matmul_tn(upstream_grad, tri="at_lower")
+        ds = self.p.masked_softmax_bwd(dp, self.mask, self.scale)
+        dq = ds.matmul(self.k, tri="a_lower")
+        dk = ds.matmul_tn(self.q, tri="at_lower")
+        return dq, dk, dv
+
+
 def use_fused_rmsnorm(x, weight) -> bool:
     if not (FUSED and x.device is Device.HIP):
         return False

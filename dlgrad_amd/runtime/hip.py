@@ -1054,6 +1054,13 @@ class HIP:
         return K.softmax_plan(L, vec)[1] > 0 and K.rmsnorm_plan(L, vec) > 0
 
     @staticmethod
+    def causal_softmax_fits(T: int) -> bool:
+        """Whether rows of T scores fit the fused masked softmax and its backward (fresh
+        allocations are 256-byte aligned, so only T decides the access width)."""
+        vec = 4 if T % 4 == 0 else 1
+        return T > 0 and K.softmax_plan(T, vec)[1] > 0 and K.rmsnorm_plan(T, vec) > 0
+
+    @staticmethod
     @dispatcher.register(CustomOps.MASKED_SOFTMAX, Device.HIP)
     def masked_softmax(x: Buffer, mask: Buffer, scale: float) -> DevicePtr:
         """softmax over the last axis of x * scale with -inf where mask > 0: the three kernels of
@@ -1317,14 +1324,14 @@ class HIP:
 
     @staticmethod
     def _launch_matmul(tile: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple,
-                       ta: bool = False, tb: bool = False) -> None:
+                       ta: bool = False, tb: bool = False, tri: str = "") -> None:
         bm, bn, threads = K.matmul_tile_shape(tile)
-        k = kernel(K.matmul_kernel, *K.MATMUL_CONFIGS[tile], veca, vecb, ta, tb)
+        k = kernel(K.matmul_kernel, *K.MATMUL_CONFIGS[tile], veca, vecb, ta, tb, tri)
         launch(k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch), threads, *args)
 
     @staticmethod
     def _tune_tile(key: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple,
-                   ta: bool, tb: bool) -> str:
+                   ta: bool, tb: bool, tri: str = "") -> str:
         """Times every plausible tile on the real operands (the output is simply rewritten:
         all tiles produce the same bits) and stores the winner in the cache directory."""
         global launch_count
@@ -1333,14 +1340,14 @@ class HIP:
         best, best_ms = None, float("inf")
         e0, e1 = l.event_create(), l.event_create()
         for tile in HIP._tile_candidates(M, N, batch):
-            HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb)          # loads the code object
+            HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri)     # loads the code object
             if COMPILE_ONLY:
                 continue
             ms, reps = 0.0, 3
             while True:
                 l.event_record(e0)
                 for _ in range(reps):
-                    HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb)
+                    HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri)
                 l.event_record(e1)
                 l.event_sync(e1)
                 ms = l.event_elapsed_ms(e0, e1) / reps
@@ -1373,25 +1380,27 @@ class HIP:
 
     @staticmethod
     def _pick_tile(M: int, N: int, Kd: int, batch: int, veca: bool, vecb: bool, args: tuple,
-                   ta: bool = False, tb: bool = False) -> str:
+                   ta: bool = False, tb: bool = False, tri: str = "") -> str:
         if HIP.MATMUL_FORCE:
             return HIP.MATMUL_FORCE
-        key = f"{batch},{M},{N},{Kd}" + (",tn" if ta else ",nt" if tb else "")
+        key = f"{batch},{M},{N},{Kd}" + (",tn" if ta else ",nt" if tb else "") + (f",{tri}" if tri else "")
         tile = HIP._tuned_table().get(key)
         if tile is not None:
             return tile
         if HIP.MATMUL_TUNE and not capturing() and 2 * M * N * Kd * batch >= HIP.MATMUL_TUNE_MIN_FLOP:
-            return HIP._tune_tile(key, veca, vecb, M, N, batch, args, ta, tb)
+            return HIP._tune_tile(key, veca, vecb, M, N, batch, args, ta, tb, tri)
         return HIP._model_tile(M, N, batch, Kd)
 
     @staticmethod
     @dispatcher.register(BinaryOps.MATMUL, Device.HIP)
-    def matmul(x: Buffer, y: Buffer, ta: bool = False, tb: bool = False) -> DevicePtr:
+    def matmul(x: Buffer, y: Buffer, ta: bool = False, tb: bool = False, tri: str = "") -> DevicePtr:
         """x (.., M, K) @ y (.., K, N) for operands already padded to the same rank 2..4
         (buffer.py:231-243); batch dims of extent 1 broadcast through a zero stride as in
         cpu.py:519-532 and :553-559.  When y carries no batch at all the batch of x is
         folded into M: one tall GEMM instead of many small ones.
-        ta: x is stored as (.., K, M) and used transposed; tb: y is stored as (.., N, K)."""
+        ta: x is stored as (.., K, M) and used transposed; tb: y is stored as (.., N, K).
+        tri: triangular structure of square (T x T) operands or outputs that the caller vouches
+        for (K.matmul_kernel); the work it lets the kernel skip never changes a kept result."""
         assert x.ndim == y.ndim and 2 <= x.ndim <= 4 and not (ta and tb)
         (Kd, M) = x.shape[-2:] if ta else x.shape[-2:][::-1]
         (N, Ky) = y.shape[-2:] if tb else y.shape[-2:][::-1]
@@ -1405,7 +1414,11 @@ class HIP:
         if Kd == 0:
             lib().fill_f32(out.addr, 0.0, B0 * B1 * M * N)
             return out
-        if yb == (1, 1) and not ta:
+        if tri:
+            square = {"out_lower": M == N, "a_lower": not ta and M == Kd, "at_lower": ta and M == Kd}.get(tri)
+            if not square:
+                raise ValueError(f"tri={tri!r} does not fit {x.shape} x {y.shape} (ta={ta}, tb={tb})")
+        if yb == (1, 1) and not ta and not tri:
             M, nbc, batch = xb[0] * xb[1] * M, 1, 1
             sa = sb = (0, 0)
         else:
@@ -1419,18 +1432,18 @@ class HIP:
         veca = (M if ta else Kd) % 4 == 0 and _addr(x) % 16 == 0
         vecb = (Kd if tb else N) % 4 == 0 and _addr(y) % 16 == 0 and out.addr % 16 == 0
         args = (_addr(x), _addr(y), out.addr, M, N, Kd, nbc, *sa, *sb)
-        tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, args, ta, tb)
-        HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb)
+        tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, args, ta, tb, tri)
+        HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri)
         return out
 
     @staticmethod
     @dispatcher.register(CustomOps.MATMUL_NT, Device.HIP)
-    def matmul_nt(x: Buffer, y: Buffer) -> DevicePtr:
+    def matmul_nt(x: Buffer, y: Buffer, tri: str = "") -> DevicePtr:
         """x (.., M, K) times the transpose of y (.., N, K), read in place."""
-        return HIP.matmul(x, y, tb=True)
+        return HIP.matmul(x, y, tb=True, tri=tri)
 
     @staticmethod
     @dispatcher.register(CustomOps.MATMUL_TN, Device.HIP)
-    def matmul_tn(x: Buffer, y: Buffer) -> DevicePtr:
+    def matmul_tn(x: Buffer, y: Buffer, tri: str = "") -> DevicePtr:
         """The transpose of x (.., K, M), read in place, times y (.., K, N)."""
-        return HIP.matmul(x, y, ta=True)
+        return HIP.matmul(x, y, ta=True, tri=tri)

@@ -24,17 +24,6 @@ class GPTConfig:
         self.learning_rate, self.device = learning_rate, device
 
 
-_mask_cache: dict = {}
-
-
-def causal_mask(T: int, device) -> Tensor:
-    """1.0 where attention is NOT allowed: tril(ones) == 0 (examples/gpt.py:52-53)."""
-    key = (T, str(device))
-    if key not in _mask_cache:
-        _mask_cache[key] = Tensor.tril(Tensor.ones((T, T), device=device), k=0.0) == Tensor(0.0)
-    return _mask_cache[key]
-
-
 class CausalSelfAttention:
     def __init__(self, c: GPTConfig) -> None:
         assert c.n_embd % c.n_head == 0
@@ -64,8 +53,9 @@ class CausalSelfAttention:
                 cache.write(layer, k_lin, v_lin, 0)
             k = k_lin.reshape(split).transpose(1, 2)
             v = v_lin.reshape(split).transpose(1, 2)
-            # (att * scale).masked_fill(mask, -inf).softmax(dim=3), one kernel on the hip device
-            att = (q @ k.transpose(2, 3)).masked_softmax(causal_mask(T, x.device), self.scale, dim=3)   # (B, h, T, T)
+            # ((q @ k^T) * scale).masked_fill(mask, -inf).softmax(dim=3) @ v (examples/gpt.py:50-55)
+            y = nn.causal_attention(q, k, v, self.scale)                                     # (B, h, T, d)
+            return self.c_proj(y.transpose(1, 2).reshape((B, T, C)))
         y = (att @ v).transpose(1, 2).reshape((B, T, C))
         return self.c_proj(y)
 

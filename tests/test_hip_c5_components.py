@@ -185,3 +185,37 @@ def test_masked_softmax_falls_back_to_the_chain_where_the_kernel_does_not_fit():
         got = t.masked_softmax(m, 0.5, dim=dim).numpy()
         want = Tensor(x).masked_softmax(Tensor(mask), 0.5, dim=dim).numpy()
         check(got, want, 1e-6, f"masked softmax chain {xs} {ms} dim {dim}")
+
+
+@pytest.mark.parametrize("shape", [(2, 4, 128, 32), (1, 12, 1024, 64), (3, 2, 100, 20), (2, 1, 257, 64), (5, 64, 16)])
+def test_causal_attention_node_equals_the_op_by_op_chain(shape, monkeypatch):
+    """nn.causal_attention on the hip device runs the chain's own kernels with the causal structure
+    known (k read in place, score tiles above the diagonal skipped, products cut at the diagonal):
+    output and the gradients of q, k and v must be bit-identical to
+    (q @ k^T).masked_softmax(mask, scale) @ v, and close to a float64 evaluation (1e-5)."""
+    require_gpu()
+    from dlgrad_amd import nn, ops
+    rng = np.random.default_rng(70)
+    q, k, v, g = (rng.standard_normal(shape, dtype=np.float32) for _ in range(4))
+    scale = shape[-1] ** -0.5
+
+    def run(fused):
+        monkeypatch.setattr(ops, "use_fused_causal_attention", (lambda *a: False) if not fused else ops.use_fused_causal_attention)
+        ts = [Tensor(a, device="hip", requires_grad=True) for a in (q, k, v)]
+        y = nn.causal_attention(*ts, scale)
+        node = type(y._ctx).__name__
+        (y * Tensor(g, device="hip")).sum().backward()
+        return node, [y.numpy()] + [t.grad.numpy() for t in ts]
+
+    (n1, fused), (n0, chain) = run(True), run(False)
+    assert n1 == "CausalAttention" and n0 != "CausalAttention"
+    if hip.COMPILE_ONLY:
+        return
+    for name, a, b in zip(("y", "dq", "dk", "dv"), fused, chain):
+        assert (a.view(np.uint32) == b.view(np.uint32)).all(), f"{name} {shape}"
+    T = shape[-2]
+    q64, k64, v64 = (a.astype(np.float64) for a in (q, k, v))
+    s = np.where(np.triu(np.ones((T, T), bool), 1), -np.inf, (q64 @ np.swapaxes(k64, -1, -2)) * scale)
+    e = np.exp(s - s.max(-1, keepdims=True))
+    want = (e / e.sum(-1, keepdims=True)) @ v64
+    assert np.abs(fused[0] - want).max() <= 1e-5 * max(1.0, np.abs(want).max())

@@ -188,3 +188,43 @@ def test_every_tile_configuration_transposed(tile, monkeypatch):
     monkeypatch.setattr(HIP, "MATMUL_FORCE", tile)
     check(xd.matmul_nt(yd).numpy(), want_nt, 0, f"NT {tile}")
     check(xd.matmul_tn(zd).numpy(), want_tn, 0, f"TN {tile}")
+
+
+@pytest.mark.parametrize("T,d,batch", [(128, 32, (2, 3)), (1024, 64, (2,)), (100, 20, (3,)), (257, 64, ()), (64, 8, (1, 2))])
+def test_triangular_hints_skip_work_without_changing_a_bit(T, d, batch):
+    """tri = out_lower / a_lower / at_lower tell the product kernel which tiles or which part of
+    the k range a triangular operand or a masked consumer makes irrelevant.  With operands that
+    really have that structure every kept entry must equal the plain product bit for bit, for
+    every tile configuration (forced one by one), ragged T included."""
+    require_gpu()
+    from dlgrad_amd.codegen import hip_kernel as K
+    from dlgrad_amd.runtime.hip import HIP
+    rng = np.random.default_rng(T + d)
+    low = np.tril(rng.standard_normal(batch + (T, T), dtype=np.float32))          # zero above the diagonal
+    x = rng.standard_normal(batch + (T, d), dtype=np.float32)
+    y = rng.standard_normal(batch + (T, d), dtype=np.float32)
+    keep = np.tril(np.ones((T, T), bool))
+    lowd, xd, yd = dev(low), dev(x), dev(y)
+    want_scores = xd.matmul_nt(yd).numpy()
+    want_av = lowd.matmul(yd).numpy()
+    want_atv = lowd.matmul_tn(yd).numpy()
+    tiles = [t for t in K.MATMUL_CONFIGS if T >= 64 or t in ("64x64", "32x32")]
+    for tile in tiles:
+        prev, HIP.MATMUL_FORCE = HIP.MATMUL_FORCE, tile
+        try:
+            got = xd.matmul_nt(yd, tri="out_lower").numpy()
+            if not hip.COMPILE_ONLY:
+                assert (got[..., keep].view(np.uint32) == want_scores[..., keep].view(np.uint32)).all(), f"out_lower {tile}"
+            check(lowd.matmul(yd, tri="a_lower").numpy(), want_av, 0, f"a_lower {tile}")
+            check(lowd.matmul_tn(yd, tri="at_lower").numpy(), want_atv, 0, f"at_lower {tile}")
+        finally:
+            HIP.MATMUL_FORCE = prev
+
+
+def test_triangular_hints_are_refused_where_they_make_no_sense():
+    require_gpu()
+    a, b = dev(f32(8, 16)), dev(f32(16, 8))
+    with pytest.raises(ValueError):
+        a.matmul(b, tri="a_lower")                      # A is not square
+    with pytest.raises(ValueError):
+        a.matmul_nt(dev(f32(4, 16)), tri="out_lower")   # the output is not square
