@@ -1338,14 +1338,17 @@ def softmax_bwd_rows_kernel(vec: int, nval: int, nt: bool = False, masked: bool 
 """
     else:
         if masked:
+            # 4-byte form: a masked entry's upstream value is never used (its memory may hold anything)
             outs = f"            const {T} mk = pm[c];\n" + "".join(
                 f"            o{c} = (mk{c} > 0.0f ? 0.0f : y[k]{c} * (g[k]{c} - s)) * scale;\n" for c in comps)
+            ldg = f"(pm[c] > 0.0f ? 0.0f : {ld('pg')})"
         else:
             outs = "".join(f"            o{c} = y[k]{c} * (g[k]{c} - s);\n" for c in comps)
+            ldg = ld('pg')
         loads = f"""    #pragma unroll
     for (u32 k = 0; k < {nval}u; ++k) {{
         const u32 c = lane + k * 64u;
-        if (c < nv) {{ y[k] = {ld('py')}; g[k] = {ld('pg')}; s += {dot}; }}
+        if (c < nv) {{ y[k] = {ld('py')}; g[k] = {ldg}; s += {dot}; }}
     }}
 """
     st = ("{ const v4f ov = {o.x, o.y, o.z, o.w}; __builtin_nontemporal_store(ov, reinterpret_cast<v4f*>(q) + c); }" if nt

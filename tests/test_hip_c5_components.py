@@ -219,3 +219,38 @@ def test_causal_attention_node_equals_the_op_by_op_chain(shape, monkeypatch):
     e = np.exp(s - s.max(-1, keepdims=True))
     want = (e / e.sum(-1, keepdims=True)) @ v64
     assert np.abs(fused[0] - want).max() <= 1e-5 * max(1.0, np.abs(want).max())
+
+
+@pytest.mark.parametrize("shape", [(2, 2, 256, 32), (2, 1, 257, 64), (1, 3, 130, 8)])
+def test_causal_attention_never_reads_what_it_skipped(shape):
+    """The score and dP tiles above the diagonal are left unwritten, so they hold whatever the
+    pool's blocks held before.  With the pool's free blocks filled with NaN first, output and
+    gradients must still be finite and bit-identical to a run on clean memory: nothing that
+    was skipped may enter a sum, whether the rows take the 16-byte or the 4-byte kernels."""
+    require_gpu()
+    from dlgrad_amd import nn
+    from dlgrad_amd.buffer import Buffer
+    from dlgrad_amd.device import Device
+    rng = np.random.default_rng(71)
+    q, k, v, g = (rng.standard_normal(shape, dtype=np.float32) for _ in range(4))
+
+    def run():
+        ts = [Tensor(a, device="hip", requires_grad=True) for a in (q, k, v)]
+        y = nn.causal_attention(*ts, 0.25)
+        assert type(y._ctx).__name__ == "CausalAttention"
+        (y * Tensor(g, device="hip")).sum().backward()
+        return [y.numpy()] + [t.grad.numpy() for t in ts]
+
+    clean = run()
+    T = shape[-2]
+    n_scores = int(np.prod(shape[:-2])) * T * T
+    poison = [Buffer.from_numpy(np.full(n, np.nan, np.float32), Device.HIP)
+              for n in (n_scores, n_scores, n_scores, int(np.prod(shape)), int(np.prod(shape)))]
+    hip.lib().sync()
+    del poison                                               # back to the pool, NaN and all
+    dirty = run()
+    if hip.COMPILE_ONLY:
+        return
+    for name, a, b in zip(("y", "dq", "dk", "dv"), dirty, clean):
+        assert np.isfinite(a).all(), name
+        assert (a.view(np.uint32) == b.view(np.uint32)).all(), name
