@@ -463,3 +463,39 @@ def test_one_launch_adam_over_a_parameter_list_is_bit_identical_to_the_per_tenso
     if not hip.COMPILE_ONLY:
         for a, b in zip(results[True], results[False]):
             np.testing.assert_array_equal(a, b)
+
+
+def gpt_losses(device, cfg_kw, steps, seed=0):
+    """Loss before each of `steps` forward + backward + Adam steps on one seeded batch."""
+    c = G.GPTConfig(device=device, **cfg_kw)
+    model = G.GPT(c)
+    G.init_weights_(model, seed)
+    opt = nn.optim.Adam(nn.utils.get_parameters(model), lr=c.learning_rate)
+    rng = np.random.default_rng(seed + 1)
+    out = []
+    idx = rng.integers(0, c.vocab_size, (c.batch_size, c.block_size)).astype(np.float32)
+    tgt = rng.integers(0, c.vocab_size, (c.batch_size, c.block_size)).astype(np.float32)
+    for _ in range(steps):
+        opt.zero_grad()
+        _, loss = model(Tensor(idx, device=device), Tensor(tgt, device=device))
+        loss.backward()
+        opt.step()
+        out.append(float(loss.numpy().reshape(-1)[0]))
+    return np.array(out)
+
+
+@pytest.mark.gpu
+def test_gpt_training_trajectory_hip_vs_cpu_oracle():
+    """Twelve consecutive training steps of a small GPT on both devices from the same weights, on
+    the same batch: the loss falls, and the loss of every step agrees to 1e-4 relative.  (Single steps are compared tensor
+    by tensor above; this holds the composition of steps, optimizer state included.)"""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    cfg = dict(vocab_size=65, block_size=32, n_layer=2, n_head=2, n_embd=64, batch_size=4)
+    cpu = gpt_losses("cpu", cfg, 12)
+    dev_ = gpt_losses("hip", cfg, 12)
+    if hip.COMPILE_ONLY:
+        return
+    assert cpu[-1] < cpu[0]                                   # it trains
+    rel = np.abs(dev_ - cpu) / np.abs(cpu)
+    assert rel.max() <= 1e-4, f"loss trajectories part: {rel}"
