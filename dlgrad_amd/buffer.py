@@ -335,6 +335,19 @@ class Buffer:
         """self is a masked_softmax output; returns the gradient of its input."""
         return self._like(self._dispatch(CustomOps.MASKED_SOFTMAX_BWD, y=self, g=upstream, mask=mask, scale=scale))
 
+    def causal_attention(self, k: "Buffer", v: "Buffer", n_head: int, scale: float) -> tuple["Buffer", "Buffer"]:
+        """self, k, v: (B, T, C) projections with C = n_head * d.  Returns the context (B, T, C) and the
+        attention probabilities (B, n_head, T, T); the heads are read and written in place."""
+        B, T, _ = self.shape
+        y, p = self._dispatch(CustomOps.CAUSAL_ATTENTION, q=self, k=k, v=v, n_head=n_head, scale=scale)
+        return self._like(y), self._like(p, (B, n_head, T, T))
+
+    def causal_attention_bwd(self, k: "Buffer", v: "Buffer", p: "Buffer", dy: "Buffer", n_head: int,
+                             scale: float) -> tuple["Buffer", "Buffer", "Buffer"]:
+        """Gradients of causal_attention for q = self, k, v, each (B, T, C)."""
+        dq, dk, dv = self._dispatch(CustomOps.CAUSAL_ATTENTION_BWD, q=self, k=k, v=v, p=p, dy=dy, n_head=n_head, scale=scale)
+        return self._like(dq), self._like(dk), self._like(dv)
+
     def log_softmax(self, dim: int) -> "Buffer":
         return self._unary(CustomOps.LOG_SOFTMAX, dim=dim)
 

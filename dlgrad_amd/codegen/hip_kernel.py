@@ -1623,7 +1623,7 @@ MATMUL_TRI = ("", "out_lower", "a_lower", "at_lower")
 
 @cache
 def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb: bool,
-                  ta: bool = False, tb: bool = False, tri: str = "") -> tuple[str, str, str]:
+                  ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False) -> tuple[str, str, str]:
     """C[z] = op(A[z]) . op(B[z]), fp32, row-major, on the matrix cores (v_mfma_f32_32x32x2_f32).
 
     Replaces the i-k-j loops of cpu_kernel.py:351-428.  Batched over blockIdx.z with two
@@ -1658,12 +1658,15 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
       out_lower  only output tiles that touch n <= m are computed (the others are left unwritten)
       a_lower    op(A) = A is lower triangular (A[m][k] = 0 for k > m): k stops at the tile's last row
       at_lower   op(A) = A^T with the stored A (K x M) lower triangular: k starts at the tile's first row
+    strided: A, B and C have their own row pitches (lda, ldb, ldc, in floats) and C its own two batch
+    strides, so operands and result can be matrices cut out of larger tensors -- the heads of a
+    (B, T, h*d) projection are (T x d) matrices with pitch h*d, batch strides T*h*d and d.
     """
     BM, BN, T = 32 * MI * WM, 32 * NJ * WN, 64 * WM * WN
     assert BK % 8 == 0 and MI in (1, 2, 3, 4) and NJ in (1, 2, 3, 4)
     assert matmul_lds_bytes(WM, WN, MI, NJ, BK, ta, tb) <= MATMUL_LDS_LIMIT
     name = (f"matmul_{BM}x{BN}x{BK}_w{WM}x{WN}_{'a4' if veca else 'a1'}{'b4' if vecb else 'b1'}"
-            f"{'_tn' if ta else ''}{'_nt' if tb else ''}{'_' + tri if tri else ''}")
+            f"{'_tn' if ta else ''}{'_nt' if tb else ''}{'_' + tri if tri else ''}{'_ld' if strided else ''}")
     assert tri in MATMUL_TRI and not (tri == "a_lower" and ta) and not (tri == "at_lower" and not ta)
     comp = ["x", "y", "z", "w"]
     vtype = {1: "float", 2: "float2", 3: "f3v", 4: "float4"}
@@ -1864,6 +1867,18 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
         }}
 }}
 """
+    if strided:
+        for was, now in (("struct MMArgs { u32 M, N, K, nbc, sa0, sa1, sb0, sb1; };",
+                          "struct MMArgs { u32 M, N, K, nbc, sa0, sa1, sb0, sb1, lda, ldb, ldc, sc0, sc1; };"),
+                         ("A + (u64)k * g.M + col" if ta else "A + (u64)row * g.K + k",
+                          "A + (u64)k * g.lda + col" if ta else "A + (u64)row * g.lda + k"),
+                         ("B + (u64)row * g.K + k" if tb else "B + (u64)k * g.N + col",
+                          "B + (u64)row * g.ldb + k" if tb else "B + (u64)k * g.ldb + col"),
+                         ("C += (u64)blockIdx.z * g.M * g.N;", "C += (u64)zb * g.sc0 + (u64)zc * g.sc1;"),
+                         ("C + (u64)row * g.N;", "C + (u64)row * g.ldc;")):
+            assert src.count(was) == 1, was
+            src = src.replace(was, now)
+        return src, name, _fmt("P", "P", "P", "13I")
     return src, name, _fmt("P", "P", "P", "8I")
 
 

@@ -68,6 +68,8 @@ class CustomOps(Enum):
     SOFTMAX_BWD = auto()            # y * (g - sum(g * y)) over the last axis, one kernel
     MASKED_SOFTMAX = auto()         # softmax(masked_fill(x * scale, mask, -inf)) over the last axis, one kernel
     MASKED_SOFTMAX_BWD = auto()     # its backward, one kernel
+    CAUSAL_ATTENTION = auto()       # softmax(mask(q k^T * scale)) v on (B, T, heads*d) projections, heads read in place
+    CAUSAL_ATTENTION_BWD = auto()
     LOG_SOFTMAX = auto()
     LOG_SOFTMAX_GATHER = auto()     # log-softmax rows + the ce_forward gather, one kernel
     CE_GRAD = auto()                # ((exp(lsm) - onehot) * upstream) / N, one kernel

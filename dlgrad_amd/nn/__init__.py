@@ -66,3 +66,16 @@ def causal_attention(q: Tensor, k: Tensor, v: Tensor, scale: float) -> Tensor:
     nd, T = q.ndim, q.shape[-2]
     mask = Tensor(ops.causal_mask(T, q.device))
     return (q @ k.transpose(nd - 2, nd - 1)).masked_softmax(mask, scale, dim=nd - 1) @ v
+
+
+def causal_self_attention(q: Tensor, k: Tensor, v: Tensor, n_head: int, scale: float) -> Tensor:
+    """Multi-head causal attention on the projections themselves: q, k, v and the result are
+    (B, T, n_head * d).  What examples/gpt.py:45-57 writes as reshape -> transpose(1, 2) for each of
+    q, k, v, the attention, and transpose(1, 2) -> reshape back.  On the hip device the heads
+    are read and written in place (ops.CausalAttentionHeads); elsewhere it is that sequence."""
+    if ops.use_fused_attention_heads(q, k, v, n_head):
+        return ops.CausalAttentionHeads.execute(q, k, v, n_head=n_head, scale=scale)
+    B, T, C = q.shape
+    split = (B, T, n_head, C // n_head)
+    qh, kh, vh = (t.reshape(split).transpose(1, 2) for t in (q, k, v))
+    return causal_attention(qh, kh, vh, scale).transpose(1, 2).reshape((B, T, C))

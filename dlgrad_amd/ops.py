@@ -427,6 +427,31 @@ class CausalAttention(OP):
         return dq, dk, dv
 
 
+def use_fused_attention_heads(q, k, v, n_head: int) -> bool:
+    if not (FUSED and q.device is Device.HIP and k.device is Device.HIP and v.device is Device.HIP):
+        return False
+    if not (q.ndim == 3 and q.shape == k.shape == v.shape and n_head > 0 and q.shape[2] % n_head == 0 and q.numel):
+        return False
+    from dlgrad_amd.runtime.hip import HIP
+    return HIP.causal_softmax_fits(q.shape[1])
+
+
+class CausalAttentionHeads(OP):
+    """CausalAttention for the (B, T, n_head * d) projections themselves: the products read each head
+    where it lies (row pitch n_head * d) and write the context and the three gradients in the same
+    layout, so the head split and merge of examples/gpt.py:46-48,57 -- four transposes forward,
+    four backward -- never run.  Same kernels, same additions in the same order: the values are
+    those of the chain with materialised transposes, bit for bit."""
+
+    def forward(self, q: Buffer, k: Buffer, v: Buffer, n_head: int, scale: float) -> Buffer:
+        self.q, self.k, self.v, self.n_head, self.scale = q, k, v, n_head, scale
+        y, self.p = q.causal_attention(k, v, n_head, scale)
+        return y
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return self.q.causal_attention_bwd(self.k, self.v, self.p, upstream_grad, self.n_head, self.scale)
+
+
 def use_fused_rmsnorm(x, weight) -> bool:
     if not (FUSED and x.device is Device.HIP):
         return False

@@ -1324,14 +1324,14 @@ class HIP:
 
     @staticmethod
     def _launch_matmul(tile: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple,
-                       ta: bool = False, tb: bool = False, tri: str = "") -> None:
+                       ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False) -> None:
         bm, bn, threads = K.matmul_tile_shape(tile)
-        k = kernel(K.matmul_kernel, *K.MATMUL_CONFIGS[tile], veca, vecb, ta, tb, tri)
+        k = kernel(K.matmul_kernel, *K.MATMUL_CONFIGS[tile], veca, vecb, ta, tb, tri, strided)
         launch(k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch), threads, *args)
 
     @staticmethod
     def _tune_tile(key: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple,
-                   ta: bool, tb: bool, tri: str = "") -> str:
+                   ta: bool, tb: bool, tri: str = "", strided: bool = False) -> str:
         """Times every plausible tile on the real operands (the output is simply rewritten:
         all tiles produce the same bits) and stores the winner in the cache directory."""
         global launch_count
@@ -1340,14 +1340,14 @@ class HIP:
         best, best_ms = None, float("inf")
         e0, e1 = l.event_create(), l.event_create()
         for tile in HIP._tile_candidates(M, N, batch):
-            HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri)     # loads the code object
+            HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri, strided)   # loads the code object
             if COMPILE_ONLY:
                 continue
             ms, reps = 0.0, 3
             while True:
                 l.event_record(e0)
                 for _ in range(reps):
-                    HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri)
+                    HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri, strided)
                 l.event_record(e1)
                 l.event_sync(e1)
                 ms = l.event_elapsed_ms(e0, e1) / reps
@@ -1380,15 +1380,15 @@ class HIP:
 
     @staticmethod
     def _pick_tile(M: int, N: int, Kd: int, batch: int, veca: bool, vecb: bool, args: tuple,
-                   ta: bool = False, tb: bool = False, tri: str = "") -> str:
+                   ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False) -> str:
         if HIP.MATMUL_FORCE:
             return HIP.MATMUL_FORCE
-        key = f"{batch},{M},{N},{Kd}" + (",tn" if ta else ",nt" if tb else "") + (f",{tri}" if tri else "")
+        key = f"{batch},{M},{N},{Kd}" + (",tn" if ta else ",nt" if tb else "") + (f",{tri}" if tri else "") + (",ld" if strided else "")
         tile = HIP._tuned_table().get(key)
         if tile is not None:
             return tile
         if HIP.MATMUL_TUNE and not capturing() and 2 * M * N * Kd * batch >= HIP.MATMUL_TUNE_MIN_FLOP:
-            return HIP._tune_tile(key, veca, vecb, M, N, batch, args, ta, tb, tri)
+            return HIP._tune_tile(key, veca, vecb, M, N, batch, args, ta, tb, tri, strided)
         return HIP._model_tile(M, N, batch, Kd)
 
     @staticmethod
@@ -1447,3 +1447,69 @@ class HIP:
     def matmul_tn(x: Buffer, y: Buffer, tri: str = "") -> DevicePtr:
         """The transpose of x (.., K, M), read in place, times y (.., K, N)."""
         return HIP.matmul(x, y, ta=True, tri=tri)
+
+    @staticmethod
+    def _gemm_strided(A: tuple, B: tuple, C: tuple, M: int, N: int, Kd: int, B0: int, B1: int,
+                      ta: bool = False, tb: bool = False, tri: str = "") -> None:
+        """C[b0, b1] = op(A[b0, b1]) . op(B[b0, b1]) for matrices cut out of larger tensors: every
+        operand is (address, row pitch, stride of b0, stride of b1) in floats.  Same kernel, same
+        order of additions as the contiguous product of the same logical matrices."""
+        (aa, lda, sa0, sa1), (ba, ldb, sb0, sb1), (ca, ldc, sc0, sc1) = A, B, C
+        if B0 * B1 > 65535 or max(lda * max(M, Kd), ldb * max(N, Kd), ldc * M) >= 2 ** 31:
+            raise ValueError("strided product too large for the grid or for 32-bit indexing")
+        al4 = lambda addr, *v: addr % 16 == 0 and all(x % 4 == 0 for x in v)     # noqa: E731
+        veca = (M if ta else Kd) % 4 == 0 and al4(aa, lda, sa0, sa1)
+        vecb = (Kd if tb else N) % 4 == 0 and al4(ba, ldb, sb0, sb1) and al4(ca, ldc, sc0, sc1)
+        args = (aa, ba, ca, M, N, Kd, B1, sa0, sa1, sb0, sb1, lda, ldb, ldc, sc0, sc1)
+        batch = B0 * B1
+        tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, args, ta, tb, tri, True)
+        HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri, True)
+
+    @staticmethod
+    def _heads(addr: int, T: int, C: int, d: int) -> tuple:
+        """The (T x d) head matrices inside a (B, T, C) tensor: pitch C, batch strides T*C and d."""
+        return (addr, C, T * C, d)
+
+    @staticmethod
+    @dispatcher.register(CustomOps.CAUSAL_ATTENTION, Device.HIP)
+    def causal_attention(q: Buffer, k: Buffer, v: Buffer, n_head: int, scale: float) -> tuple[DevicePtr, DevicePtr]:
+        """Causal attention for q, k, v given as (B, T, C) projections with C = n_head * d: the heads are
+        read where they lie and the context is written straight into (B, T, C), so the four head
+        transposes of examples/gpt.py:46-48,57 never materialise.  Returns (y, p) with the
+        probabilities p (B, n_head, T, T) kept for the backward pass.  The products and the
+        softmax are the kernels of the op-by-op chain, with the causal structure known."""
+        Bn, T, C = q.shape
+        d = C // n_head
+        p_scores = alloc(Bn * n_head * T * T)
+        dense = (p_scores.addr, T, n_head * T * T, T * T)
+        HIP._gemm_strided(HIP._heads(_addr(q), T, C, d), HIP._heads(_addr(k), T, C, d), dense, T, T, d, Bn, n_head,
+                          tb=True, tri="out_lower")
+        scores = Buffer(p_scores, (Bn, n_head, T, T), Device.HIP)
+        from dlgrad_amd.ops import causal_mask
+        p = HIP.masked_softmax(scores, causal_mask(T, Device.HIP), scale)
+        y = alloc(Bn * T * C)
+        HIP._gemm_strided((p.addr, T, n_head * T * T, T * T), HIP._heads(_addr(v), T, C, d), HIP._heads(y.addr, T, C, d),
+                          T, d, T, Bn, n_head, tri="a_lower")
+        return y, p
+
+    @staticmethod
+    @dispatcher.register(CustomOps.CAUSAL_ATTENTION_BWD, Device.HIP)
+    def causal_attention_bwd(q: Buffer, k: Buffer, v: Buffer, p: Buffer, dy: Buffer, n_head: int,
+                             scale: float) -> tuple[DevicePtr, DevicePtr, DevicePtr]:
+        """Gradients of causal_attention with respect to the (B, T, C) projections, written in that layout."""
+        Bn, T, C = q.shape
+        d = C // n_head
+        pd = (_addr(p), T, n_head * T * T, T * T)
+        heads = lambda buf_addr: HIP._heads(buf_addr, T, C, d)                     # noqa: E731
+        dp = alloc(p.numel)
+        HIP._gemm_strided(heads(_addr(dy)), heads(_addr(v)), (dp.addr, T, n_head * T * T, T * T), T, T, d, Bn, n_head,
+                          tb=True, tri="out_lower")
+        dv = alloc(Bn * T * C)
+        HIP._gemm_strided(pd, heads(_addr(dy)), heads(dv.addr), T, d, T, Bn, n_head, ta=True, tri="at_lower")
+        from dlgrad_amd.ops import causal_mask
+        ds = HIP.masked_softmax_bwd(p, Buffer(dp, p.shape, Device.HIP), causal_mask(T, Device.HIP), scale)
+        dsd = (ds.addr, T, n_head * T * T, T * T)
+        dq, dk = alloc(Bn * T * C), alloc(Bn * T * C)
+        HIP._gemm_strided(dsd, heads(_addr(k)), heads(dq.addr), T, d, T, Bn, n_head, tri="a_lower")
+        HIP._gemm_strided(dsd, heads(_addr(q)), heads(dk.addr), T, d, T, Bn, n_head, ta=True, tri="at_lower")
+        return dq, dk, dv

@@ -41,21 +41,19 @@ class CausalSelfAttention:
         (examples/gpt.py:44-66)."""
         B, T, C = x.shape
         split = (B, T, self.n_head, self.head_dim)
-        q = self.q_proj(x).reshape(split).transpose(1, 2)            # (B, h, T, d)
-        k_lin, v_lin = self.k_proj(x), self.v_proj(x)                # (B, T, C)
+        q_lin, k_lin, v_lin = self.q_proj(x), self.k_proj(x), self.v_proj(x)    # (B, T, C)
         if cache is not None and cache.length > 0:
             assert T == 1, "incremental attention takes one new position"
+            q = q_lin.reshape(split).transpose(1, 2)                  # (B, h, 1, d)
             cache.write(layer, k_lin, v_lin, cache.length)
             k, v = cache.view(layer, cache.length + 1, self.n_head)  # (B, h, n, d)
             att = ((q @ k.transpose(2, 3)) * self.scale).softmax(dim=3)
         else:
             if cache is not None:
                 cache.write(layer, k_lin, v_lin, 0)
-            k = k_lin.reshape(split).transpose(1, 2)
-            v = v_lin.reshape(split).transpose(1, 2)
-            # ((q @ k^T) * scale).masked_fill(mask, -inf).softmax(dim=3) @ v (examples/gpt.py:50-55)
-            y = nn.causal_attention(q, k, v, self.scale)                                     # (B, h, T, d)
-            return self.c_proj(y.transpose(1, 2).reshape((B, T, C)))
+            # split into heads, ((q @ k^T) * scale).masked_fill(mask, -inf).softmax(dim=3) @ v, merge the
+            # heads (examples/gpt.py:45-57): one node that works on the (B, T, C) projections in place
+            return self.c_proj(nn.causal_self_attention(q_lin, k_lin, v_lin, self.n_head, self.scale))
         y = (att @ v).transpose(1, 2).reshape((B, T, C))
         return self.c_proj(y)
 

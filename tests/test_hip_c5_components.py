@@ -254,3 +254,33 @@ def test_causal_attention_never_reads_what_it_skipped(shape):
     for name, a, b in zip(("y", "dq", "dk", "dv"), dirty, clean):
         assert np.isfinite(a).all(), name
         assert (a.view(np.uint32) == b.view(np.uint32)).all(), name
+
+
+@pytest.mark.parametrize("B,T,h,d", [(2, 128, 4, 32), (1, 1024, 12, 64), (3, 100, 2, 20), (2, 257, 1, 64), (4, 16, 2, 6), (2, 130, 3, 7)])
+def test_attention_on_the_projections_equals_split_attend_merge(B, T, h, d, monkeypatch):
+    """nn.causal_self_attention takes q, k, v as (B, T, h*d) and reads every head where it lies
+    (strided product kernels) instead of transposing to (B, h, T, d) and back.  Output and the
+    gradients of the three projections are bit-identical to reshape -> transpose -> attention ->
+    transpose -> reshape, including head sizes that force 4-byte accesses."""
+    require_gpu()
+    from dlgrad_amd import nn, ops
+    rng = np.random.default_rng(72)
+    C = h * d
+    q, k, v, g = (rng.standard_normal((B, T, C), dtype=np.float32) for _ in range(4))
+    scale = d ** -0.5
+
+    def run(fused):
+        monkeypatch.setattr(ops, "use_fused_attention_heads", (lambda *a: False) if not fused else ops.use_fused_attention_heads)
+        ts = [Tensor(a, device="hip", requires_grad=True) for a in (q, k, v)]
+        y = nn.causal_self_attention(*ts, h, scale)
+        node = type(y._ctx).__name__
+        (y * Tensor(g, device="hip")).sum().backward()
+        return node, [y.numpy()] + [t.grad.numpy() for t in ts]
+
+    (n1, fused), (n0, chain) = run(True), run(False)
+    assert n1 == "CausalAttentionHeads" and n0 != "CausalAttentionHeads"
+    if hip.COMPILE_ONLY:
+        return
+    for name, a, b in zip(("y", "dq", "dk", "dv"), fused, chain):
+        assert a.shape == (B, T, C)
+        assert (a.view(np.uint32) == b.view(np.uint32)).all(), f"{name} B{B} T{T} h{h} d{d}"
