@@ -348,6 +348,13 @@ class Buffer:
         dq, dk, dv = self._dispatch(CustomOps.CAUSAL_ATTENTION_BWD, q=self, k=k, v=v, p=p, dy=dy, n_head=n_head, scale=scale)
         return self._like(dq), self._like(dk), self._like(dv)
 
+    def cached_attention(self, k_store: "Buffer", v_store: "Buffer", n: int, n_head: int, scale: float,
+                         hidden: "Buffer | None" = None) -> "Buffer":
+        """self: (B, 1, C) query projection; k_store, v_store: (block, B, C) caches of which the first n
+        rows take part (minus those `hidden` marks).  Returns the context (B, 1, C)."""
+        return self._like(self._dispatch(CustomOps.CACHED_ATTENTION, q=self, k_store=k_store, v_store=v_store, n=n,
+                                         n_head=n_head, scale=scale, hidden=hidden))
+
     def log_softmax(self, dim: int) -> "Buffer":
         return self._unary(CustomOps.LOG_SOFTMAX, dim=dim)
 

@@ -79,3 +79,24 @@ def causal_self_attention(q: Tensor, k: Tensor, v: Tensor, n_head: int, scale: f
     split = (B, T, n_head, C // n_head)
     qh, kh, vh = (t.reshape(split).transpose(1, 2) for t in (q, k, v))
     return causal_attention(qh, kh, vh, scale).transpose(1, 2).reshape((B, T, C))
+
+
+def cached_attention(q: Tensor, k_store: Tensor, v_store: Tensor, n: int, n_head: int, scale: float,
+                     hidden: Tensor | None = None) -> Tensor:
+    """Attention of one new position per sequence over a key/value cache, for inference: q is the
+    (B, 1, C) query projection, k_store and v_store are (block, B, C) with the first n rows in use,
+    `hidden` (1, 1, 1, n) marks rows to leave out.  The else-branch of the reference's attention
+    (examples/gpt.py:58-63) without its host concatenation.  On the hip device the heads are read
+    in place from q and from the stores; elsewhere the views are materialised as there."""
+    B, _, C = q.shape
+    if ops.FUSED and q.device is Device.HIP and k_store.device is Device.HIP and v_store.device is Device.HIP \
+            and ops.softmax_row_fits(n):
+        h = None if hidden is None else hidden.data
+        return Tensor(q.data.cached_attention(k_store.data, v_store.data, n, n_head, scale, h))
+    split = (n, B, n_head, C // n_head)
+    k = k_store[0:n].reshape(split).permute((1, 2, 0, 3))                  # (B, h, n, d)
+    v = v_store[0:n].reshape(split).permute((1, 2, 0, 3))
+    qh = q.reshape((B, 1, n_head, C // n_head)).transpose(1, 2)            # (B, h, 1, d)
+    att = qh @ k.transpose(2, 3)
+    att = (att * scale).softmax(dim=3) if hidden is None else att.masked_softmax(hidden, scale, dim=3)
+    return (att @ v).transpose(1, 2).reshape((B, 1, C))

@@ -427,6 +427,12 @@ class CausalAttention(OP):
         return dq, dk, dv
 
 
+def softmax_row_fits(n: int) -> bool:
+    """Whether a row of n scores fits the register-resident masked softmax kernels."""
+    from dlgrad_amd.runtime.hip import HIP
+    return HIP.causal_softmax_fits(n)
+
+
 def use_fused_attention_heads(q, k, v, n_head: int) -> bool:
     if not (FUSED and q.device is Device.HIP and k.device is Device.HIP and v.device is Device.HIP):
         return False

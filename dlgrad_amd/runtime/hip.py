@@ -158,7 +158,7 @@ class DevicePtr:
 
     def __del__(self) -> None:
         if self.base is None and self.addr:
-            l = _state["lib"]
+            l = _state["lib"] if _state is not None else None      # module globals are gone at interpreter exit
             if l is not None:
                 try:
                     l.free(self.addr)
@@ -1491,6 +1491,34 @@ class HIP:
         HIP._gemm_strided((p.addr, T, n_head * T * T, T * T), HIP._heads(_addr(v), T, C, d), HIP._heads(y.addr, T, C, d),
                           T, d, T, Bn, n_head, tri="a_lower")
         return y, p
+
+    @staticmethod
+    @dispatcher.register(CustomOps.CACHED_ATTENTION, Device.HIP)
+    def cached_attention(q: Buffer, k_store: Buffer, v_store: Buffer, n: int, n_head: int, scale: float,
+                         hidden: Buffer | None = None) -> DevicePtr:
+        """One new position per sequence, q (B, 1, C), attending to the first n rows of key/value
+        stores laid out (block, B, C): softmax(q k^T * scale) v per head, the heads read where they
+        lie in q and in the stores and the context written as (B, 1, C).  `hidden` (.., n) marks rows
+        to leave out (-inf before the softmax).  Inference only."""
+        Bn, _, C = q.shape
+        d = C // n_head
+        store_heads = lambda buf: (_addr(buf), Bn * C, C, d)                        # noqa: E731  rows = positions
+        one_row = lambda addr: (addr, C, C, d)                                        # noqa: E731  (B, 1, C)
+        s = alloc(Bn * n_head * n)
+        dense = (s.addr, n, n_head * n, n)
+        HIP._gemm_strided(one_row(_addr(q)), store_heads(k_store), dense, 1, n, d, Bn, n_head, tb=True)
+        if hidden is None:                                   # nothing to leave out: a mask of zeros
+            if _graph_depth:
+                zeros = alloc(n, zero=True)                      # an arena's memory must not outlive it
+            else:
+                zeros = _state.get("zeros")
+                if zeros is None or zeros.nbytes < 4 * n:
+                    zeros = _state["zeros"] = alloc(max(n, 1024), zero=True)
+            hidden = Buffer(zeros, (n,), Device.HIP)
+        p = HIP.masked_softmax(Buffer(s, (Bn, n_head, 1, n), Device.HIP), hidden, scale)
+        y = alloc(Bn * C)
+        HIP._gemm_strided((p.addr, n, n_head * n, n), store_heads(v_store), one_row(y.addr), 1, d, n, Bn, n_head)
+        return y
 
     @staticmethod
     @dispatcher.register(CustomOps.CAUSAL_ATTENTION_BWD, Device.HIP)

@@ -39,22 +39,19 @@ class CausalSelfAttention:
         (whose k/v projections are stored if a cache is given).  With a filled cache and
         T == 1: the new position attends to everything cached plus itself, no mask
         (examples/gpt.py:44-66)."""
-        B, T, C = x.shape
-        split = (B, T, self.n_head, self.head_dim)
+        T = x.shape[1]
         q_lin, k_lin, v_lin = self.q_proj(x), self.k_proj(x), self.v_proj(x)    # (B, T, C)
         if cache is not None and cache.length > 0:
             assert T == 1, "incremental attention takes one new position"
-            q = q_lin.reshape(split).transpose(1, 2)                  # (B, h, 1, d)
             cache.write(layer, k_lin, v_lin, cache.length)
-            k, v = cache.view(layer, cache.length + 1, self.n_head)  # (B, h, n, d)
-            att = ((q @ k.transpose(2, 3)) * self.scale).softmax(dim=3)
+            # the heads of q against the heads of everything cached (examples/gpt.py:58-63)
+            y = nn.cached_attention(q_lin, cache.k[layer], cache.v[layer], cache.length + 1, self.n_head, self.scale)
         else:
             if cache is not None:
                 cache.write(layer, k_lin, v_lin, 0)
             # split into heads, ((q @ k^T) * scale).masked_fill(mask, -inf).softmax(dim=3) @ v, merge the
             # heads (examples/gpt.py:45-57): one node that works on the (B, T, C) projections in place
-            return self.c_proj(nn.causal_self_attention(q_lin, k_lin, v_lin, self.n_head, self.scale))
-        y = (att @ v).transpose(1, 2).reshape((B, T, C))
+            y = nn.causal_self_attention(q_lin, k_lin, v_lin, self.n_head, self.scale)
         return self.c_proj(y)
 
 
@@ -62,8 +59,9 @@ class KVCache:
     """The k and v projections of every position so far, per layer, on the model's device.
 
     Stored as (block_size, B, C): the first n positions are then one contiguous view, and
-    appending a position is a single device-to-device copy of B*C floats.  `view` hands
-    attention the same (B, h, n, d) values the reference gets by concatenating on the host."""
+    appending a position is a single device-to-device copy of B*C floats.  nn.cached_attention
+    reads the heads of those rows in place: the same (B, h, n, d) values the reference gets by
+    concatenating on the host."""
 
     def __init__(self, c: GPTConfig, batch: int) -> None:
         shape = (c.block_size, batch, c.n_embd)
@@ -77,12 +75,6 @@ class KVCache:
         for store, new in ((self.k[layer], k), (self.v[layer], v)):
             rows = new if (B == 1 or T == 1) else new.transpose(0, 1)          # (T, B, C) order
             store[at:at + T].data.copy_(rows.data)
-
-    def view(self, layer: int, n: int, n_head: int) -> tuple[Tensor, Tensor]:
-        C = self.k[layer].shape[2]
-        split = (n, self.batch, n_head, C // n_head)
-        return (self.k[layer][0:n].reshape(split).permute((1, 2, 0, 3)),
-                self.v[layer][0:n].reshape(split).permute((1, 2, 0, 3)))
 
 
 class MLP:
@@ -226,14 +218,11 @@ class StaticDecoder:
         self.seq.data.upload_(first)
 
     def _attend(self, attn: CausalSelfAttention, x: Tensor, layer: int, hidden: Tensor) -> Tensor:
-        C = x.shape[2]
         T = self.model.config.block_size
-        q = attn.q_proj(x).reshape((1, 1, attn.n_head, attn.head_dim)).transpose(1, 2)      # (1, h, 1, d)
         self.cache.k[layer].data.row_store_(attn.k_proj(x).data, self.slot.data)
         self.cache.v[layer].data.row_store_(attn.v_proj(x).data, self.slot.data)
-        k, v = self.cache.view(layer, T, attn.n_head)                                       # (1, h, T, d)
-        att = (q @ k.transpose(2, 3)).masked_softmax(hidden, attn.scale, dim=3)              # (1, h, 1, T)
-        return attn.c_proj((att @ v).transpose(1, 2).reshape((1, 1, C)))
+        y = nn.cached_attention(attn.q_proj(x), self.cache.k[layer], self.cache.v[layer], T, attn.n_head, attn.scale, hidden)
+        return attn.c_proj(y)
 
     def step(self) -> None:
         """Feeds self.tok at index self.slot; leaves the argmax in seq[slot + 1] and as the next
