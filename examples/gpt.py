@@ -192,7 +192,7 @@ class StaticDecoder:
     """Greedy decoding inside the context window as one step of fixed shape.
 
     forward_incremental attends to a cache that grows by one row per token, so every token has
-    new tensor shapes and must be issued launch by launch from Python (~170 launches per token
+    new tensor shapes and must be issued launch by launch from Python (~130 launches per token
     for the char model, which is what bounds its speed).  Here the step always attends to all
     block_size cache rows and masks the ones not written yet (-inf before the softmax, so they
     weigh exactly 0), and everything that changes from token to token -- the token, the cache
