@@ -159,6 +159,9 @@ class Relu(OP):
         return self.out
 
     def backward(self, upstream_grad: Buffer) -> tuple:
+        if FUSED and self.out.device is Device.HIP and upstream_grad.shape == self.out.shape:
+            # the 0/1 mask times the gradient as one select: the gradient where out > 0, else 0
+            return (self.out.where(inp=upstream_grad, other=0.0),)
         return (self.out.where(inp=1.0, other=0.0) * upstream_grad,)
 
 
