@@ -348,6 +348,17 @@ class Buffer:
         dq, dk, dv = self._dispatch(CustomOps.CAUSAL_ATTENTION_BWD, q=self, k=k, v=v, p=p, dy=dy, n_head=n_head, scale=scale)
         return self._like(dq), self._like(dk), self._like(dv)
 
+    def causal_attention_qkv(self, n_head: int, scale: float) -> tuple["Buffer", "Buffer"]:
+        """self: (B, T, 3C) with q, k, v side by side per position.  Returns the context (B, T, C) and the
+        probabilities (B, n_head, T, T)."""
+        B, T, C3 = self.shape
+        y, p = self._dispatch(CustomOps.CAUSAL_ATTENTION_QKV, qkv=self, n_head=n_head, scale=scale)
+        return self._like(y, (B, T, C3 // 3)), self._like(p, (B, n_head, T, T))
+
+    def causal_attention_qkv_bwd(self, p: "Buffer", dy: "Buffer", n_head: int, scale: float) -> "Buffer":
+        """Gradient of causal_attention_qkv with respect to self, same (B, T, 3C) layout."""
+        return self._like(self._dispatch(CustomOps.CAUSAL_ATTENTION_QKV_BWD, qkv=self, p=p, dy=dy, n_head=n_head, scale=scale))
+
     def cached_attention(self, k_store: "Buffer", v_store: "Buffer", n: int, n_head: int, scale: float,
                          hidden: "Buffer | None" = None) -> "Buffer":
         """self: (B, 1, C) query projection; k_store, v_store: (block, B, C) caches of which the first n

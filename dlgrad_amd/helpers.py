@@ -70,6 +70,8 @@ class CustomOps(Enum):
     MASKED_SOFTMAX_BWD = auto()     # its backward, one kernel
     CAUSAL_ATTENTION = auto()       # softmax(mask(q k^T * scale)) v on (B, T, heads*d) projections, heads read in place
     CAUSAL_ATTENTION_BWD = auto()
+    CAUSAL_ATTENTION_QKV = auto()   # the same for q, k, v interleaved as one (B, T, 3C) projection
+    CAUSAL_ATTENTION_QKV_BWD = auto()
     CACHED_ATTENTION = auto()       # one new position attending to the rows of a (block, B, heads*d) key/value cache in place
     LOG_SOFTMAX = auto()
     LOG_SOFTMAX_GATHER = auto()     # log-softmax rows + the ce_forward gather, one kernel

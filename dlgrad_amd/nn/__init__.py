@@ -100,3 +100,30 @@ def cached_attention(q: Tensor, k_store: Tensor, v_store: Tensor, n: int, n_head
     att = qh @ k.transpose(2, 3)
     att = (att * scale).softmax(dim=3) if hidden is None else att.masked_softmax(hidden, scale, dim=3)
     return (att @ v).transpose(1, 2).reshape((B, 1, C))
+
+
+def stack_parameters(tensors: list) -> None:
+    """Moves the data of equally shaped parameter tensors into one allocation, back to back in the
+    given order (values kept, each tensor now a view of its part).  Nothing else about them
+    changes -- names, shapes, gradients, optimizer and checkpoint handling -- but kernels may
+    treat them as one matrix: see self_attention_qkv.  A no-op off the hip device."""
+    first = tensors[0]
+    if first.device is not Device.HIP or any(t.shape != first.shape or t.device is not Device.HIP for t in tensors):
+        return
+    from dlgrad_amd.buffer import Buffer
+    n = first.numel
+    base = Buffer.full((len(tensors) * n,), 0.0, Device.HIP)
+    for i, t in enumerate(tensors):
+        part = Buffer(base.ptr + i * n, t.shape, Device.HIP)
+        part.copy_(t.data)
+        t.data = part
+
+
+def self_attention_qkv(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor, n_head: int, scale: float) -> Tensor:
+    """causal_self_attention(x @ wq^T, x @ wk^T, x @ wv^T, n_head, scale) for x (B, T, C) and three
+    (C, C) weights: the projections and attention of examples/gpt.py:45-57.  When the weights are
+    stacked in memory (stack_parameters) the hip device runs one projection and reads q, k, v out
+    of its result in place (ops.SelfAttentionQKV)."""
+    if ops.use_fused_qkv_attention(x, wq, wk, wv, n_head):
+        return ops.SelfAttentionQKV.execute(x, wq, wk, wv, n_head=n_head, scale=scale)
+    return causal_self_attention(x.linear(wq, None), x.linear(wk, None), x.linear(wv, None), n_head, scale)

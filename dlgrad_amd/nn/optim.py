@@ -7,6 +7,16 @@ from dlgrad_amd.device import Device
 from dlgrad_amd.tensor import Tensor
 
 
+def _rebind(p: Tensor, new) -> None:
+    """p.data = new, as the reference's optimizers do -- except for a parameter that is a view into a
+    shared allocation (nn.stack_parameters): its new value is copied into place, so it stays where the
+    kernels that rely on the stacking expect it."""
+    if getattr(p.data.ptr, "base", None) is not None:
+        p.data.copy_(new)
+    else:
+        p.data = new
+
+
 class Optimizer:
     def __init__(self, params: list[Tensor], lr: float = 1e-1) -> None:
         self.params = params
@@ -15,7 +25,7 @@ class Optimizer:
     def step(self) -> None:
         for p in self.params:
             assert p.shape == p.grad.shape, f"The shape of the parameter {p.shape} and its grad {p.grad.shape} do not match"
-            p.data = (p - p.grad * self.lr).data
+            _rebind(p, (p - p.grad * self.lr).data)
 
     def zero_grad(self) -> None:
         for p in self.params:
@@ -45,7 +55,7 @@ class SGD(Optimizer):
             if self.momentum != 0:
                 upd = self.velocities[id(p)] * self.momentum + p.grad          # v = mu * v + g
                 self.velocities[id(p)] = upd
-            p.data = (p - upd * self.lr).data
+            _rebind(p, (p - upd * self.lr).data)
 
 
 class Adam(Optimizer):
@@ -102,9 +112,10 @@ class Adam(Optimizer):
             if ops.FUSED and p.device is Device.HIP:
                 # same fp32 operations in the same order as below, in one kernel (bit-identical)
                 pb, mb, vb = p.data.adam_step(g.data, self.m[k].data, self.v[k].data, consts)
-                p.data, self.m[k], self.v[k] = pb, Tensor(mb), Tensor(vb)
+                _rebind(p, pb)
+                self.m[k], self.v[k] = Tensor(mb), Tensor(vb)
                 continue
             self.m[k] = ((self.m[k] * self.beta1) + (g * (1.0 - self.beta1))).detach()
             self.v[k] = ((self.v[k] * self.beta2) + ((g ** 2.0) * (1.0 - self.beta2))).detach()
             m_hat, v_hat = self.m[k] / c1, self.v[k] / c2
-            p.data = (p - (m_hat / (v_hat.sqrt() + self.eps)) * self.lr).data
+            _rebind(p, (p - (m_hat / (v_hat.sqrt() + self.eps)) * self.lr).data)

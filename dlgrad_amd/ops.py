@@ -461,6 +461,51 @@ class CausalAttentionHeads(OP):
         return self.q.causal_attention_bwd(self.k, self.v, self.p, upstream_grad, self.n_head, self.scale)
 
 
+def stacked(wq, wk, wv) -> bool:
+    """Whether three equal (C, C) weights lie back to back in one allocation, in this order, so that
+    together they are one (3C, C) matrix (nn.stack_parameters arranges that)."""
+    if not (wq.ndim == 2 and wq.shape == wk.shape == wv.shape and wq.device is Device.HIP):
+        return False
+    step = 4 * wq.numel
+    a = [getattr(w.data.ptr, "addr", None) for w in (wq, wk, wv)]
+    return None not in a and a[1] == a[0] + step and a[2] == a[1] + step
+
+
+def use_fused_qkv_attention(x, wq, wk, wv, n_head: int) -> bool:
+    if not (FUSED and x.device is Device.HIP and x.ndim == 3 and x.numel and n_head > 0):
+        return False
+    C = x.shape[2]
+    if wq.shape != (C, C) or C % n_head or not stacked(wq, wk, wv):
+        return False
+    return softmax_row_fits(x.shape[1])
+
+
+class SelfAttentionQKV(OP):
+    """The three projections and the causal attention of examples/gpt.py:45-57 for weights that are
+    stacked in memory: one product x W^T with W = [Wq; Wk; Wv] gives q, k, v side by side, the
+    attention kernels read their heads there (row pitch 3C), and backward is one product for dx
+    (K = 3C), one for the stacked dW and the attention gradients written into one (B, T, 3C) buffer.
+    Per layer 3 + 6 products and two gradient additions become 1 + 2.  q, k, v, the context and
+    the weight gradients have the bits of the separate products; dx adds its 3C terms in one
+    accumulator instead of three partial sums, so it differs from them by rounding."""
+
+    def forward(self, x: Buffer, wq: Buffer, wk: Buffer, wv: Buffer, n_head: int, scale: float) -> Buffer:
+        C = wq.shape[0]
+        self.x, self.n_head, self.scale = x, n_head, scale
+        self.w = Buffer(wq.ptr, (3 * C, C), x.device)                    # the three matrices as one
+        self.qkv = x.matmul_nt(self.w)
+        y, self.p = self.qkv.causal_attention_qkv(n_head, scale)
+        return y
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        C = self.w.shape[1]
+        g = self.qkv.causal_attention_qkv_bwd(self.p, upstream_grad, self.n_head, self.scale)     # (B, T, 3C)
+        dx = g @ self.w
+        dw = unbroadcast(g.matmul_tn(self.x), self.w.shape)                                       # (3C, C)
+        part = lambda i: Buffer(dw.ptr + i * C * C, (C, C), dw.device)                            # noqa: E731
+        return dx, part(0), part(1), part(2)
+
+
 def use_fused_rmsnorm(x, weight) -> bool:
     if not (FUSED and x.device is Device.HIP):
         return False

@@ -1471,6 +1471,64 @@ class HIP:
         return (addr, C, T * C, d)
 
     @staticmethod
+    def _attend(qa: int, ka: int, va: int, pitch: int, ya: int, y_pitch: int, Bn: int, T: int, n_head: int, d: int,
+                scale: float) -> DevicePtr:
+        """Causal attention over heads that lie at addresses qa, ka, va with row pitch `pitch` (batch
+        stride T * pitch, head stride d); the context goes to ya with pitch y_pitch.  Returns the
+        probabilities (Bn, n_head, T, T)."""
+        from dlgrad_amd.ops import causal_mask
+        raw = alloc(Bn * n_head * T * T)
+        dense = lambda addr: (addr, T, n_head * T * T, T * T)                       # noqa: E731
+        HIP._gemm_strided(HIP._heads(qa, T, pitch, d), HIP._heads(ka, T, pitch, d), dense(raw.addr), T, T, d, Bn, n_head,
+                          tb=True, tri="out_lower")
+        p = HIP.masked_softmax(Buffer(raw, (Bn, n_head, T, T), Device.HIP), causal_mask(T, Device.HIP), scale)
+        HIP._gemm_strided(dense(p.addr), HIP._heads(va, T, pitch, d), HIP._heads(ya, T, y_pitch, d),
+                          T, d, T, Bn, n_head, tri="a_lower")
+        return p
+
+    @staticmethod
+    def _attend_bwd(qa: int, ka: int, va: int, pitch: int, p: Buffer, dya: int, dy_pitch: int, dqa: int, dka: int,
+                    dva: int, g_pitch: int, Bn: int, T: int, n_head: int, d: int, scale: float) -> None:
+        """Gradients of _attend, written to dqa, dka, dva with row pitch g_pitch."""
+        from dlgrad_amd.ops import causal_mask
+        dense = lambda addr: (addr, T, n_head * T * T, T * T)                       # noqa: E731
+        dp = alloc(p.numel)
+        HIP._gemm_strided(HIP._heads(dya, T, dy_pitch, d), HIP._heads(va, T, pitch, d), dense(dp.addr), T, T, d, Bn, n_head,
+                          tb=True, tri="out_lower")
+        HIP._gemm_strided(dense(_addr(p)), HIP._heads(dya, T, dy_pitch, d), HIP._heads(dva, T, g_pitch, d),
+                          T, d, T, Bn, n_head, ta=True, tri="at_lower")
+        ds = HIP.masked_softmax_bwd(p, Buffer(dp, p.shape, Device.HIP), causal_mask(T, Device.HIP), scale)
+        HIP._gemm_strided(dense(ds.addr), HIP._heads(ka, T, pitch, d), HIP._heads(dqa, T, g_pitch, d),
+                          T, d, T, Bn, n_head, tri="a_lower")
+        HIP._gemm_strided(dense(ds.addr), HIP._heads(qa, T, pitch, d), HIP._heads(dka, T, g_pitch, d),
+                          T, d, T, Bn, n_head, ta=True, tri="at_lower")
+
+    @staticmethod
+    @dispatcher.register(CustomOps.CAUSAL_ATTENTION_QKV, Device.HIP)
+    def causal_attention_qkv(qkv: Buffer, n_head: int, scale: float) -> tuple[DevicePtr, DevicePtr]:
+        """causal_attention for q, k and v interleaved per position as one (B, T, 3C) tensor -- the
+        output of a single projection with the three weight matrices stacked: the heads are read
+        with row pitch 3C.  Returns (y (B, T, C), p)."""
+        Bn, T, C3 = qkv.shape
+        C = C3 // 3
+        a = _addr(qkv)
+        y = alloc(Bn * T * C)
+        p = HIP._attend(a, a + 4 * C, a + 8 * C, C3, y.addr, C, Bn, T, n_head, C // n_head, scale)
+        return y, p
+
+    @staticmethod
+    @dispatcher.register(CustomOps.CAUSAL_ATTENTION_QKV_BWD, Device.HIP)
+    def causal_attention_qkv_bwd(qkv: Buffer, p: Buffer, dy: Buffer, n_head: int, scale: float) -> DevicePtr:
+        """Gradient of causal_attention_qkv with respect to qkv, in the same (B, T, 3C) layout."""
+        Bn, T, C3 = qkv.shape
+        C = C3 // 3
+        a = _addr(qkv)
+        g = alloc(Bn * T * C3)
+        HIP._attend_bwd(a, a + 4 * C, a + 8 * C, C3, p, _addr(dy), C, g.addr, g.addr + 4 * C, g.addr + 8 * C, C3,
+                        Bn, T, n_head, C // n_head, scale)
+        return g
+
+    @staticmethod
     @dispatcher.register(CustomOps.CAUSAL_ATTENTION, Device.HIP)
     def causal_attention(q: Buffer, k: Buffer, v: Buffer, n_head: int, scale: float) -> tuple[DevicePtr, DevicePtr]:
         """Causal attention for q, k, v given as (B, T, C) projections with C = n_head * d: the heads are
@@ -1479,17 +1537,8 @@ class HIP:
         probabilities p (B, n_head, T, T) kept for the backward pass.  The products and the
         softmax are the kernels of the op-by-op chain, with the causal structure known."""
         Bn, T, C = q.shape
-        d = C // n_head
-        p_scores = alloc(Bn * n_head * T * T)
-        dense = (p_scores.addr, T, n_head * T * T, T * T)
-        HIP._gemm_strided(HIP._heads(_addr(q), T, C, d), HIP._heads(_addr(k), T, C, d), dense, T, T, d, Bn, n_head,
-                          tb=True, tri="out_lower")
-        scores = Buffer(p_scores, (Bn, n_head, T, T), Device.HIP)
-        from dlgrad_amd.ops import causal_mask
-        p = HIP.masked_softmax(scores, causal_mask(T, Device.HIP), scale)
         y = alloc(Bn * T * C)
-        HIP._gemm_strided((p.addr, T, n_head * T * T, T * T), HIP._heads(_addr(v), T, C, d), HIP._heads(y.addr, T, C, d),
-                          T, d, T, Bn, n_head, tri="a_lower")
+        p = HIP._attend(_addr(q), _addr(k), _addr(v), C, y.addr, C, Bn, T, n_head, C // n_head, scale)
         return y, p
 
     @staticmethod
@@ -1526,18 +1575,7 @@ class HIP:
                              scale: float) -> tuple[DevicePtr, DevicePtr, DevicePtr]:
         """Gradients of causal_attention with respect to the (B, T, C) projections, written in that layout."""
         Bn, T, C = q.shape
-        d = C // n_head
-        pd = (_addr(p), T, n_head * T * T, T * T)
-        heads = lambda buf_addr: HIP._heads(buf_addr, T, C, d)                     # noqa: E731
-        dp = alloc(p.numel)
-        HIP._gemm_strided(heads(_addr(dy)), heads(_addr(v)), (dp.addr, T, n_head * T * T, T * T), T, T, d, Bn, n_head,
-                          tb=True, tri="out_lower")
-        dv = alloc(Bn * T * C)
-        HIP._gemm_strided(pd, heads(_addr(dy)), heads(dv.addr), T, d, T, Bn, n_head, ta=True, tri="at_lower")
-        from dlgrad_amd.ops import causal_mask
-        ds = HIP.masked_softmax_bwd(p, Buffer(dp, p.shape, Device.HIP), causal_mask(T, Device.HIP), scale)
-        dsd = (ds.addr, T, n_head * T * T, T * T)
-        dq, dk = alloc(Bn * T * C), alloc(Bn * T * C)
-        HIP._gemm_strided(dsd, heads(_addr(k)), heads(dq.addr), T, d, T, Bn, n_head, tri="a_lower")
-        HIP._gemm_strided(dsd, heads(_addr(q)), heads(dk.addr), T, d, T, Bn, n_head, ta=True, tri="at_lower")
+        dq, dk, dv = alloc(Bn * T * C), alloc(Bn * T * C), alloc(Bn * T * C)
+        HIP._attend_bwd(_addr(q), _addr(k), _addr(v), C, p, _addr(dy), C, dq.addr, dk.addr, dv.addr, C,
+                        Bn, T, n_head, C // n_head, scale)
         return dq, dk, dv

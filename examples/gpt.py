@@ -33,6 +33,8 @@ class CausalSelfAttention:
         self.k_proj = nn.Linear(c.n_embd, c.n_embd, bias=False, device=c.device)
         self.v_proj = nn.Linear(c.n_embd, c.n_embd, bias=False, device=c.device)
         self.c_proj = nn.Linear(c.n_embd, c.n_embd, bias=False, device=c.device)
+        # same three parameters, placed back to back so that one product can serve all three projections
+        nn.stack_parameters([self.q_proj.weight, self.k_proj.weight, self.v_proj.weight])
 
     def __call__(self, x: Tensor, cache: "KVCache | None" = None, layer: int = 0) -> Tensor:
         """Without a cache, or with an empty one: causal attention over the T positions of x
@@ -40,17 +42,19 @@ class CausalSelfAttention:
         T == 1: the new position attends to everything cached plus itself, no mask
         (examples/gpt.py:44-66)."""
         T = x.shape[1]
+        if cache is None:
+            # q, k, v projections, split into heads, ((q @ k^T) * scale).masked_fill(mask, -inf).softmax(dim=3) @ v,
+            # merge the heads (examples/gpt.py:45-57): one node on the hip device
+            return self.c_proj(nn.self_attention_qkv(x, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight,
+                                                     self.n_head, self.scale))
         q_lin, k_lin, v_lin = self.q_proj(x), self.k_proj(x), self.v_proj(x)    # (B, T, C)
-        if cache is not None and cache.length > 0:
+        if cache.length > 0:
             assert T == 1, "incremental attention takes one new position"
             cache.write(layer, k_lin, v_lin, cache.length)
             # the heads of q against the heads of everything cached (examples/gpt.py:58-63)
             y = nn.cached_attention(q_lin, cache.k[layer], cache.v[layer], cache.length + 1, self.n_head, self.scale)
         else:
-            if cache is not None:
-                cache.write(layer, k_lin, v_lin, 0)
-            # split into heads, ((q @ k^T) * scale).masked_fill(mask, -inf).softmax(dim=3) @ v, merge the
-            # heads (examples/gpt.py:45-57): one node that works on the (B, T, C) projections in place
+            cache.write(layer, k_lin, v_lin, 0)               # prefill: the projections are kept for later tokens
             y = nn.causal_self_attention(q_lin, k_lin, v_lin, self.n_head, self.scale)
         return self.c_proj(y)
 
@@ -274,10 +278,9 @@ def init_weights_(model: GPT, seed: int, std: float = 0.02) -> None:
     """Overwrites every parameter with seeded numpy values: N(0, std) for matrices and
     embeddings, ones for the RMSNorm gains -- the same values on any device."""
     rng = np.random.default_rng(seed)
-    dev = model.config.device
     for name, p in nn.utils.get_state_dict(model).items():
         if ".ln" in f".{name}" and name.endswith("weight"):
             w = np.ones(p.shape, dtype=np.float32)
         else:
             w = (rng.standard_normal(p.shape) * std).astype(np.float32)
-        p.data = Tensor(w, device=dev).data
+        p.data.upload_(w)                                # in place: parameters keep their addresses (and their stacking)

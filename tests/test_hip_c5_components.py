@@ -284,3 +284,42 @@ def test_attention_on_the_projections_equals_split_attend_merge(B, T, h, d, monk
     for name, a, b in zip(("y", "dq", "dk", "dv"), fused, chain):
         assert a.shape == (B, T, C)
         assert (a.view(np.uint32) == b.view(np.uint32)).all(), f"{name} B{B} T{T} h{h} d{d}"
+
+
+@pytest.mark.parametrize("B,T,h,d", [(2, 128, 4, 32), (1, 1024, 12, 64), (3, 100, 2, 20), (2, 33, 3, 7)])
+def test_stacked_qkv_attention_equals_three_projections_and_attention(B, T, h, d, monkeypatch):
+    """nn.self_attention_qkv with weights that nn.stack_parameters placed back to back: one
+    projection, heads read out of its (B, T, 3C) result.  The context and the three weight
+    gradients have the bits of the separate route (three projections, attention on the
+    projections); dx adds its 3C terms in one accumulator instead of three partial sums and
+    agrees to 1e-5 of the largest entry (a 2304-term fp32 sum at C = 768)."""
+    require_gpu()
+    from dlgrad_amd import nn, ops
+    rng = np.random.default_rng(73)
+    C = h * d
+    x, g = (rng.standard_normal((B, T, C), dtype=np.float32) for _ in range(2))
+    ws = [rng.standard_normal((C, C), dtype=np.float32) * C ** -0.5 for _ in range(3)]
+    scale = d ** -0.5
+
+    def run(fused):
+        monkeypatch.setattr(ops, "use_fused_qkv_attention", (lambda *a: False) if not fused else ops.use_fused_qkv_attention)
+        xt = Tensor(x, device="hip", requires_grad=True)
+        wt = [Tensor(w, device="hip", requires_grad=True) for w in ws]
+        nn.stack_parameters(wt)
+        assert ops.stacked(*wt) or hip.COMPILE_ONLY
+        for t, w in zip(wt, ws):
+            check(t.numpy(), w, 0, "stacking keeps the values")
+        y = nn.self_attention_qkv(xt, *wt, h, scale)
+        node = type(y._ctx).__name__
+        (y * Tensor(g, device="hip")).sum().backward()
+        return node, [y.numpy(), xt.grad.numpy()] + [t.grad.numpy() for t in wt]
+
+    (n1, fused), (n0, chain) = run(True), run(False)
+    assert n1 == "SelfAttentionQKV" and n0 != "SelfAttentionQKV"
+    if hip.COMPILE_ONLY:
+        return
+    for name, a, b in zip(("y", "dx", "dwq", "dwk", "dwv"), fused, chain):
+        if name == "dx":
+            assert np.abs(a - b).max() <= 1e-5 * np.abs(b).max(), name
+        else:
+            assert (a.view(np.uint32) == b.view(np.uint32)).all(), f"{name} B{B} T{T} h{h} d{d}"
