@@ -242,20 +242,23 @@ class Buffer:
         do not know it compute the whole product, which gives the same kept values."""
         return {"tri": tri} if tri and self.device is Device.HIP else {}
 
-    def matmul(self, other: "Buffer", tri: str = "") -> "Buffer":
+    def matmul(self, other: "Buffer", tri: str = "", epi: str = "", e: "Buffer | None" = None) -> "Buffer":
+        """epi / e (hip only): an element-wise step fused into the store of the result, see HIP.matmul."""
         p1, p2, out_shape = broadcast_shapes(self.shape, other.shape)
         x = self if self.shape == p1 else self._like(self.ptr, p1)
         y = other if other.shape == p2 else other._like(other.ptr, p2)
-        return self._like(self._dispatch(BinaryOps.MATMUL, x=x, y=y, **self._tri(tri)), out_shape)
+        kw = {"epi": epi, "e": e} if epi else {}
+        return self._like(self._dispatch(BinaryOps.MATMUL, x=x, y=y, **self._tri(tri), **kw), out_shape)
 
-    def matmul_nt(self, other: "Buffer", tri: str = "") -> "Buffer":
+    def matmul_nt(self, other: "Buffer", tri: str = "", epi: str = "", e: "Buffer | None" = None) -> "Buffer":
         """self (.., M, K) @ other(.., N, K)^T without materialising the transpose."""
         swapped = other.shape[:-2] + (other.shape[-1], other.shape[-2])
         p1, p2, out_shape = broadcast_shapes(self.shape, swapped)
         p2 = p2[:-2] + (p2[-1], p2[-2])
         x = self if self.shape == p1 else self._like(self.ptr, p1)
         y = other if other.shape == p2 else other._like(other.ptr, p2)
-        return self._like(self._dispatch(CustomOps.MATMUL_NT, x=x, y=y, **self._tri(tri)), out_shape)
+        kw = {"epi": epi, "e": e} if epi else {}
+        return self._like(self._dispatch(CustomOps.MATMUL_NT, x=x, y=y, **self._tri(tri), **kw), out_shape)
 
     def matmul_tn(self, other: "Buffer", tri: str = "") -> "Buffer":
         """self(.., K, M)^T @ other (.., K, N) without materialising the transpose."""

@@ -1623,7 +1623,8 @@ MATMUL_TRI = ("", "out_lower", "a_lower", "at_lower")
 
 @cache
 def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb: bool,
-                  ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False) -> tuple[str, str, str]:
+                  ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False,
+                  epi: str = "") -> tuple[str, str, str]:
     """C[z] = op(A[z]) . op(B[z]), fp32, row-major, on the matrix cores (v_mfma_f32_32x32x2_f32).
 
     Replaces the i-k-j loops of cpu_kernel.py:351-428.  Batched over blockIdx.z with two
@@ -1658,6 +1659,10 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
       out_lower  only output tiles that touch n <= m are computed (the others are left unwritten)
       a_lower    op(A) = A is lower triangular (A[m][k] = 0 for k > m): k stops at the tile's last row
       at_lower   op(A) = A^T with the stored A (K x M) lower triangular: k starts at the tile's first row
+    epi: what the epilogue does to each result c on its way to memory, with e the entry at the same place of a
+    fourth operand E shaped like C: "add" stores c + e (a residual), "relu" stores max-like c > 0 ? c : 0,
+    "gate" stores e > 0 ? c : 0 (the backward of a ReLU whose output is E).  One rounding each, as the
+    separate element-wise kernel would do.
     strided: A, B and C have their own row pitches (lda, ldb, ldc, in floats) and C its own two batch
     strides, so operands and result can be matrices cut out of larger tensors -- the heads of a
     (B, T, h*d) projection are (T x d) matrices with pitch h*d, batch strides T*h*d and d.
@@ -1666,7 +1671,7 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     assert BK % 8 == 0 and MI in (1, 2, 3, 4) and NJ in (1, 2, 3, 4)
     assert matmul_lds_bytes(WM, WN, MI, NJ, BK, ta, tb) <= MATMUL_LDS_LIMIT
     name = (f"matmul_{BM}x{BN}x{BK}_w{WM}x{WN}_{'a4' if veca else 'a1'}{'b4' if vecb else 'b1'}"
-            f"{'_tn' if ta else ''}{'_nt' if tb else ''}{'_' + tri if tri else ''}{'_ld' if strided else ''}")
+            f"{'_tn' if ta else ''}{'_nt' if tb else ''}{'_' + tri if tri else ''}{'_ld' if strided else ''}{'_' + epi if epi else ''}")
     assert tri in MATMUL_TRI and not (tri == "a_lower" and ta) and not (tri == "at_lower" and not ta)
     comp = ["x", "y", "z", "w"]
     vtype = {1: "float", 2: "float2", 3: "f3v", 4: "float4"}
@@ -1867,6 +1872,52 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
         }}
 }}
 """
+    if epi:
+        assert epi in ("add", "relu", "gate") and not strided
+        macro = {"add": "((cv) + (ev))", "relu": "((cv) > 0.0f ? (cv) : 0.0f)", "gate": "((ev) > 0.0f ? (cv) : 0.0f)"}[epi]
+        edits = [("float* __restrict__ C, MMArgs g) {", "float* __restrict__ C, MMArgs g, const float* __restrict__ E) {"),
+                 ("C += (u64)blockIdx.z * g.M * g.N;", "C += (u64)blockIdx.z * g.M * g.N;\n    E += (u64)blockIdx.z * g.M * g.N;"),
+                 ("typedef float f16v __attribute__((ext_vector_type(16)));",
+                  f"typedef float f16v __attribute__((ext_vector_type(16)));\n#define EPI(cv, ev) {macro}")]
+        if tb:
+            edits.append(("crow[col] = acc[i][j][e];", "crow[col] = EPI(acc[i][j][e], ev[i][j][e]);"))
+        else:
+            edits.append(("crow[col + j] = acc[i][j][e];", "crow[col + j] = EPI(acc[i][j][e], ev[i][j][e]);"))
+            if vecb and NJ == 4:
+                edits.append(("make_float4(acc[i][0][e], acc[i][1][e], acc[i][2][e], acc[i][3][e]);",
+                              "make_float4(EPI(acc[i][0][e], ev[i][0][e]), EPI(acc[i][1][e], ev[i][1][e]), "
+                              "EPI(acc[i][2][e], ev[i][2][e]), EPI(acc[i][3][e], ev[i][3][e]));"))
+        if epi != "relu":
+            # The entries of E this lane will need, fetched with clamped (always valid) addresses and no
+            # branch, so that all loads are in flight together: ahead of the k loop where they fit in few
+            # registers, right after it otherwise.
+            if tb:
+                fetch = ("#pragma unroll\n            for (int j = 0; j < NJ; ++j) "
+                         "ev[i][j][e] = erow[min(n0 + wn0 + 32u * j + r, g.N - 1u)];")
+            elif vecb and NJ == 4:                     # vecb vouches for 16-byte alignment of E as of C, and N % 4 == 0
+                fetch = ("const float4 q = *reinterpret_cast<const float4*>(erow + min(n0 + wn0 + 4u * r, g.N - 4u));\n"
+                         "            ev[i][0][e] = q.x; ev[i][1][e] = q.y; ev[i][2][e] = q.z; ev[i][3][e] = q.w;")
+            else:
+                fetch = (f"#pragma unroll\n            for (int j = 0; j < NJ; ++j) "
+                         f"ev[i][j][e] = erow[min(n0 + wn0 + {NJ}u * r + j, g.N - 1u)];")
+            pre = f"""    float ev[MI][NJ][16];
+    #pragma unroll
+    for (int i = 0; i < MI; ++i)
+        #pragma unroll
+        for (int e = 0; e < 16; ++e) {{
+            const float* __restrict__ erow = E + (u64)min({row_expr}, g.M - 1u) * g.N;
+            {fetch}
+        }}
+
+"""
+            anchor = "    float4 ra[" if MI * NJ <= 2 else "    #pragma unroll\n    for (int i = 0; i < MI; ++i)\n        #pragma unroll\n        for (int e = 0; e < 16; ++e) {\n            const u32 row"
+            edits.append((anchor, pre + anchor))
+        else:
+            edits.append(("ev[i][", "acc[i]["))         # relu looks at the result only
+        for was, now in edits:
+            assert src.count(was) >= 1, was
+            src = src.replace(was, now)
+        return src, name, _fmt("P", "P", "P", "8I", "P")
     if strided:
         for was, now in (("struct MMArgs { u32 M, N, K, nbc, sa0, sa1, sb0, sb1; };",
                           "struct MMArgs { u32 M, N, K, nbc, sa0, sa1, sb0, sb1, lda, ldb, ldc, sc0, sc1; };"),

@@ -19,8 +19,15 @@ class Linear:
         self.bias = Tensor.uniform((1, out_features), low=-bound, high=bound,
                                    requires_grad=True, device=device) if bias else None
 
-    def __call__(self, x: Tensor) -> Tensor:
-        return x.linear(self.weight, self.bias)
+    def __call__(self, x: Tensor, residual: Tensor | None = None) -> Tensor:
+        """x @ W^T + b, plus `residual` if given (an extension: on the hip device the addition is
+        part of the product kernel, ops.LinearNTAdd)."""
+        if residual is None:
+            return x.linear(self.weight, self.bias)
+        if self.bias is None and residual.shape == x.shape[:-1] + (self.weight.shape[0],) \
+                and residual.device is x.device and ops.use_fused_epilogues(x, self.weight):
+            return ops.LinearNTAdd.execute(x, self.weight, residual)
+        return residual + x.linear(self.weight, self.bias)
 
 
 class Embedding:
@@ -127,3 +134,14 @@ def self_attention_qkv(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor, n_head: in
     if ops.use_fused_qkv_attention(x, wq, wk, wv, n_head):
         return ops.SelfAttentionQKV.execute(x, wq, wk, wv, n_head=n_head, scale=scale)
     return causal_self_attention(x.linear(wq, None), x.linear(wk, None), x.linear(wv, None), n_head, scale)
+
+
+def mlp_relu(x: Tensor, w_fc: Tensor, w_proj: Tensor, residual: Tensor | None = None) -> Tensor:
+    """relu(x @ w_fc^T) @ w_proj^T (+ residual): the bias-free feed-forward block of
+    examples/gpt.py:69-78.  On the hip device one node whose ReLU, ReLU gradient and residual addition
+    happen as the products are stored (ops.MLPRelu); elsewhere the four ops."""
+    if ops.use_fused_epilogues(x, w_fc, w_proj) and (residual is None or (residual.device is x.device and residual.shape == x.shape[:-1] + (w_proj.shape[0],))):
+        args = (x, w_fc, w_proj) if residual is None else (x, w_fc, w_proj, residual)
+        return ops.MLPRelu.execute(*args)
+    out = x.linear(w_fc, None).relu().linear(w_proj, None)
+    return out if residual is None else residual + out

@@ -343,6 +343,46 @@ class LinearNT(OP):
         return unbroadcast(grad_x, self.x.shape), unbroadcast(grad_w, self.w.shape)
 
 
+class LinearNTAdd(OP):
+    """x @ W^T + r with the addition done as the product is stored (r shaped like the result, e.g. the
+    residual stream): LinearNT followed by Add, one kernel and one pass over the result fewer, same bits."""
+
+    def forward(self, x: Buffer, w: Buffer, r: Buffer) -> Buffer:
+        self.x, self.w = x, w
+        return x.matmul_nt(w, epi="add", e=r)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        grad_x = upstream_grad @ self.w
+        grad_w = upstream_grad.matmul_tn(self.x)
+        return unbroadcast(grad_x, self.x.shape), unbroadcast(grad_w, self.w.shape), upstream_grad
+
+
+class MLPRelu(OP):
+    """relu(x @ W1^T) @ W2^T (+ r): the feed-forward block of examples/gpt.py:69-78 with the ReLU applied
+    as the first product is stored, its backward select applied as the gradient of the hidden layer
+    is stored, and the residual added as the second product is stored: the ReLU, its backward and the
+    addition no longer run as kernels of their own.  Same values as the op-by-op form: every fused
+    step is the same single fp32 operation on the same operands."""
+
+    def forward(self, x: Buffer, w1: Buffer, w2: Buffer, r: Buffer | None = None) -> Buffer:
+        self.x, self.w1, self.w2, self.has_r = x, w1, w2, r is not None
+        self.h = x.matmul_nt(w1, epi="relu")
+        self.gate = self.h                                  # positive where the ReLU let the value through
+        return self.h.matmul_nt(w2, epi="add", e=r) if r is not None else self.h.matmul_nt(w2)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        gh = upstream_grad.matmul(self.w2, epi="gate", e=self.gate)         # gradient before the ReLU
+        dw2 = unbroadcast(upstream_grad.matmul_tn(self.h), self.w2.shape)
+        dx = unbroadcast(gh @ self.w1, self.x.shape)
+        dw1 = unbroadcast(gh.matmul_tn(self.x), self.w1.shape)
+        return (dx, dw1, dw2, upstream_grad) if self.has_r else (dx, dw1, dw2)
+
+
+def use_fused_epilogues(x, *weights) -> bool:
+    return FUSED and x.device is Device.HIP and x.ndim >= 2 and x.numel > 0 and \
+        all(w.ndim == 2 and w.device is Device.HIP for w in weights)
+
+
 class Softmax(OP):
     """Fused forward along the last axis; backward dx = y * (g - sum(g * y, last))."""
 

@@ -1161,7 +1161,8 @@ class HIP:
         if _addr(dy) % 16 and L % 4 == 0:                          # a gradient view at an odd offset: realign it
             dy = Buffer(_map("copy", "x0", [dy], dy.shape), dy.shape, Device.HIP)
         dx = alloc(x.numel)
-        rows_per_wave = max(1, (R + 2047) // 2048)
+        # partial rows of dw: at most 2048, and for small inputs (launch-bound) at most the 512 that one launch folds
+        rows_per_wave = max(1, (R + 511) // 512 if R * L <= (1 << 20) else (R + 2047) // 2048)
         P = (R + rows_per_wave - 1) // rows_per_wave            # partial rows of dw, one per wavefront
         part = alloc(P * L) if w is not None else None
         vec = HIP._rms_vec(L, _addr(x), _addr(dy), dx.addr, _addr(w) if w is not None else 0,
@@ -1324,9 +1325,9 @@ class HIP:
 
     @staticmethod
     def _launch_matmul(tile: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple,
-                       ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False) -> None:
+                       ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False, epi: str = "") -> None:
         bm, bn, threads = K.matmul_tile_shape(tile)
-        k = kernel(K.matmul_kernel, *K.MATMUL_CONFIGS[tile], veca, vecb, ta, tb, tri, strided)
+        k = kernel(K.matmul_kernel, *K.MATMUL_CONFIGS[tile], veca, vecb, ta, tb, tri, strided, epi)
         launch(k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch), threads, *args)
 
     @staticmethod
@@ -1393,14 +1394,17 @@ class HIP:
 
     @staticmethod
     @dispatcher.register(BinaryOps.MATMUL, Device.HIP)
-    def matmul(x: Buffer, y: Buffer, ta: bool = False, tb: bool = False, tri: str = "") -> DevicePtr:
+    def matmul(x: Buffer, y: Buffer, ta: bool = False, tb: bool = False, tri: str = "", epi: str = "",
+               e: Buffer | None = None) -> DevicePtr:
         """x (.., M, K) @ y (.., K, N) for operands already padded to the same rank 2..4
         (buffer.py:231-243); batch dims of extent 1 broadcast through a zero stride as in
         cpu.py:519-532 and :553-559.  When y carries no batch at all the batch of x is
         folded into M: one tall GEMM instead of many small ones.
         ta: x is stored as (.., K, M) and used transposed; tb: y is stored as (.., N, K).
         tri: triangular structure of square (T x T) operands or outputs that the caller vouches
-        for (K.matmul_kernel); the work it lets the kernel skip never changes a kept result."""
+        for (K.matmul_kernel); the work it lets the kernel skip never changes a kept result.
+        epi: "add" (result + e), "relu" (result where positive, else 0) or "gate" (result where e is
+        positive, else 0), applied as the result is stored; e has the shape of the result."""
         assert x.ndim == y.ndim and 2 <= x.ndim <= 4 and not (ta and tb)
         (Kd, M) = x.shape[-2:] if ta else x.shape[-2:][::-1]
         (N, Ky) = y.shape[-2:] if tb else y.shape[-2:][::-1]
@@ -1409,10 +1413,18 @@ class HIP:
         yb = (1,) * (4 - y.ndim) + tuple(y.shape[:-2])
         B0, B1 = max(xb[0], yb[0]), max(xb[1], yb[1])
         out = alloc(B0 * B1 * M * N)
+        if epi:
+            if epi not in ("add", "relu", "gate") or tri:
+                raise ValueError(f"epilogue {epi!r} with tri={tri!r} is not provided")
+            if epi != "relu" and (e is None or e.is_host_scalar or e.numel != B0 * B1 * M * N):
+                raise ValueError(f"epilogue {epi!r} needs an operand shaped like the result ({B0 * B1 * M * N} elements)")
         if B0 * B1 * M * N == 0:
             return out
-        if Kd == 0:
-            lib().fill_f32(out.addr, 0.0, B0 * B1 * M * N)
+        if Kd == 0:                                            # an empty sum: zeros, plus e for "add"
+            if epi == "add":
+                lib().d2d(out.addr, _addr(e), 4 * B0 * B1 * M * N)
+            else:
+                lib().fill_f32(out.addr, 0.0, B0 * B1 * M * N)
             return out
         if tri:
             square = {"out_lower": M == N, "a_lower": not ta and M == Kd, "at_lower": ta and M == Kd}.get(tri)
@@ -1431,16 +1443,21 @@ class HIP:
             raise ValueError("matrix too large for 32-bit indexing")
         veca = (M if ta else Kd) % 4 == 0 and _addr(x) % 16 == 0
         vecb = (Kd if tb else N) % 4 == 0 and _addr(y) % 16 == 0 and out.addr % 16 == 0
+        if epi and e is not None and (_addr(e) % 16 or N % 4):
+            vecb = False                                       # the epilogue reads e as it writes the result
         args = (_addr(x), _addr(y), out.addr, M, N, Kd, nbc, *sa, *sb)
         tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, args, ta, tb, tri)
+        if epi:
+            HIP._launch_matmul(tile, veca, vecb, M, N, batch, (*args, out.addr if e is None else _addr(e)), ta, tb, "", False, epi)
+            return out
         HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri)
         return out
 
     @staticmethod
     @dispatcher.register(CustomOps.MATMUL_NT, Device.HIP)
-    def matmul_nt(x: Buffer, y: Buffer, tri: str = "") -> DevicePtr:
+    def matmul_nt(x: Buffer, y: Buffer, tri: str = "", epi: str = "", e: Buffer | None = None) -> DevicePtr:
         """x (.., M, K) times the transpose of y (.., N, K), read in place."""
-        return HIP.matmul(x, y, tb=True, tri=tri)
+        return HIP.matmul(x, y, tb=True, tri=tri, epi=epi, e=e)
 
     @staticmethod
     @dispatcher.register(CustomOps.MATMUL_TN, Device.HIP)

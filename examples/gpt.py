@@ -36,7 +36,8 @@ class CausalSelfAttention:
         # same three parameters, placed back to back so that one product can serve all three projections
         nn.stack_parameters([self.q_proj.weight, self.k_proj.weight, self.v_proj.weight])
 
-    def __call__(self, x: Tensor, cache: "KVCache | None" = None, layer: int = 0) -> Tensor:
+    def __call__(self, x: Tensor, cache: "KVCache | None" = None, layer: int = 0,
+                 residual: Tensor | None = None) -> Tensor:
         """Without a cache, or with an empty one: causal attention over the T positions of x
         (whose k/v projections are stored if a cache is given).  With a filled cache and
         T == 1: the new position attends to everything cached plus itself, no mask
@@ -46,7 +47,7 @@ class CausalSelfAttention:
             # q, k, v projections, split into heads, ((q @ k^T) * scale).masked_fill(mask, -inf).softmax(dim=3) @ v,
             # merge the heads (examples/gpt.py:45-57): one node on the hip device
             return self.c_proj(nn.self_attention_qkv(x, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight,
-                                                     self.n_head, self.scale))
+                                                     self.n_head, self.scale), residual)
         q_lin, k_lin, v_lin = self.q_proj(x), self.k_proj(x), self.v_proj(x)    # (B, T, C)
         if cache.length > 0:
             assert T == 1, "incremental attention takes one new position"
@@ -56,7 +57,7 @@ class CausalSelfAttention:
         else:
             cache.write(layer, k_lin, v_lin, 0)               # prefill: the projections are kept for later tokens
             y = nn.causal_self_attention(q_lin, k_lin, v_lin, self.n_head, self.scale)
-        return self.c_proj(y)
+        return self.c_proj(y, residual)
 
 
 class KVCache:
@@ -86,8 +87,9 @@ class MLP:
         self.c_fc = nn.Linear(c.n_embd, 4 * c.n_embd, bias=False, device=c.device)
         self.c_proj = nn.Linear(4 * c.n_embd, c.n_embd, bias=False, device=c.device)
 
-    def __call__(self, x: Tensor) -> Tensor:
-        return self.c_proj(self.c_fc(x).relu())
+    def __call__(self, x: Tensor, residual: Tensor | None = None) -> Tensor:
+        """c_proj(relu(c_fc(x))), plus the residual stream if given."""
+        return nn.mlp_relu(x, self.c_fc.weight, self.c_proj.weight, residual)
 
 
 class Block:
@@ -98,8 +100,8 @@ class Block:
         self.mlp = MLP(c)
 
     def __call__(self, x: Tensor, cache: KVCache | None = None, layer: int = 0) -> Tensor:
-        x = x + self.attn(self.ln1(x), cache, layer)
-        return x + self.mlp(self.ln2(x))
+        x = self.attn(self.ln1(x), cache, layer, residual=x)          # x + attention(norm(x))
+        return self.mlp(self.ln2(x), residual=x)                      # x + mlp(norm(x))
 
 
 class GPT:
@@ -221,12 +223,12 @@ class StaticDecoder:
         first[0, 0] = first_token
         self.seq.data.upload_(first)
 
-    def _attend(self, attn: CausalSelfAttention, x: Tensor, layer: int, hidden: Tensor) -> Tensor:
+    def _attend(self, attn: CausalSelfAttention, x: Tensor, layer: int, hidden: Tensor, residual: Tensor) -> Tensor:
         T = self.model.config.block_size
         self.cache.k[layer].data.row_store_(attn.k_proj(x).data, self.slot.data)
         self.cache.v[layer].data.row_store_(attn.v_proj(x).data, self.slot.data)
         y = nn.cached_attention(attn.q_proj(x), self.cache.k[layer], self.cache.v[layer], T, attn.n_head, attn.scale, hidden)
-        return attn.c_proj(y)
+        return attn.c_proj(y, residual)
 
     def step(self) -> None:
         """Feeds self.tok at index self.slot; leaves the argmax in seq[slot + 1] and as the next
@@ -238,8 +240,8 @@ class StaticDecoder:
         hidden = Tensor.arange((1, c.block_size), device=c.device) > slot                   # cache rows not written yet
         x = m.wte(self.tok) + m.wpe(pos)
         for i, block in enumerate(m.blocks):
-            x = x + self._attend(block.attn, block.ln1(x), i, hidden)
-            x = x + block.mlp(block.ln2(x))
+            x = self._attend(block.attn, block.ln1(x), i, hidden, x)
+            x = block.mlp(block.ln2(x), x)
         nxt = m.lm_head(m.ln_f(x)).reshape((1, c.vocab_size)).argmax(1)                     # (1, 1)
         nslot = slot + 1.0
         self.seq.data.row_store_(nxt.data, nslot.data)

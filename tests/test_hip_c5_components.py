@@ -323,3 +323,43 @@ def test_stacked_qkv_attention_equals_three_projections_and_attention(B, T, h, d
             assert np.abs(a - b).max() <= 1e-5 * np.abs(b).max(), name
         else:
             assert (a.view(np.uint32) == b.view(np.uint32)).all(), f"{name} B{B} T{T} h{h} d{d}"
+
+
+@pytest.mark.parametrize("B,T,C,H", [(2, 64, 48, 192), (1, 100, 36, 50), (4, 256, 384, 1536)])
+def test_feed_forward_with_fused_epilogues_equals_the_four_ops(B, T, C, H, monkeypatch):
+    """nn.mlp_relu and nn.Linear(x, residual): the ReLU, its gradient select and the residual
+    addition ride on the stores of the products.  Output and every gradient (input, both weights,
+    residual) have the bits of linear -> relu -> linear -> add run op by op."""
+    require_gpu()
+    from dlgrad_amd import nn, ops
+    rng = np.random.default_rng(B * T + C)
+    x, r, g = (rng.standard_normal((B, T, C), dtype=np.float32) for _ in range(3))
+    w1 = rng.standard_normal((H, C), dtype=np.float32) * C ** -0.5
+    w2 = rng.standard_normal((C, H), dtype=np.float32) * H ** -0.5
+    usable = ops.use_fused_epilogues
+
+    def run(fused, what):
+        monkeypatch.setattr(ops, "use_fused_epilogues", usable if fused else (lambda *a: False))
+        ts = [Tensor(a, device="hip", requires_grad=True) for a in (x, w1, w2, r)]
+        if what == "mlp":
+            y = nn.mlp_relu(*ts)
+        elif what == "mlp_plain":
+            y = nn.mlp_relu(*ts[:3])
+        else:
+            lin = nn.Linear(H, C, bias=False)
+            lin.weight = ts[2]
+            h = Tensor(np.abs(np.resize(x, (B, T, H))), device="hip", requires_grad=True)
+            ts[0] = h
+            y = lin(h, ts[3])
+        node = type(y._ctx).__name__
+        (y * Tensor(g, device="hip")).sum().backward()
+        return node, [y.numpy()] + [t.grad.numpy() for t in ts if t.grad is not None]
+
+    for what, node in (("mlp", "MLPRelu"), ("mlp_plain", "MLPRelu"), ("linear", "LinearNTAdd")):
+        (n1, fused), (n0, chain) = run(True, what), run(False, what)
+        assert n1 == node and n0 != node, (what, n1, n0)
+        assert len(fused) == len(chain) == (4 if what == "mlp_plain" else 5 if what == "mlp" else 4)
+        if hip.COMPILE_ONLY:
+            continue
+        for i, (a, b) in enumerate(zip(fused, chain)):
+            assert a.shape == b.shape and (a.view(np.uint32) == b.view(np.uint32)).all(), f"{what} output/gradient {i}"

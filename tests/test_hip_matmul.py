@@ -221,6 +221,53 @@ def test_triangular_hints_skip_work_without_changing_a_bit(T, d, batch):
             HIP.MATMUL_FORCE = prev
 
 
+@pytest.mark.parametrize("shape_x,shape_y,nt", [((256, 96), (96, 128), False), ((3, 100, 36), (50, 36), True),
+                                                ((2, 3, 65, 17), (2, 3, 17, 33), False), ((512, 384), (1536, 384), True),
+                                                ((4, 0), (0, 8), False)])
+def test_epilogues_equal_the_separate_elementwise_kernels(shape_x, shape_y, nt):
+    """epi = add / relu / gate do their one fp32 operation on the accumulator as it is stored: the bits
+    of product + e, relu(product) and where(e > 0, product, 0) computed by separate kernels, for
+    every tile configuration (forced one by one), ragged and batched shapes, NN and NT, empty k."""
+    require_gpu()
+    from dlgrad_amd.codegen import hip_kernel as K
+    from dlgrad_amd.runtime.hip import HIP
+    rng = np.random.default_rng(len(shape_x) * 1000 + shape_x[-1])
+    x = rng.standard_normal(shape_x, dtype=np.float32)
+    y = rng.standard_normal(shape_y, dtype=np.float32)
+    xd, yd = dev(x), dev(y)
+    mm = (lambda **kw: xd.matmul_nt(yd, **kw)) if nt else (lambda **kw: xd.matmul(yd, **kw))
+    plain = mm()
+    e = rng.standard_normal(plain.shape, dtype=np.float32)
+    e[..., ::3] = 0.0                                                 # gate: zero is not positive
+    ed = dev(e)
+    want_add = (plain + ed).numpy()
+    want_relu = plain.relu().numpy()
+    want_gate = (ed > 0.0).where(inp=plain, other=0.0).numpy()
+    small = min(plain.shape[-2:]) < 64
+    tiles = [None] + [t for t in K.MATMUL_CONFIGS if not small or t in ("64x64", "32x32")]
+    for tile in tiles:
+        prev, HIP.MATMUL_FORCE = HIP.MATMUL_FORCE, tile
+        try:
+            check(mm(epi="add", e=ed).numpy(), want_add, 0, f"add {tile}")
+            check(mm(epi="relu").numpy(), want_relu, 0, f"relu {tile}")
+            check(mm(epi="gate", e=ed).numpy(), want_gate, 0, f"gate {tile}")
+        finally:
+            HIP.MATMUL_FORCE = prev
+
+
+def test_epilogues_are_refused_without_a_fitting_operand():
+    require_gpu()
+    a, b = dev(f32(8, 16)), dev(f32(16, 8))
+    with pytest.raises(ValueError):
+        a.matmul(b, epi="add")                          # nothing to add
+    with pytest.raises(ValueError):
+        a.matmul(b, epi="gate", e=dev(f32(8, 4)))       # wrong size
+    with pytest.raises(ValueError):
+        a.matmul(b, epi="square")                       # no such step
+    with pytest.raises(ValueError):
+        a.matmul_nt(dev(f32(8, 16)), tri="out_lower", epi="relu")
+
+
 def test_triangular_hints_are_refused_where_they_make_no_sense():
     require_gpu()
     a, b = dev(f32(8, 16)), dev(f32(16, 8))

@@ -179,6 +179,20 @@ class ReluBranches:
 
         monkeypatch.setattr(ops.Relu, "forward", forward)
         monkeypatch.setattr(ops.Relu, "backward", backward)
+        fused0 = ops.MLPRelu.forward
+
+        def fused_forward(node, *args):                 # the feed-forward node holds its ReLU inside
+            out = fused0(node, *args)
+            if not (hip.COMPILE_ONLY or record):
+                mask = node.h.numpy() > 0
+                want = tape.masks[tape.cursor]
+                tape.cursor += 1
+                tape.differing += int((mask != want).sum())
+                tape.total += mask.size
+                node.gate = Buffer.from_numpy(want.astype(np.float32), node.h.device)
+            return out
+
+        monkeypatch.setattr(ops.MLPRelu, "forward", fused_forward)
 
 
 @pytest.mark.gpu
