@@ -1610,9 +1610,9 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 MATMUL_LDS_LIMIT = 160 * 1024          # LDS per CU on gfx950, all of it available to one block
 
 
-def matmul_lds_bytes(WM: int, WN: int, MI: int, NJ: int, BK: int, ta: bool = False, tb: bool = False) -> int:
+def matmul_lds_bytes(WM: int, WN: int, MI: int, NJ: int, BK: int, ta: bool = False, tb: bool = False, S: int = 32) -> int:
     """Static LDS of one block (both operands, double-buffered)."""
-    BM, BN = 32 * MI * WM, 32 * NJ * WN
+    BM, BN = S * MI * WM, S * NJ * WN
     a = BK * BM if ta else BM * (BK + 4)
     b = BN * (BK + 4) if tb else BK * BN
     return 2 * 4 * (a + b)
@@ -1624,8 +1624,9 @@ MATMUL_TRI = ("", "out_lower", "a_lower", "at_lower")
 @cache
 def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb: bool,
                   ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False,
-                  epi: str = "") -> tuple[str, str, str]:
-    """C[z] = op(A[z]) . op(B[z]), fp32, row-major, on the matrix cores (v_mfma_f32_32x32x2_f32).
+                  epi: str = "", S: int = 32) -> tuple[str, str, str]:
+    """C[z] = op(A[z]) . op(B[z]), fp32, row-major, on the matrix cores (v_mfma_f32_32x32x2_f32, or
+    v_mfma_f32_16x16x4_f32 for S = 16).
 
     Replaces the i-k-j loops of cpu_kernel.py:351-428.  Batched over blockIdx.z with two
     batch extents (z = zb * nbc + zc) whose operand strides may be 0, which is how the
@@ -1663,15 +1664,22 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     fourth operand E shaped like C: "add" stores c + e (a residual), "relu" stores max-like c > 0 ? c : 0,
     "gate" stores e > 0 ? c : 0 (the backward of a ReLU whose output is E).  One rounding each, as the
     separate element-wise kernel would do.
+    S: edge of the MFMA tile.  A wavefront's share of one output element's k sum is a fixed chain of
+    MFMA steps however small its tile, so a long-k product with few output tiles (2048 x 128 x 512: 64
+    tiles of 64x64) is bound by that chain on a quarter of the SIMDs.  S = 16 gives every wavefront a
+    (16*MI) x (16*NJ) tile, four times as many wavefronts and a quarter of the chain each.  One 16x16x4
+    step adds four k; the lane groups take k = 8*blk + {0, 4, 1, 5} and then {2, 6, 3, 7}, the order
+    in which two 32x32x2 steps at a time add them.
     strided: A, B and C have their own row pitches (lda, ldb, ldc, in floats) and C its own two batch
     strides, so operands and result can be matrices cut out of larger tensors -- the heads of a
     (B, T, h*d) projection are (T x d) matrices with pitch h*d, batch strides T*h*d and d.
     """
-    BM, BN, T = 32 * MI * WM, 32 * NJ * WN, 64 * WM * WN
-    assert BK % 8 == 0 and MI in (1, 2, 3, 4) and NJ in (1, 2, 3, 4)
-    assert matmul_lds_bytes(WM, WN, MI, NJ, BK, ta, tb) <= MATMUL_LDS_LIMIT
+    BM, BN, T = S * MI * WM, S * NJ * WN, 64 * WM * WN
+    NE = S * S // 64                                        # accumulator registers per MFMA tile
+    assert BK % 8 == 0 and MI in (1, 2, 3, 4) and NJ in (1, 2, 3, 4) and S in (16, 32) and T <= 1024
+    assert matmul_lds_bytes(WM, WN, MI, NJ, BK, ta, tb, S) <= MATMUL_LDS_LIMIT
     name = (f"matmul_{BM}x{BN}x{BK}_w{WM}x{WN}_{'a4' if veca else 'a1'}{'b4' if vecb else 'b1'}"
-            f"{'_tn' if ta else ''}{'_nt' if tb else ''}{'_' + tri if tri else ''}{'_ld' if strided else ''}{'_' + epi if epi else ''}")
+            f"{'_tn' if ta else ''}{'_nt' if tb else ''}{'_' + tri if tri else ''}{'_ld' if strided else ''}{'_' + epi if epi else ''}{'_m16' if S == 16 else ''}")
     assert tri in MATMUL_TRI and not (tri == "a_lower" and ta) and not (tri == "at_lower" and not ta)
     comp = ["x", "y", "z", "w"]
     vtype = {1: "float", 2: "float2", 3: "f3v", 4: "float4"}
@@ -1733,38 +1741,41 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     decl_a, idx_a, PA, load_a, stash_a = loader("A", not ta, "M", BM, "M", "M", "m0", veca)
     decl_b, idx_b, PB, load_b, stash_b = loader("B", tb, "N", BN, "N", "N", "n0", vecb)
 
-    # ---- the multiply: one group of 8 k per iteration, four MFMA steps
+    # ---- the multiply: one group of 8 k per iteration, four 32x32x2 (two 16x16x4) MFMA steps
     pre = ""
     if not ta:
         pre += (f"            float4 a[MI];\n            #pragma unroll\n            for (int i = 0; i < MI; ++i)\n"
-                f"                a[i] = *reinterpret_cast<const float4*>(&As[buf][wm0 + 32u * i + r][kb + 4u * h]);\n")
+                f"                a[i] = *reinterpret_cast<const float4*>(&As[buf][wm0 + {S}u * i + r][kb + 4u * {'h' if S == 32 else '(h & 1u)'}]);\n")
     if tb:
         pre += (f"            float4 b[NJ];\n            #pragma unroll\n            for (int j = 0; j < NJ; ++j)\n"
-                f"                b[j] = *reinterpret_cast<const float4*>(&Bs[buf][wn0 + 32u * j + r][kb + 4u * h]);\n")
+                f"                b[j] = *reinterpret_cast<const float4*>(&Bs[buf][wn0 + {S}u * j + r][kb + 4u * {'h' if S == 32 else '(h & 1u)'}]);\n")
     mfma = pre
-    for st_ in range(4):
+    for st_ in range(4 if S == 32 else 2):
+        # the k (within the group of 8) that this lane feeds to step st_, and the component of a float4 read at 4*(k/4)
+        krow = f"kb + 4u * h + {st_}u" if S == 32 else f"kb + 4u * (h & 1u) + (h >> 1) + {2 * st_}u"
+        pick = (lambda v: f"{v}.{comp[st_]}") if S == 32 else (lambda v: f"((h >> 1) ? {v}.{comp[2 * st_ + 1]} : {v}.{comp[2 * st_]})")
         mfma += "            {\n"
         if ta:
             mfma += (f"              const {vtype[MI]} av = *reinterpret_cast<const {vtype[MI]}*>"
-                     f"(&As[buf][kb + 4u * h + {st_}u][wm0 + {MI}u * r]);\n")
+                     f"(&As[buf][{krow}][wm0 + {MI}u * r]);\n")
         if not tb:
             mfma += (f"              const {vtype[NJ]} bv = *reinterpret_cast<const {vtype[NJ]}*>"
-                     f"(&Bs[buf][kb + 4u * h + {st_}u][wn0 + {NJ}u * r]);\n")
+                     f"(&Bs[buf][{krow}][wn0 + {NJ}u * r]);\n")
         for i_ in range(MI):
-            ai = (("av" if MI == 1 else f"av.{comp[i_]}") if ta else f"a[{i_}].{comp[st_]}")
+            ai = (("av" if MI == 1 else f"av.{comp[i_]}") if ta else pick(f"a[{i_}]"))
             for j_ in range(NJ):
-                bj = (f"b[{j_}].{comp[st_]}" if tb else ("bv" if NJ == 1 else f"bv.{comp[j_]}"))
-                mfma += (f"              acc[{i_}][{j_}] = __builtin_amdgcn_mfma_f32_32x32x2f32("
+                bj = (pick(f"b[{j_}]") if tb else ("bv" if NJ == 1 else f"bv.{comp[j_]}"))
+                mfma += (f"              acc[{i_}][{j_}] = __builtin_amdgcn_mfma_f32_{'32x32x2' if S == 32 else '16x16x4'}f32("
                          f"{ai}, {bj}, acc[{i_}][{j_}], 0, 0, 0);\n")
         mfma += "            }\n"
 
     # ---- epilogue: accumulator e of tile (i, j) belongs to operand-row index 8*(e/4) + 4*h + e%4
-    # of A's tile i and operand-row index lane%32 of B's tile j
-    row_expr = (f"m0 + wm0 + {MI}u * (8u * (e >> 2) + 4u * h + (e & 3)) + i" if ta
-                else "m0 + wm0 + 32u * i + 8u * (e >> 2) + 4u * h + (e & 3)")
+    # (4*h + e for the 16-wide tile) of A's tile i and operand-row index lane%S of B's tile j
+    arow = "8u * (e >> 2) + 4u * h + (e & 3)" if S == 32 else "4u * h + e"
+    row_expr = (f"m0 + wm0 + {MI}u * ({arow}) + i" if ta else f"m0 + wm0 + {S}u * i + {arow}")
     if tb:
-        store = """                #pragma unroll
-                for (int j = 0; j < NJ; ++j) { const u32 col = n0 + wn0 + 32u * j + r; if (col < g.N) crow[col] = acc[i][j][e]; }"""
+        store = f"""                #pragma unroll
+                for (int j = 0; j < NJ; ++j) {{ const u32 col = n0 + wn0 + {S}u * j + r; if (col < g.N) crow[col] = acc[i][j][e]; }}"""
     elif vecb and NJ == 4:
         store = f"""                const u32 col = n0 + wn0 + {NJ}u * r;
                 if (col + 3u < g.N) {{
@@ -1801,8 +1812,9 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     __syncthreads();
     for (u32 kt = kt0; kt < nk; ++kt) {{
         const u32 buf = (kt - kt0) & 1u;"""
+    f4v_typedef = "" if S == 32 else "\ntypedef float f4v __attribute__((ext_vector_type(4)));"
     src = f"""{PRELUDE}
-typedef float f16v __attribute__((ext_vector_type(16)));
+typedef float f16v __attribute__((ext_vector_type(16)));{f4v_typedef}
 struct f3v {{ float x, y, z; }};
 struct MMArgs {{ u32 M, N, K, nbc, sa0, sa1, sb0, sb1; }};
 #define BM {BM}u
@@ -1832,18 +1844,18 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
     C += (u64)blockIdx.z * g.M * g.N;
 
     const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const u32 r = lane & 31u, h = lane >> 5;
-    const u32 wm0 = (wave / {WN}u) * {32 * MI}u, wn0 = (wave % {WN}u) * {32 * NJ}u;
+    const u32 r = lane & {S - 1}u, h = lane >> {5 if S == 32 else 4};
+    const u32 wm0 = (wave / {WN}u) * {S * MI}u, wn0 = (wave % {WN}u) * {S * NJ}u;
     {idx_a}
     {idx_b}
 
-    f16v acc[MI][NJ];
+    {'f16v' if S == 32 else 'f4v'} acc[MI][NJ];
     #pragma unroll
     for (int i = 0; i < MI; ++i)
         #pragma unroll
         for (int j = 0; j < NJ; ++j)
             #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+            for (int e = 0; e < {NE}; ++e) acc[i][j][e] = 0.f;
 
     float4 ra[{PA}], rb[{PB}];
     auto load_tiles = [&](u32 k0) {{
@@ -1863,7 +1875,7 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
     #pragma unroll
     for (int i = 0; i < MI; ++i)
         #pragma unroll
-        for (int e = 0; e < 16; ++e) {{
+        for (int e = 0; e < {NE}; ++e) {{
             const u32 row = {row_expr};
             if (row < g.M) {{
                 float* __restrict__ crow = C + (u64)row * g.N;
@@ -1877,8 +1889,7 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
         macro = {"add": "((cv) + (ev))", "relu": "((cv) > 0.0f ? (cv) : 0.0f)", "gate": "((ev) > 0.0f ? (cv) : 0.0f)"}[epi]
         edits = [("float* __restrict__ C, MMArgs g) {", "float* __restrict__ C, MMArgs g, const float* __restrict__ E) {"),
                  ("C += (u64)blockIdx.z * g.M * g.N;", "C += (u64)blockIdx.z * g.M * g.N;\n    E += (u64)blockIdx.z * g.M * g.N;"),
-                 ("typedef float f16v __attribute__((ext_vector_type(16)));",
-                  f"typedef float f16v __attribute__((ext_vector_type(16)));\n#define EPI(cv, ev) {macro}")]
+                 ("struct f3v {", f"#define EPI(cv, ev) {macro}\nstruct f3v {{")]
         if tb:
             edits.append(("crow[col] = acc[i][j][e];", "crow[col] = EPI(acc[i][j][e], ev[i][j][e]);"))
         else:
@@ -1893,24 +1904,24 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
             # registers, right after it otherwise.
             if tb:
                 fetch = ("#pragma unroll\n            for (int j = 0; j < NJ; ++j) "
-                         "ev[i][j][e] = erow[min(n0 + wn0 + 32u * j + r, g.N - 1u)];")
+                         f"ev[i][j][e] = erow[min(n0 + wn0 + {S}u * j + r, g.N - 1u)];")
             elif vecb and NJ == 4:                     # vecb vouches for 16-byte alignment of E as of C, and N % 4 == 0
                 fetch = ("const float4 q = *reinterpret_cast<const float4*>(erow + min(n0 + wn0 + 4u * r, g.N - 4u));\n"
                          "            ev[i][0][e] = q.x; ev[i][1][e] = q.y; ev[i][2][e] = q.z; ev[i][3][e] = q.w;")
             else:
                 fetch = (f"#pragma unroll\n            for (int j = 0; j < NJ; ++j) "
                          f"ev[i][j][e] = erow[min(n0 + wn0 + {NJ}u * r + j, g.N - 1u)];")
-            pre = f"""    float ev[MI][NJ][16];
+            pre = f"""    float ev[MI][NJ][{NE}];
     #pragma unroll
     for (int i = 0; i < MI; ++i)
         #pragma unroll
-        for (int e = 0; e < 16; ++e) {{
+        for (int e = 0; e < {NE}; ++e) {{
             const float* __restrict__ erow = E + (u64)min({row_expr}, g.M - 1u) * g.N;
             {fetch}
         }}
 
 """
-            anchor = "    float4 ra[" if MI * NJ <= 2 else "    #pragma unroll\n    for (int i = 0; i < MI; ++i)\n        #pragma unroll\n        for (int e = 0; e < 16; ++e) {\n            const u32 row"
+            anchor = "    float4 ra[" if MI * NJ * NE <= 32 else f"    #pragma unroll\n    for (int i = 0; i < MI; ++i)\n        #pragma unroll\n        for (int e = 0; e < {NE}; ++e) {{\n            const u32 row"
             edits.append((anchor, pre + anchor))
         else:
             edits.append(("ev[i][", "acc[i]["))         # relu looks at the result only
@@ -1958,13 +1969,20 @@ MATMUL_CONFIGS = {
     "64x64": (2, 2, 1, 1, 16),
     "64x64k64": (2, 2, 1, 1, 64),       # same tile, K walked 64 at a time: fewer barriers when one block per CU
     "32x32": (1, 1, 1, 1, 16),          # has nobody to overlap with (1024^3: 73 against 62 TFLOP/s)
+    # sixth entry 16: wavefronts of 16x16 (v_mfma_f32_16x16x4_f32) for small outputs with a long k, where the
+    # chain of MFMA steps per wavefront is what takes the time (2048 x 128 x 512)
+    "64x64m16": (4, 4, 1, 1, 64, 16),
+    "64x32m16": (4, 2, 1, 1, 32, 16),
+    "32x32m16": (2, 2, 1, 1, 32, 16),
 }
+MATMUL_SMALL_TILES = ("64x64", "64x64k64", "32x32", "64x64m16", "64x32m16", "32x32m16")
 
 
 def matmul_tile_shape(tile: str) -> tuple[int, int, int]:
     """(rows, columns, threads) of a block of the named configuration."""
-    wm, wn, mi, nj, _ = MATMUL_CONFIGS[tile]
-    return 32 * mi * wm, 32 * nj * wn, 64 * wm * wn
+    wm, wn, mi, nj, _, *s = MATMUL_CONFIGS[tile]
+    edge = s[0] if s else 32
+    return edge * mi * wm, edge * nj * wn, 64 * wm * wn
 
 
 # (relative per-CU throughput when the chip is full, resident blocks per CU): the model that

@@ -1305,7 +1305,10 @@ class HIP:
             score = rate * (M * N) / float(tm * bm * tn * bn) * fill
             if score > best_score * 1.0001:
                 best, best_score = name, score
-        if best == "64x64" and Kd >= 512 and -(-M // 64) * -(-N // 64) * batch <= 512:
+        small = -(-M // 64) * -(-N // 64) * batch           # blocks of the smallest 32-wide tile worth using
+        if best in ("64x64", "32x32") and small <= 192 and Kd >= 64:
+            best = "32x32m16"                       # a fraction of the SIMDs busy: four times the wavefronts, 16x16 each
+        elif best == "64x64" and Kd >= 512 and small <= 512:
             best = "64x64k64"                       # few blocks, long K: the deep-K form of the same tile
         return best
 
@@ -1318,7 +1321,7 @@ class HIP:
             bm, bn, _ = K.matmul_tile_shape(name)
             if bm > max(32, 2 * M) or bn > max(32, 2 * N):
                 continue
-            if M * N * batch > (1 << 22 if name == "32x32" else 1 << 27 if name.startswith("64x64") else 1 << 62):
+            if M * N * batch > (1 << 22 if name == "32x32" or name.endswith("m16") else 1 << 27 if name.startswith("64x64") else 1 << 62):
                 continue
             out.append(name)
         return out
@@ -1327,7 +1330,8 @@ class HIP:
     def _launch_matmul(tile: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple,
                        ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False, epi: str = "") -> None:
         bm, bn, threads = K.matmul_tile_shape(tile)
-        k = kernel(K.matmul_kernel, *K.MATMUL_CONFIGS[tile], veca, vecb, ta, tb, tri, strided, epi)
+        cfg = K.MATMUL_CONFIGS[tile]                           # (WM, WN, MI, NJ, BK) and, for the 16-wide MFMA tiles, 16
+        k = kernel(K.matmul_kernel, *cfg[:5], veca, vecb, ta, tb, tri, strided, epi, *cfg[5:])
         launch(k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch), threads, *args)
 
     @staticmethod

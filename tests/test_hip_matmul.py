@@ -208,7 +208,7 @@ def test_triangular_hints_skip_work_without_changing_a_bit(T, d, batch):
     want_scores = xd.matmul_nt(yd).numpy()
     want_av = lowd.matmul(yd).numpy()
     want_atv = lowd.matmul_tn(yd).numpy()
-    tiles = [t for t in K.MATMUL_CONFIGS if T >= 64 or t in ("64x64", "32x32")]
+    tiles = [t for t in K.MATMUL_CONFIGS if T >= 64 or t in K.MATMUL_SMALL_TILES]
     for tile in tiles:
         prev, HIP.MATMUL_FORCE = HIP.MATMUL_FORCE, tile
         try:
@@ -244,7 +244,7 @@ def test_epilogues_equal_the_separate_elementwise_kernels(shape_x, shape_y, nt):
     want_relu = plain.relu().numpy()
     want_gate = (ed > 0.0).where(inp=plain, other=0.0).numpy()
     small = min(plain.shape[-2:]) < 64
-    tiles = [None] + [t for t in K.MATMUL_CONFIGS if not small or t in ("64x64", "32x32")]
+    tiles = [None] + [t for t in K.MATMUL_CONFIGS if not small or t in K.MATMUL_SMALL_TILES]
     for tile in tiles:
         prev, HIP.MATMUL_FORCE = HIP.MATMUL_FORCE, tile
         try:
