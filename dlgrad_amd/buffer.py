@@ -388,9 +388,10 @@ class Buffer:
         return self._like(y), self._like(r, (self.numel // max(self.shape[-1], 1),))
 
     def rmsnorm_bwd(self, weight: "Buffer | None", r: "Buffer", dy: "Buffer",
-                    through_mean: bool) -> tuple["Buffer", "Buffer | None"]:
-        """self is the forward input x; returns (dx, dw) with dw shaped like the weight."""
-        dx, dw = self._dispatch(CustomOps.RMSNORM_BWD, x=self, w=weight, r=r, dy=dy, through_mean=through_mean)
+                    through_mean: bool, plus: "Buffer | None" = None) -> tuple["Buffer", "Buffer | None"]:
+        """self is the forward input x; returns (dx, dw) with dw shaped like the weight.  plus: added to dx as it is stored."""
+        kw = {"plus": plus} if plus is not None else {}
+        dx, dw = self._dispatch(CustomOps.RMSNORM_BWD, x=self, w=weight, r=r, dy=dy, through_mean=through_mean, **kw)
         return self._like(dx), (None if dw is None else self._like(dw, weight.shape))
 
     # ---- selects ----------------------------------------------------------------------------------

@@ -1535,7 +1535,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 
 
 @cache
-def rmsnorm_bwd_kernel(vec: int, nval: int, affine: bool, through_mean: bool) -> tuple[str, str, str]:
+def rmsnorm_bwd_kernel(vec: int, nval: int, affine: bool, through_mean: bool, plus: bool = False) -> tuple[str, str, str]:
     """Backward of the fused RMSNorm.  Per row, with dn = dy * w:
         dx = dn * r                                         (the path through x * r)
            + (x * 2) * ((1/L) * (sum(dn * x) * (r^3 * -0.5)))   (the path through mean(x^2)),
@@ -1544,9 +1544,12 @@ def rmsnorm_bwd_kernel(vec: int, nval: int, affine: bool, through_mean: bool) ->
     RMSNorm passes no gradient through the normaliser.
     dw = sum over rows of dy * (x * r): each wavefront walks rows_per_wave consecutive rows
     with its columns' partial sums in registers and writes one row of `dwpart`; a column
-    reduction over those partial rows finishes it."""
+    reduction over those partial rows finishes it.
+    plus: what is stored is prev + dx for a given array prev shaped like x (a gradient that
+    reached x by another route, e.g. the residual connection around the norm): dx is rounded to
+    fp32 first, so the sum has the bits of a separate addition kernel."""
     T, comps, nv = _rms_lanes(vec)
-    name = f"rmsnorm_bwd_v{vec}_r{nval}{'_w' if affine else ''}{'_m' if through_mean else ''}"
+    name = f"rmsnorm_bwd_v{vec}_r{nval}{'_w' if affine else ''}{'_m' if through_mean else ''}{'_p' if plus else ''}"
     dn = lambda c: f"(d[k]{c} * g[k]{c})" if affine else f"d[k]{c}"          # noqa: E731
     dot = " + ".join(f"{dn(c)} * v[k]{c}" for c in comps)
     dxs = "".join(
@@ -1557,10 +1560,19 @@ def rmsnorm_bwd_kernel(vec: int, nval: int, affine: bool, through_mean: bool) ->
     tail = f"""    {T}* __restrict__ pw = reinterpret_cast<{T}*>(dwpart + (u64)wid * L);
     #pragma unroll
     for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = lane + k * 64u; if (c < nv) pw[c] = acc[k]; }}""" if affine else ""
+    plus_load = f"""
+        {T} e[{nval}];
+        #pragma unroll
+        for (u32 k = 0; k < {nval}u; ++k) {{
+            const u32 c = lane + k * 64u;
+            if (c < nv) e[k] = reinterpret_cast<const {T}*>(prev + (u64)row * L)[c];
+        }}""" if plus else ""
+    # the empty asm keeps the last multiply of dx from being contracted into this addition
+    plus_add = "".join(f'                asm volatile("" : "+v"(o{c}));\n                o{c} = e[k]{c} + o{c};\n' for c in comps) if plus else ""
     src = f"""{PRELUDE}
 extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
         const float* __restrict__ w, const float* __restrict__ rinv, const float* __restrict__ dy,
-        float* __restrict__ dx, float* __restrict__ dwpart, u32 R, u32 L, u32 rows_per_wave) {{
+        float* __restrict__ dx, float* __restrict__ dwpart, u32 R, u32 L, u32 rows_per_wave{', const float* __restrict__ prev' if plus else ''}) {{
     const u32 lane = threadIdx.x & 63u;
     const u32 wid = blockIdx.x * 4u + (threadIdx.x >> 6);
     const u32 row0 = wid * rows_per_wave;
@@ -1585,7 +1597,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
         for (u32 k = 0; k < {nval}u; ++k) {{
             const u32 c = lane + k * 64u;
             if (c < nv) {{ v[k] = p[c]; d[k] = pd[c]; {f's += {dot};' if through_mean else ''} }}
-        }}
+        }}{plus_load}
         {'s = wave_sum(s);' if through_mean else ''}
         const float coef = (1.0f / (float)L) * (s * ((r * r * r) * -0.5f)); (void)coef;
         #pragma unroll
@@ -1593,14 +1605,14 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
             const u32 c = lane + k * 64u;
             if (c < nv) {{
                 {T} o;
-{dxs}                q[c] = o;
+{dxs}{plus_add}                q[c] = o;
 {accs}            }}
         }}
     }}
 {tail}
 }}
 """
-    return src, name, _fmt("P", "P", "P", "P", "P", "P", "I", "I", "I")
+    return src, name, _fmt("P", "P", "P", "P", "P", "P", "I", "I", "I", *(["P"] if plus else []))
 
 
 # =====================================================================================
@@ -1974,8 +1986,13 @@ MATMUL_CONFIGS = {
     "64x64m16": (4, 4, 1, 1, 64, 16),
     "64x32m16": (4, 2, 1, 1, 32, 16),
     "32x32m16": (2, 2, 1, 1, 32, 16),
+    # the same with k walked 128 at a time: a product with k = 128 is then one round of loads (all in flight
+    # together), one barrier and one run of MFMA steps instead of four dependent rounds
+    "64x64m16k128": (4, 4, 1, 1, 128, 16),
+    "32x32m16k128": (2, 2, 1, 1, 128, 16),
+    "32x32m16k64": (2, 2, 1, 1, 64, 16),
 }
-MATMUL_SMALL_TILES = ("64x64", "64x64k64", "32x32", "64x64m16", "64x32m16", "32x32m16")
+MATMUL_SMALL_TILES = ("64x64", "64x64k64", "32x32", "64x64m16", "64x32m16", "32x32m16", "64x64m16k128", "32x32m16k128", "32x32m16k64")
 
 
 def matmul_tile_shape(tile: str) -> tuple[int, int, int]:

@@ -564,9 +564,18 @@ class RMSNorm(OP):
         y, self.r = x.rmsnorm(weight, eps)
         return y
 
-    def backward(self, upstream_grad: Buffer) -> tuple:
-        dx, dw = self.x.rmsnorm_bwd(self.weight, self.r, upstream_grad, through_mean=not STRICT_REFERENCE)
+    def _grads(self, upstream_grad: Buffer, plus: Buffer | None) -> tuple:
+        dx, dw = self.x.rmsnorm_bwd(self.weight, self.r, upstream_grad, through_mean=not STRICT_REFERENCE, plus=plus)
         return (dx,) if self.weight is None else (dx, dw)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return self._grads(upstream_grad, None)
+
+    def backward_onto(self, upstream_grad: Buffer, have: tuple) -> tuple:
+        """have[0]: the gradient x has collected so far (the residual route around the norm), or None.
+        It is added as dx is stored, and parent 0 is reported as already summed."""
+        plus = have[0] if (have[0] is not None and have[0].shape == self.x.shape and have[0].device is self.x.device) else None
+        return self._grads(upstream_grad, plus), ((0,) if plus is not None else ())
 
 
 class CrossEntropy(OP):

@@ -1153,7 +1153,8 @@ class HIP:
     @staticmethod
     @dispatcher.register(CustomOps.RMSNORM_BWD, Device.HIP)
     def rmsnorm_bwd(x: Buffer, w: Buffer | None, r: Buffer, dy: Buffer,
-                    through_mean: bool) -> tuple[DevicePtr, DevicePtr | None]:
+                    through_mean: bool, plus: Buffer | None = None) -> tuple[DevicePtr, DevicePtr | None]:
+        """plus: an array shaped like x that is added to dx as it is stored (a gradient that reached x by another route)."""
         L = x.shape[-1]
         R = x.numel // L
         if dy.numel != x.numel or r.numel != R:
@@ -1165,14 +1166,16 @@ class HIP:
         rows_per_wave = max(1, (R + 511) // 512 if R * L <= (1 << 20) else (R + 2047) // 2048)
         P = (R + rows_per_wave - 1) // rows_per_wave            # partial rows of dw, one per wavefront
         part = alloc(P * L) if w is not None else None
+        if plus is not None and (plus.numel != x.numel or plus.is_host_scalar):
+            raise ValueError(f"rmsnorm_bwd: plus {plus.shape} is not shaped like x {x.shape}")
         vec = HIP._rms_vec(L, _addr(x), _addr(dy), dx.addr, _addr(w) if w is not None else 0,
-                           part.addr if part is not None else 0)
+                           part.addr if part is not None else 0, _addr(plus) if plus is not None else 0)
         nval = K.rmsnorm_plan(L, vec)
         if nval == 0:
             raise ValueError(f"fused RMSNorm: a row of {L} unaligned floats does not fit a wavefront's registers")
-        k = kernel(K.rmsnorm_bwd_kernel, vec, nval, w is not None, bool(through_mean))
+        k = kernel(K.rmsnorm_bwd_kernel, vec, nval, w is not None, bool(through_mean), plus is not None)
         launch(k, (P + 3) // 4, 256, _addr(x), _addr(w) if w is not None else 0, _addr(r), _addr(dy), dx.addr,
-               part.addr if part is not None else 0, R, L, rows_per_wave)
+               part.addr if part is not None else 0, R, L, rows_per_wave, *([_addr(plus)] if plus is not None else []))
         if w is None:
             return dx, None
         dw = alloc(L)
@@ -1321,7 +1324,7 @@ class HIP:
             bm, bn, _ = K.matmul_tile_shape(name)
             if bm > max(32, 2 * M) or bn > max(32, 2 * N):
                 continue
-            if M * N * batch > (1 << 22 if name == "32x32" or name.endswith("m16") else 1 << 27 if name.startswith("64x64") else 1 << 62):
+            if M * N * batch > (1 << 22 if name == "32x32" or "m16" in name else 1 << 27 if name.startswith("64x64") else 1 << 62):
                 continue
             out.append(name)
         return out

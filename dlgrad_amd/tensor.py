@@ -331,12 +331,18 @@ class Tensor:
         for node in reversed(topo):
             if node.grad is None:
                 raise RuntimeError(f"Tensor {node} has no grad")
-            grads = node._ctx.backward(node.grad.data)
-            for p, g in zip(node._ctx.parents, grads):
+            ctx = node._ctx
+            onto = getattr(ctx, "backward_onto", None)
+            if onto is None:
+                grads, summed = ctx.backward(node.grad.data), ()
+            else:       # an op that can add what a parent has collected so far as it stores that parent's gradient
+                have = tuple(p.grad.data if (p.grad is not None and p.requires_grad) else None for p in ctx.parents)
+                grads, summed = onto(node.grad.data, have)
+            for i, (p, g) in enumerate(zip(ctx.parents, grads)):
                 if g is None or not p.requires_grad:
                     continue
                 gt = Tensor(g, requires_grad=False, device=g.device)
-                p.grad = gt if p.grad is None else p.grad + gt
+                p.grad = gt if (p.grad is None or i in summed) else p.grad + gt
         for node in topo:                                # release the tape
             node._ctx = None
 

@@ -81,6 +81,55 @@ def test_complete_gradient_matches_torch_float64(shape, affine):
         assert dw is None
 
 
+@pytest.mark.parametrize("shape", SHAPES + [(3, 7, 130)])
+@pytest.mark.parametrize("affine,through_mean", [(True, True), (True, False), (False, True)])
+def test_gradient_added_on_store_has_the_bits_of_a_separate_addition(shape, affine, through_mean):
+    """rmsnorm_bwd(plus=p) stores p + dx: dx is rounded before the addition, so the result equals
+    the separate element-wise kernel bit for bit, and dw is untouched."""
+    require_gpu()
+    rng = np.random.default_rng(sum(shape) + 2 * affine + through_mean)
+    x, up, prev = (rng.standard_normal(shape, dtype=np.float32) for _ in range(3))
+    w = (1 + 0.1 * rng.standard_normal((1, shape[-1]))).astype(np.float32)
+    xb, wb, pb = dev(x), (dev(w) if affine else None), dev(prev)
+    _, r = xb.rmsnorm(wb, 1e-6)
+    dx, dw = xb.rmsnorm_bwd(wb, r, dev(up), through_mean=through_mean)
+    dx2, dw2 = xb.rmsnorm_bwd(wb, r, dev(up), through_mean=through_mean, plus=pb)
+    check(dx2.numpy(), (pb + dx).numpy(), 0, "prev + dx")
+    if affine:
+        check(dw2.numpy(), dw.numpy(), 0, "dw")
+
+
+def test_a_residual_gradient_is_added_by_the_norm_backward_itself():
+    """x feeds a norm and a residual connection: x.grad = g_residual + dx_norm.  The engine hands the
+    norm what x has collected so far (OP.backward_onto) instead of running an addition: same bits,
+    one kernel fewer."""
+    require_gpu()
+    from dlgrad_amd import nn, ops
+    rng = np.random.default_rng(5)
+    x0 = rng.standard_normal((4, 32, 128), dtype=np.float32)
+    g0 = rng.standard_normal((4, 32, 128), dtype=np.float32)
+
+    def run(onto):
+        x = Tensor(x0, device="hip", requires_grad=True)
+        h = x * 1.5                                   # a non-leaf with two consumers
+        norm = nn.RMSNorm(128, device="hip")
+        if not onto:
+            norm_ctx = ops.RMSNorm.backward_onto
+            ops.RMSNorm.backward_onto = None
+        try:
+            before = hip.launch_count
+            y = h + norm(h) * 2.0
+            (y * Tensor(g0, device="hip")).sum().backward()
+            return hip.launch_count - before, x.grad.numpy()
+        finally:
+            if not onto:
+                ops.RMSNorm.backward_onto = norm_ctx
+
+    (n1, a), (n0, b) = run(True), run(False)
+    assert n1 == n0 - 1, (n1, n0)
+    check(a, b, 0, "x.grad")
+
+
 def test_rows_that_do_not_fit_fall_back_to_the_composition():
     require_gpu()
     x = np.random.default_rng(3).standard_normal((3, 4100), dtype=np.float32)
