@@ -1309,8 +1309,9 @@ class HIP:
             if score > best_score * 1.0001:
                 best, best_score = name, score
         small = -(-M // 64) * -(-N // 64) * batch           # blocks of the smallest 32-wide tile worth using
-        if best in ("64x64", "32x32") and small <= 192 and Kd >= 64:
-            best = "32x32m16"                       # a fraction of the SIMDs busy: four times the wavefronts, 16x16 each
+        if best in ("64x64", "32x32") and small <= 192 and Kd >= 32:
+            # a fraction of the SIMDs busy: four times the wavefronts, 16x16 each, and as few rounds of loads as k allows
+            best = "32x32m16k128" if Kd >= 128 else "32x32m16k64" if Kd >= 64 else "32x32m16"
         elif best == "64x64" and Kd >= 512 and small <= 512:
             best = "64x64k64"                       # few blocks, long K: the deep-K form of the same tile
         return best
