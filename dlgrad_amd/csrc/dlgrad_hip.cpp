@@ -46,7 +46,13 @@ std::vector<hipModule_t> g_modules;
 // Arena 0 is the ordinary pool.  Other arenas are private pools for captured graphs: a
 // block handed out while an arena is current returns to that arena when freed and is
 // never given to anybody else, because a graph replays writes to its addresses.
-struct Block { size_t bucket; uint64_t arena; };
+struct Block { size_t bucket; uint64_t arena; void *base; };
+// Large blocks are handed out at base + colour * 4 KiB, colour cycling 0..3 from one large allocation
+// to the next.  Driver allocations of this size all start on the same multi-MiB alignment, so element i
+// of two operands of an element-wise kernel falls on the same DRAM channel and bank at the same moment;
+// 4 KiB between them is worth 5 % of a 16384x8192 add (6.26 -> 6.60 TB/s, measured over the offsets 0..1 MiB).
+constexpr size_t kStaggerMin = size_t(8) << 20, kStagger = 4096, kColours = 4;
+unsigned g_colour = 0;
 std::map<uint64_t, std::map<size_t, std::vector<void *>>> g_free;   // arena -> bucket -> cached blocks
 std::unordered_map<void *, Block> g_live;                            // block -> bucket, arena
 std::map<uint64_t, bool> g_arena_alive;                              // arenas that still exist
@@ -104,7 +110,8 @@ void trim_locked() {                              // the ordinary pool only: gra
 }
 
 int alloc_locked(size_t nbytes, void **out) {
-    size_t b = bucket_of(nbytes);
+    const bool stagger = nbytes >= kStaggerMin;
+    size_t b = bucket_of(stagger ? nbytes + (kColours - 1) * kStagger : nbytes);
     auto &lists = g_free[g_arena];
     auto it = lists.find(b);
     if (it != lists.end() && !it->second.empty()) {
@@ -130,7 +137,9 @@ int alloc_locked(size_t nbytes, void **out) {
         ++g_device_allocs;
         *out = p;
     }
-    g_live[*out] = Block{b, g_arena};
+    void *base = *out;
+    if (stagger) *out = static_cast<char *>(base) + (g_colour++ % kColours) * kStagger;
+    g_live[*out] = Block{b, g_arena, base};
     g_bytes_in_use += b;
     return 0;
 }
@@ -255,10 +264,10 @@ int dlg_hip_free(void *ptr) {
     g_live.erase(it);
     g_bytes_in_use -= blk.bucket;
     if (blk.arena != 0 && !g_arena_alive[blk.arena]) {      // its graph is gone: give the memory back
-        (void)hipFree(ptr);
+        (void)hipFree(blk.base);
         return 0;
     }
-    g_free[blk.arena][blk.bucket].push_back(ptr);
+    g_free[blk.arena][blk.bucket].push_back(blk.base);
     g_bytes_cached += blk.bucket;
     return 0;
 }
