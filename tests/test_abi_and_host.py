@@ -277,3 +277,35 @@ def test_bench_prints_one_json_line_with_the_contract_keys():
         assert key in out, key
     assert out["n_gpus"] == 1 and out["steps"] == 2 and out["warmup"] == 1 and out["vs_baseline"] is None
     assert out["dtype"] == "f32" and out["data"] == "synthetic" and "workload" in out["config"]
+
+
+@pytest.mark.gpu
+def test_large_blocks_are_staggered_and_recycled_whole():
+    """Allocations of 8 MiB and more start 4 KiB apart (mod 16 KiB) from one to the next, so that the
+    operands of an element-wise kernel do not meet the same DRAM bank at the same moment; freeing returns
+    the whole block (the next block of that size reuses it, whatever its offset), and contents written
+    through an offset pointer read back intact up to the last byte asked for."""
+    from dlgrad_amd.runtime import hip
+    if not hip.available():
+        pytest.skip("no HIP device")
+    import numpy as np
+    from dlgrad_amd.buffer import Buffer
+    from dlgrad_amd.device import Device
+    lib = hip.lib()
+    n = (8 << 20) // 4 + 1021                                     # just over 8 MiB, not a round size
+    ptrs = [hip.alloc(n) for _ in range(5)]
+    offs = [p.addr % (4 * 4096) for p in ptrs]
+    assert all(p.addr % 4096 == 0 for p in ptrs)
+    assert [(b - a) % (4 * 4096) for a, b in zip(offs, offs[1:])] == [4096] * 4, offs
+    small = [hip.alloc(1024) for _ in range(3)]
+    assert len({p.addr % 256 for p in small}) == 1                # small blocks are left alone
+    in_use, cached, allocs = lib.pool_stats()
+    del ptrs
+    again = [hip.alloc(n) for _ in range(5)]
+    assert lib.pool_stats()[2] == allocs, "freed large blocks were not reused"
+    data = np.arange(n, dtype=np.float32)
+    for p in again:
+        b = Buffer(p, (n,), Device.HIP)
+        b.upload_(data)
+    for p in again:
+        np.testing.assert_array_equal(Buffer(p, (n,), Device.HIP).numpy(), data)
