@@ -2011,6 +2011,115 @@ MATMUL_TILE_MODEL = {
 
 
 # =====================================================================================
+# attention for one new position (decoding)
+# =====================================================================================
+
+DECODE_ATTENTION_MAX_N = 1024
+DECODE_ATTENTION_MAX_D = 64
+
+
+@cache
+def decode_attention_kernel(npl: int, masked: bool, vec: int) -> tuple[str, str, str]:
+    """softmax(q k^T * scale) v for one query position per (sequence, head) against n cached positions:
+    the three launches of the decoding branch of examples/gpt.py:58-63 (scores, softmax, context) as one.
+    One wavefront per (sequence, head).  q is (B, 1, C) with the head's d <= 64 values at b*C + head*d;
+    the stores are (rows, B, C), row r of this head at r*pitch + b*C + head*d.  Lane l scores the
+    positions l, l + 64, ... (npl of them at most, so n <= 64*npl): d multiply-adds each, times
+    scale, -inf where `hidden` says so; maximum, exponentials and their sum are reduced over the
+    wavefront; the probabilities pass through LDS.
+    vec=4 (d in 4, 8, .. 64 a power of two, 16-byte aligned rows): key rows are read 16 bytes at a
+    time, eight loads in flight; for the context the lanes form d/4 column groups times 256/d position
+    groups, each lane adds p[r] * v[r][4 floats] over its share of the positions with sixteen loads in
+    flight, and the position groups are joined by lane exchanges.
+    vec=1: any d; lane j adds p[r] * v[r][j] over the positions (two interleaved halves when d <= 32)."""
+    assert npl in (2, 4, 8, 16) and vec in (1, 4)
+    name = f"decode_attention_r{npl}{'_m' if masked else ''}_v{vec}"
+    if vec == 4:
+        dot = """                const float4* __restrict__ kr = reinterpret_cast<const float4*>(kh + (u64)pos * pitch);
+                for (u32 j0 = 0; j0 < d4; j0 += 8u) {
+                    float4 kv[8];
+                    #pragma unroll
+                    for (u32 t = 0; t < 8u; ++t) kv[t] = kr[min(j0 + t, d4 - 1u)];
+                    #pragma unroll
+                    for (u32 t = 0; t < 8u; ++t) if (j0 + t < d4) {
+                        const u32 j = 4u * (j0 + t);
+                        acc = fmaf(qs[j], kv[t].x, acc); acc = fmaf(qs[j + 1u], kv[t].y, acc);
+                        acc = fmaf(qs[j + 2u], kv[t].z, acc); acc = fmaf(qs[j + 3u], kv[t].w, acc);
+                    }
+                }"""
+        context = """    const u32 CG = d4, PG = 64u / CG, cg = lane % CG;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    #pragma unroll 16
+    for (u32 pos = lane / CG; pos < n; pos += PG) {
+        const float w = ps[pos];
+        const float4 t = reinterpret_cast<const float4*>(vh + (u64)pos * pitch)[cg];
+        o.x = fmaf(w, t.x, o.x); o.y = fmaf(w, t.y, o.y); o.z = fmaf(w, t.z, o.z); o.w = fmaf(w, t.w, o.w);
+    }
+    for (u32 off = CG; off < 64u; off <<= 1) {
+        o.x += __shfl_xor(o.x, off, WAVE); o.y += __shfl_xor(o.y, off, WAVE);
+        o.z += __shfl_xor(o.z, off, WAVE); o.w += __shfl_xor(o.w, off, WAVE);
+    }
+    if (lane < CG) reinterpret_cast<float4*>(y + at)[lane] = o;"""
+    else:
+        dot = """                const float* __restrict__ kr = kh + (u64)pos * pitch;
+                for (u32 j0 = 0; j0 < d; j0 += 8u) {
+                    float kv[8];
+                    #pragma unroll
+                    for (u32 t = 0; t < 8u; ++t) kv[t] = kr[min(j0 + t, d - 1u)];
+                    #pragma unroll
+                    for (u32 t = 0; t < 8u; ++t) if (j0 + t < d) acc = fmaf(qs[j0 + t], kv[t], acc);
+                }"""
+        context = """    const u32 W = d <= 32u ? 32u : 64u, step = 64u / W, j = lane % W;
+    float o = 0.0f;
+    if (j < d) {
+        #pragma unroll 16
+        for (u32 pos = lane / W; pos < n; pos += step) o = fmaf(ps[pos], vh[(u64)pos * pitch + j], o);
+    }
+    if (step == 2u) o += __shfl_xor(o, 32, WAVE);
+    if (lane < d) y[at + lane] = o;"""
+    hid = "if (hidden[pos] > 0.0f) acc = -__builtin_inff();" if masked else ""
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(64) void {name}(const float* __restrict__ q,
+        const float* __restrict__ ks, const float* __restrict__ vs, const float* __restrict__ hidden,
+        float* __restrict__ y, u32 n, u32 C, u32 d, u32 pitch, u32 n_head, float scale) {{
+    __shared__ float qs[{DECODE_ATTENTION_MAX_D}];
+    __shared__ float ps[{64 * npl}];
+    const u32 lane = threadIdx.x, b = blockIdx.x / n_head, at = b * C + (blockIdx.x % n_head) * d;
+    const u32 d4 = d >> 2; (void)d4;
+    const float* __restrict__ kh = ks + at;
+    const float* __restrict__ vh = vs + at;
+    if (lane < d) qs[lane] = q[at + lane];
+    __syncthreads();
+    float sc[{npl}];
+    float m = -__builtin_inff();
+    #pragma unroll
+    for (u32 k = 0; k < {npl}u; ++k) {{
+        const u32 pos = lane + 64u * k;
+        float acc = -__builtin_inff();
+        if (pos < n) {{
+            acc = 0.0f;
+{dot}
+            acc *= scale;
+            {hid}
+        }}
+        sc[k] = acc;
+        m = fmaxf(m, acc);
+    }}
+    m = wave_max(m);
+    float sum = 0.0f;
+    #pragma unroll
+    for (u32 k = 0; k < {npl}u; ++k) {{ sc[k] = expf(sc[k] - m); sum += sc[k]; }}
+    sum = wave_sum(sum);
+    #pragma unroll
+    for (u32 k = 0; k < {npl}u; ++k) ps[lane + 64u * k] = sc[k] / sum;
+    __syncthreads();
+{context}
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "P", "P", "I", "I", "I", "I", "I", "f")
+
+
+# =====================================================================================
 # optimizer
 # =====================================================================================
 

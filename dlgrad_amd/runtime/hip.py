@@ -1261,6 +1261,8 @@ class HIP:
         launch(kernel(K.sgd_inplace_kernel, v is not None), (n + 255) // 256, 256,
                _addr(p), _addr(g), _addr(v) if v is not None else 0, n, float(lr), float(momentum))
 
+    DECODE_FUSED = os.environ.get("DLGRAD_HIP_DECODE_FUSED", "1") != "0"    # "0": cached attention as product, softmax, product
+
     # ---- matmul ----------------------------------------------------------------------------------------------------------
     MATMUL_FORCE = os.environ.get("DLGRAD_HIP_MATMUL_TILE")      # e.g. "128x128": benchmarking aid
     # "1": a shape met for the first time (and large enough to matter) is timed once with every
@@ -1576,6 +1578,17 @@ class HIP:
         to leave out (-inf before the softmax).  Inference only."""
         Bn, _, C = q.shape
         d = C // n_head
+        if HIP.DECODE_FUSED and 0 < n <= K.DECODE_ATTENTION_MAX_N and d <= K.DECODE_ATTENTION_MAX_D and Bn * n_head < 2 ** 31:
+            # one wavefront per (sequence, head) does scores, softmax and context in one launch
+            if hidden is not None and hidden.numel < n:
+                raise ValueError(f"cached_attention: hidden {hidden.shape} is shorter than {n} positions")
+            y = alloc(Bn * C)
+            addrs = (_addr(q), _addr(k_store), _addr(v_store))
+            vec = 4 if (d in (4, 8, 16, 32, 64) and C % 4 == 0 and not any(a & 15 for a in addrs + (y.addr,))) else 1
+            npl = next(v for v in (2, 4, 8, 16) if 64 * v >= n)
+            launch(kernel(K.decode_attention_kernel, npl, hidden is not None, vec), Bn * n_head, 64, *addrs,
+                   _addr(hidden) if hidden is not None else 0, y.addr, n, C, d, Bn * C, n_head, float(scale))
+            return y
         store_heads = lambda buf: (_addr(buf), Bn * C, C, d)                        # noqa: E731  rows = positions
         one_row = lambda addr: (addr, C, C, d)                                        # noqa: E731  (B, 1, C)
         s = alloc(Bn * n_head * n)

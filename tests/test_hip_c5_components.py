@@ -363,3 +363,46 @@ def test_feed_forward_with_fused_epilogues_equals_the_four_ops(B, T, C, H, monke
             continue
         for i, (a, b) in enumerate(zip(fused, chain)):
             assert a.shape == b.shape and (a.view(np.uint32) == b.view(np.uint32)).all(), f"{what} output/gradient {i}"
+
+
+@pytest.mark.parametrize("B,h,d,rows,n,masked", [(1, 4, 32, 128, 128, True), (1, 4, 32, 128, 37, False), (3, 2, 64, 300, 300, True),
+                                                 (2, 3, 20, 70, 65, False), (2, 12, 64, 1024, 1000, True), (1, 1, 7, 5, 1, False)])
+def test_attention_for_one_new_position_in_one_launch(B, h, d, rows, n, masked, monkeypatch):
+    """nn.cached_attention on the hip device: scores, softmax and context of the decoding branch
+    (examples/gpt.py:58-63) by one kernel, checked against float64 numpy and against the three-launch
+    form it replaces, both to 2e-6 of the largest entry (the dot products are added in another order)."""
+    require_gpu()
+    from dlgrad_amd.runtime.hip import HIP
+    rng = np.random.default_rng(B * 100 + n)
+    C = h * d
+    q = rng.standard_normal((B, 1, C), dtype=np.float32)
+    ks, vs = (rng.standard_normal((rows, B, C), dtype=np.float32) for _ in range(2))
+    hidden = (rng.random((1, n)) < 0.3).astype(np.float32) if masked else None
+    if masked:
+        hidden[0, 0] = 0.0                                         # something is always visible
+    scale = d ** -0.5
+    qd, kd, vd = dev(q), dev(ks), dev(vs)
+    hd = dev(hidden) if masked else None
+
+    def run(fused):
+        monkeypatch.setattr(HIP, "DECODE_FUSED", fused)
+        before = hip.launch_count
+        y = qd.cached_attention(kd, vd, n, h, scale, hd)
+        return hip.launch_count - before, y.numpy()
+
+    (l1, got), (l0, chain) = run(True), run(False)
+    assert l1 == 1 and l0 >= 3, (l1, l0)
+    q64 = q.astype(np.float64).reshape(B, h, d)
+    k64 = ks[:n].astype(np.float64).reshape(n, B, h, d)
+    v64 = vs[:n].astype(np.float64).reshape(n, B, h, d)
+    s = np.einsum("bhd,nbhd->bhn", q64, k64) * scale
+    if masked:
+        s = np.where(hidden[0] > 0, -np.inf, s)
+    p = np.exp(s - s.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    want = np.einsum("bhn,nbhd->bhd", p, v64).reshape(B, 1, C)
+    if hip.COMPILE_ONLY:
+        return
+    top = np.abs(want).max()
+    assert np.abs(got - want).max() <= 2e-6 * top, "one-launch attention vs float64"
+    assert np.abs(got - chain).max() <= 2e-6 * top, "one-launch attention vs product-softmax-product"
