@@ -3,6 +3,7 @@ dlgrad/nn/__init__.py:8-41."""
 import math
 
 from dlgrad_amd import ops
+from dlgrad_amd.buffer import Buffer
 from dlgrad_amd.device import Device
 from dlgrad_amd.nn import optim, utils  # noqa: F401
 from dlgrad_amd.tensor import Tensor
@@ -117,7 +118,6 @@ def stack_parameters(tensors: list) -> None:
     first = tensors[0]
     if first.device is not Device.HIP or any(t.shape != first.shape or t.device is not Device.HIP for t in tensors):
         return
-    from dlgrad_amd.buffer import Buffer
     n = first.numel
     base = Buffer.full((len(tensors) * n,), 0.0, Device.HIP)
     for i, t in enumerate(tensors):
@@ -134,6 +134,19 @@ def self_attention_qkv(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor, n_head: in
     if ops.use_fused_qkv_attention(x, wq, wk, wv, n_head):
         return ops.SelfAttentionQKV.execute(x, wq, wk, wv, n_head=n_head, scale=scale)
     return causal_self_attention(x.linear(wq, None), x.linear(wk, None), x.linear(wv, None), n_head, scale)
+
+
+def project_qkv_row(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor) -> tuple[Tensor, Tensor, Tensor]:
+    """(x @ wq^T, x @ wk^T, x @ wv^T) for decoding.  When x is a single row and the weights are stacked
+    in memory (stack_parameters), the hip device runs one product and the three results are the
+    thirds of its output row; such results carry no tape (inference only).  Otherwise three linears."""
+    if x.numel == x.shape[-1] and x.numel and ops.FUSED and ops.stacked(wq, wk, wv) and x.device is wq.device:
+        C = wq.shape[0]
+        w = Buffer(wq.data.ptr, (3 * C, wq.shape[1]), wq.device)
+        row = x.data.matmul_nt(w)
+        shape = x.shape[:-1] + (C,)
+        return tuple(Tensor(Buffer(row.ptr + i * C, shape, x.device), requires_grad=False) for i in range(3))
+    return x.linear(wq, None), x.linear(wk, None), x.linear(wv, None)
 
 
 def mlp_relu(x: Tensor, w_fc: Tensor, w_proj: Tensor, residual: Tensor | None = None) -> Tensor:

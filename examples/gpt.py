@@ -48,7 +48,7 @@ class CausalSelfAttention:
             # merge the heads (examples/gpt.py:45-57): one node on the hip device
             return self.c_proj(nn.self_attention_qkv(x, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight,
                                                      self.n_head, self.scale), residual)
-        q_lin, k_lin, v_lin = self.q_proj(x), self.k_proj(x), self.v_proj(x)    # (B, T, C)
+        q_lin, k_lin, v_lin = nn.project_qkv_row(x, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight)   # (B, T, C)
         if cache.length > 0:
             assert T == 1, "incremental attention takes one new position"
             cache.write(layer, k_lin, v_lin, cache.length)
@@ -225,9 +225,10 @@ class StaticDecoder:
 
     def _attend(self, attn: CausalSelfAttention, x: Tensor, layer: int, hidden: Tensor, residual: Tensor) -> Tensor:
         T = self.model.config.block_size
-        self.cache.k[layer].data.row_store_(attn.k_proj(x).data, self.slot.data)
-        self.cache.v[layer].data.row_store_(attn.v_proj(x).data, self.slot.data)
-        y = nn.cached_attention(attn.q_proj(x), self.cache.k[layer], self.cache.v[layer], T, attn.n_head, attn.scale, hidden)
+        q, k, v = nn.project_qkv_row(x, attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight)
+        self.cache.k[layer].data.row_store_(k.data, self.slot.data)
+        self.cache.v[layer].data.row_store_(v.data, self.slot.data)
+        y = nn.cached_attention(q, self.cache.k[layer], self.cache.v[layer], T, attn.n_head, attn.scale, hidden)
         return attn.c_proj(y, residual)
 
     def step(self) -> None:
