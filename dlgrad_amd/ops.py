@@ -331,7 +331,8 @@ class LinearNT(OP):
     with W read in place.  The reference builds it as Transpose -> MatMul, i.e. one permute
     forward and three backward (Y^T, X^T, and the transpose of dW^T back); here
     dX = G @ W and dW = sum over the batch of G^T @ X need none.  Same products, same order
-    of additions: bit-identical to that composition."""
+    of additions: bit-identical to that composition -- except for a single row x (decoding), whose
+    product runs as one wavefront per output with the k sum split over the lanes (1e-6)."""
 
     def forward(self, x: Buffer, w: Buffer) -> Buffer:
         self.x, self.w = x, w

@@ -1261,6 +1261,7 @@ class HIP:
         launch(kernel(K.sgd_inplace_kernel, v is not None), (n + 255) // 256, 256,
                _addr(p), _addr(g), _addr(v) if v is not None else 0, n, float(lr), float(momentum))
 
+    ROW_MATMUL = os.environ.get("DLGRAD_HIP_ROW_MATMUL", "1") != "0"        # "0": one-row products on the MFMA tiles too
     DECODE_FUSED = os.environ.get("DLGRAD_HIP_DECODE_FUSED", "1") != "0"    # "0": cached attention as product, softmax, product
 
     # ---- matmul ----------------------------------------------------------------------------------------------------------
@@ -1447,6 +1448,12 @@ class HIP:
             nbc, batch = B1, B0 * B1
             sa = (xb[1] * M * Kd if xb[0] > 1 else 0, M * Kd if xb[1] > 1 else 0)
             sb = (yb[1] * Kd * N if yb[0] > 1 else 0, Kd * N if yb[1] > 1 else 0)
+        if (M == 1 and batch == 1 and tb and not ta and not tri and HIP.ROW_MATMUL and not HIP.MATMUL_FORCE and Kd % 4 == 0
+                and not ((_addr(x) | _addr(y)) & 15) and (e is None or not e.is_host_scalar)):
+            # one row against a transposed matrix (a linear layer while decoding): a wavefront per output
+            launch(kernel(K.row_matmul_nt_kernel, epi), (N + 3) // 4, 256, _addr(x), _addr(y), out.addr,
+                   _addr(e) if e is not None else 0, N, Kd)
+            return out
         if batch > 65535:
             raise ValueError(f"{batch} batches exceed the grid limit")
         if max(M * Kd, Kd * N, M * N) >= 2 ** 31:

@@ -275,3 +275,34 @@ def test_triangular_hints_are_refused_where_they_make_no_sense():
         a.matmul(b, tri="a_lower")                      # A is not square
     with pytest.raises(ValueError):
         a.matmul_nt(dev(f32(4, 16)), tri="out_lower")   # the output is not square
+
+
+@pytest.mark.parametrize("N,K,lead", [(128, 128, (1, 1)), (384, 128, (1,)), (65, 128, ()), (512, 2048, (1, 1)), (7, 12, (1,)), (130, 1000, ())])
+def test_one_row_times_a_transposed_matrix(N, K, lead, monkeypatch):
+    """The linear layers of a decoding step, x (1, K) against W (N, K): one wavefront per output
+    instead of an MFMA tile with one useful row.  Checked against float64 and against the tile path
+    (1e-6 of the largest entry: the k sum is split over the lanes), with each epilogue."""
+    require_gpu()
+    from dlgrad_amd.runtime.hip import HIP
+    rng = np.random.default_rng(N + K)
+    x = rng.standard_normal(lead + (1, K), dtype=np.float32)
+    w = rng.standard_normal((N, K), dtype=np.float32)
+    e = rng.standard_normal(lead + (1, N), dtype=np.float32)
+    e[..., ::3] = 0.0
+    xd, wd, ed = dev(x), dev(w), dev(e)
+    want = x.astype(np.float64) @ w.astype(np.float64).T
+    variants = {"": want, "add": want + e, "relu": np.maximum(want, 0), "gate": np.where(e > 0, want, 0)}
+    for epi, ref in variants.items():
+        kw = {"epi": epi, "e": ed} if epi in ("add", "gate") else {"epi": epi} if epi else {}
+        before = hip.launch_count
+        got = xd.matmul_nt(wd, **kw).numpy()
+        assert hip.launch_count - before == 1
+        monkeypatch.setattr(HIP, "ROW_MATMUL", False)
+        tiled = xd.matmul_nt(wd, **kw).numpy()
+        monkeypatch.setattr(HIP, "ROW_MATMUL", True)
+        if hip.COMPILE_ONLY:
+            continue
+        assert got.shape == ref.shape
+        top = np.abs(want).max()
+        assert np.abs(got - ref).max() <= 2e-6 * top, f"{epi or 'plain'} vs float64"
+        assert np.abs(got - tiled).max() <= 2e-6 * top, f"{epi or 'plain'} vs the tile path"

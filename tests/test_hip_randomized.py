@@ -121,7 +121,11 @@ def test_random_matmuls_plain_and_transposed(seed):
             assert np.abs(nn_ - want).max() <= 1e-4 * scale, f"matmul {x.shape} {y.shape}"
         yt = np.ascontiguousarray(np.swapaxes(y, -1, -2))
         xt = np.ascontiguousarray(np.swapaxes(x, -1, -2))
-        check(xd.matmul_nt(dev(yt)).numpy(), nn_, 0, f"NT {x.shape} {yt.shape}")          # same bits as the plain product
+        nt = xd.matmul_nt(dev(yt)).numpy()
+        if x.size == Kd and not hip.COMPILE_ONLY:           # a single row: one wavefront per output splits the k sum over its lanes
+            assert np.abs(nt - nn_).max() <= 2e-6 * scale, f"NT {x.shape} {yt.shape}"
+        else:
+            check(nt, nn_, 0, f"NT {x.shape} {yt.shape}")                                 # same bits as the plain product
         check(dev(xt).matmul_tn(yd).numpy(), nn_, 0, f"TN {xt.shape} {y.shape}")
 
 
