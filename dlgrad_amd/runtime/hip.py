@@ -1585,6 +1585,11 @@ class HIP:
         to leave out (-inf before the softmax).  Inference only."""
         Bn, _, C = q.shape
         d = C // n_head
+        if q.shape[1] != 1 or C % n_head or n < 1:
+            raise ValueError(f"cached_attention: q {q.shape} is not one position of {n_head} heads, or n = {n}")
+        for store in (k_store, v_store):
+            if store.ndim != 3 or store.shape[1:] != (Bn, C) or store.shape[0] < n:
+                raise ValueError(f"cached_attention: a store of shape {store.shape} does not hold {n} rows of ({Bn}, {C})")
         if HIP.DECODE_FUSED and 0 < n <= K.DECODE_ATTENTION_MAX_N and d <= K.DECODE_ATTENTION_MAX_D and Bn * n_head < 2 ** 31:
             # one wavefront per (sequence, head) does scores, softmax and context in one launch
             if hidden is not None and hidden.numel < n:

@@ -406,3 +406,16 @@ def test_attention_for_one_new_position_in_one_launch(B, h, d, rows, n, masked, 
     top = np.abs(want).max()
     assert np.abs(got - want).max() <= 2e-6 * top, "one-launch attention vs float64"
     assert np.abs(got - chain).max() <= 2e-6 * top, "one-launch attention vs product-softmax-product"
+
+
+def test_cached_attention_checks_its_stores_on_the_host():
+    require_gpu()
+    q = dev(np.zeros((2, 1, 8), np.float32))
+    store = dev(np.zeros((5, 2, 8), np.float32))
+    with pytest.raises(ValueError):
+        q.cached_attention(store, store, 6, 2, 1.0)                       # more positions than rows
+    with pytest.raises(ValueError):
+        q.cached_attention(dev(np.zeros((5, 1, 8), np.float32)), store, 3, 2, 1.0)   # another batch size
+    with pytest.raises(ValueError):
+        dev(np.zeros((2, 2, 8), np.float32)).cached_attention(store, store, 3, 2, 1.0)   # two positions
+    assert q.cached_attention(store, store, 5, 2, 1.0).shape == (2, 1, 8)
