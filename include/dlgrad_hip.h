@@ -66,6 +66,10 @@ int dlg_hip_shutdown(void);
  * dlg_hip_free       <- free_ptr(ptr)                 cpu_kernel.py:730-740 (the ffi.gc finaliser)
  * Blocks come from a size-bucketed pool over hipMalloc; free returns the block
  * to the pool (safe without a sync because every user is on the one stream).
+ * Blocks of 8 MiB and more start 0, 4, 8 or 12 KiB into their pool block, in
+ * turn, so that equal offsets into two large operands fall on different DRAM
+ * banks; such pointers stay 4 KiB aligned, and dlg_hip_free takes the
+ * pointer that dlg_hip_alloc returned.
  * A NULL/failed allocation is an error return, which the Python side turns
  * into MemoryError exactly where the reference does (cpu.py:104,132,189).   */
 int dlg_hip_alloc(size_t nbytes, void **out);
