@@ -436,13 +436,22 @@ class Buffer:
         """In-place Adam update of self, m and v with the constants held in device memory."""
         self._dispatch(CustomOps.ADAM_STEP_INPLACE, p=self, g=g, m=m, v=v, consts=consts)
 
-    def row_store_(self, src: "Buffer", idx: "Buffer") -> None:
+    def row_store_(self, src: "Buffer", idx: "Buffer", also: "tuple[Buffer, Buffer] | None" = None) -> None:
         """self[(int)idx, :] = src, rows being the leading dim of self; idx is a one-element
-        Buffer on the same device, read where the kernel runs."""
+        Buffer on the same device, read where the kernel runs.  also = (dst2, src2): the same for a
+        second destination of the same shape (one launch on the hip device)."""
         rows = self.shape[0]
         width = self.numel // max(rows, 1)
         if src.numel != width or idx.numel != 1 or idx.is_host_scalar:
             raise ValueError(f"row_store_: row of {src.numel} into {self.shape}, index {idx.shape}")
+        if also is not None:
+            dst2, src2 = also
+            if dst2.shape != self.shape or src2.numel != width or dst2.device is not self.device:
+                raise ValueError(f"row_store_: second pair {dst2.shape} <- {src2.shape} does not match {self.shape}")
+            if self.device is Device.HIP:
+                self._dispatch(CustomOps.ROW_STORE, dst=self, src=src, idx=idx, rows=rows, width=width, dst2=dst2, src2=src2)
+                return
+            dst2.row_store_(src2, idx)
         self._dispatch(CustomOps.ROW_STORE, dst=self, src=src, idx=idx, rows=rows, width=width)
 
     def sgd_step_(self, g: "Buffer", v: "Buffer | None", lr: float, momentum: float) -> None:

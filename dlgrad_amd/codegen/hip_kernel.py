@@ -1452,22 +1452,27 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const unsigned char* __
 
 
 @cache
-def row_store_kernel() -> tuple[str, str, str]:
+def row_store_kernel(pairs: int = 1) -> tuple[str, str, str]:
     """dst[(int)idx[0], :] = src[:] for a (R, W) dst: a row written at a position that is itself
     device data, which is what lets one captured decoding step append to the key/value cache
-    at a different place on every replay.  A row index outside [0, R) writes nothing."""
-    name = "row_store"
+    at a different place on every replay.  A row index outside [0, R) writes nothing.
+    pairs=2: a second (dst, src) of the same shape in the same launch (blockIdx.y picks the pair):
+    the key and the value row of one layer."""
+    assert pairs in (1, 2)
+    name = "row_store" + ("2" if pairs == 2 else "")
+    second = ", float* __restrict__ dst2, const float* __restrict__ src2" if pairs == 2 else ""
+    pick = "    if (blockIdx.y == 1u) { dst = dst2; src = src2; }\n" if pairs == 2 else ""
     src = f"""{PRELUDE}
 extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ dst, const float* __restrict__ src,
-        const float* __restrict__ idx, u32 R, u32 W) {{
-    const float fi = idx[0];
+        const float* __restrict__ idx, u32 R, u32 W{second}) {{
+{pick}    const float fi = idx[0];
     if (!(fi >= 0.0f) || fi >= (float)R) return;
     const u32 row = (u32)fi;
     const u32 j = blockIdx.x * 256u + threadIdx.x;
     if (j < W) dst[(u64)row * W + j] = src[j];
 }}
 """
-    return src, name, _fmt("P", "P", "P", "I", "I")
+    return src, name, _fmt("P", "P", "P", "I", "I", *(["P", "P"] if pairs == 2 else []))
 
 
 # =====================================================================================

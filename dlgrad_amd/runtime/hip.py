@@ -517,9 +517,16 @@ class HIP:
 
     @staticmethod
     @dispatcher.register(CustomOps.ROW_STORE, Device.HIP)
-    def row_store(dst: Buffer, src: Buffer, idx: Buffer, rows: int, width: int) -> None:
-        if rows and width:
+    def row_store(dst: Buffer, src: Buffer, idx: Buffer, rows: int, width: int,
+                  dst2: Buffer | None = None, src2: Buffer | None = None) -> None:
+        """dst2 / src2: a second destination and row of the same shape, stored by the same launch."""
+        if not (rows and width):
+            return
+        if dst2 is None:
             launch(kernel(K.row_store_kernel), (width + 255) // 256, 256, _addr(dst), _addr(src), _addr(idx), rows, width)
+        else:
+            launch(kernel(K.row_store_kernel, 2), ((width + 255) // 256, 2, 1), 256, _addr(dst), _addr(src), _addr(idx),
+                   rows, width, _addr(dst2), _addr(src2))
 
     @staticmethod
     @dispatcher.register(CustomOps.COPY_INTO, Device.HIP)

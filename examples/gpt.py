@@ -226,8 +226,7 @@ class StaticDecoder:
     def _attend(self, attn: CausalSelfAttention, x: Tensor, layer: int, hidden: Tensor, residual: Tensor) -> Tensor:
         T = self.model.config.block_size
         q, k, v = nn.project_qkv_row(x, attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight)
-        self.cache.k[layer].data.row_store_(k.data, self.slot.data)
-        self.cache.v[layer].data.row_store_(v.data, self.slot.data)
+        self.cache.k[layer].data.row_store_(k.data, self.slot.data, also=(self.cache.v[layer].data, v.data))
         y = nn.cached_attention(q, self.cache.k[layer], self.cache.v[layer], T, attn.n_head, attn.scale, hidden)
         return attn.c_proj(y, residual)
 
