@@ -295,3 +295,34 @@ def test_softmax_with_causal_minus_inf_mask_gives_exact_zeros():
     if not hip.COMPILE_ONLY:
         assert np.all(p[..., np.triu_indices(128, 1)[0], np.triu_indices(128, 1)[1]] == 0)
         np.testing.assert_allclose(p.sum(-1), 1.0, rtol=1e-5)
+
+
+@pytest.mark.parametrize("W", [1, 64, 384, 1000])
+def test_row_store_writes_the_row_the_device_index_names(W):
+    """dst[(int)idx, :] = src with idx read on the device (the cache append of a captured decoding
+    step), alone and for two destinations in one launch; an index outside the rows writes nothing.
+    Bit-exact."""
+    require_gpu()
+    rng = np.random.default_rng(W)
+    R = 9
+    a0, b0 = (rng.standard_normal((R, 2, W), dtype=np.float32) for _ in range(2))
+    ra, rb = (rng.standard_normal((1, 2 * W), dtype=np.float32) for _ in range(2))
+    for row in (0, 4, 8, 9, -1):
+        a, b, idx = dev(a0), dev(b0), dev(np.array([[row]], np.float32))
+        before = hip.launch_count
+        a.row_store_(dev(ra), idx, also=(b, dev(rb)))
+        launches = hip.launch_count - before
+        wa, wb = a0.copy(), b0.copy()
+        if 0 <= row < R:
+            wa[row], wb[row] = ra.reshape(2, W), rb.reshape(2, W)
+        check(a.numpy(), wa, 0, f"first destination, row {row}")
+        check(b.numpy(), wb, 0, f"second destination, row {row}")
+        assert launches == 1
+        c = dev(a0)
+        c.row_store_(dev(rb), idx)
+        wc = a0.copy()
+        if 0 <= row < R:
+            wc[row] = rb.reshape(2, W)
+        check(c.numpy(), wc, 0, f"single destination, row {row}")
+    with pytest.raises(ValueError):
+        dev(a0).row_store_(dev(ra), dev(np.zeros((1, 1), np.float32)), also=(dev(np.zeros((R, 3, W), np.float32)), dev(rb)))
