@@ -381,6 +381,19 @@ class Buffer:
         """self is a log-softmax; returns ((exp(self) - onehot(target)) * upstream) / n."""
         return self._like(self._dispatch(CustomOps.CE_GRAD, lsm=self, target=target, upstream=upstream, n=n))
 
+    def ce_stats(self, target: "Buffer") -> tuple["Buffer", "Buffer", "Buffer"]:
+        """self: (N, V) logits.  Returns per row the max, log(sum(exp(x - max))) and the target's
+        log-probability, each as (1, N) -- the cross-entropy forward without a log-softmax tensor."""
+        n = self.shape[0]
+        m, ls, picked = self._dispatch(CustomOps.CE_STATS, x=self, target=target)
+        return self._like(m, (1, n)), self._like(ls, (1, n)), self._like(picked, (1, n))
+
+    def ce_grad_logits(self, m: "Buffer", ls: "Buffer", target: "Buffer", upstream: "Buffer", n: float) -> "Buffer":
+        """self: the logits ce_stats saw, m / ls: its row statistics.  Returns
+        ((softmax(self) - onehot(target)) * upstream) / n."""
+        return self._like(self._dispatch(CustomOps.CE_GRAD_LOGITS, x=self, m=m, ls=ls, target=target,
+                                         upstream=upstream, n=n))
+
     def rmsnorm(self, weight: "Buffer | None", eps: float) -> tuple["Buffer", "Buffer"]:
         """Fused RMSNorm over the last axis; returns (y, r) with r = rsqrt(mean(x^2) + eps)
         per row, kept for the backward pass."""

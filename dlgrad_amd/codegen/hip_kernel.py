@@ -863,17 +863,21 @@ struct PArgs {{ u32 np, nq, nt, nb;        // extents: two carried dims, tile di
 def embedding_kernel() -> tuple[str, str, str]:
     """Gather: out[i, :] = x[(int)(idx[i] * W) + 0..W) (cpu_kernel.py:217-229; the
     offset is formed in float and truncated, exactly as there).  One wavefront per
-    index; 16-byte moves when W and the offset allow it."""
+    index; 16-byte moves when W and the offset allow it.  An index whose row does not lie
+    inside the table's `total` floats (negative, or >= the row count) reads nothing: its
+    output row is zeros (the reference reads whatever memory lies there)."""
     name = "embedding_gather"
     src = f"""{PRELUDE}
 extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
-        const float* __restrict__ idx, float* __restrict__ out, u32 n_idx, u32 W, u32 aligned) {{
+        const float* __restrict__ idx, float* __restrict__ out, u32 n_idx, u32 W, u32 aligned, u32 total) {{
     const u32 i = blockIdx.x * 4u + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
     if (i >= n_idx) return;
     const int x_idx = (int)(idx[i] * (float)W);
     const float* __restrict__ src = x + (long long)x_idx;
     float* __restrict__ dst = out + (u64)i * W;
-    if (aligned && ((x_idx & 3) == 0)) {{
+    if (x_idx < 0 || (u64)x_idx + W > (u64)total) {{
+        for (u32 j = lane; j < W; j += 64u) dst[j] = 0.0f;
+    }} else if (aligned && ((x_idx & 3) == 0)) {{
         for (u32 v = lane; v < (W >> 2); v += 64u)
             reinterpret_cast<float4*>(dst)[v] = reinterpret_cast<const float4*>(src)[v];
     }} else {{
@@ -881,7 +885,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
     }}
 }}
 """
-    return src, name, _fmt("P", "P", "P", "I", "I", "I")
+    return src, name, _fmt("P", "P", "P", "I", "I", "I", "I")
 
 
 @cache
@@ -890,19 +894,22 @@ def embedding_backward_kernel() -> tuple[str, str, str]:
     (cpu_kernel.py:231-243).  The row index is formed in integers; the reference forms
     idx*W + j in float, which is the same number wherever that product is exact
     (below 2^24) and a wrong column above.  Hardware fp32 atomics, one wavefront per
-    index row, so duplicate ids accumulate in an unspecified order."""
+    index row, so duplicate ids accumulate in an unspecified order.  Rows whose index is
+    outside [0, V) are skipped."""
     name = "embedding_scatter_add"
     src = f"""{PRELUDE}
 extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out,
-        const float* __restrict__ g, const float* __restrict__ idx, u32 n_idx, u32 W) {{
+        const float* __restrict__ g, const float* __restrict__ idx, u32 n_idx, u32 W, u32 V) {{
     const u32 i = blockIdx.x * 4u + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
     if (i >= n_idx) return;
-    float* __restrict__ dst = out + (long long)((int)idx[i]) * W;
+    const int row = (int)idx[i];
+    if ((u32)row >= V) return;
+    float* __restrict__ dst = out + (long long)row * W;
     const float* __restrict__ src = g + (u64)i * W;
     for (u32 j = lane; j < W; j += 64u) unsafeAtomicAdd(dst + j, src[j]);
 }}
 """
-    return src, name, _fmt("P", "P", "P", "I", "I")
+    return src, name, _fmt("P", "P", "P", "I", "I", "I")
 
 
 EMB_SEGMENT = 512          # positions per segment of the ordered scatter-add
@@ -958,7 +965,8 @@ def embedding_backward_ordered_kernel(stage: str, vec: int = 1) -> tuple[str, st
                again each for its slice of the columns.
     Ids confined to one segment are therefore bit-identical to the sequential reference; ids
     that span segments differ from it only in where the parentheses fall, and every run
-    gives the same bits.  vec=4 moves rows as float4 (W % 4 == 0, aligned bases)."""
+    gives the same bits.  vec=4 moves rows as float4 (W % 4 == 0, aligned bases).
+    Positions whose id is outside [0, V) take no part in any stage."""
     assert stage in ("mark", "ordered", "merge")
     name = f"embedding_scatter_{stage}" + ("" if stage == "mark" else f"_v{vec}")
     VT = "float4" if vec == 4 else "float"
@@ -971,9 +979,10 @@ def embedding_backward_ordered_kernel(stage: str, vec: int = 1) -> tuple[str, st
     if stage == "mark":
         body = f"""
 extern "C" __global__ __launch_bounds__(256) void {name}(u32* __restrict__ owner,
-        const float* __restrict__ idx, u32 n, u32 NS) {{
+        const float* __restrict__ idx, u32 n, u32 NS, u32 V) {{
 {head}
     const int my = (int)idx[i];
+    if ((u32)my >= V) return;
     const u32 seg = i / EMB_SEG, s0 = seg * EMB_SEG, s1 = min(n, s0 + EMB_SEG);
     u64 hit[EMB_NK];
     segment_hits(idx, my, s0, s1, n, lane, hit);
@@ -982,16 +991,17 @@ extern "C" __global__ __launch_bounds__(256) void {name}(u32* __restrict__ owner
     if (below == 0u && lane == 0u) owner[(u64)my * NS + seg] = i + 1u;
 }}
 """
-        fmt = _fmt("P", "P", "I", "I")
+        fmt = _fmt("P", "P", "I", "I", "I")
     elif stage == "ordered":
         body = f"""
 extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out,
         float* __restrict__ partial, u32* __restrict__ flag, const u32* __restrict__ owner,
-        const float* __restrict__ g, const float* __restrict__ idx, u32 n, u32 W, u32 NS) {{
+        const float* __restrict__ g, const float* __restrict__ idx, u32 n, u32 W, u32 NS, u32 V) {{
     __shared__ u32 lists[4][{EMB_SEGMENT}];
     __shared__ {VT} stage[4][{EMB_SEGMENT}];
 {head}
     const int my = (int)idx[i];
+    if ((u32)my >= V) return;                                   // wave-uniform: the whole wavefront leaves
     const u32 seg = i / EMB_SEG, s0 = seg * EMB_SEG, s1 = min(n, s0 + EMB_SEG);
     u64 hit[EMB_NK];
     segment_hits(idx, my, s0, s1, n, lane, hit);
@@ -1046,16 +1056,17 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
     }}
 }}
 """
-        fmt = _fmt("P", "P", "P", "P", "P", "P", "I", "I", "I")
+        fmt = _fmt("P", "P", "P", "P", "P", "P", "I", "I", "I", "I")
     else:
         body = f"""
 extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out,
         const float* __restrict__ partial, const u32* __restrict__ flag, const u32* __restrict__ owner,
-        const float* __restrict__ idx, u32 n, u32 W, u32 NS) {{
+        const float* __restrict__ idx, u32 n, u32 W, u32 NS, u32 V) {{
     __shared__ u32 lists[4][64];
 {head}
-    if (flag[i] == 0u) return;                                  // only the owners of an id that spans segments work
     const int my = (int)idx[i];
+    if ((u32)my >= V) return;                                   // no flag was written for it
+    if (flag[i] == 0u) return;                                  // only the owners of an id that spans segments work
     const u32 p = lane < NS ? owner[(u64)my * NS + lane] : 0u;
     const u64 present = __ballot(p != 0u);
     u32* __restrict__ list = lists[w];                          // the id's owners, in segment order
@@ -1074,33 +1085,64 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
     }}
 }}
 """
-        fmt = _fmt("P", "P", "P", "P", "P", "I", "I", "I")
+        fmt = _fmt("P", "P", "P", "P", "P", "I", "I", "I", "I")
     return f"{PRELUDE}{_ORDERED_COMMON}{body}", name, fmt
 
 
 @cache
 def ce_kernel(backward: bool) -> tuple[str, str, str]:
     """ce_forward: out[i] = x[(int)target[i] + stride0*i]; ce_backward: that element -= 1,
-    in place (cpu_kernel.py:430-457)."""
+    in place (cpu_kernel.py:430-457).  A target outside [0, cols) picks 0 and subtracts nothing."""
     if backward:
         name = "ce_backward"
         src = f"""{PRELUDE}
 extern "C" __global__ __launch_bounds__(256) void {name}(float* x, const float* __restrict__ target,
-        u32 rows, u32 stride0) {{
+        u32 rows, u32 stride0, u32 cols) {{
     const u32 i = blockIdx.x * 256u + threadIdx.x;
-    if (i < rows) x[(long long)(int)target[i] + (u64)stride0 * i] -= 1.0f;
+    if (i >= rows) return;
+    const int t = (int)target[i];
+    if ((u32)t < cols) x[(long long)t + (u64)stride0 * i] -= 1.0f;
 }}
 """
-        return src, name, _fmt("P", "P", "I", "I")
+        return src, name, _fmt("P", "P", "I", "I", "I")
     name = "ce_forward"
     src = f"""{PRELUDE}
 extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
-        const float* __restrict__ target, float* __restrict__ out, u32 rows, u32 stride0) {{
+        const float* __restrict__ target, float* __restrict__ out, u32 rows, u32 stride0, u32 cols) {{
     const u32 i = blockIdx.x * 256u + threadIdx.x;
-    if (i < rows) out[i] = x[(long long)(int)target[i] + (u64)stride0 * i];
+    if (i >= rows) return;
+    const int t = (int)target[i];
+    out[i] = (u32)t < cols ? x[(long long)t + (u64)stride0 * i] : 0.0f;
 }}
 """
-    return src, name, _fmt("P", "P", "P", "I", "I")
+    return src, name, _fmt("P", "P", "P", "I", "I", "I")
+
+
+def _row_block_reduce(NW: int) -> str:
+    """block_max / block_sum over the NW wavefronts of a block that owns one row: the per-wave
+    results meet in LDS and are combined in wave order by every thread."""
+    return f"""
+static __device__ __forceinline__ float block_max(float v, float* sm) {{
+    v = wave_max(v);
+    if ((threadIdx.x & 63u) == 0) sm[threadIdx.x >> 6] = v;
+    __syncthreads();
+    v = sm[0];
+    #pragma unroll
+    for (int w = 1; w < {NW}; ++w) v = fmaxf(v, sm[w]);
+    __syncthreads();
+    return v;
+}}
+static __device__ __forceinline__ float block_sum(float v, float* sm) {{
+    v = wave_sum(v);
+    if ((threadIdx.x & 63u) == 0) sm[threadIdx.x >> 6] = v;
+    __syncthreads();
+    v = sm[0];
+    #pragma unroll
+    for (int w = 1; w < {NW}; ++w) v += sm[w];
+    __syncthreads();
+    return v;
+}}
+"""
 
 
 @cache
@@ -1244,32 +1286,16 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     if gather:
         assert log
         body += f"""
-    if ({tid} == 0) {{ const float* __restrict__ xr = x + (u64)row * L; picked[row] = (xr[(int)target[row]] - m) - ls; }}
+    if ({tid} == 0) {{
+        const float* __restrict__ xr = x + (u64)row * L;
+        const int t = (int)target[row];
+        picked[row] = (u32)t < L ? (xr[t] - m) - ls : 0.0f;           // a target outside the row picks 0
+    }}
 """
     extra_params = ", const float* __restrict__ target, float* __restrict__ picked" if gather else ""
     if masked:
         extra_params = ", const float* __restrict__ mask, u32 mrows, float scale"
-    src = f"""{PRELUDE}
-static __device__ __forceinline__ float block_max(float v, float* sm) {{
-    v = wave_max(v);
-    if ((threadIdx.x & 63u) == 0) sm[threadIdx.x >> 6] = v;
-    __syncthreads();
-    v = sm[0];
-    #pragma unroll
-    for (int w = 1; w < {NW}; ++w) v = fmaxf(v, sm[w]);
-    __syncthreads();
-    return v;
-}}
-static __device__ __forceinline__ float block_sum(float v, float* sm) {{
-    v = wave_sum(v);
-    if ((threadIdx.x & 63u) == 0) sm[threadIdx.x >> 6] = v;
-    __syncthreads();
-    v = sm[0];
-    #pragma unroll
-    for (int w = 1; w < {NW}; ++w) v += sm[w];
-    __syncthreads();
-    return v;
-}}
+    src = f"""{PRELUDE}{_row_block_reduce(NW)}
 extern "C" __global__ __launch_bounds__({threads}) void {name}(const float* __restrict__ x,
         float* __restrict__ out, u32 R, u32 L{extra_params}) {{
     __shared__ float sm[{NW}];
@@ -1279,6 +1305,81 @@ extern "C" __global__ __launch_bounds__({threads}) void {name}(const float* __re
 }}
 """
     return src, name, _fmt("P", "P", "I", "I", *(("P", "P") if gather else ("P", "I", "f") if masked else ()))
+
+
+
+@cache
+def ce_stats_kernel(vec: int, per_block: bool, nval: int, threads: int = 256, nt: bool = False) -> tuple[str, str, str]:
+    """The forward pass of the cross-entropy loss without its log-softmax tensor (ops.py:337-357
+    composes max, sub, exp, sum, log, sub over the whole (N, V) logits and gathers one entry per
+    row).  Per row r of an (R, L) view: m[r] = max, ls[r] = log(sum(exp(x - m))) and
+    picked[r] = (x[r, t] - m) - ls with t = (int)target[r], i.e. exactly the entry the gather of
+    cpu_kernel.py:430-441 would read from the log-softmax (0 for a target outside the row).  The
+    row is read once into registers (softmax_plan's layout) and nothing of its size is written:
+    4 B per element + 12 B per row.  The backward pass rebuilds exp((x - m) - ls) from the logits
+    and these two numbers, the same operations on the same values."""
+    assert nval > 0
+    nt = nt and vec == 4
+    name = f"ce_stats_v{vec}_{f'blk{threads}' if per_block else 'wav'}_r{nval}{'nt' if nt else ''}"
+    if not per_block:
+        threads = 256
+    T = f"{threads}u" if per_block else "64u"
+    NW = threads // 64
+    tid = "threadIdx.x" if per_block else "(threadIdx.x & 63u)"
+    row = "blockIdx.x" if per_block else "(blockIdx.x * 4u + (threadIdx.x >> 6))"
+    red_max = "block_max(m, sm)" if per_block else "wave_max(m)"
+    red_sum = "block_sum(s, sm)" if per_block else "wave_sum(s)"
+    if vec == 4:
+        body = f"""
+    const float4* __restrict__ p = reinterpret_cast<const float4*>(x + (u64)row * L);
+    const u32 nv = L >> 2;
+    float4 v[{nval}];
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < nv) v[k] = {'ld4_stream(p + c)' if nt else 'p[c]'}; }}
+    float m = NEG_FLT_MAX;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < nv)
+        m = fmaxf(fmaxf(m, fmaxf(v[k].x, v[k].y)), fmaxf(v[k].z, v[k].w));
+    m = {red_max};
+    float s = 0.0f;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < nv)
+        s += (expf(v[k].x - m) + expf(v[k].y - m)) + (expf(v[k].z - m) + expf(v[k].w - m));
+    s = {red_sum};
+"""
+    else:
+        body = f"""
+    const float* __restrict__ p = x + (u64)row * L;
+    float v[{nval}];
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < L) v[k] = p[c]; }}
+    float m = NEG_FLT_MAX;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < L) m = fmaxf(m, v[k]);
+    m = {red_max};
+    float s = 0.0f;
+    #pragma unroll
+    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < L) s += expf(v[k] - m);
+    s = {red_sum};
+"""
+    src = f"""{PRELUDE}{_row_block_reduce(NW)}
+extern "C" __global__ __launch_bounds__({threads}) void {name}(const float* __restrict__ x,
+        const float* __restrict__ target, float* __restrict__ row_max, float* __restrict__ row_logsum,
+        float* __restrict__ picked, u32 R, u32 L) {{
+    __shared__ float sm[{NW}];
+    const u32 row = {row};
+    {'' if per_block else 'if (row >= R) return;'}
+{body}
+    if ({tid} == 0) {{
+        const float ls = logf(s);
+        const int t = (int)target[row];
+        row_max[row] = m;
+        row_logsum[row] = ls;
+        picked[row] = (u32)t < L ? (x[(u64)row * L + (u32)t] - m) - ls : 0.0f;
+    }}
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "P", "P", "I", "I")
 
 
 def softmax_plan(L: int, vec: int) -> tuple[bool, int, int]:

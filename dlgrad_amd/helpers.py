@@ -76,6 +76,8 @@ class CustomOps(Enum):
     LOG_SOFTMAX = auto()
     LOG_SOFTMAX_GATHER = auto()     # log-softmax rows + the ce_forward gather, one kernel
     CE_GRAD = auto()                # ((exp(lsm) - onehot) * upstream) / N, one kernel
+    CE_STATS = auto()               # per row of the logits: max, log(sum(exp(x - max))) and the target's log-prob, one read-only kernel
+    CE_GRAD_LOGITS = auto()         # ((exp((x - max) - logsum) - onehot) * upstream) / N from the logits and the two row statistics
     ADAM_STEP = auto()              # the 14 element-wise kernels of one Adam update, one kernel
     ADAM_STEP_INPLACE = auto()      # the same, in place, constants from device memory (graph replay)
     MATMUL_NT = auto()              # x @ y^T with y read in place (no materialised transpose)

@@ -582,13 +582,22 @@ class RMSNorm(OP):
 class CrossEntropy(OP):
     def forward(self, logits: Buffer, target: Buffer, dim: int = 1) -> Buffer:
         """log-softmax, gather of the target log-probs, and -SUM over rows -- not the mean
-        (ops.py:338-357); backward nevertheless scales by 1/N (ops.py:359-370)."""
+        (ops.py:338-357); backward nevertheless scales by 1/N (ops.py:359-370).
+        On the hip device the (N, V) log-softmax is never stored: the forward keeps two numbers
+        per row (max and log-sum) and the backward rebuilds each entry from the logits, which the
+        tape holds anyway -- one read of the logits forward, one read and one write backward."""
         assert logits.shape[0] == target.shape[0]
         self.target = target
         self.N = float(logits.shape[0])
         self.fused = FUSED and logits.device is Device.HIP and logits.ndim == 2 and dim == 1
+        self.stats = None
         if self.fused:
-            self.log_softmax, picked = logits.log_softmax_gather(target)
+            from dlgrad_amd.runtime.hip import HIP
+            if HIP.ce_stats_fits(logits):
+                m, ls, picked = logits.ce_stats(target)
+                self.logits, self.stats = logits, (m, ls)
+            else:                                           # rows beyond the register-resident kernels
+                self.log_softmax, picked = logits.log_softmax_gather(target)
         else:
             shifted = logits - logits.max(dim=dim, keepdim=True)
             self.log_softmax = shifted - shifted.exp().sum(dim=dim, keepdim=True).log()
@@ -596,6 +605,8 @@ class CrossEntropy(OP):
         return -picked.sum()
 
     def backward(self, upstream_grad: Buffer) -> tuple:
+        if self.stats is not None:
+            return (self.logits.ce_grad_logits(*self.stats, self.target, upstream_grad, self.N),)
         if self.fused:
             return (self.log_softmax.ce_grad(self.target, upstream_grad, self.N),)
         probs = self.log_softmax.exp()

@@ -953,20 +953,20 @@ class HIP:
                 partial, flag, owner = alloc(n_idx * W), alloc(n_idx), alloc(V * NS, zero=True)
                 vec = 4 if (W % 4 == 0 and not (_addr(upstream_grad) | out.addr | partial.addr) & 15) else 1
                 grid = (n_idx + 3) // 4
-                launch(kernel(K.embedding_backward_ordered_kernel, "mark"), grid, 256, owner.addr, _addr(idx), n_idx, NS)
+                launch(kernel(K.embedding_backward_ordered_kernel, "mark"), grid, 256, owner.addr, _addr(idx), n_idx, NS, V)
                 launch(kernel(K.embedding_backward_ordered_kernel, "ordered", vec), grid, 256, out.addr, partial.addr,
-                       flag.addr, owner.addr, _addr(upstream_grad), _addr(idx), n_idx, W, NS)
+                       flag.addr, owner.addr, _addr(upstream_grad), _addr(idx), n_idx, W, NS, V)
                 launch(kernel(K.embedding_backward_ordered_kernel, "merge", vec), grid, 256, out.addr, partial.addr,
-                       flag.addr, owner.addr, _addr(idx), n_idx, W, NS)
+                       flag.addr, owner.addr, _addr(idx), n_idx, W, NS, V)
                 return out
             launch(kernel(K.embedding_backward_kernel), (n_idx + 3) // 4, 256,
-                   out.addr, _addr(upstream_grad), _addr(idx), n_idx, W)
+                   out.addr, _addr(upstream_grad), _addr(idx), n_idx, W, x.numel // W)
             return out
         out = alloc(out_numel)
         if n_idx:
             aligned = int(W % 4 == 0 and _addr(x) % 16 == 0 and out.addr % 16 == 0)
             launch(kernel(K.embedding_kernel), (n_idx + 3) // 4, 256,
-                   _addr(x), _addr(idx), out.addr, n_idx, W, aligned)
+                   _addr(x), _addr(idx), out.addr, n_idx, W, aligned, x.numel)
         return out
 
     @staticmethod
@@ -975,14 +975,14 @@ class HIP:
         rows = x.shape[0]
         out = alloc(rows)
         launch(kernel(K.ce_kernel, False), (rows + 255) // 256, 256, _addr(x), _addr(y), out.addr,
-               rows, x.stride[0])
+               rows, x.stride[0], x.shape[-1])
         return out
 
     @staticmethod
     @dispatcher.register(CustomOps.CE_BACKWARD, Device.HIP)
     def ce_backward(x: Buffer, target: Buffer) -> None:
         rows = x.shape[0]
-        launch(kernel(K.ce_kernel, True), (rows + 255) // 256, 256, _addr(x), _addr(target), rows, x.stride[0])
+        launch(kernel(K.ce_kernel, True), (rows + 255) // 256, 256, _addr(x), _addr(target), rows, x.stride[0], x.shape[-1])
 
     # ---- fused row softmax / cross-entropy ------------------------------------------------------------------------------
     @staticmethod
@@ -1121,11 +1121,57 @@ class HIP:
         CrossEntropy.backward (exp, in-place ce_backward, mul, div; ops.py:359-370) fused.
         Same operation order, so it differs from them only through expf."""
         rows = Buffer(target.ptr, (lsm.shape[0], 1), Device.HIP)
-        expr = "((expf(x0) - (((i % C) == (u32)(int)x1) ? 1.0f : 0.0f)) * {g}) / s0"
+        # the column of element i is i % C only while the launcher keeps the (rows, V) grid: a single
+        # row collapses to a flat run whose C is 1, and there the column is i itself
+        one = lsm.shape[0] == 1
+        col = "i" if one else "(i % C)"
+        expr = "((expf(x0) - ((" + col + " == (u32)(int)x1) ? 1.0f : 0.0f)) * {g}) / s0"
+        tag = "cegrad1" if one else "cegrad"
         if upstream.is_host_scalar:
-            return _map("cegrad_v", expr.format(g="s1"), [lsm, rows], lsm.shape,
+            return _map(tag + "_v", expr.format(g="s1"), [lsm, rows], lsm.shape,
                         (n, float(upstream.ptr.value)))
-        return _map("cegrad_p", expr.format(g="x2"), [lsm, rows, upstream], lsm.shape, (n,))
+        return _map(tag + "_p", expr.format(g="x2"), [lsm, rows, upstream], lsm.shape, (n,))
+
+    @staticmethod
+    def ce_stats_fits(x: Buffer) -> bool:
+        """Rows that the register-resident row kernels hold (up to 65536 floats)."""
+        if x.ndim != 2 or not x.numel or x.numel >= 2 ** 31:
+            return False
+        L = x.shape[1]
+        return K.softmax_plan(L, 4 if (L % 4 == 0 and _addr(x) % 16 == 0) else 1)[1] > 0
+
+    @staticmethod
+    @dispatcher.register(CustomOps.CE_STATS, Device.HIP)
+    def ce_stats(x: Buffer, target: Buffer) -> tuple[DevicePtr, DevicePtr, DevicePtr]:
+        """(max, log(sum(exp(x - max))), (x[target] - max) - logsum) per row of the 2-D logits x: all
+        the forward pass of the cross-entropy loss needs (ops.py:337-357), from one read of x and with
+        no (N, V) intermediate.  picked has the bits the gather from a log-softmax tensor would have."""
+        R, L = x.shape
+        m, ls, picked = alloc(R), alloc(R), alloc(R)
+        vec = 4 if (L % 4 == 0 and _addr(x) % 16 == 0) else 1
+        blk, nval, threads = K.softmax_plan(L, vec)
+        if not nval:
+            raise ValueError(f"ce_stats: rows of {L} floats do not fit the register-resident kernels")
+        k = kernel(K.ce_stats_kernel, vec, blk, nval, threads, x.numel >= NT_STORE_MIN_ELEMENTS)
+        launch(k, R if blk else (R + 3) // 4, threads, _addr(x), _addr(target), m.addr, ls.addr, picked.addr, R, L)
+        return m, ls, picked
+
+    @staticmethod
+    @dispatcher.register(CustomOps.CE_GRAD_LOGITS, Device.HIP)
+    def ce_grad_logits(x: Buffer, m: Buffer, ls: Buffer, target: Buffer, upstream: Buffer, n: float) -> DevicePtr:
+        """((exp((x - m) - ls) - onehot(target)) * upstream) / n in one pass over the logits: the
+        log-softmax entry is rebuilt from the row statistics ce_stats kept (the same two subtractions
+        on the same values the stored tensor was made with), then the four kernels of
+        CrossEntropy.backward (exp, in-place ce_backward, mul, div; ops.py:359-370) follow fused."""
+        R = x.shape[0]
+        rows = [Buffer(b.ptr, (R, 1), Device.HIP) for b in (m, ls, target)]
+        one = R == 1                                     # a single row collapses to a flat run: the column is i itself
+        col = "i" if one else "(i % C)"
+        expr = "((expf((x0 - x1) - x2) - ((" + col + " == (u32)(int)x3) ? 1.0f : 0.0f)) * {g}) / s0"
+        tag = "cegradx1" if one else "cegradx"
+        if upstream.is_host_scalar:
+            return _map(tag + "_v", expr.format(g="s1"), [x, *rows], x.shape, (n, float(upstream.ptr.value)))
+        return _map(tag + "_p", expr.format(g="x4"), [x, *rows, upstream], x.shape, (n,))
 
     # ---- fused RMSNorm ------------------------------------------------------------------------------------------------------
     @staticmethod

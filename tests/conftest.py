@@ -12,6 +12,37 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a HIP device (run on the MI355X box)")
 
 
+def compile_only_refusal() -> str:
+    """Why this test session must not run in compile-only mode, or "" if it may.
+
+    DLGRAD_HIP_COMPILE_ONLY=1 skips every launch and every comparison, so a GPU test "passes"
+    there without having executed a kernel.  The one legitimate use is the run that records
+    which kernels the tests ask for (dlgrad_amd.codegen.manifest --record), which sets
+    DLGRAD_HIP_MANIFEST as well and runs where there is no device.  Anything else -- the
+    variable inherited by accident, or set on a machine that has a GPU -- ends the session
+    with an error instead of a green result."""
+    if os.environ.get("DLGRAD_HIP_COMPILE_ONLY") != "1":
+        return ""
+    if not os.environ.get("DLGRAD_HIP_MANIFEST"):
+        return ("DLGRAD_HIP_COMPILE_ONLY=1 is set without DLGRAD_HIP_MANIFEST: in that mode no kernel runs and no "
+                "result is compared, so the GPU tests would pass without testing anything; unset it")
+    try:
+        from dlgrad_amd.runtime import hip
+        has_device = hip.available()
+    except Exception:
+        has_device = False
+    if has_device:
+        return ("DLGRAD_HIP_COMPILE_ONLY=1 on a machine with a HIP device: the tests would pass without executing "
+                "a kernel; unset it (a run with DLGRAD_HIP_MANIFEST alone records the kernels while really running)")
+    return ""
+
+
+def pytest_sessionstart(session):
+    why = compile_only_refusal()
+    if why:
+        pytest.exit(why, returncode=3)
+
+
 @pytest.fixture(scope="session")
 def rng_seed():
     return 1234

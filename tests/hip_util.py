@@ -8,8 +8,12 @@ from dlgrad_amd.runtime import hip
 
 
 def require_gpu():
+    """Skips where there is no device.  Compile-only mode (the kernel-recording run, admitted by
+    conftest only without a device and with DLGRAD_HIP_MANIFEST set) goes through the host side
+    of the test so that the kernels it asks for are listed; it executes and compares nothing."""
     if not (hip.available() or hip.COMPILE_ONLY):
         pytest.skip("no HIP device")
+    assert not (hip.COMPILE_ONLY and hip.available()), "compile-only mode with a device present tests nothing"
 
 
 def dev(a) -> Buffer:
@@ -27,7 +31,7 @@ def rel_err(got, want) -> float:
 
 
 def check(got, want, tol: float, what: str = "") -> None:
-    if hip.COMPILE_ONLY:
+    if hip.COMPILE_ONLY:                     # the recording run: nothing was computed
         return
     got = np.asarray(got)
     assert got.shape == np.asarray(want).shape, f"{what}: shape {got.shape} vs {np.asarray(want).shape}"

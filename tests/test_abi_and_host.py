@@ -309,3 +309,21 @@ def test_large_blocks_are_staggered_and_recycled_whole():
         b.upload_(data)
     for p in again:
         np.testing.assert_array_equal(Buffer(p, (n,), Device.HIP).numpy(), data)
+
+
+def _run_pytest_subprocess(env_extra: dict):
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = {k: v for k, v in os.environ.items() if k not in ("DLGRAD_HIP_COMPILE_ONLY", "DLGRAD_HIP_MANIFEST")}
+    env.update(env_extra)
+    return subprocess.run([sys.executable, "-m", "pytest", "tests/test_hip_elementwise.py", "-m", "gpu", "-q", "-x",
+                           "-p", "no:cacheprovider", "-k", "test_fills"], capture_output=True, text=True, env=env,
+                          cwd=root, timeout=600)
+
+
+def test_a_stray_compile_only_variable_fails_the_gpu_tests_instead_of_passing_them():
+    """Compile-only mode launches nothing and compares nothing; only the kernel-recording run
+    (which also names a manifest file, on a machine without a device) may use it for the tests."""
+    r = _run_pytest_subprocess({"DLGRAD_HIP_COMPILE_ONLY": "1"})
+    assert r.returncode == 3 and "DLGRAD_HIP_COMPILE_ONLY" in (r.stdout + r.stderr), (r.returncode, r.stdout[-500:])

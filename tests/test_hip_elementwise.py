@@ -201,3 +201,140 @@ def test_dropout_mask_comes_from_the_seeded_stream():
     check(y.numpy(), np.where(keep, x, np.float32(0)) * scale, 0, "dropout forward")
     check(t.grad.numpy(), np.where(keep, np.float32(1), np.float32(0)) * scale, 0, "dropout backward")
     assert 0.6 < keep.mean() < 0.8
+
+
+# ---- the streaming ("nt") forms -------------------------------------------------------------------
+# From NT_STORE_MIN_ELEMENTS (2^25) elements on, the launcher picks kernel variants that read
+# and write with nontemporal accesses and walk one 16-byte item per thread.  They are the
+# variants the C2 benchmark times at 16384 x 8192, so they are compared with the oracle twice:
+# every variant at a small size (threshold lowered), and the suite's shapes at full size.
+
+@pytest.fixture
+def streaming_everywhere(monkeypatch):
+    """Lowers the streaming threshold so that tensors of a few thousand elements take the nt
+    kernels; launch plans made under the other threshold are set aside for the test."""
+    monkeypatch.setattr(hip, "NT_STORE_MIN_ELEMENTS", 1024)
+    monkeypatch.setattr(hip, "_map_plans", {})
+    yield
+
+
+def test_streaming_map_variants_match_the_oracle(streaming_everywhere):
+    require_gpu()
+    R, C = 96, 520                                                 # 49920 elements: a ragged last block
+    x, same = f32(R, C), f32(R, C) + 3
+    col, row = f32(R, 1) + 3, f32(1, C) + 3
+    one = dev((f32(1, 1) + 3))
+    bx = dev(x)
+    n0 = len(hip.requested_kernels)
+    for op in OPS:
+        tol = 1e-6 if op == "div" else 0
+        for name, y in (("same", same), ("(R,1)", col), ("(1,C)", row)):
+            check(OPS[op](bx, dev(y)).numpy(), cref.binary(op, x, y), tol, f"nt {op} {name}")
+        check(OPS[op](bx, 1.5).numpy(), cref.binary(op, x, np.float32(1.5)), tol, f"nt {op} scalar")
+        check(OPS[op](bx, one).numpy(), cref.binary(op, x, one.numpy()), tol, f"nt {op} device scalar")
+    pos = np.abs(x) + np.float32(1e-3)
+    check(bx.exp().numpy(), cref.unary("exp", x), 1e-6, "nt exp")
+    check(dev(pos).log().numpy(), cref.unary("log", pos), 1e-6, "nt log")
+    check(dev(pos).sqrt().numpy(), cref.unary("sqrt", pos), 1e-6, "nt sqrt")
+    check(dev(pos).rsqrt().numpy(), cref.unary("rsqrt", pos), 1e-6, "nt rsqrt")
+    check((-bx).numpy(), cref.unary("neg", x), 0, "nt neg")
+    check((dev(pos) ** 3.0).numpy(), cref.unary("pow", pos, 3.0), 1e-6, "nt pow")
+    check(bx.clamp(-0.5, 0.25).numpy(), cref.clamp(x, -0.5, 0.25), 0, "nt clamp")
+    check(bx.relu().numpy(), cref.where(x, x, np.float32(0)), 0, "nt relu")
+    check(bx.where(dev(same), dev(x)).numpy(), cref.where(x, same, x), 0, "nt where, three tensors")
+    check((bx > 0.0).numpy(), cref.binary("gt", x, np.float32(0)), 0, "nt gt")
+    m = (RNG.random((1, C)) > 0.5).astype(np.float32)
+    check(Buffer.masked_fill(bx, dev(m), float("-inf")).numpy(), cref.masked_fill(x, m, -np.inf), 0, "nt masked_fill")
+    check(Buffer.full((R, C), 2.0, Device.HIP).numpy(), cref.full((R, C), 2.0), 0, "nt full")
+    names = {hip_kernel_name(g, p) for g, p in hip.requested_kernels}
+    if len(hip.requested_kernels) > n0 or not hip.COMPILE_ONLY:
+        assert any(n.endswith("u1nt") for n in names), "the streaming variants were not selected"
+
+
+def hip_kernel_name(gen_name: str, params: tuple) -> str:
+    from dlgrad_amd.codegen import hip_kernel as K
+    return getattr(K, gen_name)(*params)[1]
+
+
+def test_streaming_reduce_argmax_permute_softmax_variants_match_the_oracle(streaming_everywhere):
+    require_gpu()
+    x = f32(192, 2304)                                             # rows long enough for the block-per-row forms
+    bx = dev(x)
+    f64 = x.astype(np.float64)
+    def close_sum(got, want, what):          # sums of N(0,1) values cancel: measured against the largest |sum|
+        if not hip.COMPILE_ONLY:
+            assert got.shape == want.shape and np.abs(got - want).max() <= 1e-5 * np.abs(want).max() + 1e-4, what
+    for dim in (0, 1, None):
+        args = () if dim is None else (dim,)
+        check(bx.max(*args).numpy(), np.asarray(x.max(*args)), 0, f"nt max {dim}")
+        close_sum(bx.sum(*args).numpy(), np.asarray(f64.sum(*args)), f"nt sum {dim}")
+    ones = np.ones((192, 2304), np.float32)
+    check(dev(ones).sum(0).numpy(), ones.sum(0), 0, "nt sum axis 0 of ones")
+    check(dev(ones).sum(1).numpy(), ones.sum(1), 0, "nt sum axis 1 of ones")
+    check(dev(ones).sum().numpy(), np.asarray(ones.sum()), 0, "nt sum of ones")
+    planted = x.copy()
+    planted[:, 7] = planted[:, 900] = 9.0                          # ties: the first maximum wins
+    planted[5, :] = -np.inf
+    bp = dev(planted)
+    check(bp.argmax(1).numpy(), cref.argmax(planted, 1).reshape(-1, 1), 0, "nt argmax rows")
+    tall = f32(4096, 256)
+    tall[100] = tall[3000] = 9.0
+    check(dev(tall).argmax(0).numpy(), cref.argmax(tall, 0).reshape(1, -1), 0, "nt argmax columns")
+    check(bx.permute((1, 0)).numpy(), cref.permute(x, (1, 0)), 0, "nt transpose")
+    sq = f32(1024, 2048)                                           # a 2 KiB-multiple pitch: the diagonal 128 x 128 tiles
+    check(dev(sq).permute((1, 0)).numpy(), cref.permute(sq, (1, 0)), 0, "nt transpose, diagonal tiles")
+    h = f32(4, 64, 6, 32)
+    check(dev(h).permute((0, 2, 1, 3)).numpy(), cref.permute(h, (0, 2, 1, 3)), 0, "nt head permute")
+    rows = f32(64, 1024)
+    e = np.exp(rows.astype(np.float64) - rows.astype(np.float64).max(1, keepdims=True))
+    want = e / e.sum(1, keepdims=True)
+    got = dev(rows).softmax(1)
+    check(got.numpy(), want, 2e-6, "nt softmax")
+    g = f32(64, 1024)
+    y64 = want
+    dwant = y64 * (g - (g * y64).sum(1, keepdims=True))
+    dgot = got.softmax_bwd(dev(g)).numpy()
+    if not hip.COMPILE_ONLY:                                       # cancellation: measured against the largest entry
+        assert np.abs(dgot - dwant).max() <= 2e-6 * np.abs(dwant).max(), "nt softmax backward"
+    mask = np.triu(np.ones((64, 1024), np.float32), 1)
+    z = np.where(mask > 0, -np.inf, rows.astype(np.float64) * 0.125)
+    ez = np.exp(z - z.max(1, keepdims=True))
+    check(dev(rows).masked_softmax(dev(mask), 0.125).numpy(), ez / ez.sum(1, keepdims=True), 2e-6, "nt masked softmax")
+
+
+@pytest.mark.parametrize("case", ["add_same", "sub_rowvec", "mul_colvec", "div_scalar", "exp", "relu", "log", "sqrt"])
+def test_c2_suite_at_16384x8192_matches_the_oracle(case):
+    """The benchmark's own size: 134 M elements per tensor, the streaming kernels as the launcher
+    picks them with its default threshold."""
+    require_gpu()
+    R, C = 16384, 8192
+    rng = np.random.default_rng(2)
+    a = rng.standard_normal((R, C), dtype=np.float32)
+    da = dev(a)
+    if case == "add_same":
+        b = rng.standard_normal((R, C), dtype=np.float32)
+        got, want, tol = (da + dev(b)).numpy(), cref.binary("add", a, b), 0
+    elif case == "sub_rowvec":
+        v = rng.standard_normal((R, 1), dtype=np.float32)
+        got, want, tol = (da - dev(v)).numpy(), cref.binary("sub", a, v), 0
+    elif case == "mul_colvec":
+        v = rng.standard_normal((1, C), dtype=np.float32)
+        got, want, tol = (da * dev(v)).numpy(), cref.binary("mul", a, v), 0
+    elif case == "div_scalar":
+        got, want, tol = (da / 1.5).numpy(), cref.binary("div", a, np.float32(1.5)), 1e-6
+    elif case == "exp":
+        got, want, tol = da.exp().numpy(), cref.unary("exp", a), 1e-6
+    elif case == "relu":
+        got, want, tol = da.relu().numpy(), cref.where(a, a, np.float32(0)), 0
+    else:
+        pos = np.abs(a) + np.float32(1e-3)
+        got, want, tol = getattr(dev(pos), case)().numpy(), cref.unary(case, pos), 1e-6
+    if hip.COMPILE_ONLY:
+        return
+    assert got.shape == want.shape
+    if tol == 0:
+        assert np.array_equal(got, want), case
+    else:
+        with np.errstate(all="ignore"):
+            err = np.abs(got.astype(np.float64) - want) / np.maximum(np.abs(want), 1e-30)
+        assert float(np.nanmax(np.where(got == want, 0.0, err))) <= tol, case

@@ -95,8 +95,13 @@ def test_square_sweep_vs_float64_blas(n):
     require_gpu()
     x, y = f32(n, n), f32(n, n, scale=n ** -0.5)
     got = (dev(x) @ dev(y)).numpy()
-    want = x.astype(np.float64) @ y.astype(np.float64) if n <= 2048 else (x @ y)
-    check_mm(got, want, f"{n}^3")
+    if n <= 2048:
+        check_mm(got, x.astype(np.float64) @ y.astype(np.float64), f"{n}^3")
+    elif not hip.COMPILE_ONLY:                                  # float64 on every 37th row: each tile row, all columns
+        rows = np.arange(0, n, 37)
+        want = x[rows].astype(np.float64) @ y.astype(np.float64)
+        err = np.abs(got[rows] - want).max() / np.abs(want).max()
+        assert err <= 1e-4, f"{n}^3: {err:.3e}"
 
 
 def test_tall_skinny():
@@ -306,3 +311,48 @@ def test_one_row_times_a_transposed_matrix(N, K, lead, monkeypatch):
         top = np.abs(want).max()
         assert np.abs(got - ref).max() <= 2e-6 * top, f"{epi or 'plain'} vs float64"
         assert np.abs(got - tiled).max() <= 2e-6 * top, f"{epi or 'plain'} vs the tile path"
+
+
+def _rows_vs_float64(got: np.ndarray, rows: np.ndarray, a_rows: np.ndarray, b: np.ndarray, what: str) -> None:
+    """`got[rows]` against the float64 product of the matching rows of the left operand: a full
+    float64 product of these sizes is a teraflop on the host, a sample of rows (spread over
+    every tile row, all columns) is not."""
+    if hip.COMPILE_ONLY:
+        return
+    want = a_rows.astype(np.float64) @ b.astype(np.float64)
+    err = np.abs(got[rows] - want).max() / (np.abs(want).max() + 1e-30)
+    assert err <= 1e-4, f"{what}: {err:.3e}"
+    assert np.isfinite(got).all(), what
+
+
+def test_8192_cubed_against_float64_on_a_row_sample():
+    require_gpu()
+    n = 8192
+    rng = np.random.default_rng(31)
+    x = rng.standard_normal((n, n), dtype=np.float32)
+    y = rng.standard_normal((n, n), dtype=np.float32) * np.float32(n ** -0.5)
+    got = (dev(x) @ dev(y)).numpy()
+    rows = np.unique(np.concatenate([np.arange(0, n, 67), [n - 1]]))        # every 256-row tile is hit
+    _rows_vs_float64(got, rows, x[rows], y, "8192^3")
+    if not hip.COMPILE_ONLY:                                                # linearity: (x @ y) 1 = x (y 1), every row
+        lhs = got.astype(np.float64).sum(1)
+        rhs = x.astype(np.float64) @ y.astype(np.float64).sum(1)
+        assert np.abs(lhs - rhs).max() <= 1e-4 * np.abs(rhs).max() + 1e-3
+
+
+def test_4096_backward_shapes_in_place_against_float64_on_a_row_sample():
+    """A^T G (TN kernel) and G B^T (NT kernel) at the benchmark's 4096 size, and the same two
+    products as the reference issues them (materialised transpose, then NN)."""
+    require_gpu()
+    n = 4096
+    rng = np.random.default_rng(32)
+    a = rng.standard_normal((n, n), dtype=np.float32) * np.float32(n ** -0.5)
+    g = rng.standard_normal((n, n), dtype=np.float32) * np.float32(n ** -0.5)
+    da, dg = dev(a), dev(g)
+    rows = np.unique(np.concatenate([np.arange(0, n, 61), [n - 1]]))
+    tn = da.matmul_tn(dg).numpy()                                           # a^T g
+    _rows_vs_float64(tn, rows, np.ascontiguousarray(a.T[rows]), g, "4096 TN in place")
+    nt = dg.matmul_nt(da).numpy()                                           # g a^T
+    _rows_vs_float64(nt, rows, g[rows], np.ascontiguousarray(a.T), "4096 NT in place")
+    check(((da.T) @ dg).numpy(), tn, 0, "permute + NN gives the TN kernel's bits")
+    check((dg @ da.T).numpy(), nt, 0, "permute + NN gives the NT kernel's bits")

@@ -326,3 +326,99 @@ def test_row_store_writes_the_row_the_device_index_names(W):
         check(c.numpy(), wc, 0, f"single destination, row {row}")
     with pytest.raises(ValueError):
         dev(a0).row_store_(dev(ra), dev(np.zeros((1, 1), np.float32)), also=(dev(np.zeros((R, 3, W), np.float32)), dev(rb)))
+
+
+def _ce_float64(logits, t):
+    """(sum of the row losses, mean-scaled gradient) in float64 (ops.py:337-370: forward sums, backward divides by N)."""
+    z = logits.astype(np.float64)
+    z = z - z.max(1, keepdims=True)
+    lsm = z - np.log(np.exp(z).sum(1, keepdims=True))
+    n = logits.shape[0]
+    grad = np.exp(lsm)
+    grad[np.arange(n), t] -= 1.0
+    return -lsm[np.arange(n), t].sum(), grad / n
+
+
+@pytest.mark.parametrize("N,V", [(1, 65), (1, 64), (1, 50304), (2, 65), (4, 64), (300, 1000), (3, 50304)])
+@pytest.mark.parametrize("fused", [True, False])
+def test_cross_entropy_loss_and_gradient_single_rows_included(N, V, fused, monkeypatch):
+    """A single row collapses to a flat index space in the launcher, where the one-hot column must
+    still be found; targets 0, V-1 and in between."""
+    require_gpu()
+    from dlgrad_amd import Tensor, ops
+    monkeypatch.setattr(ops, "FUSED", fused)
+    logits = f32(N, V) * 2
+    for t0 in (0, V - 1, V // 3):
+        t = (np.arange(N) * 7 + t0) % V
+        a = Tensor(logits, requires_grad=True, device="hip")
+        loss = a.cross_entropy_loss(Tensor(t.astype(np.float32).reshape(N, 1), device="hip"))
+        loss.backward()
+        got_loss, got_grad = float(loss.numpy()), a.grad.numpy()
+        if hip.COMPILE_ONLY:
+            continue
+        want_loss, want_grad = _ce_float64(logits, t)
+        assert abs(got_loss - want_loss) <= 1e-5 * abs(want_loss), (N, V, t0)
+        assert np.abs(got_grad - want_grad).max() <= 1e-5 * np.abs(want_grad).max(), (N, V, t0)
+        assert (got_grad[np.arange(N), t] < 0).all() and (np.delete(got_grad[0], t[0]) > 0).all()
+
+
+@pytest.mark.parametrize("N,V", [(1, 64), (1, 65), (2048, 65), (64, 50304), (33, 4100)])
+def test_ce_row_statistics_give_the_bits_of_the_stored_log_softmax(N, V):
+    """The forward keeps (max, log-sum) per row instead of the (N, V) log-softmax; picked log-probs and
+    the gradient rebuilt from the logits must be the very numbers the stored tensor gave."""
+    require_gpu()
+    logits = f32(N, V) * 3
+    t = RNG.integers(0, V, (N, 1)).astype(np.float32)
+    x, dt = dev(logits), dev(t)
+    lsm, picked_old = x.log_softmax_gather(dt)
+    m, ls, picked = x.ce_stats(dt)
+    check(picked.numpy(), picked_old.numpy(), 0, "picked")
+    check(m.numpy().ravel(), cref.reduce("max", logits, 1), 0, "row max")
+    one = Buffer.from_scalar(1.0)
+    check(x.ce_grad_logits(m, ls, dt, one, float(N)).numpy(), lsm.ce_grad(dt, one, float(N)).numpy(), 0, "gradient, scalar upstream")
+    up = dev(np.float32(0.37).reshape(1, 1))
+    check(x.ce_grad_logits(m, ls, dt, up, float(N)).numpy(), lsm.ce_grad(dt, up, float(N)).numpy(), 0, "gradient, device upstream")
+
+
+def test_indices_outside_their_table_touch_nothing():
+    """Token ids and class targets are data: one that is negative or too large must not read or
+    write outside its tensor.  Gather gives a row of zeros, scatter-add skips the row, the
+    cross-entropy helpers pick 0 and subtract nothing; every in-range entry is unaffected."""
+    require_gpu()
+    V, W, n = 50, 64, 700                                          # two segments of the ordered scatter-add
+    table, g = f32(V, W), f32(n, W)
+    idx = RNG.integers(0, V, n).astype(np.float32)
+    bad = np.array([3, 100, 511, 512, 650])
+    idx[bad] = [-1.0, float(V), 1e9, -7.0, float(V + 3)]
+    ok = np.ones(n, bool)
+    ok[bad] = False
+    got = dev(table).embedding(dev(idx)).numpy()
+    if not hip.COMPILE_ONLY:
+        np.testing.assert_array_equal(got[ok], table[idx[ok].astype(int)])
+        assert not got[bad].any()
+    want = cref.embedding_backward((V, W), idx[ok], g[ok])
+    for ordered in (True, False):
+        old = hip.EMB_ORDERED
+        hip.EMB_ORDERED = ordered
+        try:
+            got = dev(table).embedding(dev(idx), backward=True, upstream_grad=dev(g)).numpy()
+        finally:
+            hip.EMB_ORDERED = old
+        if not hip.COMPILE_ONLY:
+            np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5, err_msg=f"ordered={ordered}")
+    lsm = f32(6, 10)
+    t = np.array([0, 9, -1, 10, 3, 1e6], np.float32).reshape(6, 1)
+    inside = np.array([True, True, False, False, True, False])
+    picked = Buffer.ce_forward(dev(lsm), dev(t)).numpy().ravel()
+    p = dev(lsm)
+    Buffer.ce_backward(op=CustomOps.CE_BACKWARD, device=p.device, x=p, target=dev(t))
+    after = p.numpy()
+    _, _, picked2 = dev(lsm).ce_stats(dev(t))
+    _, picked3 = dev(lsm).log_softmax_gather(dev(t))
+    if not hip.COMPILE_ONLY:
+        want_pick = np.where(inside, lsm[np.arange(6), np.where(inside, t.ravel(), 0).astype(int)], 0)
+        np.testing.assert_array_equal(picked, want_pick)
+        want_after = lsm.copy()
+        want_after[np.arange(6)[inside], t.ravel()[inside].astype(int)] -= 1
+        np.testing.assert_array_equal(after, want_after)
+        assert not picked2.numpy().ravel()[~inside].any() and not picked3.numpy().ravel()[~inside].any()
