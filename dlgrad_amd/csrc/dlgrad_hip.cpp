@@ -16,6 +16,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hiprtc.h>
 
+#include <cstddef>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -467,6 +468,71 @@ int dlg_hip_kernel_attrs(uint64_t handle, int32_t *num_regs, int32_t *lds_bytes,
     if (scratch_bytes) { HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, fn)); *scratch_bytes = v; }
     if (max_threads) { HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_MAX_THREADS_PER_BLOCK, fn)); *max_threads = v; }
     return 0;
+}
+
+// ---- full reduction as one call ---------------------------------------------------------------
+namespace {
+
+struct ReduceArgs {                               // argument block of hip_kernel.reduce_full_kernel
+    const void *x;
+    void *out;
+    uint32_t n;
+    float divisor;
+    uint32_t chunk;
+};
+constexpr size_t kReduceArgsSize = offsetof(ReduceArgs, chunk) + sizeof(uint32_t);
+constexpr uint32_t kReduceChunk = 2048;           // vector items one block of the first stage folds
+constexpr uint64_t kReduceMaxBlocks = 65536;      // partials one block of the second stage folds
+
+int launch_reduce_stage(hipFunction_t fn, uint32_t blocks, ReduceArgs a) {
+    size_t size = kReduceArgsSize;
+    void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &a, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+    HIP_TRY(hipModuleLaunchKernel(fn, blocks, 1, 1, 256, 1, 1, 0, g_stream, nullptr, config));
+    return 0;
+}
+
+// Both entry points: the first stage writes one partial per block into `part`, the second folds them.
+int reduce_full_into(uint64_t k_stage, uint64_t k_fold, const void *x, uint64_t n, uint32_t vec, float divisor,
+                     void *out, void *part, size_t part_bytes, const char *who) {
+    if (!x || !out) return fail_msg(-1, std::string(who) + ": NULL operand");
+    if (vec != 1 && vec != 4) return fail_msg(-41, std::string(who) + ": vec must be 1 or 4");
+    if (n == 0 || n >= (uint64_t(1) << 31)) return fail_msg(-42, std::string(who) + ": n must be in [1, 2^31)");
+    if (vec == 4 && ((uintptr_t)x & 15)) return fail_msg(-43, std::string(who) + ": vec = 4 needs a 16-byte aligned input");
+    hipFunction_t f_stage, f_fold;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        if (k_stage == 0 || k_stage > g_kernels.size() || k_fold == 0 || k_fold > g_kernels.size())
+            return fail_msg(-20, "bad kernel handle");
+        f_stage = g_kernels[k_stage - 1].fn;
+        f_fold = g_kernels[k_fold - 1].fn;
+    }
+    const uint64_t items = (n + vec - 1) / vec;
+    const uint64_t blocks = (items + kReduceChunk - 1) / kReduceChunk;
+    if (blocks == 1)                                              // one block folds everything: no partials
+        return launch_reduce_stage(f_stage, 1, ReduceArgs{x, out, (uint32_t)n, divisor, (uint32_t)items});
+    if (blocks > kReduceMaxBlocks) {
+        char buf[200];
+        std::snprintf(buf, sizeof buf, "%s: %llu elements need %llu partial results, at most %llu fit one call", who,
+                      (unsigned long long)n, (unsigned long long)blocks, (unsigned long long)kReduceMaxBlocks);
+        return fail_msg(-44, buf);
+    }
+    if (!part || ((uintptr_t)part & 15) || part_bytes < blocks * sizeof(float)) {
+        char buf[200];
+        std::snprintf(buf, sizeof buf, "%s: the partial results need %llu bytes, 16-byte aligned (got %zu)", who,
+                      (unsigned long long)(blocks * sizeof(float)), part_bytes);
+        return fail_msg(-45, buf);
+    }
+    int rc = launch_reduce_stage(f_stage, (uint32_t)blocks, ReduceArgs{x, part, (uint32_t)n, 1.0f, kReduceChunk});
+    if (rc) return rc;
+    return launch_reduce_stage(f_fold, 1, ReduceArgs{part, out, (uint32_t)blocks, divisor, (uint32_t)((blocks + 3) / 4)});
+}
+
+}  // namespace
+
+int dlg_hip_reduce_full(uint64_t k_stage, uint64_t k_fold, const void *x, uint64_t n, uint32_t vec,
+                        float divisor, void *out, void *workspace, size_t workspace_bytes) {
+    NEED_INIT();
+    return reduce_full_into(k_stage, k_fold, x, n, vec, divisor, out, workspace, workspace_bytes, "dlg_hip_reduce_full");
 }
 
 // ---- arenas and graphs ----------------------------------------------------------------

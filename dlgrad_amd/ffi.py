@@ -44,6 +44,8 @@ _SIGS = {
                                        _c.POINTER(_c.c_uint64)]),
     "dlg_hip_launch": (_c.c_int, [_c.c_uint64] + [_c.c_uint32] * 7 + [_c.c_char_p, _c.c_size_t]),
     "dlg_hip_kernel_attrs": (_c.c_int, [_c.c_uint64] + [_c.POINTER(_c.c_int32)] * 4),
+    "dlg_hip_reduce_full": (_c.c_int, [_c.c_uint64, _c.c_uint64, _c.c_void_p, _c.c_uint64, _c.c_uint32, _c.c_float,
+                                       _c.c_void_p, _c.c_void_p, _c.c_size_t]),
     "dlg_hip_arena_create": (_c.c_int, [_c.POINTER(_c.c_uint64)]),
     "dlg_hip_arena_set": (_c.c_int, [_c.c_uint64]),
     "dlg_hip_arena_destroy": (_c.c_int, [_c.c_uint64]),
@@ -259,6 +261,14 @@ class HipLib:
         self._check(self._lib.dlg_hip_kernel_attrs(handle, *[o[0] for o in outs]))
         return dict(zip(("num_regs", "lds_bytes", "scratch_bytes", "max_threads"),
                         (int(o[1]()) for o in outs)))
+
+    def reduce_full(self, k_stage: int, k_fold: int, x: int, n: int, vec: int, divisor: float, out: int,
+                    workspace: int, workspace_bytes: int) -> None:
+        """Sum or max of n floats at x into out[0] / divisor: both launches in one call."""
+        rc = self._lib.dlg_hip_reduce_full(k_stage, k_fold, self._vp(x), n, vec, divisor, self._vp(out),
+                                           self._vp(workspace), workspace_bytes)
+        if rc != 0:
+            self._check(rc)
 
     # -- arenas and graphs ----------------------------------------------------------------
     def arena_create(self) -> int:

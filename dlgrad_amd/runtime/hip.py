@@ -740,20 +740,24 @@ class HIP:
     # ---- reductions ------------------------------------------------------------------------------------
     @staticmethod
     def _reduce_full_into(kop: str, x_addr: int, n: int, divisor: float, out_addr: int) -> None:
-        """Two launches: blocks of 2048 vector items (32 KiB) -> partials -> one block."""
+        """Two launches: blocks of 2048 vector items (32 KiB) -> partials -> one block; both are
+        issued by one call into the library (dlg_hip_reduce_full), the partials in a pool block."""
+        global launch_count
         vec = 4 if x_addr % 16 == 0 else 1
         items = (n + vec - 1) // vec
         G = (items + 2047) // 2048
-        if G == 1:
-            launch(kernel(K.reduce_full_kernel, kop, vec), 1, 256, x_addr, out_addr, n, float(divisor), items)
-            return
-        part = alloc(G)
-        nt = vec == 4 and n >= NT_STORE_MIN_ELEMENTS                # streamed once: keep it out of the caches
-        launch(kernel(K.reduce_full_kernel, kop, vec, nt), G, 256, x_addr, part.addr, n, 1.0, 2048)
-        if G > 65536:                                    # > 537 M elements: fold the partials recursively
+        if G > 65536:                                    # > 537 M elements: fold the partials of the pieces recursively
+            part = alloc(G)
+            nt = vec == 4 and n >= NT_STORE_MIN_ELEMENTS
+            launch(kernel(K.reduce_full_kernel, kop, vec, nt), G, 256, x_addr, part.addr, n, 1.0, 2048)
             HIP._reduce_full_into(kop, part.addr, G, divisor, out_addr)
             return
-        launch(kernel(K.reduce_full_kernel, kop, 4), 1, 256, part.addr, out_addr, G, float(divisor), (G + 3) // 4)
+        nt = G > 1 and vec == 4 and n >= NT_STORE_MIN_ELEMENTS        # streamed once: keep it out of the caches
+        k_stage, k_fold = kernel(K.reduce_full_kernel, kop, vec, nt)[0], kernel(K.reduce_full_kernel, kop, 4)[0]
+        part = alloc(G) if G > 1 else None
+        launch_count += 2 if G > 1 else 1
+        (_state["lib"] or lib()).reduce_full(k_stage, k_fold, x_addr, n, vec, float(divisor), out_addr,
+                                             part.addr if part is not None else 0, 4 * G if part is not None else 0)
 
     @staticmethod
     def _reduce_cols(kop: str, x_addr: int, O: int, L: int, I: int, divisor: float, out_addr: int) -> None:

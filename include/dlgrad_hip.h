@@ -131,6 +131,20 @@ int dlg_hip_launch(uint64_t handle,
 int dlg_hip_kernel_attrs(uint64_t handle, int32_t *num_regs, int32_t *lds_bytes,
                          int32_t *scratch_bytes, int32_t *max_threads);
 
+/* ---- full reduction (sum or max of n floats into one) as one call ----------------------
+ * dlg_hip_reduce_full <- CPU.sum / CPU.max with dim = -1 (dlgrad/runtime/cpu.py:604-650) calling
+ *      the generated `reduce` loop (dlgrad/codegen/cpu_kernel.py:150-177).  On the GPU it is two
+ *      launches of the caller's stage kernel (hip_kernel.reduce_full_kernel, argument block
+ *      {x, out, u32 n, float divisor, u32 chunk}): blocks of 2048 vector items each write one
+ *      partial result, then one block folds the partials, divides by `divisor` (1, or n for a
+ *      mean) and writes out[0].  k_stage reads x with `vec` floats per access (1, or 4 for a
+ *      16-byte aligned x); k_fold is the same generator with vec = 4.  `workspace` receives the
+ *      partials: ceil(ceil(n / vec) / 2048) floats, 16-byte aligned, device memory; it may be NULL
+ *      when that count is 1.  More than 65536 partials (n > 2048 * vec * 65536) is an error: fold
+ *      in pieces.  Asynchronous on the library's stream; allocates nothing itself.           */
+int dlg_hip_reduce_full(uint64_t k_stage, uint64_t k_fold, const void *x, uint64_t n, uint32_t vec,
+                        float divisor, void *out, void *workspace, size_t workspace_bytes);
+
 /* ---- arenas and captured graphs ------------------------------------------------
  * No counterpart in the reference, whose CPU kernels have no launch cost to remove; on a
  * GPU a char-GPT training step is ~900 tiny launches and is bound by issuing them.

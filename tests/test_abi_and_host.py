@@ -327,3 +327,40 @@ def test_a_stray_compile_only_variable_fails_the_gpu_tests_instead_of_passing_th
     (which also names a manifest file, on a machine without a device) may use it for the tests."""
     r = _run_pytest_subprocess({"DLGRAD_HIP_COMPILE_ONLY": "1"})
     assert r.returncode == 3 and "DLGRAD_HIP_COMPILE_ONLY" in (r.stdout + r.stderr), (r.returncode, r.stdout[-500:])
+
+
+@pytest.mark.gpu
+def test_reduce_full_checks_its_arguments_on_the_host():
+    """dlg_hip_reduce_full launches twice on the caller's word; what the kernels and their grid assume
+    (access width, alignment, element count, room for the partial results) is checked before."""
+    from dlgrad_amd.runtime import hip
+    if not hip.available():
+        pytest.skip("no HIP device")
+    import numpy as np
+    from dlgrad_amd.codegen import hip_kernel as K
+    from dlgrad_amd.ffi import HipError
+    lib = hip.lib()
+    k1, k4 = hip.kernel(K.reduce_full_kernel, "sum", 1)[0], hip.kernel(K.reduce_full_kernel, "sum", 4)[0]
+    n = 100_000
+    x, out, ws = hip.alloc(n + 1), hip.alloc(1), hip.alloc(64)
+    ones = np.ones(n + 1, np.float32)                                           # kept alive across the copy
+    lib.h2d(x.addr, ones.ctypes.data, 4 * (n + 1))
+    G = ((n + 3) // 4 + 2047) // 2048
+    lib.reduce_full(k4, k4, x.addr, n, 4, 1.0, out.addr, ws.addr, 4 * G)
+    got = np.empty(1, np.float32)
+    lib.d2h(got.ctypes.data, out.addr, 4)
+    assert got[0] == n
+    lib.reduce_full(k1, k4, x.addr + 4, n, 1, 2.0, out.addr, ws.addr, 256)      # unaligned input, 4-byte reads, a mean-like divisor
+    lib.d2h(got.ctypes.data, out.addr, 4)
+    assert got[0] == n / 2
+    for args, msg in (((k4, k4, x.addr + 4, n, 4, 1.0, out.addr, ws.addr, 256), "aligned"),
+                      ((k4, k4, x.addr, n, 3, 1.0, out.addr, ws.addr, 256), "vec"),
+                      ((k4, k4, x.addr, 0, 4, 1.0, out.addr, ws.addr, 256), "n must"),
+                      ((k4, k4, x.addr, n, 4, 1.0, out.addr, ws.addr, 4 * G - 4), "partial results need"),
+                      ((k4, k4, x.addr, n, 4, 1.0, out.addr, 0, 0), "partial results need"),
+                      ((k4, k4, x.addr, n, 4, 1.0, out.addr, ws.addr + 4, 256), "partial results need"),
+                      ((k4, 10 ** 6, x.addr, n, 4, 1.0, out.addr, ws.addr, 256), "handle"),
+                      ((k4, k4, x.addr, 2048 * 4 * 65536 + 1, 4, 1.0, out.addr, ws.addr, 256), "at most")):
+        with pytest.raises(HipError, match=msg):
+            lib.reduce_full(*args)
+    lib.sync()
