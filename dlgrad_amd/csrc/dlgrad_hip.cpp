@@ -1,7 +1,8 @@
 // libdlgrad_hip.so -- device layer under dlgrad's `device="hip"` runtime.
 //
-// Host-only C++ (no device code lives here: kernels arrive as HIP source strings
-// from dlgrad_amd/codegen/hip_kernel.py and are compiled by hiprtc for gfx950).
+// Host C++ plus one device-side object, the static scratch array of the allocation-free
+// reduction (no kernels live here: they arrive as HIP source strings from
+// dlgrad_amd/codegen/hip_kernel.py and are compiled by hiprtc for gfx950).
 // Implements include/dlgrad_hip.h: a size-bucketed caching allocator over
 // hipMalloc, synchronous transfers, hiprtc compile, code-object load, kernel
 // launch from a packed argument block, events and error strings.
@@ -26,7 +27,16 @@
 #include <unordered_map>
 #include <vector>
 
+// Partial results of dlg_hip_reduce_full_static: one float per block of the first stage.  Device
+// memory that belongs to the library's code object; every GPU the library is loaded on holds its
+// own copy until the process ends.  Host code never uses this name as an address: the device
+// address is looked up once per device (dlg_hip_init) and kept in g_scratch_ptr.
+static __device__ __align__(256) unsigned char scratch[DLG_HIP_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices] = {};            // device address of `scratch`, per device
 
 thread_local std::string g_err;
 thread_local std::string g_log;
@@ -176,7 +186,14 @@ int dlg_hip_init(int device) {
         return fail_msg(-5, "no HIP device available");
     }
     if (device < 0 || device >= n) return fail_msg(-6, "device index out of range");
+    if (device >= kMaxDevices) return fail_msg(-6, "device index out of range");
     HIP_TRY(hipSetDevice(device));
+    {                                             // with this device current: where its copy of `scratch` lives
+        void *p = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail_msg(-40, "hipGetSymbolAddress returned no address for the static scratch array");
+        g_scratch_ptr[device] = p;
+    }
     HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
     g_device = device;
     g_inited = true;
@@ -533,6 +550,15 @@ int dlg_hip_reduce_full(uint64_t k_stage, uint64_t k_fold, const void *x, uint64
                         float divisor, void *out, void *workspace, size_t workspace_bytes) {
     NEED_INIT();
     return reduce_full_into(k_stage, k_fold, x, n, vec, divisor, out, workspace, workspace_bytes, "dlg_hip_reduce_full");
+}
+
+int dlg_hip_reduce_full_static(uint64_t k_stage, uint64_t k_fold, const void *x, uint64_t n, uint32_t vec,
+                               float divisor, void *out) {
+    NEED_INIT();
+    void *part = g_scratch_ptr[g_device];                         // never the array's name: that is a host-side stand-in
+    if (!part) return fail_msg(-40, "dlg_hip_reduce_full_static: the static scratch array was not located at init");
+    return reduce_full_into(k_stage, k_fold, x, n, vec, divisor, out, part, DLG_HIP_STATIC_SCRATCH_BYTES,
+                            "dlg_hip_reduce_full_static");
 }
 
 // ---- arenas and graphs ----------------------------------------------------------------

@@ -46,6 +46,8 @@ _SIGS = {
     "dlg_hip_kernel_attrs": (_c.c_int, [_c.c_uint64] + [_c.POINTER(_c.c_int32)] * 4),
     "dlg_hip_reduce_full": (_c.c_int, [_c.c_uint64, _c.c_uint64, _c.c_void_p, _c.c_uint64, _c.c_uint32, _c.c_float,
                                        _c.c_void_p, _c.c_void_p, _c.c_size_t]),
+    "dlg_hip_reduce_full_static": (_c.c_int, [_c.c_uint64, _c.c_uint64, _c.c_void_p, _c.c_uint64, _c.c_uint32, _c.c_float,
+                                              _c.c_void_p]),
     "dlg_hip_arena_create": (_c.c_int, [_c.POINTER(_c.c_uint64)]),
     "dlg_hip_arena_set": (_c.c_int, [_c.c_uint64]),
     "dlg_hip_arena_destroy": (_c.c_int, [_c.c_uint64]),
@@ -267,6 +269,12 @@ class HipLib:
         """Sum or max of n floats at x into out[0] / divisor: both launches in one call."""
         rc = self._lib.dlg_hip_reduce_full(k_stage, k_fold, self._vp(x), n, vec, divisor, self._vp(out),
                                            self._vp(workspace), workspace_bytes)
+        if rc != 0:
+            self._check(rc)
+
+    def reduce_full_static(self, k_stage: int, k_fold: int, x: int, n: int, vec: int, divisor: float, out: int) -> None:
+        """reduce_full with the partial results in the library's static device array: allocates nothing."""
+        rc = self._lib.dlg_hip_reduce_full_static(k_stage, k_fold, self._vp(x), n, vec, divisor, self._vp(out))
         if rc != 0:
             self._check(rc)
 

@@ -141,9 +141,23 @@ int dlg_hip_kernel_attrs(uint64_t handle, int32_t *num_regs, int32_t *lds_bytes,
  *      16-byte aligned x); k_fold is the same generator with vec = 4.  `workspace` receives the
  *      partials: ceil(ceil(n / vec) / 2048) floats, 16-byte aligned, device memory; it may be NULL
  *      when that count is 1.  More than 65536 partials (n > 2048 * vec * 65536) is an error: fold
- *      in pieces.  Asynchronous on the library's stream; allocates nothing itself.           */
+ *      in pieces.  Asynchronous on the library's stream; allocates nothing itself.
+ *
+ * dlg_hip_reduce_full_static has NO counterpart in the reference.  It is the same call for
+ *      callers that cannot allocate device memory or hand one in: code under stream capture,
+ *      tight serving loops, harnesses that forbid hipMalloc.  The partials go to a 256 KiB array
+ *      that is part of the library's device code (DLG_HIP_STATIC_SCRATCH_BYTES; every GPU the
+ *      library is initialised on holds it until the process ends), so the call allocates
+ *      nothing and records no memset; the same limit of 65536 partials applies and larger
+ *      inputs are refused with a message.  The array is shared by every call on that GPU and
+ *      keeps the last call's partials (each call overwrites the part it reads, so nothing needs
+ *      clearing).  Calls on the library's one stream are ordered; calls that overlap on one GPU
+ *      by any other route would race on the array.                                          */
+#define DLG_HIP_STATIC_SCRATCH_BYTES (65536 * 4)
 int dlg_hip_reduce_full(uint64_t k_stage, uint64_t k_fold, const void *x, uint64_t n, uint32_t vec,
                         float divisor, void *out, void *workspace, size_t workspace_bytes);
+int dlg_hip_reduce_full_static(uint64_t k_stage, uint64_t k_fold, const void *x, uint64_t n, uint32_t vec,
+                               float divisor, void *out);
 
 /* ---- arenas and captured graphs ------------------------------------------------
  * No counterpart in the reference, whose CPU kernels have no launch cost to remove; on a
