@@ -45,6 +45,7 @@ from dlgrad_amd.helpers import (
 
 _state = {"lib": None, "ready": False, "props": None}
 _handles: dict = {}            # (generator, params) -> (kernel handle, struct.Struct)
+kernel_names: dict = {}        # id of such a pair -> the kernel's name in its code object (what a profiler shows)
 launch_count = 0               # launches issued since import (read by the benchmarks)
 
 # Ahead-of-time mode for the build step: no device is touched, every kernel a workload
@@ -356,6 +357,7 @@ def kernel(gen, *params):
         requested_kernels.add((gen.__name__, params))
         l = lib()
         h = _handles[key] = (l.module_load(code_object(src, name, l), name), struct.Struct(fmt))
+        kernel_names[id(h)] = name
     return h
 
 
@@ -1331,6 +1333,7 @@ class HIP:
     _tuned_new: dict = {}
 
     MATMUL_TUNED_FILE = os.path.join(CACHE_DIR, "matmul_tuned.json")
+    last_matmul_kernel: str | None = None      # name of the most recently launched product kernel (reported by the benchmark)
 
     @staticmethod
     def _tuned_path() -> str:
@@ -1396,6 +1399,7 @@ class HIP:
         bm, bn, threads = K.matmul_tile_shape(tile)
         cfg = K.MATMUL_CONFIGS[tile]                           # (WM, WN, MI, NJ, BK) and, for the 16-wide MFMA tiles, 16
         k = kernel(K.matmul_kernel, *cfg[:5], veca, vecb, ta, tb, tri, strided, epi, *cfg[5:])
+        HIP.last_matmul_kernel = kernel_names.get(id(k))
         launch(k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch), threads, *args)
 
     @staticmethod
