@@ -17,6 +17,8 @@ buffer.py:86-90).  Buffers are always contiguous: `stride` is derived from
 """
 from __future__ import annotations
 
+from functools import lru_cache
+
 import numpy as np
 
 from dlgrad_amd.device import Device, as_device
@@ -36,6 +38,10 @@ from dlgrad_amd.helpers import (
 )
 
 
+_new_buffer = object.__new__
+_dispatch_table = dispatcher._dispatch_table      # (op, device) -> runtime function: the table dispatcher.dispatch reads
+
+
 class HostScalar:
     """One fp32 value that lives on the host and is passed to kernels by value."""
     __slots__ = ("value",)
@@ -50,18 +56,16 @@ class HostScalar:
         return f"HostScalar({float(self.value)!r})"
 
 
-class BufferMetadata:
-    """shape / numel / stride / ndim / dtype / device / nbytes of a Buffer (buffer.py:24-32)."""
-    __slots__ = ("shape", "numel", "stride", "ndim", "dtype", "device", "nbytes")
-
-    def __init__(self, shape: tuple, numel: int, stride: tuple, ndim: int, dtype: DType, device: Device,
-                 nbytes: int) -> None:
-        self.shape, self.numel, self.stride, self.ndim = shape, numel, stride, ndim
-        self.dtype, self.device, self.nbytes = dtype, device, nbytes
+@lru_cache(maxsize=16384)
+def _shape_info(shape: tuple) -> tuple:
+    """(numel, stride, ndim, nbytes) of a contiguous fp32 array of this shape."""
+    n = prod_(shape)
+    return n, calculate_stride(shape), len(shape), n * 4
 
 
 def _is_scalar(v) -> bool:
-    return isinstance(v, (int, float, np.floating)) and not isinstance(v, bool)
+    c = v.__class__
+    return c is float or c is int or (c is not bool and isinstance(v, (int, float, np.floating)) and not isinstance(v, bool))
 
 
 # 0-d host values never reach a device: scalar-with-scalar arithmetic is done here in
@@ -86,6 +90,12 @@ _HOST_UNARY = {
 
 
 class Buffer:
+    """shape / numel / stride / ndim / dtype / device / nbytes are attributes of the Buffer itself;
+    `metadata` (the reference keeps them in a separate BufferMetadata object, buffer.py:24-32, and
+    reads and writes them as `buf.metadata.shape`) is the Buffer again, so both spellings work and
+    creating a Buffer -- which happens for every op output -- allocates one object, not two."""
+    __slots__ = ("ptr", "shape", "numel", "stride", "ndim", "dtype", "device", "nbytes", "__weakref__")
+
     def __init__(self, data: CDataPtr, shape: tuple, device: str | Device | None = Device.CPU,
                  dtype: str | DType | None = None, **kwargs) -> None:
         self.ptr = data
@@ -94,34 +104,55 @@ class Buffer:
             dtype = DType.from_str(dtype) if dtype else DType.FLOAT32
         if device.__class__ is not Device:
             device = as_device(device)
-        n = prod_(shape)
+        n, stride, ndim, nbytes = _shape_info(shape)
         room = getattr(data, "nbytes", None)               # device pointers know how much of their block is left
-        if room is not None and n * 4 > room:
-            raise ValueError(f"a Buffer of shape {shape} needs {n * 4} bytes, the pointer has {room}")
+        if room is not None and nbytes > room:
+            raise ValueError(f"a Buffer of shape {shape} needs {nbytes} bytes, the pointer has {room}")
         if kwargs:
-            stride, ndim = kwargs.get("stride", calculate_stride(shape)), kwargs.get("ndim", len(shape))
-        else:
-            stride, ndim = calculate_stride(shape), len(shape)
-        self.metadata = BufferMetadata(shape, n, stride, ndim, dtype, device, n * 4)
+            stride, ndim = kwargs.get("stride", stride), kwargs.get("ndim", ndim)
+        self.shape, self.numel, self.stride, self.ndim = shape, n, stride, ndim
+        self.dtype, self.device, self.nbytes = dtype, device, nbytes
+
+    @property
+    def metadata(self) -> "Buffer":
+        return self
+
+    @staticmethod
+    def fresh(ptr: CDataPtr, shape: tuple, device: Device, dtype: DType = DType.FLOAT32) -> "Buffer":
+        """A Buffer around a pointer the runtime has just made for exactly this (tuple) shape: no
+        conversions and no size check."""
+        b = _new_buffer(Buffer)
+        b.ptr, b.shape, b.dtype, b.device = ptr, shape, dtype, device
+        b.numel, b.stride, b.ndim, b.nbytes = _shape_info(shape)
+        return b
 
     # ---- plumbing -------------------------------------------------------------------
     def _dispatch(self, op, **kw):
-        return dispatcher.dispatch(op=op, device=self.device, **kw)
+        return _dispatch_table[(op, self.device)](**kw)            # what dispatcher.dispatch does, one call less
 
     def _like(self, ptr, shape: tuple | None = None, **kw) -> "Buffer":
-        return Buffer(data=ptr, shape=self.shape if shape is None else shape,
-                      device=self.device, dtype=self.dtype, **kw)
+        if kw or (shape is not None and shape.__class__ is not tuple):
+            return Buffer(data=ptr, shape=self.shape if shape is None else shape,
+                          device=self.device, dtype=self.dtype, **kw)
+        b = _new_buffer(Buffer)
+        b.ptr, b.dtype, b.device = ptr, self.dtype, self.device
+        if shape is None:
+            b.shape, b.numel, b.stride, b.ndim, b.nbytes = self.shape, self.numel, self.stride, self.ndim, self.nbytes
+        else:
+            b.shape = shape
+            b.numel, b.stride, b.ndim, b.nbytes = _shape_info(shape)
+            room = getattr(ptr, "nbytes", None)
+            if room is not None and b.nbytes > room:
+                raise ValueError(f"a Buffer of shape {shape} needs {b.nbytes} bytes, the pointer has {room}")
+        return b
 
     @property
     def is_host_scalar(self) -> bool:
-        return isinstance(self.ptr, HostScalar)
+        return self.ptr.__class__ is HostScalar
 
     def _set_shape(self, shape: tuple) -> None:
-        md = self.metadata
-        md.shape = tuple(shape)
-        md.numel = prod_(shape)
-        md.stride = calculate_stride(shape)
-        md.ndim = len(shape)
+        self.shape = tuple(shape)
+        self.numel, self.stride, self.ndim, _ = _shape_info(self.shape)
 
     # ---- host boundary ----------------------------------------------------------------
     @staticmethod
@@ -152,7 +183,7 @@ class Buffer:
 
     @staticmethod
     def from_scalar(val: Scalar) -> "Buffer":
-        return Buffer(data=HostScalar(val), shape=(), device=Device.CPU, dtype=DType.FLOAT32)
+        return Buffer.fresh(HostScalar(val), (), Device.CPU)
 
     # ---- creation -----------------------------------------------------------------------
     @staticmethod
@@ -471,6 +502,11 @@ class Buffer:
         """In-place SGD update of self (and of the velocity v when momentum is used)."""
         self._dispatch(CustomOps.SGD_STEP_INPLACE, p=self, g=g, v=v, lr=lr, momentum=momentum)
 
+    def set_values_(self, values: tuple) -> None:
+        """Writes up to eight floats, given by value, into the first elements of this Buffer with a kernel
+        launch (hip): nothing is transferred and the host does not wait."""
+        self._dispatch(CustomOps.SET_VALUES, dst=self, values=tuple(values))
+
     def upload_(self, arr: np.ndarray) -> None:
         """Overwrites this Buffer's memory with `arr` (same element count); the address stays."""
         if arr.size != self.numel:
@@ -489,20 +525,22 @@ class Buffer:
         """x is the operand with more elements and fixes the output shape (buffer.py:402-448).
         A smaller left operand of SUB is handled as -(other - self), as there."""
         check_broadcast(self.shape, other.shape)
-        if self.is_host_scalar and other.is_host_scalar:
+        a_host, b_host = self.ptr.__class__ is HostScalar, other.ptr.__class__ is HostScalar
+        if a_host and b_host:
             with np.errstate(all="ignore"):
                 return self._like(HostScalar(_HOST_BINARY[op](self.ptr.value, other.ptr.value)))
-        big, small = (self, other) if self.numel >= other.numel else (other, self)
-        dev = small.device if big.is_host_scalar else big.device
-        ptr = dispatcher.dispatch(op=op, device=dev, x=big, y=small)
-        out = Buffer(data=ptr, shape=big.shape, device=dev, dtype=self.dtype)
-        if op == BinaryOps.SUB and big is not self:
+        if self.numel >= other.numel:
+            big, small, dev = self, other, (other.device if a_host else self.device)
+        else:
+            big, small, dev = other, self, (self.device if b_host else other.device)
+        out = Buffer.fresh(_dispatch_table[(op, dev)](x=big, y=small), big.shape, dev, self.dtype)
+        if op is BinaryOps.SUB and big is not self:
             out = -out
         return out
 
     @staticmethod
     def _coerce(v) -> "Buffer":
-        return Buffer.from_scalar(v) if _is_scalar(v) else v
+        return v if v.__class__ is Buffer else (Buffer.from_scalar(v) if _is_scalar(v) else v)
 
     def __add__(self, other) -> "Buffer":
         return self._binary_op(Buffer._coerce(other), BinaryOps.ADD)
@@ -554,31 +592,3 @@ class Buffer:
     @property
     def T(self) -> "Buffer":  # noqa: N802
         return self.transpose(0, 1)
-
-    @property
-    def numel(self) -> int:
-        return self.metadata.numel
-
-    @property
-    def shape(self) -> tuple:
-        return self.metadata.shape
-
-    @property
-    def stride(self) -> tuple:
-        return self.metadata.stride
-
-    @property
-    def ndim(self) -> int:
-        return self.metadata.ndim
-
-    @property
-    def dtype(self) -> DType:
-        return self.metadata.dtype
-
-    @property
-    def device(self) -> Device:
-        return self.metadata.device
-
-    @property
-    def nbytes(self) -> int:
-        return self.metadata.nbytes

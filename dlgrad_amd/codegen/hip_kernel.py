@@ -1309,67 +1309,75 @@ extern "C" __global__ __launch_bounds__({threads}) void {name}(const float* __re
 
 
 @cache
-def ce_stats_kernel(vec: int, per_block: bool, nval: int, threads: int = 256, nt: bool = False) -> tuple[str, str, str]:
+def ce_stats_kernel(vec: int, per_block: bool, nt: bool = False) -> tuple[str, str, str]:
     """The forward pass of the cross-entropy loss without its log-softmax tensor (ops.py:337-357
     composes max, sub, exp, sum, log, sub over the whole (N, V) logits and gathers one entry per
     row).  Per row r of an (R, L) view: m[r] = max, ls[r] = log(sum(exp(x - m))) and
-    picked[r] = (x[r, t] - m) - ls with t = (int)target[r], i.e. exactly the entry the gather of
-    cpu_kernel.py:430-441 would read from the log-softmax (0 for a target outside the row).  The
-    row is read once into registers (softmax_plan's layout) and nothing of its size is written:
-    4 B per element + 12 B per row.  The backward pass rebuilds exp((x - m) - ls) from the logits
-    and these two numbers, the same operations on the same values."""
-    assert nval > 0
+    picked[r] = (x[r, t] - m) - ls with t = (int)target[r], i.e. the entry the gather of
+    cpu_kernel.py:430-441 reads from the log-softmax (0 for a target outside the row).
+
+    One pass over the row, nothing of its size written: 4 B per element + 12 B per row.  Each
+    thread walks its items sixteen values at a time with a running maximum and a running sum
+    that is rescaled whenever the maximum rises (s <- s * exp(m_old - m_new)), so a row needs
+    no second read and no registers of its own: many wavefronts are resident and the exp of one
+    overlaps the loads of the others.  The threads' (m, s) pairs are joined the same way.  The
+    sum is therefore added in another order than max-then-sum would add it (a few ulp); the
+    maximum is exact.  The backward pass rebuilds exp((x - m) - ls) from the logits and these
+    two numbers.  One wavefront per row, or one 256-thread block per long row."""
     nt = nt and vec == 4
-    name = f"ce_stats_v{vec}_{f'blk{threads}' if per_block else 'wav'}_r{nval}{'nt' if nt else ''}"
-    if not per_block:
-        threads = 256
-    T = f"{threads}u" if per_block else "64u"
-    NW = threads // 64
+    name = f"ce_stats_v{vec}_{'blk' if per_block else 'wav'}{'nt' if nt else ''}"
+    T = "256u" if per_block else "64u"
     tid = "threadIdx.x" if per_block else "(threadIdx.x & 63u)"
     row = "blockIdx.x" if per_block else "(blockIdx.x * 4u + (threadIdx.x >> 6))"
     red_max = "block_max(m, sm)" if per_block else "wave_max(m)"
     red_sum = "block_sum(s, sm)" if per_block else "wave_sum(s)"
     if vec == 4:
+        ld = "ld4_stream(p + c)" if nt else "p[c]"
         body = f"""
     const float4* __restrict__ p = reinterpret_cast<const float4*>(x + (u64)row * L);
     const u32 nv = L >> 2;
-    float4 v[{nval}];
-    #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < nv) v[k] = {'ld4_stream(p + c)' if nt else 'p[c]'}; }}
-    float m = NEG_FLT_MAX;
-    #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < nv)
-        m = fmaxf(fmaxf(m, fmaxf(v[k].x, v[k].y)), fmaxf(v[k].z, v[k].w));
-    m = {red_max};
-    float s = 0.0f;
-    #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < nv)
-        s += (expf(v[k].x - m) + expf(v[k].y - m)) + (expf(v[k].z - m) + expf(v[k].w - m));
-    s = {red_sum};
+    float m = NEG_FLT_MAX, s = 0.0f;
+    u32 c = {tid};
+    for (; c + 3u * {T} < nv; c += 4u * {T}) {{                    // four loads in flight, sixteen values per round
+        float4 v[4];
+        #pragma unroll
+        for (u32 k = 0; k < 4u; ++k) {{ const u32 cc = c + k * {T}; v[k] = {ld.replace('p + c', 'p + cc').replace('p[c]', 'p[cc]')}; }}
+        float gm = fmaxf(fmaxf(v[0].x, v[0].y), fmaxf(v[0].z, v[0].w));
+        #pragma unroll
+        for (u32 k = 1; k < 4u; ++k) gm = fmaxf(gm, fmaxf(fmaxf(v[k].x, v[k].y), fmaxf(v[k].z, v[k].w)));
+        if (gm > m) {{ s *= expf(m - gm); m = gm; }}
+        #pragma unroll
+        for (u32 k = 0; k < 4u; ++k) s += (expf(v[k].x - m) + expf(v[k].y - m)) + (expf(v[k].z - m) + expf(v[k].w - m));
+    }}
+    for (; c < nv; c += {T}) {{
+        const float4 v = {ld};
+        const float gm = fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w));
+        if (gm > m) {{ s *= expf(m - gm); m = gm; }}
+        s += (expf(v.x - m) + expf(v.y - m)) + (expf(v.z - m) + expf(v.w - m));
+    }}
 """
     else:
         body = f"""
     const float* __restrict__ p = x + (u64)row * L;
-    float v[{nval}];
-    #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; if (c < L) v[k] = p[c]; }}
-    float m = NEG_FLT_MAX;
-    #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < L) m = fmaxf(m, v[k]);
-    m = {red_max};
-    float s = 0.0f;
-    #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < L) s += expf(v[k] - m);
-    s = {red_sum};
+    float m = NEG_FLT_MAX, s = 0.0f;
+    for (u32 c = {tid}; c < L; c += {T}) {{
+        const float v = p[c];
+        if (v > m) {{ s *= expf(m - v); m = v; }}
+        s += expf(v - m);
+    }}
 """
-    src = f"""{PRELUDE}{_row_block_reduce(NW)}
-extern "C" __global__ __launch_bounds__({threads}) void {name}(const float* __restrict__ x,
+    src = f"""{PRELUDE}{_row_block_reduce(4)}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
         const float* __restrict__ target, float* __restrict__ row_max, float* __restrict__ row_logsum,
         float* __restrict__ picked, u32 R, u32 L) {{
-    __shared__ float sm[{NW}];
+    __shared__ float sm[4];
     const u32 row = {row};
     {'' if per_block else 'if (row >= R) return;'}
 {body}
+    const float mine = m;
+    m = {red_max};
+    s *= expf(mine - m);                                          // this thread's sum on the row's scale
+    s = {red_sum};
     if ({tid} == 0) {{
         const float ls = logf(s);
         const int t = (int)target[row];

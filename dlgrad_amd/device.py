@@ -8,6 +8,8 @@ from enum import Enum, auto
 
 
 class Device(Enum):
+    __hash__ = object.__hash__          # members are singletons; this keys the dispatch table on every op
+
     CPU = auto()
     METAL = auto()
     HIP = auto()

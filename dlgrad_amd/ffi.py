@@ -122,6 +122,12 @@ class HipLib:
         self.raw_launch = self._lib.dlg_hip_launch
 
     # -- helpers -----------------------------------------------------------------------
+    def function_address(self, name: str) -> int:
+        """Where an exported function lives in this process (for a compiled binding that calls it directly)."""
+        if self._cffi is not None:
+            return int(self._cffi.cast("uintptr_t", self._cffi.addressof(self._lib, name)))
+        return ctypes.cast(getattr(self._lib, name), ctypes.c_void_p).value
+
     def last_error(self) -> str:
         e = self._lib.dlg_hip_last_error()
         if self._cffi is not None:

@@ -17,7 +17,13 @@ from functools import lru_cache
 from math import prod
 
 
-class UnaryOps(Enum):
+class _Op(Enum):
+    """Members are singletons compared by identity, so the identity hash serves; Enum's own
+    __hash__ is a Python-level function and these objects key a dict on every op."""
+    __hash__ = object.__hash__
+
+
+class UnaryOps(_Op):
     SUM = auto()
     MAX = auto()
     NEG = auto()
@@ -36,14 +42,14 @@ class UnaryOps(Enum):
     PERMUTE = auto()
 
 
-class BufferOps(Enum):
+class BufferOps(_Op):
     CREATE = auto()
     UNIFORM = auto()
     ARANGE = auto()
     FULL = auto()
 
 
-class BinaryOps(Enum):
+class BinaryOps(_Op):
     ADD = auto()
     SUB = auto()
     MUL = auto()
@@ -55,7 +61,7 @@ class BinaryOps(Enum):
     CMP = auto()
 
 
-class CustomOps(Enum):
+class CustomOps(_Op):
     INDEX = auto()
     CE_FORWARD = auto()
     CE_BACKWARD = auto()
@@ -87,6 +93,7 @@ class CustomOps(Enum):
     COPY_INTO = auto()              # device-to-device copy into an existing buffer (a KV-cache row)
     ADAM_MULTI_INPLACE = auto()     # one launch for a whole parameter list (addresses in a device table)
     SGD_STEP_INPLACE = auto()       # p -= (momentum-filtered) g * lr where p is (graph replay)
+    SET_VALUES = auto()             # a few floats given by value written into an existing buffer by a kernel (no transfer, no wait)
     RMSNORM = auto()                # (x * rsqrt(mean(x^2) + eps)) * w over the last axis, one kernel
     RMSNORM_BWD = auto()            # its backward: dx in one kernel, dw by partial rows + a column sum
 
@@ -109,6 +116,7 @@ def calculate_stride(shape: tuple | list) -> tuple:
     return _stride_of(tuple(shape))
 
 
+@lru_cache(maxsize=4096)
 def check_broadcast(x_shape: tuple, y_shape: tuple) -> bool:
     """True, or AssertionError when a trailing-aligned pair of dims is neither
     equal nor 1 (helpers.py:64-82)."""
@@ -119,6 +127,7 @@ def check_broadcast(x_shape: tuple, y_shape: tuple) -> bool:
     return True
 
 
+@lru_cache(maxsize=4096)
 def broadcast_shapes_2(s1: tuple, s2: tuple) -> tuple:
     """numpy-style broadcast of two shapes (helpers.py:311-334)."""
     n = max(len(s1), len(s2))
@@ -152,6 +161,7 @@ def get_broadcast_strides_2(out_shape: tuple, in_shape: tuple, in_stride: tuple)
     return tuple(res)
 
 
+@lru_cache(maxsize=4096)
 def broadcast_shapes(s1: tuple, s2: tuple) -> tuple[tuple, tuple, tuple]:
     """Matmul operand alignment: left-pad both to equal rank, broadcast the batch
     dims, check the inner dims; returns (padded1, padded2, out) (helpers.py:114-133)."""

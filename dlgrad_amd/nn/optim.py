@@ -62,15 +62,20 @@ class Adam(Optimizer):
     """m = b1 m + (1-b1) g;  v = b2 v + (1-b2) g^2;  p -= lr * m_hat / (sqrt(v_hat) + eps)."""
 
     def __init__(self, params: list[Tensor], lr: float = 1e-3, betas: tuple[float, float] = (0.9, 0.999),
-                 eps: float = 1e-8, graph_safe: bool = False) -> None:
-        """graph_safe (hip only): parameters and moments are updated in place and the
-        step-dependent constants live in device memory, so that a captured step can be
-        replayed: call advance() before each replay.  Same arithmetic, same bits."""
+                 eps: float = 1e-8, graph_safe: bool | None = None) -> None:
+        """graph_safe (hip only): parameters and moments are updated in place -- all of them by one
+        launch -- and the step-dependent constants live in device memory, so that a captured step can
+        be replayed: call advance() before each replay.  Same arithmetic, same bits as the
+        per-parameter expressions.  None (the default) chooses it whenever every parameter is on
+        the hip device and the fused kernels are on; False keeps one update per parameter that
+        rebinds `param.data`, as the reference does."""
         self.params, self.lr, self.eps = params, lr, eps
         self.beta1, self.beta2 = betas
         self.m = {id(p): Tensor.zeros_like(p) for p in params}
         self.v = {id(p): Tensor.zeros_like(p) for p in params}
         self.t = 0
+        if graph_safe is None:
+            graph_safe = bool(ops.FUSED and params and all(p.device is Device.HIP for p in params))
         self.graph_safe = graph_safe
         self.consts = Tensor(np.zeros(8, np.float32), device=params[0].device) if graph_safe else None
         self._table = None                 # device-side address table of the one-launch update
@@ -81,9 +86,10 @@ class Adam(Optimizer):
         return (self.beta1, 1.0 - self.beta1, self.beta2, 1.0 - self.beta2, c1, c2, self.eps, self.lr)
 
     def advance(self) -> None:
-        """graph_safe: moves to the next step and uploads its constants (not capturable)."""
+        """graph_safe: moves to the next step and writes its constants into device memory with a small
+        launch (not capturable: a captured graph reads them from there on every replay)."""
         self.t += 1
-        self.consts.data.upload_(np.asarray(self._consts(), dtype=np.float32))
+        self.consts.data.set_values_(self._consts())
 
     def step(self) -> None:
         if self.graph_safe:

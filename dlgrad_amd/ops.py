@@ -596,7 +596,7 @@ class CrossEntropy(OP):
             if HIP.ce_stats_fits(logits):
                 m, ls, picked = logits.ce_stats(target)
                 self.logits, self.stats = logits, (m, ls)
-            else:                                           # rows beyond the register-resident kernels
+            else:                                           # more than 2^31 elements
                 self.log_softmax, picked = logits.log_softmax_gather(target)
         else:
             shifted = logits - logits.max(dim=dim, keepdim=True)

@@ -117,14 +117,28 @@ if os.environ.get("DLGRAD_HIP_MANIFEST"):
     atexit.register(_dump_manifest)
 
 
+try:                                   # the compiled binding of alloc / free / launch (csrc/dlgfast.c)
+    from dlgrad_amd import _dlgfast as _fast
+except ImportError:                    # not built: the same three calls go through ffi.py's binding
+    _fast = None
+if os.environ.get("DLGRAD_HIP_FAST_BINDING", "1") == "0":
+    _fast = None
+_bound = False                         # _fast holds the library's function addresses
+
+
 def lib() -> _ffi.HipLib:
     """The loaded library with the device initialised; raises when there is no GPU."""
+    global _bound
     if not _state["ready"]:
         l = _ffi.get_lib()
         if COMPILE_ONLY:
             l = _CompileOnlyLib(l)
         else:
             l.init(int(os.environ.get("DLGRAD_HIP_DEVICE", "0")))
+            if _fast is not None:
+                _fast.bind(*[l.function_address(f) for f in ("dlg_hip_alloc", "dlg_hip_free", "dlg_hip_launch",
+                                                             "dlg_hip_last_error")])
+                _bound = True
         _state["lib"], _state["ready"] = l, True
     return _state["lib"]
 
@@ -142,10 +156,10 @@ def props() -> dict:
     return _state["props"]
 
 
-class DevicePtr:
+class _PyDevicePtr:
     """An address in HBM.  Owning pointers give their block back to the pool when
     collected; views (`ptr + n_elements`, as tensor.py:816-821 slices) keep their
-    base alive instead."""
+    base alive instead.  (The form used when the compiled binding is not built.)"""
     __slots__ = ("addr", "nbytes", "base", "__weakref__")
 
     def __init__(self, addr: int, nbytes: int, base: "DevicePtr | None" = None) -> None:
@@ -170,15 +184,24 @@ class DevicePtr:
         return f"DevicePtr(0x{self.addr:x}, {self.nbytes} B{', view' if self.base else ''})"
 
 
+# The compiled type does the same with its finaliser in C (it calls dlg_hip_free directly); in
+# compile-only mode its addresses are made up and nothing is bound, so it frees nothing.
+DevicePtr = _fast.DevPtr if _fast is not None else _PyDevicePtr
+
+
 def alloc(numel: int, zero: bool = False) -> DevicePtr:
     nbytes = 4 * numel if numel > 0 else 4
-    l = _state["lib"] or lib()
-    if zero and _graph_depth:
+    if not zero:
+        if _bound:
+            return _fast.alloc(nbytes)
+        l = _state["lib"] or lib()                              # the first call initialises (and binds)
+        return _fast.alloc(nbytes) if _bound else DevicePtr(l.alloc(nbytes, False), nbytes)
+    if _graph_depth:
         # a memset node must not enter a captured graph: clear with a kernel instead
-        p = DevicePtr(l.alloc(nbytes, False), nbytes)
+        p = alloc(numel)
         _map("full", "s0", [], (max(numel, 1),), (0.0,), out=p)
         return p
-    return DevicePtr(l.alloc(nbytes, zero), nbytes)
+    return DevicePtr((_state["lib"] or lib()).alloc(nbytes, True), nbytes)
 
 
 # ---- pinned host staging ------------------------------------------------------------------
@@ -375,10 +398,44 @@ def launch(k, grid, block, *args) -> None:
         bx, by, bz = block, 1, 1
     else:
         bx, by, bz = block if len(block) == 3 else (tuple(block) + (1, 1))[:3]
+    if _bound:
+        _fast.launch(handle, gx, gy, gz, bx, by, bz, packed)
+        return
     l = _state["lib"]
     rc = l.raw_launch(handle, gx, gy, gz, bx, by, bz, 0, packed, len(packed))
     if rc:
         l._check(rc)
+
+
+def launch_out(k, grid, block, out_offset: int, out_numel: int, *args) -> DevicePtr:
+    """A launch whose output is allocated by the same call: `args` holds 0 where the kernel expects
+    the output pointer, at byte `out_offset` of its argument block.  grid / block: an int (x extent)
+    or a 3-tuple.  Returns the freshly allocated block of out_numel floats."""
+    global launch_count
+    launch_count += 1
+    handle, st = k
+    gx, gy, gz = (grid, 1, 1) if grid.__class__ is int else grid
+    bx, by, bz = (block, 1, 1) if block.__class__ is int else block
+    if _bound:
+        return _fast.launch_out(handle, gx, gy, gz, bx, by, bz, st.pack(*args), out_offset, 4 * out_numel if out_numel > 0 else 4)
+    out = alloc(out_numel)
+    packed = bytearray(st.pack(*args))
+    struct.pack_into("@P", packed, out_offset, out.addr)
+    l = _state["lib"]
+    rc = l.raw_launch(handle, gx, gy, gz, bx, by, bz, 0, bytes(packed), len(packed))
+    if rc:
+        l._check(rc)
+    return out
+
+
+def field_offset(fmt: str, index: int) -> int:
+    """Byte offset of the index-th value of a native-alignment struct format such as "@PPfPI4I"
+    (what the kernel generators return; a count repeats its letter)."""
+    import re
+    assert fmt[0] == "@"
+    codes = "".join(c * int(n or 1) for n, c in re.findall(r"(\d*)([a-zA-Z])", fmt[1:]))
+    code = codes[index]
+    return struct.calcsize("@" + codes[:index] + code) - struct.calcsize("@" + code)
 
 
 def _addr(b: Buffer) -> int:
@@ -461,16 +518,14 @@ def _map(tag: str, expr: str, operands: list[Buffer], out_shape: tuple, svals: t
     plan = _map_plans.get(key)
     if plan is None:
         plan = _map_plans[key] = _MapPlan(tag, expr, operands, out_shape, len(svals))
-    if out is None:
-        out = alloc(plan.n)
     if plan.n == 0:
-        return out
+        return alloc(0) if out is None else out
     args = [float(b.ptr.value) if sc else b.ptr.addr for b, sc in zip(operands, plan.is_scalar)]
     var = plan.wide
     if var is not None:
-        if out.addr & 15:
+        if out is not None and out.addr & 15:
             var = plan.narrow
-        else:
+        else:                                  # a fresh output block is at least 256-byte aligned
             for a, needs in zip(args, var[4]):
                 if needs and a & 15:
                     var = plan.narrow
@@ -480,11 +535,16 @@ def _map(tag: str, expr: str, operands: list[Buffer], out_shape: tuple, svals: t
     k = var[3]
     if k is None:
         k = var[3] = kernel(*var[0])
-    launch(k, var[1], 256, *args, *[float(v) for v in svals], out.addr, *var[2])
+        var.append(field_offset(k[1].format, len(operands) + len(svals)))       # where the output pointer goes
+    if out is None:                            # output allocation and launch in one call into the library
+        return launch_out(k, var[1], 256, var[5], plan.n, *args, *svals, 0, *var[2])
+    launch(k, var[1], 256, *args, *svals, out.addr, *var[2])
     return out
 
 
 _U64 = (1 << 64) - 1
+_gemm_plans: dict = {}             # the same for products of matrices cut out of larger tensors
+_matmul_plans: dict = {}           # (shapes, flags, alignment bits) -> (kernel, grid, threads, fixed arguments, ...) of a product seen before
 ARGMAX_COL_BLOCKS = 512            # blocks of 64 x 16 threads the column argmax aims for; more only lengthen the fold
 _permute_plans: dict = {}
 PERMUTE_DIAG = os.environ.get("DLGRAD_HIP_PERMUTE_DIAG", "1") != "0"     # diagonal tile order for power-of-two pitches
@@ -623,39 +683,43 @@ class HIP:
         return _map(op, K.BINARY_EXPR[op], [x, y], broadcast_shapes_2(x.shape, y.shape))
 
     @staticmethod
-    @dispatcher.register(BinaryOps.ADD, Device.HIP)
-    def add(x: Buffer, y: Buffer) -> DevicePtr:
-        return HIP._binary_op(x, y, "add")
+    def _binary_entry(op: str):
+        """The dispatch-table entry of one binary op: after the first call for a pair of shapes the launch
+        plan is found with one dictionary lookup on (shape, shape) and nothing else is recomputed."""
+        expr, plans = K.BINARY_EXPR[op], {}
 
-    @staticmethod
-    @dispatcher.register(BinaryOps.SUB, Device.HIP)
-    def sub(x: Buffer, y: Buffer) -> DevicePtr:
-        return HIP._binary_op(x, y, "sub")
+        def run(x: Buffer, y: Buffer) -> DevicePtr:
+            xp, yp = x.ptr, y.ptr
+            y_host = yp.__class__ is HostScalar
+            if xp.__class__ is HostScalar:
+                return _map(op, expr, [x, y], broadcast_shapes_2(x.shape, y.shape))
+            plan = plans.get((x.shape, None if y_host else y.shape))
+            if plan is None:                                   # the general launcher builds and runs it once
+                out_shape = broadcast_shapes_2(x.shape, y.shape)
+                out = _map(op, expr, [x, y], out_shape)
+                plans[(x.shape, None if y_host else y.shape)] = _map_plans[(op, out_shape, (x.shape, None if y_host else y.shape), 0)]
+                return out
+            if plan.n == 0:
+                return alloc(0)
+            xa = xp.addr
+            ya = float(yp.value) if y_host else yp.addr
+            var = plan.wide
+            if var is None or (xa & 15 and var[4][0]) or (not y_host and ya & 15 and var[4][1]):
+                var = plan.narrow
+            k = var[3]
+            if k is None:
+                return _map(op, expr, [x, y], broadcast_shapes_2(x.shape, y.shape))
+            return launch_out(k, var[1], 256, 16, plan.n, xa, ya, 0, *var[2])
+        run.__name__ = op
+        return run
 
-    @staticmethod
-    @dispatcher.register(BinaryOps.MUL, Device.HIP)
-    def mul(x: Buffer, y: Buffer) -> DevicePtr:
-        return HIP._binary_op(x, y, "mul")
-
-    @staticmethod
-    @dispatcher.register(BinaryOps.DIV, Device.HIP)
-    def div(x: Buffer, y: Buffer) -> DevicePtr:
-        return HIP._binary_op(x, y, "div")
-
-    @staticmethod
-    @dispatcher.register(BinaryOps.GT, Device.HIP)
-    def gt(x: Buffer, y: Buffer) -> DevicePtr:
-        return HIP._binary_op(x, y, "gt")
-
-    @staticmethod
-    @dispatcher.register(BinaryOps.GTE, Device.HIP)
-    def gte(x: Buffer, y: Buffer) -> DevicePtr:
-        return HIP._binary_op(x, y, "gte")
-
-    @staticmethod
-    @dispatcher.register(BinaryOps.EQT, Device.HIP)
-    def eqt(x: Buffer, y: Buffer) -> DevicePtr:
-        return HIP._binary_op(x, y, "eq")
+    add = dispatcher.register(BinaryOps.ADD, Device.HIP)(_binary_entry.__func__("add"))
+    sub = dispatcher.register(BinaryOps.SUB, Device.HIP)(_binary_entry.__func__("sub"))
+    mul = dispatcher.register(BinaryOps.MUL, Device.HIP)(_binary_entry.__func__("mul"))
+    div = dispatcher.register(BinaryOps.DIV, Device.HIP)(_binary_entry.__func__("div"))
+    gt = dispatcher.register(BinaryOps.GT, Device.HIP)(_binary_entry.__func__("gt"))
+    gte = dispatcher.register(BinaryOps.GTE, Device.HIP)(_binary_entry.__func__("gte"))
+    eqt = dispatcher.register(BinaryOps.EQT, Device.HIP)(_binary_entry.__func__("eq"))
 
     @staticmethod
     @dispatcher.register(BinaryOps.CMP, Device.HIP)
@@ -670,34 +734,32 @@ class HIP:
         return _map(tag, expr, [x], x.shape, svals)
 
     @staticmethod
-    @dispatcher.register(UnaryOps.NEG, Device.HIP)
-    def neg(x: Buffer) -> DevicePtr:
-        return HIP._unary(x, "neg", K.UNARY_EXPR["neg"])
+    def _unary_entry(tag: str):
+        """The dispatch-table entry of one parameterless unary op: one dictionary lookup on the shape finds the
+        launch plan of a call seen before."""
+        expr, plans = K.UNARY_EXPR[tag], {}
 
-    @staticmethod
-    @dispatcher.register(UnaryOps.EXP, Device.HIP)
-    def exp(x: Buffer) -> DevicePtr:
-        return HIP._unary(x, "exp", K.UNARY_EXPR["exp"])
+        def run(x: Buffer) -> DevicePtr:
+            plan = plans.get(x.shape)
+            if plan is None:
+                out = _map(tag, expr, [x], x.shape)
+                plans[x.shape] = _map_plans[(tag, x.shape, (x.shape,), 0)]
+                return out
+            xa = x.ptr.addr
+            var = plan.narrow if (plan.wide is None or xa & 15) else plan.wide
+            k = var[3]
+            if k is None or plan.n == 0:
+                return _map(tag, expr, [x], x.shape)
+            return launch_out(k, var[1], 256, 8, plan.n, xa, 0, *var[2])
+        run.__name__ = tag
+        return run
 
-    @staticmethod
-    @dispatcher.register(UnaryOps.LOG, Device.HIP)
-    def log(x: Buffer) -> DevicePtr:
-        return HIP._unary(x, "log", K.UNARY_EXPR["log"])
-
-    @staticmethod
-    @dispatcher.register(UnaryOps.SQRT, Device.HIP)
-    def sqrt(x: Buffer) -> DevicePtr:
-        return HIP._unary(x, "sqrt", K.UNARY_EXPR["sqrt"])
-
-    @staticmethod
-    @dispatcher.register(UnaryOps.RSQRT, Device.HIP)
-    def rsqrt(x: Buffer) -> DevicePtr:
-        return HIP._unary(x, "rsqrt", K.UNARY_EXPR["rsqrt"])
-
-    @staticmethod
-    @dispatcher.register(UnaryOps.RELU, Device.HIP)
-    def relu(x: Buffer) -> DevicePtr:
-        return HIP._unary(x, "relu", K.UNARY_EXPR["relu"])
+    neg = dispatcher.register(UnaryOps.NEG, Device.HIP)(_unary_entry.__func__("neg"))
+    exp = dispatcher.register(UnaryOps.EXP, Device.HIP)(_unary_entry.__func__("exp"))
+    log = dispatcher.register(UnaryOps.LOG, Device.HIP)(_unary_entry.__func__("log"))
+    sqrt = dispatcher.register(UnaryOps.SQRT, Device.HIP)(_unary_entry.__func__("sqrt"))
+    rsqrt = dispatcher.register(UnaryOps.RSQRT, Device.HIP)(_unary_entry.__func__("rsqrt"))
+    relu = dispatcher.register(UnaryOps.RELU, Device.HIP)(_unary_entry.__func__("relu"))
 
     @staticmethod
     @dispatcher.register(UnaryOps.POW, Device.HIP)
@@ -1140,26 +1202,20 @@ class HIP:
 
     @staticmethod
     def ce_stats_fits(x: Buffer) -> bool:
-        """Rows that the register-resident row kernels hold (up to 65536 floats)."""
-        if x.ndim != 2 or not x.numel or x.numel >= 2 ** 31:
-            return False
-        L = x.shape[1]
-        return K.softmax_plan(L, 4 if (L % 4 == 0 and _addr(x) % 16 == 0) else 1)[1] > 0
+        return x.ndim == 2 and 0 < x.numel < 2 ** 31
 
     @staticmethod
     @dispatcher.register(CustomOps.CE_STATS, Device.HIP)
     def ce_stats(x: Buffer, target: Buffer) -> tuple[DevicePtr, DevicePtr, DevicePtr]:
         """(max, log(sum(exp(x - max))), (x[target] - max) - logsum) per row of the 2-D logits x: all
         the forward pass of the cross-entropy loss needs (ops.py:337-357), from one read of x and with
-        no (N, V) intermediate.  picked has the bits the gather from a log-softmax tensor would have."""
+        no (N, V) intermediate."""
         R, L = x.shape
         m, ls, picked = alloc(R), alloc(R), alloc(R)
         vec = 4 if (L % 4 == 0 and _addr(x) % 16 == 0) else 1
-        blk, nval, threads = K.softmax_plan(L, vec)
-        if not nval:
-            raise ValueError(f"ce_stats: rows of {L} floats do not fit the register-resident kernels")
-        k = kernel(K.ce_stats_kernel, vec, blk, nval, threads, x.numel >= NT_STORE_MIN_ELEMENTS)
-        launch(k, R if blk else (R + 3) // 4, threads, _addr(x), _addr(target), m.addr, ls.addr, picked.addr, R, L)
+        blk = L >= 2048
+        k = kernel(K.ce_stats_kernel, vec, blk, x.numel >= NT_STORE_MIN_ELEMENTS)
+        launch(k, R if blk else (R + 3) // 4, 256, _addr(x), _addr(target), m.addr, ls.addr, picked.addr, R, L)
         return m, ls, picked
 
     @staticmethod
@@ -1310,6 +1366,20 @@ class HIP:
         return table
 
     @staticmethod
+    @dispatcher.register(CustomOps.SET_VALUES, Device.HIP)
+    def set_values(dst: Buffer, values: tuple) -> None:
+        """dst[i] = values[i] for up to eight Python floats, written by a launch: unlike an upload the host
+        does not wait for the stream, and the values are ordered with the kernels around them.  Inside a
+        capture the values would be frozen into the graph, so it is refused there."""
+        n = len(values)
+        if not 0 < n <= 8 or dst.numel < n:
+            raise ValueError(f"set_values: {n} values into a buffer of {dst.numel}")
+        if capturing():
+            raise RuntimeError("set_values inside a captured graph would replay the same values on every launch")
+        expr = " : ".join(f"(i == {k}u) ? s{k}" for k in range(n - 1)) + (" : " if n > 1 else "") + f"s{n - 1}"
+        _map(f"set{n}", expr, [], (n,), tuple(float(v) for v in values), out=dst.ptr)
+
+    @staticmethod
     @dispatcher.register(CustomOps.SGD_STEP_INPLACE, Device.HIP)
     def sgd_step_inplace(p: Buffer, g: Buffer, v: Buffer | None, lr: float, momentum: float) -> None:
         n = p.numel
@@ -1396,11 +1466,18 @@ class HIP:
     @staticmethod
     def _launch_matmul(tile: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple,
                        ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False, epi: str = "") -> None:
+        k, grid, threads = HIP._matmul_kernel(tile, veca, vecb, M, N, batch, ta, tb, tri, strided, epi)
+        HIP.last_matmul_kernel = kernel_names.get(id(k))
+        launch(k, grid, threads, *args)
+
+    @staticmethod
+    def _matmul_kernel(tile: str, veca: bool, vecb: bool, M: int, N: int, batch: int, ta: bool = False, tb: bool = False,
+                       tri: str = "", strided: bool = False, epi: str = "") -> tuple:
+        """(loaded kernel, grid, threads per block) of one product."""
         bm, bn, threads = K.matmul_tile_shape(tile)
         cfg = K.MATMUL_CONFIGS[tile]                           # (WM, WN, MI, NJ, BK) and, for the 16-wide MFMA tiles, 16
         k = kernel(K.matmul_kernel, *cfg[:5], veca, vecb, ta, tb, tri, strided, epi, *cfg[5:])
-        HIP.last_matmul_kernel = kernel_names.get(id(k))
-        launch(k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch), threads, *args)
+        return k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch), threads
 
     @staticmethod
     def _tune_tile(key: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple,
@@ -1477,6 +1554,20 @@ class HIP:
         for (K.matmul_kernel); the work it lets the kernel skip never changes a kept result.
         epi: "add" (result + e), "relu" (result where positive, else 0) or "gate" (result where e is
         positive, else 0), applied as the result is stored; e has the shape of the result."""
+        xa, ya = x.ptr.addr, y.ptr.addr
+        ea = 0 if e is None or e.ptr.__class__ is HostScalar else e.ptr.addr
+        key = (x.shape, y.shape, ta, tb, tri, epi, None if e is None else e.shape, xa & 15, ya & 15, ea & 15,
+               HIP.MATMUL_FORCE, HIP.ROW_MATMUL)
+        plan = _matmul_plans.get(key)
+        if plan is not None:                                   # a shape seen before: pack the addresses and go
+            k, grid, threads, tail, out_numel, e_at, name = plan
+            if e_at == 0:                                      # (x, y, out, sizes and strides)
+                HIP.last_matmul_kernel = name
+                return launch_out(k, grid, threads, 16, out_numel, xa, ya, 0, *tail)
+            if e_at == 1:                                      # the same with the epilogue's operand at the end
+                HIP.last_matmul_kernel = name
+                return launch_out(k, grid, threads, 16, out_numel, xa, ya, 0, *tail, ea)
+            return launch_out(k, grid, threads, 16, out_numel, xa, ya, 0, ea, *tail)        # the single-row kernel: (x, W, out, e, N, K)
         assert x.ndim == y.ndim and 2 <= x.ndim <= 4 and not (ta and tb)
         (Kd, M) = x.shape[-2:] if ta else x.shape[-2:][::-1]
         (N, Ky) = y.shape[-2:] if tb else y.shape[-2:][::-1]
@@ -1484,7 +1575,8 @@ class HIP:
         xb = (1,) * (4 - x.ndim) + tuple(x.shape[:-2])
         yb = (1,) * (4 - y.ndim) + tuple(y.shape[:-2])
         B0, B1 = max(xb[0], yb[0]), max(xb[1], yb[1])
-        out = alloc(B0 * B1 * M * N)
+        out_numel = B0 * B1 * M * N
+        out = alloc(out_numel)
         if epi:
             if epi not in ("add", "relu", "gate") or tri:
                 raise ValueError(f"epilogue {epi!r} with tri={tri!r} is not provided")
@@ -1512,8 +1604,9 @@ class HIP:
         if (M == 1 and batch == 1 and tb and not ta and not tri and HIP.ROW_MATMUL and not HIP.MATMUL_FORCE and Kd % 4 == 0
                 and not ((_addr(x) | _addr(y)) & 15) and (e is None or not e.is_host_scalar)):
             # one row against a transposed matrix (a linear layer while decoding): a wavefront per output
-            launch(kernel(K.row_matmul_nt_kernel, epi), (N + 3) // 4, 256, _addr(x), _addr(y), out.addr,
-                   _addr(e) if e is not None else 0, N, Kd)
+            k = kernel(K.row_matmul_nt_kernel, epi)
+            launch(k, (N + 3) // 4, 256, _addr(x), _addr(y), out.addr, _addr(e) if e is not None else 0, N, Kd)
+            _matmul_plans[key] = (k, ((N + 3) // 4, 1, 1), (256, 1, 1), (N, Kd), N, 2, None)
             return out
         if batch > 65535:
             raise ValueError(f"{batch} batches exceed the grid limit")
@@ -1527,8 +1620,11 @@ class HIP:
         tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, args, ta, tb, tri)
         if epi:
             HIP._launch_matmul(tile, veca, vecb, M, N, batch, (*args, out.addr if e is None else _addr(e)), ta, tb, "", False, epi)
-            return out
-        HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri)
+        else:
+            HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri)
+        if not capturing():                                    # (while capturing, a shape met for the first time is not timed)
+            k, grid, threads = HIP._matmul_kernel(tile, veca, vecb, M, N, batch, ta, tb, "" if epi else tri, False, epi)
+            _matmul_plans[key] = (k, grid, threads, args[3:], out_numel, 1 if epi else 0, HIP.last_matmul_kernel)
         return out
 
     @staticmethod
@@ -1550,6 +1646,12 @@ class HIP:
         operand is (address, row pitch, stride of b0, stride of b1) in floats.  Same kernel, same
         order of additions as the contiguous product of the same logical matrices."""
         (aa, lda, sa0, sa1), (ba, ldb, sb0, sb1), (ca, ldc, sc0, sc1) = A, B, C
+        key = (A[1:], B[1:], C[1:], M, N, Kd, B0, B1, ta, tb, tri, aa & 15, ba & 15, ca & 15, HIP.MATMUL_FORCE)
+        plan = _gemm_plans.get(key)
+        if plan is not None:
+            k, grid, threads, tail = plan
+            launch(k, grid, threads, aa, ba, ca, *tail)
+            return
         if B0 * B1 > 65535 or max(lda * max(M, Kd), ldb * max(N, Kd), ldc * M) >= 2 ** 31:
             raise ValueError("strided product too large for the grid or for 32-bit indexing")
         al4 = lambda addr, *v: addr % 16 == 0 and all(x % 4 == 0 for x in v)     # noqa: E731
@@ -1559,6 +1661,8 @@ class HIP:
         batch = B0 * B1
         tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, args, ta, tb, tri, True)
         HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri, True)
+        if not capturing():
+            _gemm_plans[key] = (*HIP._matmul_kernel(tile, veca, vecb, M, N, batch, ta, tb, tri, True), args[3:])
 
     @staticmethod
     def _heads(addr: int, T: int, C: int, d: int) -> tuple:

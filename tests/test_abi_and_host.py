@@ -128,13 +128,15 @@ def test_collapse_dims_finds_the_row_and_column_broadcast_patterns():
 
 
 def test_device_pointer_views_keep_their_base_and_check_bounds():
-    base = hip.DevicePtr(0x1000, 64)
-    base.base = base          # pretend it is a view so __del__ frees nothing
+    owner = hip.DevicePtr(0, 0)                     # address 0: nothing to free
+    base = hip.DevicePtr(0x1000, 64, owner)         # a made-up address as a view, so nothing is freed for it either
     v = base + 4
-    assert v.addr == 0x1010 and v.nbytes == 48 and v.base is base
+    assert v.addr == 0x1010 and v.nbytes == 48 and v.base is owner and base.base is owner and owner.base is None
     with pytest.raises(IndexError):
         base + 17
-    base.base = base
+    with pytest.raises(IndexError):
+        base + -1
+    assert "view" in repr(v) and "0x1010" in repr(v)
 
 
 def test_pow_expression_is_repeated_multiplication():

@@ -362,22 +362,32 @@ def test_cross_entropy_loss_and_gradient_single_rows_included(N, V, fused, monke
         assert (got_grad[np.arange(N), t] < 0).all() and (np.delete(got_grad[0], t[0]) > 0).all()
 
 
-@pytest.mark.parametrize("N,V", [(1, 64), (1, 65), (2048, 65), (64, 50304), (33, 4100)])
-def test_ce_row_statistics_give_the_bits_of_the_stored_log_softmax(N, V):
-    """The forward keeps (max, log-sum) per row instead of the (N, V) log-softmax; picked log-probs and
-    the gradient rebuilt from the logits must be the very numbers the stored tensor gave."""
+@pytest.mark.parametrize("N,V", [(1, 64), (1, 65), (2048, 65), (64, 50304), (33, 4100), (7, 2048), (5, 100003)])
+def test_ce_row_statistics_stand_in_for_the_stored_log_softmax(N, V):
+    """The forward keeps (max, log-sum) per row instead of the (N, V) log-softmax.  The max is exact; the
+    sum is added in one pass with a running maximum, so log-sum, picked log-probs and the gradient rebuilt
+    from the logits agree with the stored-tensor route to rounding (1e-6 of the largest entry), and with
+    float64 to the tolerance of the element-wise ops."""
     require_gpu()
     logits = f32(N, V) * 3
+    logits[0, :min(V, 40)] = -np.inf                                # exp gives exact zeros; the row still has finite entries
     t = RNG.integers(0, V, (N, 1)).astype(np.float32)
+    t[0] = V - 1
     x, dt = dev(logits), dev(t)
     lsm, picked_old = x.log_softmax_gather(dt)
     m, ls, picked = x.ce_stats(dt)
-    check(picked.numpy(), picked_old.numpy(), 0, "picked")
     check(m.numpy().ravel(), cref.reduce("max", logits, 1), 0, "row max")
+    if hip.COMPILE_ONLY:
+        return
+    z = logits.astype(np.float64)
+    ls64 = np.log(np.exp(z - z.max(1, keepdims=True)).sum(1))
+    assert np.abs(ls.numpy().ravel() - ls64).max() <= 2e-6 * max(1.0, np.abs(ls64).max())
+    assert np.abs(picked.numpy() - picked_old.numpy()).max() <= 2e-6 * np.abs(picked_old.numpy()).max()
     one = Buffer.from_scalar(1.0)
-    check(x.ce_grad_logits(m, ls, dt, one, float(N)).numpy(), lsm.ce_grad(dt, one, float(N)).numpy(), 0, "gradient, scalar upstream")
-    up = dev(np.float32(0.37).reshape(1, 1))
-    check(x.ce_grad_logits(m, ls, dt, up, float(N)).numpy(), lsm.ce_grad(dt, up, float(N)).numpy(), 0, "gradient, device upstream")
+    for up in (one, dev(np.float32(0.37).reshape(1, 1))):
+        new, old = x.ce_grad_logits(m, ls, dt, up, float(N)).numpy(), lsm.ce_grad(dt, up, float(N)).numpy()
+        assert np.abs(new - old).max() <= 2e-6 * np.abs(old).max()
+        assert (new[0, :min(V, 40)] == 0).all()
 
 
 def test_indices_outside_their_table_touch_nothing():
