@@ -912,8 +912,8 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
     return src, name, _fmt("P", "P", "P", "I", "I", "I")
 
 
-EMB_SEGMENT = 512          # positions per segment of the ordered scatter-add
-EMB_ORDERED_MAX = 32768    # at most 64 segments: one lane per segment when an id's segments are listed
+EMB_SEGMENT = 512          # positions whose indices one round of the ordered scatter-add compares (eight ballots of 64)
+EMB_ORDERED_MAX = 32768    # longest index list the ordered scatter-add takes: every position scans the whole list
 
 _ORDERED_COMMON = f"""
 #define EMB_SEG {EMB_SEGMENT}u
@@ -947,81 +947,136 @@ static __device__ __forceinline__ void wave_lds_fence() {{
 
 
 @cache
-def embedding_backward_ordered_kernel(stage: str, vec: int = 1) -> tuple[str, str, str]:
-    """Deterministic scatter-add for up to EMB_ORDERED_MAX indices, without atomics.
+def embedding_backward_ordered_kernel(stage: str, vec: int = 1, nt: bool = False, ivec: int = 1) -> tuple[str, str, str]:
+    """Deterministic scatter-add into a (V, W) table for up to EMB_ORDERED_MAX indices, without
+    atomics on memory and without a zero-fill pass: three launches that together write every
+    element of the table exactly once (cpu_kernel.py:231-243 zero-fills the table, then adds row i
+    of the gradient to row idx[i]).
 
-    The index array is cut into segments of EMB_SEGMENT positions; one wavefront works per
-    position.  An id's positions inside one segment are found from the segment's 512 indices
-    (ballots); the lowest of them is the id's owner in that segment.
-      mark     the owner writes owner[id][segment] = position + 1 (zeroed by the launcher), so
-               the row owner[id][*] lists the segments an id occurs in.
-      ordered  the rows of an id's occurrences in a segment are added in index order starting
-               from 0 -- exactly the order of the reference's loop (cpu_kernel.py:231-243).
-               The id's m wavefronts in the segment split the columns between them (each sums
-               all m rows for its slice), so a hot id costs its wavefronts no more than a rare
-               one.  If the id occurs in no other segment the sum is the final table row,
-               otherwise it goes to partial[owner position] and flag[i] = 1 marks the owner.
-      merge    the owners of an id that spans segments add its partial rows in segment order,
-               again each for its slice of the columns.
-    Ids confined to one segment are therefore bit-identical to the sequential reference; ids
-    that span segments differ from it only in where the parentheses fall, and every run
-    gives the same bits.  vec=4 moves rows as float4 (W % 4 == 0, aligned bases).
-    Positions whose id is outside [0, V) take no part in any stage."""
-    assert stage in ("mark", "ordered", "merge")
-    name = f"embedding_scatter_{stage}" + ("" if stage == "mark" else f"_v{vec}")
+    The index list is cut into segments of EMB_SEGMENT positions.
+      "mark"      a block per 64 consecutive table rows reads the index list once and collects, in
+                  LDS, for each of its rows the set of segments the row's id occurs in; it writes
+                  that set (a 64-bit mask, 0 = the id does not occur) to idsegs[row].  Every entry
+                  of idsegs is written, so nothing needs clearing first.
+      "segments"  two kinds of blocks share the grid.
+         sum blocks: one wavefront per position i.  From the 512 indices of its segment (eight
+           ballots) it learns r, how many earlier positions of the segment hold the same id, and
+           m, how many hold it in all, and lists them in LDS.  The id's m wavefronts in the segment
+           split the row's columns into m slices; the r-th adds, for its slice, the gradient rows
+           of all m positions in index order starting from 0 -- the order of the reference's loop
+           -- so a hot id costs its wavefronts no more than a rare one.  The (row, column) items of
+           a slice are spread over all 64 lanes so that every load of a pass is in flight at once,
+           meet in LDS, and each column is added in row order.  If idsegs says the id occurs in no
+           other segment the sum is the final table row; otherwise it goes to partial[first
+           position of the id in the segment], and that first position records the set of segments
+           in segmask (0 for every other position) and the id's first position in each of them.
+         zero blocks: each owns 64 consecutive table rows and writes zeros to those whose idsegs
+           entry is 0.  They are spread evenly among the sum blocks, so that the stream of zeros
+           (bandwidth-bound) and the sums (latency-bound) run side by side.
+      "merge"     the first positions of an id that spans segments (segmask != 0) split the columns
+                  again and add the id's partial rows in segment order, starting from the first.
+    Every table row is written once: by a zero block, by the sum wavefronts of its only segment, or
+    by the merge; the three sets are disjoint, so nothing races inside a launch.  An id confined to
+    one segment has exactly the bits of the sequential reference loop; one that spans segments
+    differs from it only in where the parentheses fall, and every run gives the same bits.  Ids
+    outside [0, V) take no part.  vec = 4 moves rows as float4 (W % 4 == 0, 16-byte aligned bases);
+    nt writes the zeros with nontemporal stores (tables far larger than the caches); ivec = 4 lets
+    "mark" read the index list 16 bytes at a time (a 16-byte aligned list)."""
+    assert stage in ("mark", "segments", "merge")
+    name = (f"embedding_scatter_{stage}" + (f"_i{ivec}" if stage == "mark" else
+            f"_v{vec}{'nt' if (nt and stage == 'segments' and vec == 4) else ''}"))
     VT = "float4" if vec == 4 else "float"
     zero = "make_float4(0.f, 0.f, 0.f, 0.f)" if vec == 4 else "0.0f"
     add = ("acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;" if vec == 4 else "acc += t;")
     add_ = add.replace("t.", "t_.").replace("+= t;", "+= t_;")
-    head = """    const u32 w = threadIdx.x >> 6, lane = threadIdx.x & 63u;
-    const u32 i = blockIdx.x * 4u + w;                          // one wavefront per position
-    if (i >= n) return;"""
+    zstore = ("{ const v4f z = {0.f, 0.f, 0.f, 0.f}; __builtin_nontemporal_store(z, reinterpret_cast<v4f*>(zrow) + c); }"
+              if (nt and vec == 4) else f"zrow[c] = {zero};")
+    if ivec == 4:
+        # positions 4 * item .. 4 * item + 3 per thread; an item that sticks out past n is judged value by value
+        mscan = """    for (u32 t = threadIdx.x; 4u * t < n; t += 256u) {
+        if (4u * t + 3u < n) { const float4 q = reinterpret_cast<const float4*>(idx)[t]; MARK(q.x, 4u * t) MARK(q.y, 4u * t + 1u) MARK(q.z, 4u * t + 2u) MARK(q.w, 4u * t + 3u) }
+        else for (u32 p = 4u * t; p < n; ++p) MARK(idx[p], p)
+    }"""
+    else:
+        mscan = """    for (u32 t = threadIdx.x; t < n; t += 256u) MARK(idx[t], t)"""
     if stage == "mark":
         body = f"""
-extern "C" __global__ __launch_bounds__(256) void {name}(u32* __restrict__ owner,
-        const float* __restrict__ idx, u32 n, u32 NS, u32 V) {{
-{head}
-    const int my = (int)idx[i];
-    if ((u32)my >= V) return;
-    const u32 seg = i / EMB_SEG, s0 = seg * EMB_SEG, s1 = min(n, s0 + EMB_SEG);
-    u64 hit[EMB_NK];
-    segment_hits(idx, my, s0, s1, n, lane, hit);
-    u32 below, total;
-    hit_rank(hit, i - s0, below, total);
-    if (below == 0u && lane == 0u) owner[(u64)my * NS + seg] = i + 1u;
+extern "C" __global__ __launch_bounds__(256) void {name}(u64* __restrict__ idsegs,
+        const float* __restrict__ idx, u32 n, u32 V) {{
+    __shared__ u32 lo[64], hi[64];                              // per row of this block: the segments its id occurs in
+    const u32 v0 = blockIdx.x * 64u;
+    if (threadIdx.x < 64u) {{ lo[threadIdx.x] = 0u; hi[threadIdx.x] = 0u; }}
+    __syncthreads();
+#define MARK(val, pos) {{ const int id = (int)(val); if (id >= (int)v0 && id < (int)v0 + 64) {{ const u32 sg = (pos) / EMB_SEG; \\
+        atomicOr(sg < 32u ? &lo[id - (int)v0] : &hi[id - (int)v0], 1u << (sg & 31u)); }} }}
+{mscan}
+    __syncthreads();
+    if (threadIdx.x < 64u && v0 + threadIdx.x < V) idsegs[v0 + threadIdx.x] = (u64)lo[threadIdx.x] | ((u64)hi[threadIdx.x] << 32);
 }}
 """
-        fmt = _fmt("P", "P", "I", "I", "I")
-    elif stage == "ordered":
+        return f"{PRELUDE}{_ORDERED_COMMON}{body}", name, _fmt("P", "P", "I", "I")
+    if stage == "segments":
         body = f"""
 extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out,
-        float* __restrict__ partial, u32* __restrict__ flag, const u32* __restrict__ owner,
-        const float* __restrict__ g, const float* __restrict__ idx, u32 n, u32 W, u32 NS, u32 V) {{
+        float* __restrict__ partial, u64* __restrict__ segmask, u32* __restrict__ firsts, const u64* __restrict__ idsegs,
+        const float* __restrict__ g, const float* __restrict__ idx, u32 n, u32 W, u32 V, u32 n_zero_blocks, u32 every) {{
     __shared__ u32 lists[4][{EMB_SEGMENT}];
     __shared__ {VT} stage[4][{EMB_SEGMENT}];
-{head}
+    const u32 w = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    const u32 Wv = W / {vec}u;
+    // every `every`-th block is a zero block until all n_zero_blocks of them are placed
+    const u32 grp = blockIdx.x / every;
+    if (blockIdx.x % every == every - 1u && grp < n_zero_blocks) {{
+        // ---- a zero block: 64 table rows, zeros for those no index names
+        const u32 v0 = grp * 64u;
+        const u32 rows = min(64u, V - v0);
+        for (u32 r = w; r < rows; r += 4u) {{                     // a wavefront per row, rows four apart
+            if (idsegs[v0 + r] != 0ull) continue;               // some index names this row: its sum is written instead
+            {VT}* __restrict__ zrow = reinterpret_cast<{VT}*>(out + (u64)(v0 + r) * W);
+            for (u32 c = lane; c < Wv; c += 64u) {zstore}
+        }}
+        return;
+    }}
+    // ---- a sum block: one wavefront per position
+    const u32 i = (blockIdx.x - min(n_zero_blocks, grp)) * 4u + w;
+    if (i >= n) return;
     const int my = (int)idx[i];
-    if ((u32)my >= V) return;                                   // wave-uniform: the whole wavefront leaves
     const u32 seg = i / EMB_SEG, s0 = seg * EMB_SEG, s1 = min(n, s0 + EMB_SEG);
     u64 hit[EMB_NK];
-    segment_hits(idx, my, s0, s1, n, lane, hit);
+    segment_hits(idx, my, s0, s1, n, lane, hit);                // (its loads do not wait for `my`)
+    if ((u32)my >= V) {{ if (lane == 0u) segmask[i] = 0ull; return; }}     // wave-uniform: the whole wavefront leaves
     u32 r, m;                                                   // this position is the r-th of the id's m in the segment
     hit_rank(hit, i - s0, r, m);
     u32* __restrict__ list = lists[w];                          // the id's positions in the segment, ascending
-    u32 at = 0;
-    #pragma unroll
-    for (u32 k = 0; k < EMB_NK; ++k) {{
-        if ((hit[k] >> lane) & 1ull) list[at + (u32)__popcll(hit[k] & ((1ull << lane) - 1ull))] = s0 + 64u * k + lane;
-        at += (u32)__popcll(hit[k]);
+    if (m == 1u) {{
+        if (lane == 0u) list[0] = i;
+    }} else {{
+        u32 at = 0;
+        #pragma unroll
+        for (u32 k = 0; k < EMB_NK; ++k) {{
+            if ((hit[k] >> lane) & 1ull) list[at + (u32)__popcll(hit[k] & ((1ull << lane) - 1ull))] = s0 + 64u * k + lane;
+            at += (u32)__popcll(hit[k]);
+        }}
     }}
+    const u64 segs = idsegs[my];                                // the segments the id occurs in (this one among them)
     wave_lds_fence();
-    const u32 mine = lane < NS ? owner[(u64)my * NS + lane] : 0u;
-    const u64 present = __ballot(mine != 0u);                   // the segments the id occurs in (this one among them)
-    const bool other = (present & ~(1ull << seg)) != 0ull;
-    if (lane == 0u) flag[i] = (r == 0u && other) ? 1u : 0u;
-    {VT}* __restrict__ dst = reinterpret_cast<{VT}*>(other ? partial + (u64)list[0] * W : out + (long long)my * W);
-    const u32 Wv = W / {vec}u;
-    const u32 c0 = (u32)((u64)r * Wv / m), c1 = (u32)((u64)(r + 1u) * Wv / m);      // this wavefront's slice of the columns
+    const bool other = segs != (1ull << seg);
+    if (lane == 0u) segmask[i] = (r == 0u && other) ? segs : 0ull;
+    if (r == 0u && other) {{                                     // the merge adds the partial rows of these first positions
+        const u32 NS = (n + EMB_SEG - 1u) / EMB_SEG;
+        u32 k = 0;
+        for (u64 rest = segs; rest; rest &= rest - 1ull, ++k) {{
+            const u32 t0 = (u32)__builtin_ctzll(rest) * EMB_SEG;
+            u64 h2[EMB_NK];
+            segment_hits(idx, my, t0, min(n, t0 + EMB_SEG), n, lane, h2);
+            u32 first = 0xFFFFFFFFu;
+            #pragma unroll
+            for (u32 j = EMB_NK; j-- > 0u;) if (h2[j]) first = t0 + 64u * j + (u32)__builtin_ctzll(h2[j]);
+            if (lane == 0u) firsts[(u64)i * NS + k] = first;
+        }}
+    }}
+    {VT}* __restrict__ dst = reinterpret_cast<{VT}*>(other ? partial + (u64)list[0] * W : out + (u64)my * W);
+    const u32 c0 = r * Wv / m, c1 = (r + 1u) * Wv / m;        /* r < 512 and Wv < 2^22: no overflow */      // this wavefront's slice of the columns
     // The (row, column) items of the slice are spread over all 64 lanes, so every load of a pass
     // is in flight at once whatever m is; they meet in LDS, where each column is added in row order.
     {VT}* __restrict__ st = stage[w];
@@ -1056,27 +1111,25 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
     }}
 }}
 """
-        fmt = _fmt("P", "P", "P", "P", "P", "P", "I", "I", "I", "I")
+        fmt = _fmt("P", "P", "P", "P", "P", "P", "P", "I", "I", "I", "I", "I")
     else:
         body = f"""
 extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out,
-        const float* __restrict__ partial, const u32* __restrict__ flag, const u32* __restrict__ owner,
-        const float* __restrict__ idx, u32 n, u32 W, u32 NS, u32 V) {{
-    __shared__ u32 lists[4][64];
-{head}
+        const float* __restrict__ partial, const u64* __restrict__ segmask, const u32* __restrict__ firsts,
+        const float* __restrict__ idx, u32 n, u32 W, u32 V) {{
+    const u32 w = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    const u32 i = blockIdx.x * 4u + w;                          // one wavefront per position
+    if (i >= n) return;
+    const u64 segs = segmask[i];
+    if (segs == 0ull) return;                                   // only the first positions of an id that spans segments work
     const int my = (int)idx[i];
-    if ((u32)my >= V) return;                                   // no flag was written for it
-    if (flag[i] == 0u) return;                                  // only the owners of an id that spans segments work
-    const u32 p = lane < NS ? owner[(u64)my * NS + lane] : 0u;
-    const u64 present = __ballot(p != 0u);
-    u32* __restrict__ list = lists[w];                          // the id's owners, in segment order
-    if (p != 0u) list[__popcll(present & ((1ull << lane) - 1ull))] = p - 1u;
-    wave_lds_fence();
-    const u32 m = (u32)__popcll(present);
-    const u32 r = (u32)__popcll(present & ((1ull << (i / EMB_SEG)) - 1ull));        // this owner's rank among them
-    {VT}* __restrict__ dst = reinterpret_cast<{VT}*>(out + (long long)my * W);
+    const u32 m = (u32)__popcll(segs);
+    const u32 r = (u32)__popcll(segs & ((1ull << (i / EMB_SEG)) - 1ull));           // this segment's rank among them
+    // the id's first position in each of its segments, in segment order, as the first launch listed them
+    const u32* __restrict__ list = firsts + (u64)i * ((n + EMB_SEG - 1u) / EMB_SEG);
     const u32 Wv = W / {vec}u;
-    const u32 c0 = (u32)((u64)r * Wv / m), c1 = (u32)((u64)(r + 1u) * Wv / m);      // the owners split the columns
+    {VT}* __restrict__ dst = reinterpret_cast<{VT}*>(out + (u64)my * W);
+    const u32 c0 = r * Wv / m, c1 = (r + 1u) * Wv / m;        /* r < 512 and Wv < 2^22: no overflow */      // the first positions split the columns
     for (u32 c = c0 + lane; c < c1; c += 64u) {{
         {VT} acc = reinterpret_cast<const {VT}*>(partial + (u64)list[0] * W)[c];
         #pragma unroll 8
@@ -1085,7 +1138,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
     }}
 }}
 """
-        fmt = _fmt("P", "P", "P", "P", "P", "I", "I", "I", "I")
+        fmt = _fmt("P", "P", "P", "P", "P", "I", "I", "I")
     return f"{PRELUDE}{_ORDERED_COMMON}{body}", name, fmt
 
 

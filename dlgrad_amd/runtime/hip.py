@@ -1010,25 +1010,27 @@ class HIP:
                   upstream_grad: Buffer = None) -> DevicePtr:
         W, n_idx = x.shape[-1], idx.numel
         if backward:
-            out = alloc(x.numel, zero=True)                    # init_with_scalar(0), cpu.py:1031
-            if not n_idx:
-                return out
-            NS = (n_idx + K.EMB_SEGMENT - 1) // K.EMB_SEGMENT
-            if n_idx <= K.EMB_ORDERED_MAX and NS <= W and EMB_ORDERED:
-                # ordered, atomic-free: same bits every run (and the reference's bits for ids
-                # that stay inside one 512-position segment)
-                V = x.numel // W
-                partial, flag, owner = alloc(n_idx * W), alloc(n_idx), alloc(V * NS, zero=True)
+            V = x.numel // W
+            if n_idx and n_idx <= K.EMB_ORDERED_MAX and EMB_ORDERED and x.numel < 2 ** 31 and W <= 1 << 22:
+                # two launches write every element of the table exactly once -- sums in index order where an id
+                # occurs, zeros elsewhere -- without a zero-fill pass and without atomics
+                NS = (n_idx + K.EMB_SEGMENT - 1) // K.EMB_SEGMENT
+                out, partial, segmask, firsts, idsegs = alloc(x.numel), alloc(n_idx * W), alloc(2 * n_idx), alloc(n_idx * NS), alloc(2 * V)
                 vec = 4 if (W % 4 == 0 and not (_addr(upstream_grad) | out.addr | partial.addr) & 15) else 1
-                grid = (n_idx + 3) // 4
-                launch(kernel(K.embedding_backward_ordered_kernel, "mark"), grid, 256, owner.addr, _addr(idx), n_idx, NS, V)
-                launch(kernel(K.embedding_backward_ordered_kernel, "ordered", vec), grid, 256, out.addr, partial.addr,
-                       flag.addr, owner.addr, _addr(upstream_grad), _addr(idx), n_idx, W, NS, V)
-                launch(kernel(K.embedding_backward_ordered_kernel, "merge", vec), grid, 256, out.addr, partial.addr,
-                       flag.addr, owner.addr, _addr(idx), n_idx, W, NS, V)
+                n_sum, n_zero = (n_idx + 3) // 4, (V + 63) // 64
+                every = max(1, (n_sum + n_zero) // n_zero)     # one zero block among every so many
+                launch(kernel(K.embedding_backward_ordered_kernel, "mark", 1, False, 4 if _addr(idx) % 16 == 0 else 1),
+                       n_zero, 256, idsegs.addr, _addr(idx), n_idx, V)
+                launch(kernel(K.embedding_backward_ordered_kernel, "segments", vec, x.numel >= NT_STORE_MIN_ELEMENTS),
+                       n_sum + n_zero, 256, out.addr, partial.addr, segmask.addr, firsts.addr, idsegs.addr, _addr(upstream_grad),
+                       _addr(idx), n_idx, W, V, n_zero, every)
+                launch(kernel(K.embedding_backward_ordered_kernel, "merge", vec), n_sum, 256, out.addr, partial.addr,
+                       segmask.addr, firsts.addr, _addr(idx), n_idx, W, V)
                 return out
-            launch(kernel(K.embedding_backward_kernel), (n_idx + 3) // 4, 256,
-                   out.addr, _addr(upstream_grad), _addr(idx), n_idx, W, x.numel // W)
+            out = alloc(x.numel, zero=True)                    # init_with_scalar(0), cpu.py:1031
+            if n_idx:                                          # very long index lists: hardware fp32 atomics
+                launch(kernel(K.embedding_backward_kernel), (n_idx + 3) // 4, 256,
+                       out.addr, _addr(upstream_grad), _addr(idx), n_idx, W, V)
             return out
         out = alloc(out_numel)
         if n_idx:
