@@ -412,11 +412,12 @@ class Buffer:
         """self is a log-softmax; returns ((exp(self) - onehot(target)) * upstream) / n."""
         return self._like(self._dispatch(CustomOps.CE_GRAD, lsm=self, target=target, upstream=upstream, n=n))
 
-    def ce_stats(self, target: "Buffer") -> tuple["Buffer", "Buffer", "Buffer"]:
+    def ce_stats(self, target: "Buffer", negate: bool = False) -> tuple["Buffer", "Buffer", "Buffer"]:
         """self: (N, V) logits.  Returns per row the max, log(sum(exp(x - max))) and the target's
-        log-probability, each as (1, N) -- the cross-entropy forward without a log-softmax tensor."""
+        log-probability (its negative, the row's loss, with negate), each as (1, N) -- the
+        cross-entropy forward without a log-softmax tensor."""
         n = self.shape[0]
-        m, ls, picked = self._dispatch(CustomOps.CE_STATS, x=self, target=target)
+        m, ls, picked = self._dispatch(CustomOps.CE_STATS, x=self, target=target, negate=negate)
         return self._like(m, (1, n)), self._like(ls, (1, n)), self._like(picked, (1, n))
 
     def ce_grad_logits(self, m: "Buffer", ls: "Buffer", target: "Buffer", upstream: "Buffer", n: float) -> "Buffer":

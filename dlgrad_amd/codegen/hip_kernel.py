@@ -542,6 +542,28 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 }}
 """
         return src, name, _fmt("P", "P", "I", "I")
+    if mode == "rows_direct":
+        # rows of an even number of floats up to cap, 8-byte aligned: every load of a row is issued before the first compare
+        name = f"argmax_rows_direct_c{cap}"
+        src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
+        float* __restrict__ out, u32 R, u32 L) {{
+    const u32 row = blockIdx.x * 256u + threadIdx.x;
+    if (row >= R) return;
+    const float2* __restrict__ p = reinterpret_cast<const float2*>(x + (u64)row * L);
+    float2 v[{cap // 2}];
+    #pragma unroll
+    for (u32 k = 0; k < {cap // 2}u; ++k) if (2u * k < L) v[k] = p[k];
+    float best = NEG_FLT_MAX; u32 bi = 0;
+    #pragma unroll
+    for (u32 k = 0; k < {cap // 2}u; ++k) if (2u * k < L) {{
+        if (v[k].x > best) {{ best = v[k].x; bi = 2u * k; }}
+        if (v[k].y > best) {{ best = v[k].y; bi = 2u * k + 1u; }}
+    }}
+    out[row] = (float)bi;
+}}
+"""
+        return src, name, _fmt("P", "P", "I", "I")
     if mode == "rows_staged":
         # rows of at most cap floats (sizes the LDS stage), loads of vec floats
         width = vec
@@ -660,7 +682,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 #define VEC {vec}
 extern "C" __global__ __launch_bounds__(1024) void {name}(const float* __restrict__ x,
         float* __restrict__ out, float* __restrict__ pv, u32* __restrict__ pi, u32 L, u32 I, u32 chunk, u32 final) {{
-    __shared__ float sv[16][64 * VEC + 1]; __shared__ u32 si[16][64 * VEC + 1];
+    __shared__ float sv[16][VEC][64]; __shared__ u32 si[16][VEC][64];     // [thread row][component][lane]: a wavefront's accesses fall on 64 consecutive words
     const u32 tx = threadIdx.x, ty = threadIdx.y, o = blockIdx.z;
     const u32 col = (blockIdx.x * 64u + tx) * VEC;
     const u32 l0 = blockIdx.y * chunk, l1 = min(L, l0 + chunk);
@@ -671,13 +693,13 @@ extern "C" __global__ __launch_bounds__(1024) void {name}(const float* __restric
         const float* __restrict__ xp = x + (u64)o * L * I + col;{scan}
     }}
     #pragma unroll
-    for (int c = 0; c < VEC; ++c) {{ sv[ty][tx * VEC + c] = best[c]; si[ty][tx * VEC + c] = bi[c]; }}
+    for (int c = 0; c < VEC; ++c) {{ sv[ty][c][tx] = best[c]; si[ty][c][tx] = bi[c]; }}
     __syncthreads();
     if (ty == 0 && col < I) {{
         #pragma unroll
         for (int c = 0; c < VEC; ++c) {{
             #pragma unroll
-            for (int k = 1; k < 16; ++k) TAKE(best[c], bi[c], sv[k][tx * VEC + c], si[k][tx * VEC + c])
+            for (int k = 1; k < 16; ++k) TAKE(best[c], bi[c], sv[k][c][tx], si[k][c][tx])
             if (final) out[(u64)o * I + col + c] = (float)bi[c];
             else {{ const u64 at = ((u64)o * gridDim.y + blockIdx.y) * I + col + c; pv[at] = best[c]; pi[at] = bi[c]; }}
         }}
@@ -1362,7 +1384,7 @@ extern "C" __global__ __launch_bounds__({threads}) void {name}(const float* __re
 
 
 @cache
-def ce_stats_kernel(vec: int, per_block: bool, nt: bool = False) -> tuple[str, str, str]:
+def ce_stats_kernel(vec: int, per_block: bool, nt: bool = False, negate: bool = False) -> tuple[str, str, str]:
     """The forward pass of the cross-entropy loss without its log-softmax tensor (ops.py:337-357
     composes max, sub, exp, sum, log, sub over the whole (N, V) logits and gathers one entry per
     row).  Per row r of an (R, L) view: m[r] = max, ls[r] = log(sum(exp(x - m))) and
@@ -1376,9 +1398,11 @@ def ce_stats_kernel(vec: int, per_block: bool, nt: bool = False) -> tuple[str, s
     overlaps the loads of the others.  The threads' (m, s) pairs are joined the same way.  The
     sum is therefore added in another order than max-then-sum would add it (a few ulp); the
     maximum is exact.  The backward pass rebuilds exp((x - m) - ls) from the logits and these
-    two numbers.  One wavefront per row, or one 256-thread block per long row."""
+    two numbers.  One wavefront per row, or one 256-thread block per long row.
+    negate: picked[r] is written with its sign flipped, i.e. as the row's loss term, so that the
+    loss is a plain sum of it (-(a + b) and (-a) + (-b) are the same float)."""
     nt = nt and vec == 4
-    name = f"ce_stats_v{vec}_{'blk' if per_block else 'wav'}{'nt' if nt else ''}"
+    name = f"ce_stats_v{vec}_{'blk' if per_block else 'wav'}{'nt' if nt else ''}{'_neg' if negate else ''}"
     T = "256u" if per_block else "64u"
     tid = "threadIdx.x" if per_block else "(threadIdx.x & 63u)"
     row = "blockIdx.x" if per_block else "(blockIdx.x * 4u + (threadIdx.x >> 6))"
@@ -1436,7 +1460,8 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
         const int t = (int)target[row];
         row_max[row] = m;
         row_logsum[row] = ls;
-        picked[row] = (u32)t < L ? (x[(u64)row * L + (u32)t] - m) - ls : 0.0f;
+        const float lp = (u32)t < L ? (x[(u64)row * L + (u32)t] - m) - ls : 0.0f;
+        picked[row] = {'-lp' if negate else 'lp'};
     }}
 }}
 """

@@ -594,8 +594,9 @@ class CrossEntropy(OP):
         if self.fused:
             from dlgrad_amd.runtime.hip import HIP
             if HIP.ce_stats_fits(logits):
-                m, ls, picked = logits.ce_stats(target)
+                m, ls, row_loss = logits.ce_stats(target, negate=True)
                 self.logits, self.stats = logits, (m, ls)
+                return row_loss.sum()                       # = -(sum of the picked log-probs), bit for bit
             else:                                           # more than 2^31 elements
                 self.log_softmax, picked = logits.log_softmax_gather(target)
         else:

@@ -104,6 +104,18 @@ class Block:
         return self.mlp(self.ln2(x), residual=x)                      # x + mlp(norm(x))
 
 
+_position_ids: dict = {}
+
+
+def _positions(T: int, device) -> Tensor:
+    """0 .. T-1 as a tensor on `device`, made there once per length (the reference builds it anew, and on
+    the host, in every forward; examples/gpt.py:96-97)."""
+    key = (T, str(device))
+    if key not in _position_ids:
+        _position_ids[key] = Tensor.arange((T,), device=device)
+    return _position_ids[key]
+
+
 class GPT:
     def __init__(self, c: GPTConfig) -> None:
         self.config = c
@@ -116,8 +128,7 @@ class GPT:
     def __call__(self, idx: Tensor, targets: Tensor | None = None):
         """idx, targets: (B, T) token ids stored as fp32.  Returns (logits, loss)."""
         B, T = idx.shape
-        pos = Tensor.arange((T,), device=idx.device)            # 0..T-1 made on the device (no upload per step)
-        x = self.wte(idx) + self.wpe(pos)
+        x = self.wte(idx) + self.wpe(_positions(T, idx.device))
         for block in self.blocks:
             x = block(x)
         logits = self.lm_head(self.ln_f(x))
@@ -140,7 +151,7 @@ class GPT:
         examples/gpt.py:103-112, which slices the last position out on the host)."""
         B, T = idx.shape
         cache = KVCache(self.config, B)
-        x = self._hidden(idx, Tensor.arange((T,), device=idx.device), cache)
+        x = self._hidden(idx, _positions(T, idx.device), cache)
         cache.length = T
         C = x.shape[2]
         last = x.reshape((T, C))[T - 1:T] if B == 1 else x.transpose(0, 1)[T - 1:T]
@@ -195,26 +206,39 @@ class GPT:
 
 
 class StaticDecoder:
-    """Greedy decoding inside the context window as one step of fixed shape.
+    """Greedy decoding as steps of fixed shape, inside the context window and beyond it.
 
     forward_incremental attends to a cache that grows by one row per token, so every token has
     new tensor shapes and must be issued launch by launch from Python (~130 launches per token
-    for the char model, which is what bounds its speed).  Here the step always attends to all
-    block_size cache rows and masks the ones not written yet (-inf before the softmax, so they
-    weigh exactly 0), and everything that changes from token to token -- the token, the cache
-    row to write, the position id, the mask -- is device data updated by the step itself.  The
-    step therefore has no host input at all and can be captured once as a HIP graph and
-    replayed per token.  Same tokens as generate_greedy_cached (the probabilities differ only
-    in the order of the softmax sums)."""
+    for the char model, which is what bounds its speed).  Here there are two steps, both of fixed
+    shape and without any host input, so each can be captured once as a HIP graph and replayed
+    per token:
 
-    def __init__(self, model: GPT, reference_positions: bool = STRICT_REFERENCE) -> None:
+      step()         while the sequence is shorter than block_size: one new token against the
+                     key/value cache.  It always attends to all block_size cache rows and masks
+                     the ones not written yet (-inf before the softmax, so they weigh exactly 0).
+      step_window()  once block_size tokens exist: the reference keeps no cache from there on
+                     (the position embeddings are absolute, so sliding the window by one changes
+                     every key and value) and runs the whole model over the last block_size
+                     tokens for every new one (examples/gpt.py:176-180, :246-256).  The step
+                     gathers that window out of the token buffer at an offset held on the
+                     device, runs the full forward and appends the argmax of the last position.
+
+    Everything that changes from token to token -- the token, the cache row to write, the
+    position id, the mask, the window offset -- is device data updated by the steps themselves.
+    Same tokens as generate_greedy_cached (the probabilities differ only in the order of the
+    softmax sums) and, with reference_positions=False, as full recompute (generate_greedy)."""
+
+    def __init__(self, model: GPT, reference_positions: bool = STRICT_REFERENCE, capacity: int | None = None) -> None:
         c = model.config
         self.model, self.reference_positions = model, reference_positions
+        self.capacity = int(capacity) if capacity is not None else 2 * c.block_size + 1     # tokens the buffer holds
         self.cache = KVCache(c, 1)
         self.tok = Tensor.full((1, 1), 0.0, device=c.device)          # token to feed
         self.slot = Tensor.full((1, 1), 0.0, device=c.device)         # its index = cache row to write
-        self.seq = Tensor.full((c.block_size + 1, 1), 0.0, device=c.device)
+        self.seq = Tensor.full((max(self.capacity, c.block_size + 1), 1), 0.0, device=c.device)
         self.graph = None
+        self.window_graph = None
 
     def reset(self, first_token: int) -> None:
         self.tok.data.upload_(np.array([[first_token]], np.float32))
@@ -230,6 +254,12 @@ class StaticDecoder:
         y = nn.cached_attention(q, self.cache.k[layer], self.cache.v[layer], T, attn.n_head, attn.scale, hidden)
         return attn.c_proj(y, residual)
 
+    def _append(self, nxt: Tensor) -> None:
+        nslot = self.slot + 1.0
+        self.seq.data.row_store_(nxt.data, nslot.data)
+        self.tok.data.copy_(nxt.data)
+        self.slot.data.copy_(nslot.data)
+
     def step(self) -> None:
         """Feeds self.tok at index self.slot; leaves the argmax in seq[slot + 1] and as the next
         token, and advances slot.  Reads and writes device memory only."""
@@ -242,38 +272,54 @@ class StaticDecoder:
         for i, block in enumerate(m.blocks):
             x = self._attend(block.attn, block.ln1(x), i, hidden, x)
             x = block.mlp(block.ln2(x), x)
-        nxt = m.lm_head(m.ln_f(x)).reshape((1, c.vocab_size)).argmax(1)                     # (1, 1)
-        nslot = slot + 1.0
-        self.seq.data.row_store_(nxt.data, nslot.data)
-        self.tok.data.copy_(nxt.data)
-        self.slot.data.copy_(nslot.data)
+        self._append(m.lm_head(m.ln_f(x)).reshape((1, c.vocab_size)).argmax(1))             # (1, 1)
+
+    def step_window(self) -> None:
+        """The step for a full window: tokens slot - block_size + 1 .. slot go through the whole model
+        at positions 0 .. block_size - 1; the argmax of the last position becomes token slot + 1."""
+        m, c = self.model, self.model.config
+        T = c.block_size
+        where = Tensor.arange((1, T), device=c.device) + (self.slot - float(T - 1))        # indices into the token buffer
+        window = Tensor.embedding(self.seq, where).reshape((1, T))                          # the tokens themselves
+        logits, _ = m(window)
+        self._append(logits.reshape((T, c.vocab_size))[T - 1:T].argmax(1))
 
     def capture(self) -> None:
-        """hip only: records step() into a graph (one warm-up step fixes every address first)."""
+        """hip only: records both steps into graphs (one warm-up run of each fixes every address first).
+        The warm-up tokens are overwritten by the next reset()."""
         from dlgrad_amd.runtime import hip
-        self.graph = hip.Graph()
+        T = self.model.config.block_size
         self.reset(0)
+        self.graph = hip.Graph()
         with self.graph.arena():
             self.step()
         with self.graph.capture():
             self.step()
+        if self.capacity > T:
+            self.slot.data.upload_(np.array([[T - 1]], np.float32))       # a full window, wherever its tokens come from
+            self.window_graph = hip.Graph()
+            with self.window_graph.arena():
+                self.step_window()
+            with self.window_graph.capture():
+                self.step_window()
 
     def generate(self, first_token: int, max_new_tokens: int) -> list[int]:
         c = self.model.config
-        if not 0 <= max_new_tokens <= c.block_size - 1:
-            raise ValueError(f"the static step decodes inside the window: at most {c.block_size - 1} new tokens")
+        if not 0 <= max_new_tokens <= self.capacity - 1:
+            raise ValueError(f"this decoder holds {self.capacity} tokens: at most {self.capacity - 1} new ones")
         self.reset(first_token)
-        for _ in range(max_new_tokens):
-            if self.graph is not None:
-                self.graph.replay()
+        for t in range(max_new_tokens):
+            if t < c.block_size - 1:                      # t + 1 tokens so far: still inside the window
+                self.graph.replay() if self.graph is not None else self.step()
             else:
-                self.step()
+                self.window_graph.replay() if self.window_graph is not None else self.step_window()
         return [int(v) for v in self.seq.numpy().reshape(-1)[:max_new_tokens + 1]]
 
     def close(self) -> None:
-        if self.graph is not None:
-            self.graph.close()
-            self.graph = None
+        for g in (self.graph, self.window_graph):
+            if g is not None:
+                g.close()
+        self.graph = self.window_graph = None
 
 
 def init_weights_(model: GPT, seed: int, std: float = 0.02) -> None:

@@ -92,12 +92,15 @@ def test_argmax_bit_exact_with_ties(shape):
     check(dev(y).argmax(1).numpy(), y.argmax(1).astype(np.float32).reshape(-1, 1), 0, "argmax random")
 
 
+@pytest.mark.parametrize("form", ["direct", "staged"])
 @pytest.mark.parametrize("L", [1, 2, 7, 8, 9, 10, 16, 17, 31, 32])
-def test_argmax_of_many_short_rows(L):
-    """Row counts above 4096 with L <= 32 go through LDS, 256 rows a block; the last block is
-    ragged (row counts that are no multiple of 256, of 4, and an odd total) and a view that
-    starts 4 bytes into its block takes the narrow loads."""
+def test_argmax_of_many_short_rows(L, form, monkeypatch):
+    """Row counts above 4096 with L <= 32: a thread per row with 8-byte loads where the length is
+    even and the rows are 8-byte aligned ("direct"), else -- and wherever "staged" is chosen -- through
+    LDS, 256 rows a block; the last block is ragged (row counts that are no multiple of 256, of 4,
+    and an odd total) and a view that starts 4 bytes into its block takes the narrow loads."""
     require_gpu()
+    monkeypatch.setattr(hip, "ARGMAX_SHORT_ROWS", form)
     for R in (4096, 4099, 10001):
         x = RNG.integers(0, 4, (R, L)).astype(np.float32)
         want = cref.argmax(x, 1).reshape(R, 1)

@@ -308,24 +308,32 @@ def test_cached_decode_reproduces_full_recompute_on_the_cpu_oracle():
 
 
 @pytest.mark.parametrize("reference_positions", [True, False])
-def test_fixed_shape_decoding_step_reproduces_cached_decoding_on_the_cpu_oracle(reference_positions):
-    """Attending to the whole (masked) cache instead of its filled part changes no token."""
+def test_fixed_shape_decoding_steps_reproduce_cached_decoding_on_the_cpu_oracle(reference_positions):
+    """Attending to the whole (masked) cache instead of its filled part changes no token, and beyond the
+    window the fixed-shape full-forward step over the last block_size tokens continues exactly as the
+    reference's loop does (no cache from there on); with each token at its own position the whole
+    sequence is also what full recompute gives."""
     model = G.GPT(G.GPTConfig(device="cpu", **dict(TINY, n_embd=32, block_size=12)))
     G.init_weights_(model, 3, std=0.5)
-    want = model.generate_greedy_cached(3, 11, reference_positions=reference_positions)
-    dec = G.StaticDecoder(model, reference_positions=reference_positions)
-    assert dec.generate(3, 11) == want
+    want = model.generate_greedy_cached(3, 30, reference_positions=reference_positions)
+    dec = G.StaticDecoder(model, reference_positions=reference_positions, capacity=31)
+    assert dec.generate(3, 30) == want
+    assert dec.generate(3, 11) == want[:12]                  # the last token decided inside the window
+    assert dec.generate(3, 12) == want[:13]                  # the first one decided by a full window
     assert dec.generate(7, 5) == model.generate_greedy_cached(7, 5, reference_positions=reference_positions)
+    if not reference_positions:
+        assert want == model.generate_greedy(3, 30)
     with pytest.raises(ValueError):
-        dec.generate(3, 12)                              # would leave the window (and the position table)
+        dec.generate(3, 31)                                  # more than the token buffer holds
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("reference_positions", [True, False])
 def test_decoding_step_replayed_as_a_graph_gives_the_eager_tokens(reference_positions):
-    """hip: the fixed-shape step eager, the same step captured once and replayed per token,
-    and the growing-cache loop on the C oracle's cpu device all produce the same ids; the
-    captured step is reused for a second sequence."""
+    """hip: the two fixed-shape steps eager, the same steps captured once and replayed per token, and the
+    reference's loop on the C oracle's cpu device (growing cache, then full forwards once the window is
+    full) all produce the same ids, inside the window and far beyond it; the captured steps are reused
+    for a second sequence."""
     if not (hip.available() or hip.COMPILE_ONLY):
         pytest.skip("no HIP device")
     cfg = dict(TINY, n_embd=64, block_size=32)
@@ -333,17 +341,20 @@ def test_decoding_step_replayed_as_a_graph_gives_the_eager_tokens(reference_posi
     for dev in ("cpu", "hip"):
         models[dev] = G.GPT(G.GPTConfig(device=dev, **cfg))
         G.init_weights_(models[dev], 3, std=0.2)
-    want = {t: models["cpu"].generate_greedy_cached(t, 31, reference_positions=reference_positions) for t in (0, 9)}
-    dec = G.StaticDecoder(models["hip"], reference_positions=reference_positions)
-    eager = dec.generate(0, 31)
+    want = {t: models["cpu"].generate_greedy_cached(t, 80, reference_positions=reference_positions) for t in (0, 9)}
+    dec = G.StaticDecoder(models["hip"], reference_positions=reference_positions, capacity=81)
+    eager = dec.generate(0, 80)                             # 31 tokens against the cache, 49 full windows
     if hip.COMPILE_ONLY:
         return
     assert eager == want[0]
     dec.capture()
-    assert dec.graph.nodes > 20
-    assert dec.generate(0, 31) == want[0]
-    assert dec.generate(9, 31) == want[9]
+    assert dec.graph.nodes > 20 and dec.window_graph.nodes > 20
+    assert dec.generate(0, 80) == want[0]
+    assert dec.generate(9, 80) == want[9]
+    assert dec.generate(0, 31) == want[0][:32]
     assert dec.generate(0, 4) == want[0][:5]
+    if not reference_positions:
+        assert want[0] == models["cpu"].generate_greedy(0, 80)        # the oracle's full recompute, token for token
     dec.close()
 
 
