@@ -518,7 +518,7 @@ def run_decode(n_tokens: int = 256) -> dict:
     cached = model.generate_greedy_cached(0, 120, reference_positions=False)
     dt = time.perf_counter() - t0
     out["kv_cached_120_tokens"] = {"ms_per_token": round(dt / 120 * 1e3, 3), "tokens_per_s": round(120 / dt, 1)}
-    dec = G.StaticDecoder(model, reference_positions=False, capacity=n_tokens + 1)
+    dec = G.StaticDecoder(model, reference_positions=False, capacity=max(n_tokens, 120) + 1)
     if not hip.COMPILE_ONLY:
         dec.capture()
     dec.generate(0, 8)

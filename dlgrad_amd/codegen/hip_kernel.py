@@ -1250,9 +1250,16 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     red_max = "block_max(m, sm)" if per_block else "wave_max(m)"
     red_sum = "block_sum(s, sm)" if per_block else "wave_sum(s)"
 
+    # Register-resident softmax (not log-softmax): each exp(x - m) is computed once, kept in the register
+    # that held x, summed, and divided by the sum afterwards -- the values and the order of the
+    # five-kernel composition (the exp kernel's output is what its sum and its division read).
+    keep = bool(nval) and not log
+
     def outexpr(v: str) -> str:
-        return f"(({v}) - m) - ls" if log else f"expf(({v}) - m) / s"
+        return f"(({v}) - m) - ls" if log else (f"({v}) / s" if keep else f"expf(({v}) - m) / s")
     comps = ("x", "y", "z", "w")
+    keep_exp4 = "".join(f"        v[k].{c} = expf(v[k].{c} - m);\n" for c in comps) if keep else ""
+    keep_exp1 = "v[k] = expf(v[k] - m); " if keep else ""
     mask4 = mask1 = ""
     if masked:
         sel4 = " ".join(f"v[k].{c} = (mb[k] & {1 << j}u) ? -__builtin_inff() : v[k].{c} * scale;" for j, c in enumerate(comps))
@@ -1296,8 +1303,9 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     m = {red_max};
     float s = 0.0f;
     #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) if ({live})
-        s += (expf(v[k].x - m) + expf(v[k].y - m)) + (expf(v[k].z - m) + expf(v[k].w - m));
+    for (u32 k = 0; k < {nval}u; ++k) if ({live}) {{
+{keep_exp4}        s += (E(v[k].x) + E(v[k].y)) + (E(v[k].z) + E(v[k].w));
+    }}
     s = {red_sum};
     const float ls = logf(s); (void)ls;
     #pragma unroll
@@ -1322,7 +1330,7 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     m = {red_max};
     float s = 0.0f;
     #pragma unroll
-    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < L) s += expf(v[k] - m);
+    for (u32 k = 0; k < {nval}u; ++k) if ({tid} + k * {T} < L) {{ {keep_exp1}s += E(v[k]); }}
     s = {red_sum};
     const float ls = logf(s); (void)ls;
     #pragma unroll
@@ -1371,6 +1379,7 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     if masked:
         extra_params = ", const float* __restrict__ mask, u32 mrows, float scale"
     src = f"""{PRELUDE}{_row_block_reduce(NW)}
+#define E(t) {'(t)' if keep else 'expf((t) - m)'}
 extern "C" __global__ __launch_bounds__({threads}) void {name}(const float* __restrict__ x,
         float* __restrict__ out, u32 R, u32 L{extra_params}) {{
     __shared__ float sm[{NW}];

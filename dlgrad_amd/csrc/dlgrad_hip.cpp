@@ -17,6 +17,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hiprtc.h>
 
+#include <atomic>
 #include <cstddef>
 #include <cstdio>
 #include <cstdlib>
@@ -69,9 +70,10 @@ std::unordered_map<void *, Block> g_live;                            // block ->
 std::map<uint64_t, bool> g_arena_alive;                              // arenas that still exist
 uint64_t g_arena = 0, g_next_arena = 1;
 uint64_t g_bytes_in_use = 0, g_bytes_cached = 0, g_device_allocs = 0;
-bool g_capturing = false;
+std::atomic<bool> g_capturing{false};                            // read by calls that refuse to run inside a capture
 std::map<void *, size_t> g_pinned;                                   // page-locked host blocks handed out
 std::vector<hipGraphExec_t> g_graphs;                                // handle = index + 1 (null once destroyed)
+std::vector<hipEvent_t> g_events;                                    // handle = index + 1 (null once destroyed)
 
 int fail(const char *what, hipError_t e) {
     char buf[512];
@@ -206,6 +208,8 @@ int dlg_hip_shutdown(void) {
     (void)hipStreamSynchronize(g_stream);
     for (hipGraphExec_t ge : g_graphs) if (ge) (void)hipGraphExecDestroy(ge);
     g_graphs.clear();
+    for (hipEvent_t ev : g_events) if (ev) (void)hipEventDestroy(ev);
+    g_events.clear();
     while (!g_free.empty()) trim_arena_locked(g_free.begin()->first);
     g_arena = 0;
     g_capturing = false;
@@ -228,6 +232,12 @@ int dlg_hip_props(dlg_hip_props_t *out) {
     HIP_TRY(hipGetDeviceProperties(&p, g_device));
     std::memset(out, 0, sizeof *out);
     std::snprintf(out->name, sizeof out->name, "%s", p.name);
+    if (!out->name[0]) {                          // some driver stacks leave the property empty: ask by name, then fall back to the arch
+        char nm[128] = {0};
+        if (hipDeviceGetName(nm, sizeof nm, g_device) == hipSuccess && nm[0]) std::snprintf(out->name, sizeof out->name, "%s", nm);
+        else std::snprintf(out->name, sizeof out->name, "%s", p.gcnArchName);
+        (void)hipGetLastError();
+    }
     std::snprintf(out->arch, sizeof out->arch, "%s", p.gcnArchName);
     out->compute_units = p.multiProcessorCount;
     out->wavefront_size = p.warpSize;
@@ -624,17 +634,27 @@ int dlg_hip_graph_end(uint64_t *graph, uint64_t *n_nodes) {
 
 int dlg_hip_graph_launch(uint64_t graph) {
     NEED_INIT();
-    if (graph == 0 || graph > g_graphs.size() || !g_graphs[graph - 1]) return fail_msg(-32, "bad graph handle");
-    HIP_TRY(hipGraphLaunch(g_graphs[graph - 1], g_stream));
+    hipGraphExec_t ge;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        if (graph == 0 || graph > g_graphs.size() || !g_graphs[graph - 1]) return fail_msg(-32, "bad graph handle");
+        ge = g_graphs[graph - 1];
+    }
+    HIP_TRY(hipGraphLaunch(ge, g_stream));
     return 0;
 }
 
 int dlg_hip_graph_destroy(uint64_t graph) {
     NEED_INIT();
-    if (graph == 0 || graph > g_graphs.size() || !g_graphs[graph - 1]) return fail_msg(-32, "bad graph handle");
+    hipGraphExec_t ge;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        if (graph == 0 || graph > g_graphs.size() || !g_graphs[graph - 1]) return fail_msg(-32, "bad graph handle");
+        ge = g_graphs[graph - 1];
+        g_graphs[graph - 1] = nullptr;
+    }
     HIP_TRY(hipStreamSynchronize(g_stream));
-    HIP_TRY(hipGraphExecDestroy(g_graphs[graph - 1]));
-    g_graphs[graph - 1] = nullptr;
+    HIP_TRY(hipGraphExecDestroy(ge));
     return 0;
 }
 
@@ -646,37 +666,64 @@ int dlg_hip_sync(void) {
     return 0;
 }
 
+namespace {
+// The event behind a handle, or nullptr (with the error text set) for a handle this library never gave out.
+hipEvent_t event_of(uint64_t handle) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (handle == 0 || handle > g_events.size() || !g_events[handle - 1]) {
+        g_err = "bad event handle";
+        return nullptr;
+    }
+    return g_events[handle - 1];
+}
+}  // namespace
+
 int dlg_hip_event_create(uint64_t *event) {
     NEED_INIT();
     if (!event) return fail_msg(-1, "event is NULL");
     hipEvent_t ev;
     HIP_TRY(hipEventCreate(&ev));
-    *event = (uint64_t)(uintptr_t)ev;
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_events.push_back(ev);
+    *event = (uint64_t)g_events.size();
     return 0;
 }
 
 int dlg_hip_event_record(uint64_t event) {
     NEED_INIT();
-    HIP_TRY(hipEventRecord((hipEvent_t)(uintptr_t)event, g_stream));
+    hipEvent_t ev = event_of(event);
+    if (!ev) return -33;
+    HIP_TRY(hipEventRecord(ev, g_stream));
     return 0;
 }
 
 int dlg_hip_event_sync(uint64_t event) {
     NEED_INIT();
-    HIP_TRY(hipEventSynchronize((hipEvent_t)(uintptr_t)event));
+    hipEvent_t ev = event_of(event);
+    if (!ev) return -33;
+    HIP_TRY(hipEventSynchronize(ev));
     return 0;
 }
 
 int dlg_hip_event_elapsed_ms(uint64_t start, uint64_t stop, float *ms) {
     NEED_INIT();
     if (!ms) return fail_msg(-1, "ms is NULL");
-    HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)(uintptr_t)start, (hipEvent_t)(uintptr_t)stop));
+    hipEvent_t a = event_of(start), b = event_of(stop);
+    if (!a || !b) return -33;
+    HIP_TRY(hipEventElapsedTime(ms, a, b));
     return 0;
 }
 
 int dlg_hip_event_destroy(uint64_t event) {
     NEED_INIT();
-    HIP_TRY(hipEventDestroy((hipEvent_t)(uintptr_t)event));
+    hipEvent_t ev;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        if (event == 0 || event > g_events.size() || !g_events[event - 1]) return fail_msg(-33, "bad event handle");
+        ev = g_events[event - 1];
+        g_events[event - 1] = nullptr;
+    }
+    HIP_TRY(hipEventDestroy(ev));
     return 0;
 }
 

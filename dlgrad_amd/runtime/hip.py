@@ -1407,11 +1407,12 @@ class HIP:
     # "1": a shape met for the first time (and large enough to matter) is timed once with every
     # plausible tile and the fastest is remembered; "0": shipped table, then the model
     MATMUL_TUNE = os.environ.get("DLGRAD_HIP_MATMUL_TUNE", "1") != "0"
+    MATMUL_TABLE = os.environ.get("DLGRAD_HIP_MATMUL_TABLE", "1") != "0"    # "0": ignore the measured tables (model, or first-use timing, only)
     MATMUL_TUNE_MIN_FLOP = 1 << 24
     _tuned: dict | None = None
     _tuned_new: dict = {}
 
-    MATMUL_TUNED_FILE = os.path.join(CACHE_DIR, "matmul_tuned.json")
+    MATMUL_TUNED_FILE = os.environ.get("DLGRAD_HIP_MATMUL_TUNED_FILE", os.path.join(CACHE_DIR, "matmul_tuned.json"))
     last_matmul_kernel: str | None = None      # name of the most recently launched product kernel (reported by the benchmark)
 
     @staticmethod
@@ -1424,7 +1425,7 @@ class HIP:
         MI355X) overlaid with what this machine's own tuning runs have stored in the cache."""
         if HIP._tuned is None:
             table = {}
-            for path in (os.path.join(os.path.dirname(K.__file__), "matmul_tuned.json"), HIP._tuned_path()):
+            for path in (os.path.join(os.path.dirname(K.__file__), "matmul_tuned.json"), HIP._tuned_path()) if HIP.MATMUL_TABLE else ():
                 try:
                     with open(path) as f:
                         table.update({k: v for k, v in json.load(f).items() if v in K.MATMUL_CONFIGS})

@@ -366,3 +366,29 @@ def test_reduce_full_checks_its_arguments_on_the_host():
         with pytest.raises(HipError, match=msg):
             lib.reduce_full(*args)
     lib.sync()
+
+
+@pytest.mark.gpu
+def test_event_and_graph_handles_are_checked():
+    """Handles are indices into the library's own tables: a number it never gave out, or one that
+    was destroyed, is refused with a message instead of being used as a pointer."""
+    from dlgrad_amd.runtime import hip
+    if not hip.available():
+        pytest.skip("no HIP device")
+    from dlgrad_amd.ffi import HipError
+    lib = hip.lib()
+    e0, e1 = lib.event_create(), lib.event_create()
+    lib.event_record(e0)
+    lib.event_record(e1)
+    lib.event_sync(e1)
+    assert lib.event_elapsed_ms(e0, e1) >= 0.0
+    lib.event_destroy(e1)
+    for bad in (e1, 0, 10 ** 9):
+        with pytest.raises(HipError, match="bad event handle"):
+            lib.event_record(bad)
+        with pytest.raises(HipError, match="bad event handle"):
+            lib.event_elapsed_ms(e0, bad)
+    with pytest.raises(HipError, match="bad graph handle"):
+        lib.graph_launch(10 ** 9)
+    lib.event_destroy(e0)
+    assert hip.props()["name"], "the device name must not be empty"
