@@ -436,7 +436,12 @@ class Buffer:
                     through_mean: bool, plus: "Buffer | None" = None) -> tuple["Buffer", "Buffer | None"]:
         """self is the forward input x; returns (dx, dw) with dw shaped like the weight.  plus: added to dx as it is stored."""
         kw = {"plus": plus} if plus is not None else {}
+        if weight is not None and self.device is Device.HIP and PENDING_SUMS:
+            kw["partial_dw"] = True             # dw may come back as the partial rows themselves: (pointer, rows)
         dx, dw = self._dispatch(CustomOps.RMSNORM_BWD, x=self, w=weight, r=r, dy=dy, through_mean=through_mean, **kw)
+        if dw.__class__ is tuple:
+            part, rows = dw
+            return self._like(dx), PartialSum.of(self._like(part, (rows, weight.numel)), weight.shape)
         return self._like(dx), (None if dw is None else self._like(dw, weight.shape))
 
     # ---- selects ----------------------------------------------------------------------------------
@@ -593,3 +598,51 @@ class Buffer:
     @property
     def T(self) -> "Buffer":  # noqa: N802
         return self.transpose(0, 1)
+
+
+# Sums over a leading dim that the hip runtime can leave pending (see PartialSum)
+PENDING_SUMS = True
+PENDING_SUM_MAX_ROWS = 512          # what one column-sum launch folds; the pending form must mean exactly that launch
+
+
+class PartialSum(Buffer):
+    """A Buffer whose value is `parts.sum(0)` -- the sum over the leading dim of a (rows, *shape)
+    Buffer -- and that runs that sum only when somebody asks for its memory.
+
+    The weight gradients of a step are such sums (over the batch for a linear layer, ops.py:287-295;
+    over per-wavefront partial rows for an RMSNorm gain), and nothing reads them before the optimizer.
+    The one-launch Adam of the hip runtime takes the parts themselves and adds them up as it reads
+    the gradient, in the very order the column-sum kernel uses, so the separate launch per weight (a
+    quarter of the launches of a char-GPT step) disappears and the bits stay.  Every other reader --
+    numpy(), another op, a per-tensor optimizer -- touches `ptr`, which runs the sum then, once."""
+    __slots__ = ("parts", "_sum")
+
+    @staticmethod
+    def of(parts: Buffer, shape: tuple) -> Buffer:
+        """The pending sum of `parts` over its leading dim, shaped `shape`; the plain sum where pending
+        sums do not apply (another device, too many rows, nothing to add)."""
+        rows = parts.shape[0] if parts.ndim else 0
+        if (not PENDING_SUMS or parts.device is not Device.HIP or parts.__class__ is PartialSum or not 1 < rows <= PENDING_SUM_MAX_ROWS
+                or parts.numel != rows * prod_(shape) or parts.numel == 0):
+            out = parts.sum(0, keepdim=False)
+            return out if out.shape == tuple(shape) else out.reshape(shape)
+        b = _new_buffer(PartialSum)
+        b.parts, b._sum = parts, None
+        b.shape, b.dtype, b.device = tuple(shape), parts.dtype, parts.device
+        b.numel, b.stride, b.ndim, b.nbytes = _shape_info(b.shape)
+        return b
+
+    @property
+    def pending(self) -> bool:
+        return self._sum is None
+
+    @property
+    def ptr(self):
+        if self._sum is None:
+            self._sum = self.parts.sum(0, keepdim=False).ptr
+            self.parts = None
+        return self._sum
+
+    @ptr.setter
+    def ptr(self, value) -> None:
+        self._sum, self.parts = value, None

@@ -2370,13 +2370,53 @@ def adam_multi_inplace_kernel() -> tuple[str, str, str]:
     addresses (p, g, m, v) per tensor, `sizes` the element counts, `first` the first block of each
     tensor and `owner` the tensor of every block; a block updates 1024 consecutive elements of its
     tensor (16-byte accesses: every address is 16-byte aligned, the n % 4 tail is done by the
-    tensor's first block).  Same arithmetic as the per-tensor kernel, so the same bits."""
+    tensor's first block).  Same arithmetic as the per-tensor kernel, so the same bits.
+
+    `rows` says how many rows of `size` floats a tensor's gradient pointer holds.  1: the gradient
+    itself.  More: its parts, whose sum over the rows is the gradient (the batch entries of a weight
+    gradient, the partial rows of an RMSNorm gain).  They are added up here, element by element, in
+    exactly the order reduce_cols_kernel adds a column of that many rows (thread rows 4 or 16 apart,
+    four running sums each, joined pairwise, then the thread rows in order), so the update has the bits
+    it would have had with the column-sum launch in between."""
     src, _, _ = adam_kernel(4)
     head = src[:src.index('extern "C"')]
     name = "adam_multi_inplace"
-    src2 = f"""{head}extern "C" __global__ __launch_bounds__(256) void {name}(const u64* __restrict__ ptrs,
+    colsum = r"""
+// Sum over l of row l of a (rows, n) array at one place -- element j, or the four elements of 16-byte item j when
+// n is a multiple of 4 -- in reduce_cols_kernel's order.
+static __device__ __forceinline__ float ld_at(const float* __restrict__ g, u64 row_off, u32 j, float) { return g[row_off + j]; }
+static __device__ __forceinline__ float4 ld_at(const float* __restrict__ g, u64 row_off, u32 j, float4) {
+    return reinterpret_cast<const float4*>(g + row_off)[j];
+}
+static __device__ __forceinline__ float add2(float a, float b) { return a + b; }
+static __device__ __forceinline__ float4 add2(float4 a, float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
+static __device__ __forceinline__ void zero_of(float& z) { z = 0.0f; }
+static __device__ __forceinline__ void zero_of(float4& z) { z = make_float4(0.f, 0.f, 0.f, 0.f); }
+template <int TY, typename T> static __device__ __forceinline__ T colsum(const float* __restrict__ g, u32 rows, u32 n, u32 j) {
+    T r; zero_of(r);
+    #pragma unroll 1
+    for (u32 ty = 0; ty < (u32)TY; ++ty) {
+        T a0, a1, a2, a3; zero_of(a0); zero_of(a1); zero_of(a2); zero_of(a3);
+        u32 l = ty;
+        for (; l + 3u * TY < rows; l += 4u * TY) {
+            const T t0 = ld_at(g, (u64)l * n, j, T()), t1 = ld_at(g, (u64)(l + TY) * n, j, T());
+            const T t2 = ld_at(g, (u64)(l + 2u * TY) * n, j, T()), t3 = ld_at(g, (u64)(l + 3u * TY) * n, j, T());
+            a0 = add2(a0, t0); a1 = add2(a1, t1); a2 = add2(a2, t2); a3 = add2(a3, t3);
+        }
+        for (; l < rows; l += TY) a0 = add2(a0, ld_at(g, (u64)l * n, j, T()));
+        a0 = add2(a0, a1); a2 = add2(a2, a3); a0 = add2(a0, a2);
+        r = ty == 0u ? a0 : add2(r, a0);
+    }
+    return r;
+}
+template <typename T> static __device__ __forceinline__ T grad_at(const float* __restrict__ g, u32 rows, u32 n, u32 j) {
+    if (rows == 1u) return ld_at(g, 0, j, T());
+    return rows > 64u ? colsum<16, T>(g, rows, n, j) : colsum<4, T>(g, rows, n, j);
+}
+"""
+    src2 = f"""{head}{colsum}extern "C" __global__ __launch_bounds__(256) void {name}(const u64* __restrict__ ptrs,
         const u32* __restrict__ sizes, const u32* __restrict__ first, const u32* __restrict__ owner,
-        u32 n_tensors, const AdamArgs* __restrict__ ap) {{
+        const u32* __restrict__ rows_of, u32 n_tensors, const AdamArgs* __restrict__ ap) {{
     const AdamArgs a = *ap;
     const u32 t = owner[blockIdx.x];
     const u32 lb = blockIdx.x - first[t];
@@ -2384,10 +2424,14 @@ def adam_multi_inplace_kernel() -> tuple[str, str, str]:
     const float* __restrict__ g = reinterpret_cast<const float*>(ptrs[n_tensors + t]);
     float* m = reinterpret_cast<float*>(ptrs[2u * n_tensors + t]);
     float* v = reinterpret_cast<float*>(ptrs[3u * n_tensors + t]);
-    const u32 n = sizes[t], nv = n >> 2;
+    const u32 n = sizes[t], nv = n >> 2, rows = rows_of[t];
     const u32 i = lb * 256u + threadIdx.x;
     if (i < nv) {{
-        const float4 p4 = reinterpret_cast<float4*>(p)[i], g4 = reinterpret_cast<const float4*>(g)[i];
+        float4 g4;
+        if ((n & 3u) == 0u) g4 = grad_at<float4>(g, rows, n, i);          // every row starts 16-byte aligned
+        else {{ g4.x = grad_at<float>(g, rows, n, 4u * i); g4.y = grad_at<float>(g, rows, n, 4u * i + 1u);
+               g4.z = grad_at<float>(g, rows, n, 4u * i + 2u); g4.w = grad_at<float>(g, rows, n, 4u * i + 3u); }}
+        const float4 p4 = reinterpret_cast<float4*>(p)[i];
         const float4 m4 = reinterpret_cast<float4*>(m)[i], v4 = reinterpret_cast<float4*>(v)[i];
         float4 po, mo, vo;
         adam1(p4.x, g4.x, m4.x, v4.x, a, po.x, mo.x, vo.x);
@@ -2401,12 +2445,12 @@ def adam_multi_inplace_kernel() -> tuple[str, str, str]:
     if (lb == 0 && threadIdx.x < (n & 3u)) {{
         const u32 j = (nv << 2) + threadIdx.x;
         float po, mo, vo;
-        adam1(p[j], g[j], m[j], v[j], a, po, mo, vo);
+        adam1(p[j], grad_at<float>(g, rows, n, j), m[j], v[j], a, po, mo, vo);
         p[j] = po; m[j] = mo; v[j] = vo;
     }}
 }}
 """
-    return src2, name, _fmt("P", "P", "P", "P", "I", "P")
+    return src2, name, _fmt("P", "P", "P", "P", "P", "I", "P")
 
 
 @cache

@@ -12,7 +12,7 @@ from __future__ import annotations
 
 import os
 
-from dlgrad_amd.buffer import Buffer
+from dlgrad_amd.buffer import Buffer, PartialSum
 from dlgrad_amd.device import Device
 from dlgrad_amd.dtype import Scalar
 from dlgrad_amd.helpers import STRICT_REFERENCE, CustomOps, broadcast_shapes, check_broadcast
@@ -293,7 +293,11 @@ class Div(_Binary):
 
 
 def unbroadcast(grad: Buffer, original_shape: tuple) -> Buffer:
-    """Sum a matmul gradient back to an operand that was batch-broadcast (ops.py:287-295)."""
+    """Sum a matmul gradient back to an operand that was batch-broadcast (ops.py:287-295).  On the
+    hip device the sum over one leading batch dim is left pending (buffer.PartialSum): the one-launch
+    optimizer adds the batch entries up as it reads the gradient, any other reader runs the sum."""
+    if FUSED and grad.ndim == len(original_shape) + 1 and grad.shape[1:] == tuple(original_shape):
+        return PartialSum.of(grad, tuple(original_shape))
     while grad.ndim > len(original_shape):
         grad = grad.sum(0, keepdim=False)
     for i, (g, o) in enumerate(zip(grad.shape, original_shape)):

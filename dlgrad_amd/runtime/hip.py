@@ -1277,8 +1277,10 @@ class HIP:
     @staticmethod
     @dispatcher.register(CustomOps.RMSNORM_BWD, Device.HIP)
     def rmsnorm_bwd(x: Buffer, w: Buffer | None, r: Buffer, dy: Buffer,
-                    through_mean: bool, plus: Buffer | None = None) -> tuple[DevicePtr, DevicePtr | None]:
-        """plus: an array shaped like x that is added to dx as it is stored (a gradient that reached x by another route)."""
+                    through_mean: bool, plus: Buffer | None = None, partial_dw: bool = False) -> tuple:
+        """plus: an array shaped like x that is added to dx as it is stored (a gradient that reached x by another route).
+        partial_dw: where one column-sum launch would finish dw, hand back (partial rows, their count) instead of
+        running it, so that the caller can leave the sum pending."""
         L = x.shape[-1]
         R = x.numel // L
         if dy.numel != x.numel or r.numel != R:
@@ -1302,6 +1304,8 @@ class HIP:
                part.addr if part is not None else 0, R, L, rows_per_wave, *([_addr(plus)] if plus is not None else []))
         if w is None:
             return dx, None
+        if partial_dw and 1 < P <= 512:
+            return dx, (part, P)
         dw = alloc(L)
         HIP._reduce_cols("sum", part.addr, 1, P, L, 1.0, dw.addr)
         return dx, dw
@@ -1341,18 +1345,31 @@ class HIP:
         """tensors: (p, g, m, v) Buffers per parameter.  `table` is what the previous call
         returned: the device-side address table is rewritten (a host-to-device upload) only when
         some address differs from it.  A table written for a captured step is never touched
-        again (the caller keeps it alive as long as the graph); later eager steps get their own."""
-        addrs = tuple(_addr(b) for quad in tensors for b in quad)
+        again (the caller keeps it alive as long as the graph); later eager steps get their own.
+        A gradient that is a pending sum (buffer.PartialSum) is taken as its parts: the kernel adds
+        them up as it reads, in the order of the column-sum launch that would otherwise have run."""
+        from dlgrad_amd.buffer import PartialSum
+        rows_of = []                                     # per tensor: how many rows of its size the gradient pointer holds
+        addrs = []
+        for pb, gb, mb, vb in tensors:
+            if gb.__class__ is PartialSum and gb.pending:
+                g_addr, rows = gb.parts.ptr.addr, gb.parts.shape[0]
+            else:
+                g_addr, rows = gb.ptr.addr, 1
+            rows_of.append(rows)
+            addrs += [pb.ptr.addr, g_addr, mb.ptr.addr, vb.ptr.addr]
+        addrs = tuple(addrs)
         if any(a & 15 for a in addrs):
             raise ValueError("adam_multi_inplace needs 16-byte aligned tensors")
-        if table is None or table["addrs"] != addrs:
+        key = (addrs, tuple(rows_of))
+        if table is None or table["key"] != key:
             nt = len(tensors)
             sizes = np.array([q[0].numel for q in tensors], dtype=np.uint32)
             nblk = np.maximum(1, (sizes.astype(np.int64) // 4 + 255) // 256)
             first = np.concatenate([[0], np.cumsum(nblk)[:-1]]).astype(np.uint32)
             owner = np.repeat(np.arange(nt, dtype=np.uint32), nblk)
-            ptrs = np.array([[_addr(q[k]) for q in tensors] for k in range(4)], dtype=np.uint64).reshape(-1)
-            arrays = [np.ascontiguousarray(a).view(np.float32) for a in (ptrs, sizes, first, owner)]     # raw bits
+            ptrs = np.array(addrs, dtype=np.uint64).reshape(nt, 4).T.reshape(-1)        # four rows: p, g, m, v
+            arrays = [np.ascontiguousarray(a).view(np.float32) for a in (ptrs, sizes, first, owner, np.array(rows_of, dtype=np.uint32))]     # raw bits
             reuse = (table is not None and not table["frozen"]
                      and [a.size for a in arrays] == [b.nbytes // 4 for b in table["bufs"]])
             bufs = table["bufs"] if reuse else [alloc(a.size) for a in arrays]
@@ -1367,10 +1384,10 @@ class HIP:
                 _after_capture.append(upload)
             else:
                 upload()
-            table = {"addrs": addrs, "grid": int(nblk.sum()), "nt": nt, "bufs": bufs, "frozen": capturing()}
+            table = {"key": key, "grid": int(nblk.sum()), "nt": nt, "bufs": bufs, "frozen": capturing()}
         if table["nt"]:
             b = table["bufs"]
-            launch(kernel(K.adam_multi_inplace_kernel), table["grid"], 256, b[0].addr, b[1].addr, b[2].addr, b[3].addr,
+            launch(kernel(K.adam_multi_inplace_kernel), table["grid"], 256, b[0].addr, b[1].addr, b[2].addr, b[3].addr, b[4].addr,
                    table["nt"], _addr(consts))
         return table
 

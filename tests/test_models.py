@@ -586,3 +586,50 @@ def test_gpt_training_trajectory_hip_vs_cpu_oracle():
     assert cpu[-1] < cpu[0]                                   # it trains
     rel = np.abs(dev_ - cpu) / np.abs(cpu)
     assert rel.max() <= 1e-4, f"loss trajectories part: {rel}"
+
+
+@pytest.mark.gpu
+def test_adam_adds_up_pending_gradient_sums_with_the_bits_of_the_column_sum_launch():
+    """A gradient left as a pending sum over a leading dim (the batch entries of a weight gradient, the
+    partial rows of an RMSNorm gain) goes to the one-launch Adam as its parts.  The update must equal,
+    bit for bit, the update from the gradient that the column-sum launch produces -- for row counts on
+    both sides of the kernel's 4- and 16-row forms, sizes with an n % 4 tail, and plain gradients in
+    the same list -- and reading such a gradient any other way must still give that sum."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    from dlgrad_amd.buffer import Buffer, PartialSum
+    from dlgrad_amd.device import Device
+    cases = [((65, 128), 16), ((128,), 512), ((7,), 2), ((513, 3), 8), ((33, 20), 64), ((40, 25), 65), ((1024, 96), 200), ((6, 6), 1), ((129,), 3)]
+    rng = np.random.default_rng(21)
+    values = [rng.standard_normal(shape).astype(np.float32) for shape, _ in cases]
+    parts = [rng.standard_normal((rows, *shape)).astype(np.float32) for shape, rows in cases]
+    results = {}
+    for pending in (True, False):
+        ps = [Tensor(v, requires_grad=True, device="hip") for v in values]
+        opt = nn.optim.Adam(ps, lr=1e-2, graph_safe=True)
+        n0 = hip.launch_count
+        for step in range(2):
+            for p, part, (shape, rows) in zip(ps, parts, cases):
+                b = Buffer.from_numpy(part * np.float32(step + 1), Device.HIP)
+                if rows == 1:
+                    g = b.reshape(shape)
+                elif pending:
+                    g = PartialSum.of(b, shape)
+                    assert g.__class__ is PartialSum and g.pending
+                else:
+                    g = b.sum(0)
+                p.grad = Tensor(g, device="hip")
+            opt.step()
+            if pending and not hip.COMPILE_ONLY:
+                assert all(p.grad.data.pending for p, (_, rows) in zip(ps, cases) if rows > 1), "the optimizer ran the sums"
+        if pending:
+            assert hip.launch_count - n0 == 2 * 2                  # per step: the constants, the update -- no column sums
+            for p, part, (shape, rows) in zip(ps, parts, cases):   # any other reader gets the sum the launch gives
+                if rows > 1 and not hip.COMPILE_ONLY:
+                    want = Buffer.from_numpy(part * np.float32(2), Device.HIP).sum(0).numpy()
+                    np.testing.assert_array_equal(p.grad.numpy(), want.reshape(shape))
+                    assert not p.grad.data.pending
+        results[pending] = [p.numpy() for p in ps] + [opt.m[id(p)].numpy() for p in ps] + [opt.v[id(p)].numpy() for p in ps]
+    if not hip.COMPILE_ONLY:
+        for a, b in zip(results[True], results[False]):
+            np.testing.assert_array_equal(a, b)
