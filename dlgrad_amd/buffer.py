@@ -377,9 +377,9 @@ class Buffer:
         return self._like(y), self._like(p, (B, n_head, T, T))
 
     def causal_attention_bwd(self, k: "Buffer", v: "Buffer", p: "Buffer", dy: "Buffer", n_head: int,
-                             scale: float) -> tuple["Buffer", "Buffer", "Buffer"]:
-        """Gradients of causal_attention for q = self, k, v, each (B, T, C)."""
-        dq, dk, dv = self._dispatch(CustomOps.CAUSAL_ATTENTION_BWD, q=self, k=k, v=v, p=p, dy=dy, n_head=n_head, scale=scale)
+                             scale: float, y: "Buffer | None" = None) -> tuple["Buffer", "Buffer", "Buffer"]:
+        """Gradients of causal_attention for q = self, k, v, each (B, T, C); y: its context, if kept."""
+        dq, dk, dv = self._dispatch(CustomOps.CAUSAL_ATTENTION_BWD, q=self, k=k, v=v, p=p, dy=dy, n_head=n_head, scale=scale, y=y)
         return self._like(dq), self._like(dk), self._like(dv)
 
     def causal_attention_qkv(self, n_head: int, scale: float) -> tuple["Buffer", "Buffer"]:
@@ -389,9 +389,9 @@ class Buffer:
         y, p = self._dispatch(CustomOps.CAUSAL_ATTENTION_QKV, qkv=self, n_head=n_head, scale=scale)
         return self._like(y, (B, T, C3 // 3)), self._like(p, (B, n_head, T, T))
 
-    def causal_attention_qkv_bwd(self, p: "Buffer", dy: "Buffer", n_head: int, scale: float) -> "Buffer":
+    def causal_attention_qkv_bwd(self, p: "Buffer", dy: "Buffer", n_head: int, scale: float, y: "Buffer | None" = None) -> "Buffer":
         """Gradient of causal_attention_qkv with respect to self, same (B, T, 3C) layout."""
-        return self._like(self._dispatch(CustomOps.CAUSAL_ATTENTION_QKV_BWD, qkv=self, p=p, dy=dy, n_head=n_head, scale=scale))
+        return self._like(self._dispatch(CustomOps.CAUSAL_ATTENTION_QKV_BWD, qkv=self, p=p, dy=dy, n_head=n_head, scale=scale, y=y))
 
     def cached_attention(self, k_store: "Buffer", v_store: "Buffer", n: int, n_head: int, scale: float,
                          hidden: "Buffer | None" = None) -> "Buffer":

@@ -937,7 +937,15 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
 EMB_SEGMENT = 512          # positions whose indices one round of the ordered scatter-add compares (eight ballots of 64)
 EMB_ORDERED_MAX = 32768    # longest index list the ordered scatter-add takes: every position scans the whole list
 
-_ORDERED_COMMON = f"""
+WAVE_LDS_FENCE = r"""
+// Values written to LDS by some lanes of a wavefront and read by others of the same wavefront
+static __device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+"""
+
+_ORDERED_COMMON = WAVE_LDS_FENCE + f"""
 #define EMB_SEG {EMB_SEGMENT}u
 #define EMB_NK {EMB_SEGMENT // 64}
 // Which positions of the segment [s0, s1) hold the id `my`: bit l of hit[k] stands for position
@@ -959,11 +967,6 @@ static __device__ __forceinline__ void hit_rank(const u64 (&hit)[EMB_NK], u32 li
         if (64u * k + 64u <= li) below += (u32)__popcll(hit[k]);
         else if (64u * k <= li) below += (u32)__popcll(hit[k] & ((1ull << (li - 64u * k)) - 1ull));
     }}
-}}
-// Lists written by some lanes of a wavefront and read by others of the same wavefront
-static __device__ __forceinline__ void wave_lds_fence() {{
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
 }}
 """
 
@@ -2363,6 +2366,251 @@ extern "C" __global__ __launch_bounds__(64) void {name}(const float* __restrict_
 # =====================================================================================
 # optimizer
 # =====================================================================================
+
+ATTN_SMALL_T = 128         # longest sequence, and
+ATTN_SMALL_D = 32          # widest head, that the one-launch attention kernels hold in LDS
+
+
+@cache
+def attention_small_kernel(stage: str) -> tuple[str, str, str]:
+    """Causal self-attention with the scores never leaving the chip (examples/gpt.py:50-55 run it as
+    product, scale, mask, softmax, product; here for T <= 128 and a head width d <= 32 with
+    d % 4 == 0, the char-GPT shapes): one launch forward, one backward.
+
+    The heads are read where they lie inside (B, T, pitch) tensors -- row pitch `pitch`, batch stride
+    T * pitch, head stride d -- zero-padded in LDS (row pitch 33).  The T x T score matrix of a head
+    is cut into 32 x 32 tiles; only the tiles (ti, tj <= ti) on or below the diagonal are ever
+    computed, the others are exact zeros.  One block of 8 wavefronts per (sequence, head, tile row
+    i); grid = B * n_head * ceil(T / 32).  All products are 32 x 32 x 32 tile products on
+    v_mfma_f32_32x32x2_f32 (lane l feeds A[l % 32][l / 32] and B[l / 32][l % 32] of a step; accumulator
+    e of a lane is row 8 (e / 4) + 4 (l / 32) + e % 4, column l % 32), one wavefront per tile; partial
+    tiles of one output are handed over through LDS and added in ascending tile order.
+
+      "fwd"  block i: S(i, j) = q_i k_j^T * scale for j <= i, -inf above the diagonal -> LDS; row
+             softmax, a wavefront per row (max, exp once, sum, divide); the probabilities go to
+             p (B, n_head, T, T), zeros above the diagonal, for the backward pass; y_i = sum_j P(i, j) v_j
+             goes to the (B, T, y_pitch) context in place.
+      "bwd"  block i owns dq_i, dk_i and dv_i, so it needs dS(i, j <= i) and dS(t >= i, i): four tiles at
+             most, a wavefront each.  delta = rowsum(dy * y) (equal to rowsum(dP * P), since y = P v);
+             per tile dP = dy v^T and dS = P * (dP - delta) * scale; dq_i = sum_j dS(i, j) k_j;
+             dk_i = sum_t dS(t, i)^T q_t; dv_i = sum_t P(t, i)^T dy_t (four more wavefronts, P read
+             from memory in operand layout).  The gradients go into (B, T, g_pitch) tensors in place.
+    Same mathematics as the chain of kernels, other order of additions inside the dot products."""
+    assert stage in ("fwd", "bwd")
+    name = f"attention_small_{stage}"
+    common = r"""
+typedef float f16v __attribute__((ext_vector_type(16)));
+#define DP 33u                       /* LDS row pitch of the operand tiles (32 columns) */
+#define SP 129u                      /* LDS row pitch of a tile row of scores (128 columns) */
+#define TILE (32u * DP)
+#define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0)
+#define ZERO16(a) { _Pragma("unroll") for (int z_ = 0; z_ < 16; ++z_) a[z_] = 0.0f; }
+// item `it` of a head's rows [row0, row0 + ..): row row0 + it / 8, columns 4 (it % 8) ..; zeros outside [0, T) x [0, d)
+static __device__ __forceinline__ float4 head_part(const float* __restrict__ src, u32 it, u32 row0, u32 T, u32 d, u32 pitch) {
+    const u32 row = row0 + (it >> 3), c4 = (it & 7u) << 2;
+    return (row < T && c4 < d) ? *reinterpret_cast<const float4*>(src + (u64)row * pitch + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
+}
+static __device__ __forceinline__ void put_part(float* __restrict__ dst, u32 it, const float4 v) {     // dst: LDS row of item 0
+    float* q = dst + (it >> 3) * DP + ((it & 7u) << 2);
+    q[0] = v.x; q[1] = v.y; q[2] = v.z; q[3] = v.w;
+}
+// acc += A B over 32 steps of k with A[m][k] = a[m * am + k * ak] and B[k][n] = b[k * bk + n * bn]; operands fetched first
+static __device__ __forceinline__ void tile_product(f16v& acc, const float* __restrict__ a, u32 am, u32 ak,
+                                                    const float* __restrict__ b, u32 bk, u32 bn, u32 r, u32 h) {
+    float av[16], bv[16];
+    #pragma unroll
+    for (u32 s = 0; s < 16u; ++s) { av[s] = a[r * am + (2u * s + h) * ak]; bv[s] = b[(2u * s + h) * bk + r * bn]; }
+    #pragma unroll
+    for (u32 s = 0; s < 16u; ++s) acc = MFMA(av[s], bv[s], acc);
+}
+// partial tiles change hands as [slot][e][lane]
+static __device__ __forceinline__ void put_partial(float* __restrict__ box, u32 slot, const f16v& acc, u32 lane) {
+    #pragma unroll
+    for (u32 e = 0; e < 16u; ++e) box[(slot * 16u + e) * 64u + lane] = acc[e];
+}
+// accumulator entries 4 g .. 4 g + 3 (rows row0 + 8 g + 4 h ..) of the sum of slots [s0, s1) -> a head in global memory
+static __device__ __forceinline__ void sum_and_store(float* __restrict__ dst, const float* __restrict__ box, u32 s0, u32 s1,
+                                                     u32 g, u32 row0, u32 T, u32 d, u32 pitch, u32 lane) {
+    const u32 r = lane & 31u, h = lane >> 5;
+    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (u32 sl = s0; sl < s1; ++sl) {
+        #pragma unroll
+        for (u32 c = 0; c < 4u; ++c) v[c] += box[(sl * 16u + 4u * g + c) * 64u + lane];
+    }
+    #pragma unroll
+    for (u32 c = 0; c < 4u; ++c) {
+        const u32 row = row0 + 8u * g + 4u * h + c;
+        if (row < T && r < d) dst[(u64)row * pitch + r] = v[c];
+    }
+}
+"""
+    if stage == "fwd":
+        body = r"""
+extern "C" __global__ __launch_bounds__(512) void attention_small_fwd(const float* __restrict__ q,
+        const float* __restrict__ k, const float* __restrict__ v, float* __restrict__ y, float* __restrict__ p,
+        u32 T, u32 d, u32 pitch, u32 y_pitch, u32 n_head, u32 nt, float scale) {
+    __shared__ float Qs[TILE], Ks[4u * TILE], Vs[4u * TILE], Ss[32u * SP], box[4u * 1024u];
+    const u32 bh = blockIdx.x / nt, i = blockIdx.x % nt, b = bh / n_head, hd = bh % n_head;
+    const u32 t = threadIdx.x, w = t >> 6, lane = t & 63u, r = lane & 31u, h = lane >> 5;
+    const u64 in_off = (u64)b * T * pitch + (u64)hd * d;
+    {
+        const u32 n_kv = 256u * (i + 1u);                   // 16-byte items of the key and value rows this tile row sees
+        const float4 q4 = t < 256u ? head_part(q + in_off, t, 32u * i, T, d, pitch) : make_float4(0.f, 0.f, 0.f, 0.f);
+        float4 k4[2], v4[2];
+        #pragma unroll
+        for (u32 n = 0; n < 2u; ++n)
+            if (t + 512u * n < n_kv) { k4[n] = head_part(k + in_off, t + 512u * n, 0u, T, d, pitch); v4[n] = head_part(v + in_off, t + 512u * n, 0u, T, d, pitch); }
+        if (t < 256u) put_part(Qs, t, q4);
+        #pragma unroll
+        for (u32 n = 0; n < 2u; ++n)
+            if (t + 512u * n < n_kv) { put_part(Ks, t + 512u * n, k4[n]); put_part(Vs, t + 512u * n, v4[n]); }
+    }
+    __syncthreads();
+    if (w <= i) {                                           // S(i, w) = q_i k_w^T
+        f16v acc; ZERO16(acc)
+        tile_product(acc, Qs, DP, 1u, Ks + w * TILE, 1u, DP, r, h);
+        #pragma unroll
+        for (u32 e = 0; e < 16u; ++e) {
+            const u32 lr = 8u * (e >> 2) + 4u * h + (e & 3u), col = 32u * w + r;
+            Ss[lr * SP + col] = col > 32u * i + lr ? -__builtin_inff() : acc[e] * scale;
+        }
+    }
+    __syncthreads();
+    {   // softmax: wavefront w takes rows w, w + 8, .. of the tile row; a lane holds columns lane and lane + 64 of each.
+        // Columns 0 .. row are live, the rest of the row is 0
+        float* __restrict__ pout = p + (u64)bh * T * T;
+        const bool wide = i >= 2u;                          // the rows reach beyond column 63
+        float x0[4], x1[4], m[4], sum[4];
+        #pragma unroll
+        for (u32 c = 0; c < 4u; ++c) {
+            const u32 lr = w + 8u * c, row = 32u * i + lr;
+            x0[c] = lane <= row ? Ss[lr * SP + lane] : -__builtin_inff();
+            x1[c] = (wide && lane + 64u <= row) ? Ss[lr * SP + lane + 64u] : -__builtin_inff();
+        }
+        #pragma unroll
+        for (u32 c = 0; c < 4u; ++c) m[c] = wave_max(fmaxf(fmaxf(x0[c], x1[c]), NEG_FLT_MAX));
+        #pragma unroll
+        for (u32 c = 0; c < 4u; ++c) {
+            const u32 row = 32u * i + w + 8u * c;
+            x0[c] = lane <= row ? expf(x0[c] - m[c]) : 0.0f;
+            x1[c] = (wide && lane + 64u <= row) ? expf(x1[c] - m[c]) : 0.0f;
+        }
+        #pragma unroll
+        for (u32 c = 0; c < 4u; ++c) sum[c] = wave_sum(x0[c] + x1[c]);
+        #pragma unroll
+        for (u32 c = 0; c < 4u; ++c) {
+            const u32 lr = w + 8u * c, row = 32u * i + lr;
+            if (row < T) {
+                const float p0 = x0[c] / sum[c], p1 = x1[c] / sum[c];
+                Ss[lr * SP + lane] = p0;
+                if (wide) Ss[lr * SP + lane + 64u] = p1;
+                if (lane < T) pout[row * T + lane] = p0;
+                if (lane + 64u < T) pout[row * T + lane + 64u] = p1;
+            }
+        }
+    }
+    __syncthreads();
+    if (w <= i) {                                           // the part of y_i that comes from the keys of tile w
+        f16v acc; ZERO16(acc)
+        tile_product(acc, Ss + 32u * w, SP, 1u, Vs + w * TILE, DP, 1u, r, h);
+        put_partial(box, w, acc, lane);
+    }
+    __syncthreads();
+    if (w < 4u) sum_and_store(y + (u64)b * T * y_pitch + (u64)hd * d, box, 0u, i + 1u, w, 32u * i, T, d, y_pitch, lane);
+}
+"""
+        fmt = _fmt("P", "P", "P", "P", "P", "I", "I", "I", "I", "I", "I", "f")
+    else:
+        body = r"""
+extern "C" __global__ __launch_bounds__(512) void attention_small_bwd(const float* __restrict__ q,
+        const float* __restrict__ k, const float* __restrict__ v, const float* __restrict__ p, const float* __restrict__ y,
+        const float* __restrict__ dy, float* __restrict__ dq, float* __restrict__ dk, float* __restrict__ dv,
+        u32 T, u32 d, u32 pitch, u32 y_pitch, u32 g_pitch, u32 n_head, u32 nt, float scale) {
+    __shared__ float Qs[4u * TILE], Ks[4u * TILE], Vs[4u * TILE], Gs[4u * TILE], dSs[4u * TILE], box[12u * 1024u], delta[128];
+    const u32 bh = blockIdx.x / nt, i = blockIdx.x % nt, b = bh / n_head, hd = bh % n_head;
+    const u32 t = threadIdx.x, w = t >> 6, lane = t & 63u, r = lane & 31u, h = lane >> 5;
+    const u64 in_off = (u64)b * T * pitch + (u64)hd * d, y_off = (u64)b * T * y_pitch + (u64)hd * d;
+    const u64 g_off = (u64)b * T * g_pitch + (u64)hd * d;
+    const float* __restrict__ pin = p + (u64)bh * T * T;
+    {   // q, dy (and delta) for rows from tile i on; k, v for rows up to tile i
+        const u32 n_lo = 256u * (i + 1u), n_hi = 256u * (nt - i);
+        float4 q4[2], g4[2], y4[2], k4[2], v4[2];
+        #pragma unroll
+        for (u32 n = 0; n < 2u; ++n) {
+            const u32 it = t + 512u * n;
+            if (it < n_hi) {
+                q4[n] = head_part(q + in_off, it, 32u * i, T, d, pitch);
+                g4[n] = head_part(dy + y_off, it, 32u * i, T, d, y_pitch);
+                y4[n] = head_part(y + y_off, it, 32u * i, T, d, y_pitch);
+            }
+            if (it < n_lo) { k4[n] = head_part(k + in_off, it, 0u, T, d, pitch); v4[n] = head_part(v + in_off, it, 0u, T, d, pitch); }
+        }
+        #pragma unroll
+        for (u32 n = 0; n < 2u; ++n) {
+            const u32 it = t + 512u * n;
+            if (it < n_hi) {
+                put_part(Qs + i * TILE, it, q4[n]); put_part(Gs + i * TILE, it, g4[n]);
+                float part = (g4[n].x * y4[n].x + g4[n].y * y4[n].y) + (g4[n].z * y4[n].z + g4[n].w * y4[n].w);
+                part += dpp_f<DPP_XOR1>(part); part += dpp_f<DPP_XOR2>(part); part += dpp_f<DPP_HALF_MIRROR>(part);   // the row's 8 threads
+                if ((it & 7u) == 0u) delta[32u * i + (it >> 3)] = part;
+            }
+            if (it < n_lo) { put_part(Ks, it, k4[n]); put_part(Vs, it, v4[n]); }
+        }
+    }
+    __syncthreads();
+    // wavefronts c and 4 + c share score tile (ti, tj): (i, c) for c <= i, (c, i) below it
+    const u32 c = w & 3u, ti = c <= i ? i : c, tj = c <= i ? c : i;
+    const bool live = ti < nt, column = tj == i;           // column: the tile feeds dk_i and dv_i (the diagonal tile does both)
+    if (live && w < 4u) {
+        f16v ds; ZERO16(ds)
+        tile_product(ds, Gs + ti * TILE, DP, 1u, Vs + tj * TILE, 1u, DP, r, h);               // dP = dy_ti v_tj^T
+        #pragma unroll
+        for (u32 e = 0; e < 16u; ++e) {
+            const u32 lr = 8u * (e >> 2) + 4u * h + (e & 3u), row = 32u * ti + lr, col = 32u * tj + r;
+            const float pe = (row < T && col <= row) ? pin[row * T + col] : 0.0f;
+            dSs[c * TILE + lr * DP + r] = (pe * (ds[e] - delta[row])) * scale;
+        }
+        wave_lds_fence();
+        f16v acc; ZERO16(acc)
+        if (ti == i) {                                      // dq_i, the part from the keys of tile tj
+            tile_product(acc, dSs + c * TILE, DP, 1u, Ks + tj * TILE, DP, 1u, r, h);
+            put_partial(box, tj, acc, lane);
+        } else {                                            // dk_i, the part from the queries of tile ti
+            tile_product(acc, dSs + c * TILE, 1u, DP, Qs + ti * TILE, DP, 1u, r, h);
+            put_partial(box, 4u + ti, acc, lane);
+        }
+    }
+    if (live && column && w >= 4u) {                        // dv_i, the part from the rows of tile ti: P(ti, i)^T dy_ti
+        f16v acc; ZERO16(acc)
+        float av[16], bv[16];
+        #pragma unroll
+        for (u32 s = 0; s < 16u; ++s) {
+            const u32 row = 32u * ti + 2u * s + h, col = 32u * tj + r;
+            av[s] = (row < T && col <= row) ? pin[row * T + col] : 0.0f;
+            bv[s] = Gs[ti * TILE + (2u * s + h) * DP + r];
+        }
+        #pragma unroll
+        for (u32 s = 0; s < 16u; ++s) acc = MFMA(av[s], bv[s], acc);
+        put_partial(box, 8u + ti, acc, lane);
+    }
+    __syncthreads();
+    if (w == 4u + i) {                                      // dk_i, the part from the diagonal tile, whose dS wavefront i wrote
+        f16v acc; ZERO16(acc)
+        tile_product(acc, dSs + i * TILE, 1u, DP, Qs + i * TILE, DP, 1u, r, h);
+        put_partial(box, 4u + i, acc, lane);
+    }
+    __syncthreads();
+    for (u32 job = w; job < 12u; job += 8u) {               // 3 outputs x 4 groups of accumulator entries
+        const u32 out = job >> 2, g = job & 3u;
+        if (out == 0u) sum_and_store(dq + g_off, box, 0u, i + 1u, g, 32u * i, T, d, g_pitch, lane);
+        else if (out == 1u) sum_and_store(dk + g_off, box, 4u + i, 4u + nt, g, 32u * i, T, d, g_pitch, lane);
+        else sum_and_store(dv + g_off, box, 8u + i, 8u + nt, g, 32u * i, T, d, g_pitch, lane);
+    }
+}
+"""
+        fmt = _fmt("P", "P", "P", "P", "P", "P", "P", "P", "P", "I", "I", "I", "I", "I", "I", "I", "f")
+    return f"{PRELUDE}{WAVE_LDS_FENCE}{common}{body}", name, fmt
+
 
 @cache
 def adam_multi_inplace_kernel() -> tuple[str, str, str]:

@@ -499,11 +499,11 @@ class CausalAttentionHeads(OP):
 
     def forward(self, q: Buffer, k: Buffer, v: Buffer, n_head: int, scale: float) -> Buffer:
         self.q, self.k, self.v, self.n_head, self.scale = q, k, v, n_head, scale
-        y, self.p = q.causal_attention(k, v, n_head, scale)
-        return y
+        self.y, self.p = q.causal_attention(k, v, n_head, scale)
+        return self.y
 
     def backward(self, upstream_grad: Buffer) -> tuple:
-        return self.q.causal_attention_bwd(self.k, self.v, self.p, upstream_grad, self.n_head, self.scale)
+        return self.q.causal_attention_bwd(self.k, self.v, self.p, upstream_grad, self.n_head, self.scale, self.y)
 
 
 def stacked(wq, wk, wv) -> bool:
@@ -539,12 +539,12 @@ class SelfAttentionQKV(OP):
         self.x, self.n_head, self.scale = x, n_head, scale
         self.w = Buffer(wq.ptr, (3 * C, C), x.device)                    # the three matrices as one
         self.qkv = x.matmul_nt(self.w)
-        y, self.p = self.qkv.causal_attention_qkv(n_head, scale)
-        return y
+        self.y, self.p = self.qkv.causal_attention_qkv(n_head, scale)
+        return self.y
 
     def backward(self, upstream_grad: Buffer) -> tuple:
         C = self.w.shape[1]
-        g = self.qkv.causal_attention_qkv_bwd(self.p, upstream_grad, self.n_head, self.scale)     # (B, T, 3C)
+        g = self.qkv.causal_attention_qkv_bwd(self.p, upstream_grad, self.n_head, self.scale, self.y)     # (B, T, 3C)
         dx = g @ self.w
         dw = unbroadcast(g.matmul_tn(self.x), self.w.shape)                                       # (3C, C)
         part = lambda i: Buffer(dw.ptr + i * C * C, (C, C), dw.device)                            # noqa: E731

@@ -1418,6 +1418,7 @@ class HIP:
 
     ROW_MATMUL = os.environ.get("DLGRAD_HIP_ROW_MATMUL", "1") != "0"        # "0": one-row products on the MFMA tiles too
     DECODE_FUSED = os.environ.get("DLGRAD_HIP_DECODE_FUSED", "1") != "0"    # "0": cached attention as product, softmax, product
+    ATTENTION_FUSED = os.environ.get("DLGRAD_HIP_ATTENTION_FUSED", "1") != "0"   # "0": short causal attention as products and softmax launches too
 
     # ---- matmul ----------------------------------------------------------------------------------------------------------
     MATMUL_FORCE = os.environ.get("DLGRAD_HIP_MATMUL_TILE")      # e.g. "128x128": benchmarking aid
@@ -1697,12 +1698,26 @@ class HIP:
         return (addr, C, T * C, d)
 
     @staticmethod
+    def _attention_fits(T: int, d: int, heads: int, read_addrs: tuple, read_pitches: tuple) -> bool:
+        """Whether the one-block-per-head attention kernels take the case: the head fits their LDS tiles
+        and every tensor they read with 16-byte loads is laid out for that."""
+        return (HIP.ATTENTION_FUSED and 0 < T <= K.ATTN_SMALL_T and 0 < d <= K.ATTN_SMALL_D and d % 4 == 0
+                and 0 < heads < 2 ** 29 and not any(a & 15 for a in read_addrs) and not any(q & 3 for q in read_pitches))
+
+    @staticmethod
     def _attend(qa: int, ka: int, va: int, pitch: int, ya: int, y_pitch: int, Bn: int, T: int, n_head: int, d: int,
                 scale: float) -> DevicePtr:
         """Causal attention over heads that lie at addresses qa, ka, va with row pitch `pitch` (batch
         stride T * pitch, head stride d); the context goes to ya with pitch y_pitch.  Returns the
         probabilities (Bn, n_head, T, T)."""
         from dlgrad_amd.ops import causal_mask
+        if HIP._attention_fits(T, d, Bn * n_head, (qa, ka, va), (pitch,)):
+            # one block per (sequence, head, 32 rows): scores, softmax and context without leaving the chip
+            p = alloc(Bn * n_head * T * T)
+            nt = (T + 31) // 32
+            launch(kernel(K.attention_small_kernel, "fwd"), Bn * n_head * nt, 512, qa, ka, va, ya, p.addr, T, d, pitch, y_pitch,
+                   n_head, nt, float(scale))
+            return p
         raw = alloc(Bn * n_head * T * T)
         dense = lambda addr: (addr, T, n_head * T * T, T * T)                       # noqa: E731
         HIP._gemm_strided(HIP._heads(qa, T, pitch, d), HIP._heads(ka, T, pitch, d), dense(raw.addr), T, T, d, Bn, n_head,
@@ -1714,9 +1729,15 @@ class HIP:
 
     @staticmethod
     def _attend_bwd(qa: int, ka: int, va: int, pitch: int, p: Buffer, dya: int, dy_pitch: int, dqa: int, dka: int,
-                    dva: int, g_pitch: int, Bn: int, T: int, n_head: int, d: int, scale: float) -> None:
-        """Gradients of _attend, written to dqa, dka, dva with row pitch g_pitch."""
+                    dva: int, g_pitch: int, Bn: int, T: int, n_head: int, d: int, scale: float, ya: int | None = None) -> None:
+        """Gradients of _attend, written to dqa, dka, dva with row pitch g_pitch.  ya: the context that
+        _attend wrote, laid out like dy, if the caller kept it (the one-launch kernel wants it)."""
         from dlgrad_amd.ops import causal_mask
+        if ya is not None and HIP._attention_fits(T, d, Bn * n_head, (qa, ka, va, dya, ya), (pitch, dy_pitch)):
+            nt = (T + 31) // 32
+            launch(kernel(K.attention_small_kernel, "bwd"), Bn * n_head * nt, 512, qa, ka, va, _addr(p), ya, dya, dqa, dka, dva,
+                   T, d, pitch, dy_pitch, g_pitch, n_head, nt, float(scale))
+            return
         dense = lambda addr: (addr, T, n_head * T * T, T * T)                       # noqa: E731
         dp = alloc(p.numel)
         HIP._gemm_strided(HIP._heads(dya, T, dy_pitch, d), HIP._heads(va, T, pitch, d), dense(dp.addr), T, T, d, Bn, n_head,
@@ -1744,14 +1765,15 @@ class HIP:
 
     @staticmethod
     @dispatcher.register(CustomOps.CAUSAL_ATTENTION_QKV_BWD, Device.HIP)
-    def causal_attention_qkv_bwd(qkv: Buffer, p: Buffer, dy: Buffer, n_head: int, scale: float) -> DevicePtr:
-        """Gradient of causal_attention_qkv with respect to qkv, in the same (B, T, 3C) layout."""
+    def causal_attention_qkv_bwd(qkv: Buffer, p: Buffer, dy: Buffer, n_head: int, scale: float, y: Buffer | None = None) -> DevicePtr:
+        """Gradient of causal_attention_qkv with respect to qkv, in the same (B, T, 3C) layout.  y: the
+        context of the forward pass, if kept."""
         Bn, T, C3 = qkv.shape
         C = C3 // 3
         a = _addr(qkv)
         g = alloc(Bn * T * C3)
         HIP._attend_bwd(a, a + 4 * C, a + 8 * C, C3, p, _addr(dy), C, g.addr, g.addr + 4 * C, g.addr + 8 * C, C3,
-                        Bn, T, n_head, C // n_head, scale)
+                        Bn, T, n_head, C // n_head, scale, None if y is None else _addr(y))
         return g
 
     @staticmethod
@@ -1814,10 +1836,10 @@ class HIP:
     @staticmethod
     @dispatcher.register(CustomOps.CAUSAL_ATTENTION_BWD, Device.HIP)
     def causal_attention_bwd(q: Buffer, k: Buffer, v: Buffer, p: Buffer, dy: Buffer, n_head: int,
-                             scale: float) -> tuple[DevicePtr, DevicePtr, DevicePtr]:
+                             scale: float, y: Buffer | None = None) -> tuple[DevicePtr, DevicePtr, DevicePtr]:
         """Gradients of causal_attention with respect to the (B, T, C) projections, written in that layout."""
         Bn, T, C = q.shape
         dq, dk, dv = alloc(Bn * T * C), alloc(Bn * T * C), alloc(Bn * T * C)
         HIP._attend_bwd(_addr(q), _addr(k), _addr(v), C, p, _addr(dy), C, dq.addr, dk.addr, dv.addr, C,
-                        Bn, T, n_head, C // n_head, scale)
+                        Bn, T, n_head, C // n_head, scale, None if y is None else _addr(y))
         return dq, dk, dv

@@ -264,6 +264,7 @@ def test_attention_on_the_projections_equals_split_attend_merge(B, T, h, d, monk
     transpose -> reshape, including head sizes that force 4-byte accesses."""
     require_gpu()
     from dlgrad_amd import nn, ops
+    monkeypatch.setattr(hip.HIP, "ATTENTION_FUSED", False)       # the one-launch kernels for short sequences add in another order
     rng = np.random.default_rng(72)
     C = h * d
     q, k, v, g = (rng.standard_normal((B, T, C), dtype=np.float32) for _ in range(4))
@@ -284,6 +285,91 @@ def test_attention_on_the_projections_equals_split_attend_merge(B, T, h, d, monk
     for name, a, b in zip(("y", "dq", "dk", "dv"), fused, chain):
         assert a.shape == (B, T, C)
         assert (a.view(np.uint32) == b.view(np.uint32)).all(), f"{name} B{B} T{T} h{h} d{d}"
+
+
+def attention_float64(q, k, v, g, h, scale):
+    """Causal attention on (B, T, h*d) projections and its gradients for upstream g, in float64."""
+    B, T, C = q.shape
+    d = C // h
+    q, k, v, g = (a.astype(np.float64).reshape(B, T, h, d).transpose(0, 2, 1, 3) for a in (q, k, v, g))
+    s = np.where(np.triu(np.ones((T, T), bool), 1), -np.inf, (q @ k.transpose(0, 1, 3, 2)) * scale)
+    e = np.exp(s - s.max(-1, keepdims=True))
+    p = e / e.sum(-1, keepdims=True)
+    y = p @ v
+    dv = p.transpose(0, 1, 3, 2) @ g
+    dp = g @ v.transpose(0, 1, 3, 2)
+    ds = p * (dp - (dp * p).sum(-1, keepdims=True)) * scale
+    dq, dk = ds @ k, ds.transpose(0, 1, 3, 2) @ q
+    return [a.transpose(0, 2, 1, 3).reshape(B, T, C) for a in (y, dq, dk, dv)]
+
+
+@pytest.mark.parametrize("B,T,h,d", [(2, 128, 4, 32), (64, 128, 4, 32), (3, 100, 2, 20), (1, 1, 1, 4), (2, 33, 3, 8), (5, 65, 2, 28),
+                                     (2, 31, 8, 4)])
+@pytest.mark.parametrize("stacked", [False, True])
+def test_short_attention_in_one_launch_per_pass(B, T, h, d, stacked, monkeypatch):
+    """Up to 128 positions and head widths up to 32 (multiples of 4): one block per (sequence, head)
+    holds q, k, v and the scores in LDS, so attention is one launch forward and one backward,
+    from separate (B, T, C) projections or from one interleaved (B, T, 3C) projection.  The dot
+    products add in another order than the chain of launches does, so the check is against
+    float64: 2e-6 of the largest entry for the context and each gradient; the probabilities
+    above the diagonal are exact zeros and nothing unwritten is read (free memory full of NaN)."""
+    require_gpu()
+    from dlgrad_amd import nn, ops
+    from dlgrad_amd.buffer import Buffer
+    from dlgrad_amd.device import Device
+    rng = np.random.default_rng(74)
+    C = h * d
+    q, k, v, g = (rng.standard_normal((B, T, C), dtype=np.float32) for _ in range(4))
+    scale = d ** -0.5
+    want = None if hip.COMPILE_ONLY else attention_float64(q, k, v, g, h, scale)
+    poison = [Buffer.from_numpy(np.full(n, np.nan, np.float32), Device.HIP) for n in (B * h * T * T, 3 * B * T * C, B * T * C)]
+    hip.lib().sync()
+    del poison
+
+    def run():
+        if stacked:
+            qkv = Buffer.from_numpy(np.ascontiguousarray(np.concatenate([q, k, v], axis=2)), Device.HIP)
+            before = hip.launch_count
+            y, p = qkv.causal_attention_qkv(h, scale)
+            dg = qkv.causal_attention_qkv_bwd(p, Buffer.from_numpy(g, Device.HIP), h, scale, y)
+            launches = hip.launch_count - before
+            if hip.COMPILE_ONLY:
+                return launches, None, None
+            dg = dg.numpy()
+            return launches, [y.numpy(), dg[:, :, :C], dg[:, :, C:2 * C], dg[:, :, 2 * C:]], p.numpy()
+        bufs = [Buffer.from_numpy(a, Device.HIP) for a in (q, k, v, g)]
+        before = hip.launch_count
+        y, p = bufs[0].causal_attention(bufs[1], bufs[2], h, scale)
+        grads = bufs[0].causal_attention_bwd(bufs[1], bufs[2], p, bufs[3], h, scale, y)
+        launches = hip.launch_count - before
+        if hip.COMPILE_ONLY:
+            return launches, None, None
+        return launches, [y.numpy()] + [a.numpy() for a in grads], p.numpy()
+
+    launches, got, p = run()
+    assert launches == 2, launches
+    monkeypatch.setattr(hip.HIP, "ATTENTION_FUSED", False)
+    chain_launches, chain, _ = run()
+    assert chain_launches > 2
+    if hip.COMPILE_ONLY:
+        return
+    assert p.shape == (B, h, T, T) and not np.triu(p, 1).any() and np.isfinite(p).all()
+    assert np.abs(p.sum(-1, dtype=np.float64) - 1).max() <= 1e-5
+    for name, a, w, c in zip(("y", "dq", "dk", "dv"), got, want, chain):
+        assert np.isfinite(a).all(), name
+        bound = 2e-6 * max(1.0, np.abs(w).max())
+        assert np.abs(a - w).max() <= bound, f"{name}: {np.abs(a - w).max():.3g} > {bound:.3g}"
+        assert np.abs(c - w).max() <= bound, f"chain {name}"
+
+
+def test_short_attention_leaves_other_shapes_to_the_chain_of_launches():
+    """Longer sequences, wider heads, head widths that are no multiple of 4 and operands that do not
+    sit on 16-byte boundaries do not fit the LDS tiles or the 16-byte loads of the one-block kernels."""
+    from dlgrad_amd.runtime.hip import HIP
+    fits = HIP._attention_fits
+    assert fits(128, 32, 256, (0, 16, 4096), (96,))
+    assert not fits(129, 32, 256, (0,), (96,)) and not fits(128, 36, 256, (0,), (108,)) and not fits(64, 6, 8, (0,), (12,))
+    assert not fits(64, 8, 8, (4,), (24,)) and not fits(64, 8, 8, (0,), (25,)) and not fits(64, 8, 0, (0,), (24,))
 
 
 @pytest.mark.parametrize("B,T,h,d", [(2, 128, 4, 32), (1, 1024, 12, 64), (3, 100, 2, 20), (2, 33, 3, 7)])

@@ -463,7 +463,7 @@ def test_captured_graph_replays_match_eager_steps_bit_for_bit():
     assert float(loss.numpy()) == eager[0][0]
     with g.capture():
         loss = step()                                    # recorded only
-    assert g.nodes > 60
+    assert g.nodes > 40
     scratch = Tensor(rng.standard_normal((257, 33)).astype(np.float32), device="hip")
     for k in range(1, n_steps):
         opt.advance()
