@@ -2562,13 +2562,18 @@ extern "C" __global__ __launch_bounds__(512) void attention_small_bwd(const floa
     const u32 c = w & 3u, ti = c <= i ? i : c, tj = c <= i ? c : i;
     const bool live = ti < nt, column = tj == i;           // column: the tile feeds dk_i and dv_i (the diagonal tile does both)
     if (live && w < 4u) {
+        float pe[16];                                       // the tile of P in accumulator layout, on its way while dP is computed
+        #pragma unroll
+        for (u32 e = 0; e < 16u; ++e) {
+            const u32 row = 32u * ti + 8u * (e >> 2) + 4u * h + (e & 3u), col = 32u * tj + r;
+            pe[e] = (row < T && col <= row) ? pin[row * T + col] : 0.0f;
+        }
         f16v ds; ZERO16(ds)
         tile_product(ds, Gs + ti * TILE, DP, 1u, Vs + tj * TILE, 1u, DP, r, h);               // dP = dy_ti v_tj^T
         #pragma unroll
         for (u32 e = 0; e < 16u; ++e) {
-            const u32 lr = 8u * (e >> 2) + 4u * h + (e & 3u), row = 32u * ti + lr, col = 32u * tj + r;
-            const float pe = (row < T && col <= row) ? pin[row * T + col] : 0.0f;
-            dSs[c * TILE + lr * DP + r] = (pe * (ds[e] - delta[row])) * scale;
+            const u32 lr = 8u * (e >> 2) + 4u * h + (e & 3u);
+            dSs[c * TILE + lr * DP + r] = (pe[e] * (ds[e] - delta[32u * ti + lr])) * scale;
         }
         wave_lds_fence();
         f16v acc; ZERO16(acc)
