@@ -1396,6 +1396,52 @@ extern "C" __global__ __launch_bounds__({threads}) void {name}(const float* __re
 
 
 @cache
+def ce_grad_rows_kernel(items: int, nt: bool, g_by_value: bool) -> tuple[str, str, str]:
+    """Gradient of the summed cross-entropy with respect to 2-D logits whose rows are multiples of
+    four floats: out = ((exp((x - max) - logsum) - onehot(target)) * g) / n -- the four kernels of
+    CrossEntropy.backward (ops.py:359-370) on a log-softmax rebuilt from the row statistics -- with a
+    block per (row, run of 1024 * items columns): the row's three values are read once per block,
+    no index is divided, and a thread has `items` 16-byte loads in flight before its first store.
+    The same fp32 operations in the same order as the element-wise form of the expression.
+    nt: streaming loads and stores (tensors beyond the caches)."""
+    assert items in (1, 2, 4)
+    name = f"ce_grad_rows_u{items}" + ("nt" if nt else "") + ("_v" if g_by_value else "_p")
+    ld = "ld4_stream(reinterpret_cast<const float4*>(xr + c))" if nt else "*reinterpret_cast<const float4*>(xr + c)"
+    st = ("{ const v4f ov = {o.x, o.y, o.z, o.w}; __builtin_nontemporal_store(ov, reinterpret_cast<v4f*>(orow + c)); }" if nt
+          else "*reinterpret_cast<float4*>(orow + c) = o;")
+    garg = "float g" if g_by_value else "const float* __restrict__ gp"
+    gval = "" if g_by_value else "    const float g = *gp;\n"
+    src = f"""{PRELUDE}
+#define ITEMS {items}u
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x, const float* __restrict__ row_max,
+        const float* __restrict__ row_logsum, const float* __restrict__ target, {garg}, float* __restrict__ out,
+        u32 C, u32 runs, float n) {{
+    const u32 row = blockIdx.x / runs, c0 = (blockIdx.x - row * runs) * (1024u * ITEMS) + 4u * threadIdx.x;
+    const float* __restrict__ xr = x + (u64)row * C;
+    float* __restrict__ orow = out + (u64)row * C;
+    float4 v[ITEMS];
+    #pragma unroll
+    for (u32 k = 0; k < ITEMS; ++k) {{ const u32 c = c0 + 1024u * k; if (c < C) v[k] = {ld}; }}
+    const float m = row_max[row], ls = row_logsum[row];
+    const u32 t = (u32)(int)target[row];
+{gval}    #pragma unroll
+    for (u32 k = 0; k < ITEMS; ++k) {{
+        const u32 c = c0 + 1024u * k;
+        if (c < C) {{
+            float4 o;
+            o.x = ((expf((v[k].x - m) - ls) - (c == t ? 1.0f : 0.0f)) * g) / n;
+            o.y = ((expf((v[k].y - m) - ls) - (c + 1u == t ? 1.0f : 0.0f)) * g) / n;
+            o.z = ((expf((v[k].z - m) - ls) - (c + 2u == t ? 1.0f : 0.0f)) * g) / n;
+            o.w = ((expf((v[k].w - m) - ls) - (c + 3u == t ? 1.0f : 0.0f)) * g) / n;
+            {st}
+        }}
+    }}
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "P", "f" if g_by_value else "P", "P", "I", "I", "f")
+
+
+@cache
 def ce_stats_kernel(vec: int, per_block: bool, nt: bool = False, negate: bool = False) -> tuple[str, str, str]:
     """The forward pass of the cross-entropy loss without its log-softmax tensor (ops.py:337-357
     composes max, sub, exp, sum, log, sub over the whole (N, V) logits and gathers one entry per

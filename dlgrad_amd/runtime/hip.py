@@ -19,6 +19,7 @@ from __future__ import annotations
 
 import hashlib
 import json
+import math
 import os
 import struct
 
@@ -1234,7 +1235,16 @@ class HIP:
         log-softmax entry is rebuilt from the row statistics ce_stats kept (the same two subtractions
         on the same values the stored tensor was made with), then the four kernels of
         CrossEntropy.backward (exp, in-place ce_backward, mul, div; ops.py:359-370) follow fused."""
-        R = x.shape[0]
+        R, C = x.shape
+        items = 1 if C <= 1024 else 2 if C <= 2048 else 4
+        runs = -(-C // (1024 * items))
+        if HIP.CE_GRAD_ROWS and C % 4 == 0 and not (_addr(x) & 15) and 0 < R * runs < 2 ** 31 and x.numel < 2 ** 31:
+            # a block per (row, run of columns): the row's statistics are read once per block and no index is divided
+            by_value = upstream.is_host_scalar
+            k = kernel(K.ce_grad_rows_kernel, items, x.numel >= NT_STORE_MIN_ELEMENTS, by_value)
+            g = float(upstream.ptr.value) if by_value else _addr(upstream)
+            return launch_out(k, R * runs, 256, field_offset(k[1].format, 5), x.numel, _addr(x), _addr(m), _addr(ls), _addr(target),
+                              g, 0, C, runs, float(n))
         rows = [Buffer(b.ptr, (R, 1), Device.HIP) for b in (m, ls, target)]
         one = R == 1                                     # a single row collapses to a flat run: the column is i itself
         col = "i" if one else "(i % C)"
@@ -1418,6 +1428,7 @@ class HIP:
 
     ROW_MATMUL = os.environ.get("DLGRAD_HIP_ROW_MATMUL", "1") != "0"        # "0": one-row products on the MFMA tiles too
     DECODE_FUSED = os.environ.get("DLGRAD_HIP_DECODE_FUSED", "1") != "0"    # "0": cached attention as product, softmax, product
+    CE_GRAD_ROWS = os.environ.get("DLGRAD_HIP_CE_GRAD_ROWS", "1") != "0"       # "0": the cross-entropy gradient as an element-wise launch
     ATTENTION_FUSED = os.environ.get("DLGRAD_HIP_ATTENTION_FUSED", "1") != "0"   # "0": short causal attention as products and softmax launches too
 
     # ---- matmul ----------------------------------------------------------------------------------------------------------

@@ -375,7 +375,7 @@ def test_cross_entropy_loss_and_gradient_single_rows_included(N, V, fused, monke
         assert (got_grad[np.arange(N), t] < 0).all() and (np.delete(got_grad[0], t[0]) > 0).all()
 
 
-@pytest.mark.parametrize("N,V", [(1, 64), (1, 65), (2048, 65), (64, 50304), (33, 4100), (7, 2048), (5, 100003)])
+@pytest.mark.parametrize("N,V", [(1, 64), (1, 65), (2048, 65), (64, 50304), (33, 4100), (7, 2048), (5, 100003), (9, 1028), (3, 44)])
 def test_ce_row_statistics_stand_in_for_the_stored_log_softmax(N, V):
     """The forward keeps (max, log-sum) per row instead of the (N, V) log-softmax.  The max is exact; the
     sum is added in one pass with a running maximum, so log-sum, picked log-probs and the gradient rebuilt
@@ -401,6 +401,15 @@ def test_ce_row_statistics_stand_in_for_the_stored_log_softmax(N, V):
         new, old = x.ce_grad_logits(m, ls, dt, up, float(N)).numpy(), lsm.ce_grad(dt, up, float(N)).numpy()
         assert np.abs(new - old).max() <= 2e-6 * np.abs(old).max()
         assert (new[0, :min(V, 40)] == 0).all()
+        # rows of whole 16-byte items take a kernel with a block per (row, run of columns): the same operations
+        # in the same order as the element-wise launch, so the same bits
+        rows_kernel = hip.HIP.CE_GRAD_ROWS
+        hip.HIP.CE_GRAD_ROWS = False
+        try:
+            flat = x.ce_grad_logits(m, ls, dt, up, float(N)).numpy()
+        finally:
+            hip.HIP.CE_GRAD_ROWS = rows_kernel
+        np.testing.assert_array_equal(new.view(np.uint32), flat.view(np.uint32))
 
 
 def test_indices_outside_their_table_touch_nothing():
