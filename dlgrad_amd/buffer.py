@@ -300,6 +300,36 @@ class Buffer:
         y = other if other.shape == p2 else other._like(other.ptr, p2)
         return self._like(self._dispatch(CustomOps.MATMUL_TN, x=x, y=y, **self._tri(tri)), out_shape)
 
+    @staticmethod
+    def _product_operands(kind: str, a: "Buffer", b: "Buffer") -> tuple:
+        """(x, y, ta, tb, out_shape) of a @ b ("nn"), a @ b^T ("nt") or a^T @ b ("tn") with the operands padded
+        to one rank, as matmul / matmul_nt / matmul_tn hand them to the runtime."""
+        sa = a.shape[:-2] + (a.shape[-1], a.shape[-2]) if kind == "tn" else a.shape
+        sb = b.shape[:-2] + (b.shape[-1], b.shape[-2]) if kind == "nt" else b.shape
+        p1, p2, out_shape = broadcast_shapes(sa, sb)
+        if kind == "tn":
+            p1 = p1[:-2] + (p1[-1], p1[-2])
+        if kind == "nt":
+            p2 = p2[:-2] + (p2[-1], p2[-2])
+        x = a if a.shape == p1 else a._like(a.ptr, p1)
+        y = b if b.shape == p2 else b._like(b.ptr, p2)
+        return x, y, kind == "tn", kind == "nt", out_shape
+
+    @staticmethod
+    def matmul_pair(first: tuple, second: tuple) -> tuple["Buffer", "Buffer"]:
+        """Two independent products as one launch on the hip device: each is (kind, a, b) or (kind, a, b,
+        epi, e) with kind "nn" (a @ b), "nt" (a @ b^T) or "tn" (a^T @ b) and the epilogues of matmul.
+        The results are those of the separate calls, bit for bit."""
+        specs, shapes = [], []
+        for kind, a, b, *rest in (first, second):
+            x, y, ta, tb, out_shape = Buffer._product_operands(kind, a, b)
+            epi, e = (rest + ["", None])[:2] if rest else ("", None)
+            specs.append((x, y, ta, tb, epi, e))
+            shapes.append(out_shape)
+        a0 = first[1]
+        p0, p1 = a0._dispatch(CustomOps.MATMUL_PAIR, first=specs[0], second=specs[1])
+        return a0._like(p0, shapes[0]), a0._like(p1, shapes[1])
+
     def permute(self, order: tuple) -> "Buffer":
         order = tuple(order)
         return self._like(self._dispatch(UnaryOps.PERMUTE, x=self, order=order),

@@ -2206,6 +2206,73 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
     return src, name, _fmt("P", "P", "P", "8I")
 
 
+@cache
+def matmul_pair_kernel(first: tuple, second: tuple) -> tuple[str, str, str]:
+    """Two independent products in one launch: the blocks of `first` followed by the blocks of `second`,
+    each given as the argument tuple of matmul_kernel (tile, access widths, transposed forms, epilogue).
+
+    The backward pass of a linear layer is such a pair -- dX = G W and dW = G^T X share G and nothing
+    else -- and each of them alone leaves most of the chip idle for the few microseconds a short k loop
+    takes; launched together they overlap.  The two bodies are the product kernels themselves, compiled as
+    device functions in namespaces of their own and called with the block index they would have had
+    (x = b % tiles, z = b / tiles), so every output element is computed by the same instructions in the
+    same order as in a launch of its own: same bits.  Both bodies stage their operands in one LDS
+    buffer sized for the larger; the block has the thread count of the larger body, and the wavefronts
+    the smaller one does not use leave at once (a barrier waits only for the wavefronts still running).
+    Arguments: those of the first product (A, B, C, its sizes and strides, E if it has an epilogue), those
+    of the second, then the number of blocks of the first and the tile counts per batch entry of both."""
+    import re
+    parts = []
+    for tag, a in (("p0", first), ("p1", second)):
+        WM, WN, MI, NJ, BK, veca, vecb, ta, tb, tri, strided, epi, S = a
+        assert not tri and not strided
+        src, name, fmt = matmul_kernel(WM, WN, MI, NJ, BK, veca, vecb, ta, tb, tri, strided, epi, S)
+        assert src.startswith(PRELUDE)
+        body = src[len(PRELUDE):]
+        body, n = re.subn(r'extern "C" __global__ __launch_bounds__\(\d+\) void \w+\(',
+                          "static __device__ __forceinline__ void body(const u32 bid_x, const u32 bid_z, float* __restrict__ lds, ", body)
+        assert n == 1
+        assert "blockIdx.y" not in body
+        body = body.replace("blockIdx.x", "bid_x").replace("blockIdx.z", "bid_z")
+        decls = re.findall(r"__shared__ __attribute__\(\(aligned\(16\)\)\) float (\w+)\[2\]\[(\d+)\]\[(\d+)\];", body)
+        assert [d[0] for d in decls] == ["As", "Bs"], decls
+        at = 0
+        for nm, r_, c_ in decls:
+            body = body.replace(f"__shared__ __attribute__((aligned(16))) float {nm}[2][{r_}][{c_}];",
+                                f"float (*{nm})[{r_}][{c_}] = reinterpret_cast<float (*)[{r_}][{c_}]>(lds + {at}u);")
+            at += 2 * int(r_) * int(c_)
+        assert 4 * at == matmul_lds_bytes(WM, WN, MI, NJ, BK, ta, tb, S)
+        parts.append({"tag": tag, "name": name, "body": body, "threads": 64 * WM * WN, "lds": at, "epi": bool(epi), "fmt": fmt})
+    threads = max(p["threads"] for p in parts)
+    lds = max(p["lds"] for p in parts)
+    assert 4 * lds <= MATMUL_LDS_LIMIT
+    name = "pair_" + parts[0]["name"].replace("matmul_", "") + "__" + parts[1]["name"].replace("matmul_", "")
+    undef = "#undef BM\n#undef BN\n#undef BK\n#undef MI\n#undef NJ\n#undef EPI\n"
+    src = PRELUDE
+    params, calls = [], []
+    for i, p in enumerate(parts):
+        src += f"namespace {p['tag']} {{\n{p['body']}}}\n{undef}"
+        params.append(f"const float* __restrict__ A{i}, const float* __restrict__ B{i}, float* __restrict__ C{i}, {p['tag']}::MMArgs g{i}"
+                      + (f", const float* __restrict__ E{i}" if p["epi"] else ""))
+        calls.append(f"{p['tag']}::body(b % tiles{i}, b / tiles{i}, lds, A{i}, B{i}, C{i}, g{i}" + (f", E{i}" if p["epi"] else "") + ");")
+    src += f"""
+extern "C" __global__ __launch_bounds__({threads}) void {name}({params[0]},
+        {params[1]}, u32 nblk0, u32 tiles0, u32 tiles1) {{
+    __shared__ __attribute__((aligned(16))) float lds[{lds}];
+    if (blockIdx.x < nblk0) {{
+        if (threadIdx.x >= {parts[0]['threads']}u) return;
+        const u32 b = blockIdx.x;
+        {calls[0]}
+    }} else {{
+        if (threadIdx.x >= {parts[1]['threads']}u) return;
+        const u32 b = blockIdx.x - nblk0;
+        {calls[1]}
+    }}
+}}
+"""
+    return src, name, "@" + parts[0]["fmt"][1:] + parts[1]["fmt"][1:] + "III"
+
+
 # name -> (WM, WN, MI, NJ, BK): block tile = (32*MI*WM) x (32*NJ*WN), 64*WM*WN threads.
 # Kept after sweeps on MI355X (TFLOP/s at 4096^3 / 8192x768x768 / batch 8 of 768x3072x1024):
 #   256x256 (8 waves, 128 acc regs)   136 /  .. /  ..    largest problems, one block per CU

@@ -88,6 +88,7 @@ class CustomOps(_Op):
     ADAM_STEP_INPLACE = auto()      # the same, in place, constants from device memory (graph replay)
     MATMUL_NT = auto()              # x @ y^T with y read in place (no materialised transpose)
     MATMUL_TN = auto()              # x^T @ y with x read in place
+    MATMUL_PAIR = auto()            # two independent products (the dX and dW of a linear layer) as one launch
     FROM_U8 = auto()                # host uint8 array -> device fp32 buffer, cast on the device
     ROW_STORE = auto()              # dst[(int)idx, :] = src with idx read on the device (KV cache inside a graph)
     COPY_INTO = auto()              # device-to-device copy into an existing buffer (a KV-cache row)

@@ -330,6 +330,21 @@ class MatMul(OP):
         return unbroadcast(grad_x, self.x.shape), unbroadcast(grad_y, self.y.shape)
 
 
+def product_pair(first: tuple, second: tuple) -> tuple:
+    """Two independent products, each (kind, a, b[, epi, e]) as Buffer.matmul_pair takes them: one launch
+    on the hip device while the fused kernels are on, two calls otherwise.  Same bits either way."""
+    a = first[1]
+    if FUSED and a.device is Device.HIP:
+        from dlgrad_amd.runtime.hip import HIP
+        if HIP.MATMUL_PAIRS:
+            return Buffer.matmul_pair(first, second)
+    out = []
+    for kind, x, y, *rest in (first, second):
+        kw = {"epi": rest[0], "e": rest[1]} if rest and rest[0] else {}
+        out.append(x.matmul(y, **kw) if kind == "nn" else x.matmul_nt(y, **kw) if kind == "nt" else x.matmul_tn(y))
+    return tuple(out)
+
+
 class LinearNT(OP):
     """x @ W^T for W stored (out, in), the product inside Tensor.linear (tensor.py:549-563),
     with W read in place.  The reference builds it as Transpose -> MatMul, i.e. one permute
@@ -343,8 +358,7 @@ class LinearNT(OP):
         return x.matmul_nt(w)
 
     def backward(self, upstream_grad: Buffer) -> tuple:
-        grad_x = upstream_grad @ self.w
-        grad_w = upstream_grad.matmul_tn(self.x)
+        grad_x, grad_w = product_pair(("nn", upstream_grad, self.w), ("tn", upstream_grad, self.x))
         return unbroadcast(grad_x, self.x.shape), unbroadcast(grad_w, self.w.shape)
 
 
@@ -357,8 +371,7 @@ class LinearNTAdd(OP):
         return x.matmul_nt(w, epi="add", e=r)
 
     def backward(self, upstream_grad: Buffer) -> tuple:
-        grad_x = upstream_grad @ self.w
-        grad_w = upstream_grad.matmul_tn(self.x)
+        grad_x, grad_w = product_pair(("nn", upstream_grad, self.w), ("tn", upstream_grad, self.x))
         return unbroadcast(grad_x, self.x.shape), unbroadcast(grad_w, self.w.shape), upstream_grad
 
 
@@ -376,10 +389,11 @@ class MLPRelu(OP):
         return self.h.matmul_nt(w2, epi="add", e=r) if r is not None else self.h.matmul_nt(w2)
 
     def backward(self, upstream_grad: Buffer) -> tuple:
-        gh = upstream_grad.matmul(self.w2, epi="gate", e=self.gate)         # gradient before the ReLU
-        dw2 = unbroadcast(upstream_grad.matmul_tn(self.h), self.w2.shape)
-        dx = unbroadcast(gh @ self.w1, self.x.shape)
-        dw1 = unbroadcast(gh.matmul_tn(self.x), self.w1.shape)
+        # each gradient of an input travels with the weight gradient that reads the same upstream tensor
+        gh, dw2 = product_pair(("nn", upstream_grad, self.w2, "gate", self.gate),      # gradient before the ReLU
+                               ("tn", upstream_grad, self.h))
+        dx, dw1 = product_pair(("nn", gh, self.w1), ("tn", gh, self.x))
+        dw2, dx, dw1 = unbroadcast(dw2, self.w2.shape), unbroadcast(dx, self.x.shape), unbroadcast(dw1, self.w1.shape)
         return (dx, dw1, dw2, upstream_grad) if self.has_r else (dx, dw1, dw2)
 
 
@@ -545,8 +559,8 @@ class SelfAttentionQKV(OP):
     def backward(self, upstream_grad: Buffer) -> tuple:
         C = self.w.shape[1]
         g = self.qkv.causal_attention_qkv_bwd(self.p, upstream_grad, self.n_head, self.scale, self.y)     # (B, T, 3C)
-        dx = g @ self.w
-        dw = unbroadcast(g.matmul_tn(self.x), self.w.shape)                                       # (3C, C)
+        dx, dw = product_pair(("nn", g, self.w), ("tn", g, self.x))
+        dw = unbroadcast(dw, self.w.shape)                                                        # (3C, C)
         part = lambda i: Buffer(dw.ptr + i * C * C, (C, C), dw.device)                            # noqa: E731
         return dx, part(0), part(1), part(2)
 

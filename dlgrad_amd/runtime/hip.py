@@ -545,6 +545,7 @@ def _map(tag: str, expr: str, operands: list[Buffer], out_shape: tuple, svals: t
 
 _U64 = (1 << 64) - 1
 _gemm_plans: dict = {}             # the same for products of matrices cut out of larger tensors
+_pair_plans: dict = {}             # the same for two products that travel as one launch
 _matmul_plans: dict = {}           # (shapes, flags, alignment bits) -> (kernel, grid, threads, fixed arguments, ...) of a product seen before
 # short rows of an even length: "direct" = a thread per row with 8-byte loads straight from memory (7.2 us for
 # 1 000 000 x 10 against 8.1 for "staged", 256 rows per block through LDS, which remains the form for odd lengths)
@@ -1428,6 +1429,8 @@ class HIP:
 
     ROW_MATMUL = os.environ.get("DLGRAD_HIP_ROW_MATMUL", "1") != "0"        # "0": one-row products on the MFMA tiles too
     DECODE_FUSED = os.environ.get("DLGRAD_HIP_DECODE_FUSED", "1") != "0"    # "0": cached attention as product, softmax, product
+    MATMUL_PAIRS = os.environ.get("DLGRAD_HIP_MATMUL_PAIRS", "1") != "0"       # "0": the two products of a linear layer's backward as two launches
+    MATMUL_PAIR_MAX_FLOP = 1 << 30        # per product: beyond it a product fills the chip by itself
     CE_GRAD_ROWS = os.environ.get("DLGRAD_HIP_CE_GRAD_ROWS", "1") != "0"       # "0": the cross-entropy gradient as an element-wise launch
     ATTENTION_FUSED = os.environ.get("DLGRAD_HIP_ATTENTION_FUSED", "1") != "0"   # "0": short causal attention as products and softmax launches too
 
@@ -1665,6 +1668,89 @@ class HIP:
             k, grid, threads = HIP._matmul_kernel(tile, veca, vecb, M, N, batch, ta, tb, "" if epi else tri, False, epi)
             _matmul_plans[key] = (k, grid, threads, args[3:], out_numel, 1 if epi else 0, HIP.last_matmul_kernel)
         return out
+
+    @staticmethod
+    def _pair_part(x: Buffer, y: Buffer, ta: bool, tb: bool, epi: str, e: Buffer | None):
+        """Sizes and strides of one product of a pair as HIP.matmul lays it out -- (M, N, K, nbc, batch, sa, sb,
+        out_numel) -- or None where that product takes one of HIP.matmul's special routes or is too
+        large to gain from company."""
+        if x.ndim != y.ndim or not 2 <= x.ndim <= 4 or (ta and tb):
+            return None
+        (Kd, M) = x.shape[-2:] if ta else x.shape[-2:][::-1]
+        (N, Ky) = y.shape[-2:] if tb else y.shape[-2:][::-1]
+        xb = (1,) * (4 - x.ndim) + tuple(x.shape[:-2])
+        yb = (1,) * (4 - y.ndim) + tuple(y.shape[:-2])
+        B0, B1 = max(xb[0], yb[0]), max(xb[1], yb[1])
+        out_numel = B0 * B1 * M * N
+        if Ky != Kd or Kd == 0 or out_numel == 0:
+            return None
+        if epi and (epi not in ("add", "relu", "gate") or (epi != "relu" and (e is None or e.is_host_scalar or e.numel != out_numel))):
+            return None
+        if yb == (1, 1) and not ta:
+            M, nbc, batch = xb[0] * xb[1] * M, 1, 1
+            sa = sb = (0, 0)
+        else:
+            nbc, batch = B1, B0 * B1
+            sa = (xb[1] * M * Kd if xb[0] > 1 else 0, M * Kd if xb[1] > 1 else 0)
+            sb = (yb[1] * Kd * N if yb[0] > 1 else 0, Kd * N if yb[1] > 1 else 0)
+        if (M == 1 and batch == 1 and tb) or batch > 65535 or max(M * Kd, Kd * N, M * N) >= 2 ** 31:
+            return None
+        if 2 * M * N * Kd * batch > HIP.MATMUL_PAIR_MAX_FLOP:
+            return None
+        return M, N, Kd, nbc, batch, sa, sb, out_numel
+
+    @staticmethod
+    @dispatcher.register(CustomOps.MATMUL_PAIR, Device.HIP)
+    def matmul_pair(first: tuple, second: tuple) -> tuple[DevicePtr, DevicePtr]:
+        """Two independent products (x, y, ta, tb, epi, e), operands prepared as for HIP.matmul, as one launch
+        (K.matmul_pair_kernel): the backward of a linear layer needs dX = G W and dW = G^T X, which share
+        an input and nothing else, and either alone leaves most of the chip idle while its short k loop
+        runs.  Each product keeps the tile it would have on its own and its bits.  Large products, and the
+        shapes HIP.matmul treats specially, go out as two launches."""
+        specs = (first, second)
+        addrs = tuple((x.ptr.addr, y.ptr.addr, 0 if e is None or e.ptr.__class__ is HostScalar else e.ptr.addr)
+                      for x, y, _, _, _, e in specs)
+        key = tuple((x.shape, y.shape, ta, tb, epi, None if e is None else e.shape, a[0] & 15, a[1] & 15, a[2] & 15)
+                    for (x, y, ta, tb, epi, e), a in zip(specs, addrs)) + (HIP.MATMUL_FORCE,)
+        plan = _pair_plans.get(key)
+        if plan is None:
+            parts = [HIP._pair_part(*sp) for sp in specs]
+            if None in parts:
+                plan = _pair_plans[key] = False
+            elif capturing():                             # a pair met for the first time while capturing: tiles are not timed now
+                plan = False
+            else:
+                cfgs, tails, grids, numels, has_e = [], [], [], [], []
+                for (x, y, ta, tb, epi, e), a, (M, N, Kd, nbc, batch, sa, sb, out_numel) in zip(specs, addrs, parts):
+                    veca = (M if ta else Kd) % 4 == 0 and a[0] % 16 == 0
+                    vecb = (Kd if tb else N) % 4 == 0 and a[1] % 16 == 0
+                    if epi and e is not None and (a[2] % 16 or N % 4):
+                        vecb = False
+                    probe = alloc(out_numel)              # tiles are timed on a result of the real size
+                    tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, (a[0], a[1], probe.addr, M, N, Kd, nbc, *sa, *sb), ta, tb)
+                    bm, bn, _ = K.matmul_tile_shape(tile)
+                    cfg = K.MATMUL_CONFIGS[tile]
+                    cfgs.append((*cfg[:5], veca, vecb, ta, tb, "", False, epi, cfg[5] if len(cfg) > 5 else 32))
+                    tails.append((M, N, Kd, nbc, *sa, *sb))
+                    grids.append((((M + bm - 1) // bm) * ((N + bn - 1) // bn), batch))
+                    numels.append(out_numel)
+                    has_e.append(bool(epi))
+                k = kernel(K.matmul_pair_kernel, cfgs[0], cfgs[1])
+                nb0, nb1 = grids[0][0] * grids[0][1], grids[1][0] * grids[1][1]
+                plan = _pair_plans[key] = (k, nb0 + nb1, max(64 * c[0] * c[1] for c in cfgs), tails, numels, has_e,
+                                           (nb0, grids[0][0], grids[1][0]), kernel_names.get(id(k)))
+        if not plan:
+            return tuple(HIP.matmul(x, y, ta=ta, tb=tb, epi=epi, e=e) for x, y, ta, tb, epi, e in specs)
+        k, nblk, threads, tails, numels, has_e, tail, name = plan
+        outs = (alloc(numels[0]), alloc(numels[1]))
+        args = []
+        for a, out, t, he in zip(addrs, outs, tails, has_e):
+            args += [a[0], a[1], out.addr, *t]
+            if he:
+                args.append(a[2] or out.addr)             # "relu" looks at the result only
+        HIP.last_matmul_kernel = name
+        launch(k, nblk, threads, *args, *tail)
+        return outs
 
     @staticmethod
     @dispatcher.register(CustomOps.MATMUL_NT, Device.HIP)

@@ -356,3 +356,67 @@ def test_4096_backward_shapes_in_place_against_float64_on_a_row_sample():
     _rows_vs_float64(nt, rows, g[rows], np.ascontiguousarray(a.T), "4096 NT in place")
     check(((da.T) @ dg).numpy(), tn, 0, "permute + NN gives the TN kernel's bits")
     check((dg @ da.T).numpy(), nt, 0, "permute + NN gives the NT kernel's bits")
+
+
+PAIR_CASES = [
+    # (shape of g, shape of w, shape of x, epilogue of the first product)
+    ((16, 128, 128), (128, 128), (16, 128, 128), ""),          # the attention projection of the char-GPT step
+    ((16, 128, 384), (384, 128), (16, 128, 128), ""),          # its stacked q/k/v projection
+    ((16, 128, 128), (128, 512), (16, 128, 512), "gate"),      # its feed-forward block: hidden gradient with the ReLU select
+    ((16, 128, 512), (512, 128), (16, 128, 128), ""),
+    ((3, 50, 36), (36, 20), (3, 50, 20), ""),                  # extents that are no multiple of a tile
+    ((2, 33, 7), (7, 5), (2, 33, 5), "gate"),                  # 4-byte accesses
+    ((1, 1, 64), (64, 32), (1, 1, 32), ""),                    # a single row
+    ((256, 64), (64, 10), (256, 10), "relu"),                  # 2-D operands (the MLP)
+]
+
+
+@pytest.mark.parametrize("gs,ws,xs,epi", PAIR_CASES)
+def test_two_products_in_one_launch_keep_their_bits(gs, ws, xs, epi):
+    """dX = G W (optionally with an epilogue) and dW = G^T X of a linear layer go out as one launch of two
+    tile grids.  Each block runs the product kernel's own code on the block index it would have had, so both
+    results must equal those of the separate launches bit for bit, and the pair must be one launch."""
+    require_gpu()
+    from dlgrad_amd.buffer import Buffer
+    rng = np.random.default_rng(91)
+    g, w, x = (rng.standard_normal(s, dtype=np.float32) for s in (gs, ws, xs))
+    gate = rng.standard_normal(gs[:-1] + ws[-1:], dtype=np.float32)
+    gb, wb, xb, eb = (dev(a) for a in (g, w, x, gate))
+    first = ("nn", gb, wb, epi, eb if epi != "relu" else None) if epi else ("nn", gb, wb)
+    before = hip.launch_count
+    dx, dw = Buffer.matmul_pair(first, ("tn", gb, xb))
+    launches = hip.launch_count - before
+    kw = {"epi": epi, "e": eb if epi != "relu" else None} if epi else {}
+    dx0, dw0 = gb.matmul(wb, **kw), gb.matmul_tn(xb)
+    assert dx.shape == dx0.shape and dw.shape == dw0.shape
+    if hip.COMPILE_ONLY:
+        return
+    if gs[-2] > 1:
+        assert launches == 1, launches
+    np.testing.assert_array_equal(dx.numpy().view(np.uint32), dx0.numpy().view(np.uint32))
+    np.testing.assert_array_equal(dw.numpy().view(np.uint32), dw0.numpy().view(np.uint32))
+    want = (g.astype(np.float64) @ w.astype(np.float64))
+    if epi == "gate":
+        want = np.where(gate > 0, want, 0.0)
+    elif epi == "relu":
+        want = np.maximum(want, 0.0)
+    check_mm(dx.numpy(), want, "dx against float64")
+    want_w = np.swapaxes(g.astype(np.float64), -1, -2) @ x.astype(np.float64)
+    check_mm(dw.numpy(), want_w, "dw against float64")
+
+
+def test_large_products_do_not_travel_in_pairs():
+    """Beyond about a GFLOP a product fills the chip by itself: the pair entry then issues two launches
+    (and gives the same bits, being the same two calls)."""
+    require_gpu()
+    from dlgrad_amd.buffer import Buffer
+    rng = np.random.default_rng(92)
+    g, w, x = (rng.standard_normal(s, dtype=np.float32) for s in ((4, 1024, 512), (512, 384), (4, 1024, 384)))
+    gb, wb, xb = dev(g), dev(w), dev(x)
+    before = hip.launch_count
+    dx, dw = Buffer.matmul_pair(("nn", gb, wb), ("tn", gb, xb))
+    assert hip.launch_count - before == 2
+    if hip.COMPILE_ONLY:
+        return
+    np.testing.assert_array_equal(dx.numpy().view(np.uint32), gb.matmul(wb).numpy().view(np.uint32))
+    np.testing.assert_array_equal(dw.numpy().view(np.uint32), gb.matmul_tn(xb).numpy().view(np.uint32))
