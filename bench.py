@@ -286,7 +286,8 @@ def run_c5(steps: int, warmup: int) -> dict:
     one = Buffer.from_scalar(1.0)
     row_max, row_logsum, _ = logits.ce_stats(tgt)
     att4 = att.reshape((8, 12, 1024, 1024))
-    causal = Buffer.from_numpy(np.triu(np.ones((1024, 1024), np.float32), 1), Device.HIP)
+    from dlgrad_amd.ops import causal_mask
+    causal = causal_mask(1024, Device.HIP)                     # the mask the attention layers use (built once per size, kept)
     probs = att4.masked_softmax(causal, 0.125)
     work = [("embedding_gather", lambda: table.embedding(idx), 4 * n + 8 * n * W),
             ("embedding_scatter_add", lambda: table.embedding(idx, backward=True, upstream_grad=g),

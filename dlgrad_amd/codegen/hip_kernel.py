@@ -1239,13 +1239,19 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
     ce_forward gather of cpu_kernel.py:430-441, fused.
     masked (register-resident forms): the row is x * scale with -inf where mask > 0, the
     attention chain `(att * scale).masked_fill(mask, -inf).softmax()` of examples/gpt.py:51-54
-    in one pass; the mask has `mrows` rows of L and row r of x uses mask row r % mrows."""
+    in one pass; the mask has `mrows` rows of L and row r of x uses mask row r % mrows.
+    masked = "causal" (16-byte items): the mask is known to be 1 exactly where column > r % mrows (what
+    ops.causal_mask builds), so it is computed from the indices and never read: same values, and the
+    pass over the mask through the L2 -- as many bytes as the output -- disappears."""
     if not per_block:
         threads = 256
+    causal = masked == "causal"                           # the mask is "column > row % mrows": computed, not read
+    masked = bool(masked)
     assert not masked or (nval and not gather)
+    assert not causal or vec == 4
     nt = nt and bool(nval) and vec == 4                   # streaming loads/stores: register-resident float4 form only
     name = (f"{'log_' if log else ''}softmax_rows_v{vec}_{f'blk{threads}' if per_block else 'wav'}"
-            f"{f'_r{nval}' if nval else ''}{'_g' if gather else ''}{'_m' if masked else ''}{'nt' if nt else ''}")
+            f"{f'_r{nval}' if nval else ''}{'_g' if gather else ''}{'_c' if causal else '_m' if masked else ''}{'nt' if nt else ''}")
     T = f"{threads}u" if per_block else "64u"
     NW = threads // 64
     tid = "threadIdx.x" if per_block else "(threadIdx.x & 63u)"
@@ -1269,13 +1275,18 @@ def softmax_rows_kernel(log: bool, vec: int, per_block: bool, nval: int = 0, gat
         ldx = "ld4_stream(p + c)" if nt else "p[c]"
         # the mask is read first (a few rows, cache resident); items that are masked in all four
         # lanes are never loaded, which halves the reads of a causal mask
-        mask4 = f"""    const float4* __restrict__ pm = reinterpret_cast<const float4*>(mask + (u64)(row % mrows) * L);
-    u32 mb[{nval}];
+        if causal:
+            mask_bits = ("    const u32 last = row % mrows;                             // the last column this row may look at\n",
+                         "mb[k] = (4u * c > last ? 1u : 0u) | (4u * c + 1u > last ? 2u : 0u) | (4u * c + 2u > last ? 4u : 0u) | (4u * c + 3u > last ? 8u : 0u);")
+        else:
+            mask_bits = ("    const float4* __restrict__ pm = reinterpret_cast<const float4*>(mask + (u64)(row % mrows) * L);\n",
+                         "const float4 mk = pm[c]; mb[k] = (mk.x > 0.0f ? 1u : 0u) | (mk.y > 0.0f ? 2u : 0u) | (mk.z > 0.0f ? 4u : 0u) | (mk.w > 0.0f ? 8u : 0u);")
+        mask4 = f"""{mask_bits[0]}    u32 mb[{nval}];
     #pragma unroll
     for (u32 k = 0; k < {nval}u; ++k) {{
         const u32 c = {tid} + k * {T};
         mb[k] = 15u;
-        if (c < nv) {{ const float4 mk = pm[c]; mb[k] = (mk.x > 0.0f ? 1u : 0u) | (mk.y > 0.0f ? 2u : 0u) | (mk.z > 0.0f ? 4u : 0u) | (mk.w > 0.0f ? 8u : 0u); }}
+        if (c < nv) {{ {mask_bits[1]} }}
     }}
     #pragma unroll
     for (u32 k = 0; k < {nval}u; ++k) {{ const u32 c = {tid} + k * {T}; v[k] = make_float4(0.f, 0.f, 0.f, 0.f); if (mb[k] != 15u) v[k] = {ldx}; }}
@@ -1554,7 +1565,10 @@ def softmax_bwd_rows_kernel(vec: int, nval: int, nt: bool = False, masked: bool 
     so they add nothing to the sum) are not loaded: a causal mask halves the reads."""
     T, comps, nvx = _rms_lanes(vec)
     nt = nt and vec == 4
-    name = f"softmax_bwd_rows_v{vec}_r{nval}{'_m' if masked else ''}{'nt' if nt else ''}"
+    causal = masked == "causal"                           # as in softmax_rows_kernel: the mask is computed from the indices
+    masked = bool(masked)
+    assert not causal or vec == 4
+    name = f"softmax_bwd_rows_v{vec}_r{nval}{'_c' if causal else '_m' if masked else ''}{'nt' if nt else ''}"
     ld = (lambda p: f"ld4_stream({p} + c)") if nt else (lambda p: f"{p}[c]")
     # the row's dot product, with its roundings spelled out (one product, then fused multiply-adds in
     # lane order) so that every variant of this kernel adds the same numbers in the same way
@@ -1565,12 +1579,15 @@ def softmax_bwd_rows_kernel(vec: int, nval: int, nt: bool = False, masked: bool 
     if skip:
         outs = "".join(f"            o{c} = ((mb[k] & {1 << j}u) ? 0.0f : y[k]{c} * (g[k]{c} - s)) * scale;\n"
                        for j, c in enumerate(comps))
+        bits = ("mb[k] = (4u * c > last ? 1u : 0u) | (4u * c + 1u > last ? 2u : 0u) | (4u * c + 2u > last ? 4u : 0u) | (4u * c + 3u > last ? 8u : 0u);"
+                if causal else
+                "const float4 mk = pm[c]; mb[k] = (mk.x > 0.0f ? 1u : 0u) | (mk.y > 0.0f ? 2u : 0u) | (mk.z > 0.0f ? 4u : 0u) | (mk.w > 0.0f ? 8u : 0u);")
         loads = f"""    u32 mb[{nval}];
     #pragma unroll
     for (u32 k = 0; k < {nval}u; ++k) {{
         const u32 c = lane + k * 64u;
         mb[k] = 15u;
-        if (c < nv) {{ const float4 mk = pm[c]; mb[k] = (mk.x > 0.0f ? 1u : 0u) | (mk.y > 0.0f ? 2u : 0u) | (mk.z > 0.0f ? 4u : 0u) | (mk.w > 0.0f ? 8u : 0u); }}
+        if (c < nv) {{ {bits} }}
     }}
     #pragma unroll
     for (u32 k = 0; k < {nval}u; ++k) {{
@@ -1604,7 +1621,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
     const u32 lane = threadIdx.x & 63u;
     const u32 row = blockIdx.x * 4u + (threadIdx.x >> 6);
     if (row >= R) return;
-    {f"const {T}* __restrict__ pm = reinterpret_cast<const {T}*>(mask + (u64)(row % mrows) * L);" if masked else ""}
+    {"const u32 last = row % mrows;" if causal else f"const {T}* __restrict__ pm = reinterpret_cast<const {T}*>(mask + (u64)(row % mrows) * L);" if masked else ""}
     const {T}* __restrict__ py = reinterpret_cast<const {T}*>(yp + (u64)row * L);
     const {T}* __restrict__ pg = reinterpret_cast<const {T}*>(gp + (u64)row * L);
     {T}* __restrict__ q = reinterpret_cast<{T}*>(dx + (u64)row * L);

@@ -1160,9 +1160,20 @@ class HIP:
         blk, nval, threads = K.softmax_plan(L, vec)
         if not mrows or not nval:
             raise ValueError(f"fused masked softmax does not take x {x.shape} with mask {mask.shape}")
-        k = kernel(K.softmax_rows_kernel, False, vec, blk, nval, False, threads, x.numel >= NT_STORE_MIN_ELEMENTS, True)
+        how = "causal" if vec == 4 and HIP._is_causal_mask(mask, L, mrows) else True
+        k = kernel(K.softmax_rows_kernel, False, vec, blk, nval, False, threads, x.numel >= NT_STORE_MIN_ELEMENTS, how)
         launch(k, R if blk else (R + 3) // 4, threads, _addr(x), out.addr, R, L, _addr(mask), mrows, float(scale))
         return out
+
+    @staticmethod
+    def _is_causal_mask(mask: Buffer, L: int, mrows: int) -> bool:
+        """Whether `mask` is the (L, L) causal mask this package built and keeps (ops.causal_mask): its contents are then
+        known -- 1 where column > row -- and the softmax kernels compute them instead of reading them."""
+        if not HIP.CAUSAL_MASK_KNOWN or mrows != L:
+            return False
+        from dlgrad_amd.ops import _causal_masks
+        kept = _causal_masks.get((L, Device.HIP))
+        return kept is not None and kept.ptr is mask.ptr
 
     @staticmethod
     @dispatcher.register(CustomOps.MASKED_SOFTMAX_BWD, Device.HIP)
@@ -1177,7 +1188,8 @@ class HIP:
         nval = K.rmsnorm_plan(L, vec)
         if not mrows or nval == 0 or g.numel != y.numel or g.is_host_scalar:
             raise ValueError(f"fused masked softmax backward does not take y {y.shape} with mask {mask.shape}")
-        launch(kernel(K.softmax_bwd_rows_kernel, vec, nval, y.numel >= NT_STORE_MIN_ELEMENTS, True), (R + 3) // 4, 256,
+        how = "causal" if vec == 4 and HIP._is_causal_mask(mask, L, mrows) else True
+        launch(kernel(K.softmax_bwd_rows_kernel, vec, nval, y.numel >= NT_STORE_MIN_ELEMENTS, how), (R + 3) // 4, 256,
                _addr(y), _addr(g), dx.addr, R, L, _addr(mask), mrows, float(scale))
         return dx
 
@@ -1431,6 +1443,7 @@ class HIP:
     DECODE_FUSED = os.environ.get("DLGRAD_HIP_DECODE_FUSED", "1") != "0"    # "0": cached attention as product, softmax, product
     MATMUL_PAIRS = os.environ.get("DLGRAD_HIP_MATMUL_PAIRS", "1") != "0"       # "0": the two products of a linear layer's backward as two launches
     MATMUL_PAIR_MAX_FLOP = 1 << 30        # per product: beyond it a product fills the chip by itself
+    CAUSAL_MASK_KNOWN = os.environ.get("DLGRAD_HIP_CAUSAL_MASK_KNOWN", "1") != "0"   # "0": the cached causal mask is read like any other mask
     CE_GRAD_ROWS = os.environ.get("DLGRAD_HIP_CE_GRAD_ROWS", "1") != "0"       # "0": the cross-entropy gradient as an element-wise launch
     ATTENTION_FUSED = os.environ.get("DLGRAD_HIP_ATTENTION_FUSED", "1") != "0"   # "0": short causal attention as products and softmax launches too
 

@@ -168,6 +168,43 @@ def test_fused_masked_softmax_is_the_three_op_chain(xs, ms, monkeypatch):
     assert np.abs(g1[sl] - gw).max() <= 2e-6 * max(1.0, np.abs(gw).max())
 
 
+@pytest.mark.parametrize("shape", [(2, 3, 64, 64), (1, 2, 1024, 1024), (3, 128, 128), (2, 100, 100), (8, 12, 1024, 1024)])
+def test_the_kept_causal_mask_is_computed_instead_of_read(shape):
+    """The (T, T) causal mask that ops.causal_mask builds once and keeps is recognised by its allocation: the scaled
+    masked softmax and its backward then form "column > row" from the indices instead of reading a mask row per
+    score row.  Same kernels otherwise: the results must have the bits of a run with an equal mask that lives
+    in another buffer (and is therefore read)."""
+    require_gpu()
+    from dlgrad_amd import ops
+    from dlgrad_amd.buffer import Buffer
+    from dlgrad_amd.device import Device
+    T = shape[-1]
+    rng = np.random.default_rng(75)
+    big = int(np.prod(shape)) > 1 << 24
+    x = rng.standard_normal(shape, dtype=np.float32)
+    g = rng.standard_normal(shape, dtype=np.float32)
+    kept = ops.causal_mask(T, Device.HIP)
+    other = Buffer.from_numpy(np.triu(np.ones((T, T), np.float32), 1), Device.HIP)
+    xb, gb = Buffer.from_numpy(x, Device.HIP), Buffer.from_numpy(g, Device.HIP)
+    seen = set(hip.requested_kernels)
+    y1 = xb.masked_softmax(kept, 0.125)
+    d1 = y1.masked_softmax_bwd(gb, kept, 0.125)
+    new = {(n, p) for n, p in hip.requested_kernels - seen if "softmax" in n} if not seen >= hip.requested_kernels else set()
+    y0 = xb.masked_softmax(other, 0.125)
+    d0 = y0.masked_softmax_bwd(gb, other, 0.125)
+    assert hip.HIP._is_causal_mask(kept, T, T) and not hip.HIP._is_causal_mask(other, T, T)
+    assert all(p[-1] in ("causal", True) for _, p in new)
+    if hip.COMPILE_ONLY:
+        return
+    if not big:
+        np.testing.assert_array_equal(kept.numpy(), other.numpy())
+    for name, a, b in (("y", y1, y0), ("dx", d1, d0)):
+        a, b = a.numpy(), b.numpy()
+        assert (a.view(np.uint32) == b.view(np.uint32)).all(), name
+        if name == "y":
+            assert not np.triu(a.reshape(-1, T, T)[0], 1).any()
+
+
 def test_masked_softmax_falls_back_to_the_chain_where_the_kernel_does_not_fit():
     """Rows too long for registers, a mask that does not line up with the trailing dims, or
     another axis: the op-by-op chain runs, with the same result as on the CPU oracle (1e-6)."""
