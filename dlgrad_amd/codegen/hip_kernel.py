@@ -1055,8 +1055,11 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
         // ---- a zero block: 64 table rows, zeros for those no index names
         const u32 v0 = grp * 64u;
         const u32 rows = min(64u, V - v0);
+        // which of the rows some index names, read by every wavefront in one go (sixteen reads one after the other, each
+        // deciding the next row's fate, would make the stream of zeros wait for sixteen round trips to memory)
+        const u64 named = __ballot(lane < rows ? idsegs[v0 + lane] != 0ull : true);
         for (u32 r = w; r < rows; r += 4u) {{                     // a wavefront per row, rows four apart
-            if (idsegs[v0 + r] != 0ull) continue;               // some index names this row: its sum is written instead
+            if ((named >> r) & 1ull) continue;                  // some index names this row: its sum is written instead
             {VT}* __restrict__ zrow = reinterpret_cast<{VT}*>(out + (u64)(v0 + r) * W);
             for (u32 c = lane; c < Wv; c += 64u) {zstore}
         }}
