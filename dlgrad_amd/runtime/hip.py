@@ -813,6 +813,9 @@ class HIP:
         """Two launches: blocks of 2048 vector items (32 KiB) -> partials -> one block; both are
         issued by one call into the library (dlg_hip_reduce_full), the partials in a pool block."""
         global launch_count
+        if n == 0:                                       # nothing to add or compare: what the reference's loop leaves in its accumulator
+            lib().fill_f32(out_addr, -3.4028234663852886e+38 if kop == "max" else float("nan") if divisor == 0 else 0.0, 1)    # (a mean of nothing is 0 / 0)
+            return
         vec = 4 if x_addr % 16 == 0 else 1
         items = (n + vec - 1) // vec
         G = (items + 2047) // 2048

@@ -454,3 +454,27 @@ def test_indices_outside_their_table_touch_nothing():
         want_after[np.arange(6)[inside], t.ravel()[inside].astype(int)] -= 1
         np.testing.assert_array_equal(after, want_after)
         assert not picked2.numpy().ravel()[~inside].any() and not picked3.numpy().ravel()[~inside].any()
+
+
+def test_tensors_without_elements_and_with_one():
+    """Extents of 0 and 1 in every op family: no launch of an empty grid, the shapes the oracle gives, and for
+    the reductions what an empty loop leaves behind (0 for a sum, -FLT_MAX for a max, 0 / 0 for a mean)."""
+    require_gpu()
+    e, one = np.zeros((0, 4), np.float32), np.full((1, 1), 3.0, np.float32)
+    for a, b in ((e, e), (one, one), (np.zeros((3, 0), np.float32), np.zeros((3, 0), np.float32))):
+        check((dev(a) + dev(b)).numpy(), cref.binary("add", a, b), 0, f"add {a.shape}")
+        check(dev(a).exp().numpy(), cref.unary("exp", a), 1e-6, f"exp {a.shape}")
+        check(dev(a).permute((1, 0)).numpy(), cref.permute(a, (1, 0)), 0, f"transpose {a.shape}")
+        for dim in (0, 1):
+            for op in ("sum", "max"):
+                check(getattr(dev(a), op)(dim).numpy(), cref.reduce(op, a, dim), 0, f"{op} {a.shape} over {dim}")
+    for op in ("sum", "max"):
+        check(getattr(dev(e), op)(-1).numpy(), cref.reduce(op, e), 0, f"{op} of nothing")
+        check(getattr(dev(one), op)(-1).numpy(), cref.reduce(op, one), 0, f"{op} of one element")
+    if not hip.COMPILE_ONLY:
+        assert np.isnan(dev(e).mean(-1).numpy())
+    check(dev(e).matmul(dev(np.ones((4, 3), np.float32))).numpy(), np.zeros((0, 3), np.float32), 0, "no rows times a matrix")
+    check(dev(np.ones((2, 0), np.float32)).matmul(dev(np.ones((0, 3), np.float32))).numpy(), np.zeros((2, 3), np.float32), 0, "empty k")
+    check(dev(one).matmul(dev(one)).numpy(), np.full((1, 1), 9.0, np.float32), 0, "1 x 1")
+    check(dev(e).softmax(1).numpy(), e, 0, "softmax of no rows")
+    check(dev(e).argmax(1).numpy(), np.zeros((0, 1), np.float32), 0, "argmax of no rows")
