@@ -645,7 +645,7 @@ class PartialSum(Buffer):
     the gradient, in the very order the column-sum kernel uses, so the separate launch per weight (a
     quarter of the launches of a char-GPT step) disappears and the bits stay.  Every other reader --
     numpy(), another op, a per-tensor optimizer -- touches `ptr`, which runs the sum then, once."""
-    __slots__ = ("parts", "_sum")
+    __slots__ = ("parts", "_sum", "offset", "pitch", "whole")
 
     @staticmethod
     def of(parts: Buffer, shape: tuple) -> Buffer:
@@ -657,19 +657,35 @@ class PartialSum(Buffer):
             out = parts.sum(0, keepdim=False)
             return out if out.shape == tuple(shape) else out.reshape(shape)
         b = _new_buffer(PartialSum)
-        b.parts, b._sum = parts, None
+        b.parts, b._sum, b.offset, b.whole = parts, None, 0, None
         b.shape, b.dtype, b.device = tuple(shape), parts.dtype, parts.device
+        b.numel, b.stride, b.ndim, b.nbytes = _shape_info(b.shape)
+        b.pitch = b.numel                                  # floats from one part to the next
+        return b
+
+    def piece(self, start: int, shape: tuple) -> Buffer:
+        """Elements [start, start + prod(shape)) of the flat value as a Buffer of their own (the thirds of a
+        stacked weight gradient).  While the sum is pending the piece is pending too: it names the same parts,
+        `start` floats in, one whole value apart."""
+        if self._sum is not None:
+            return Buffer(self._sum + start, shape, self.device)
+        b = _new_buffer(PartialSum)
+        b.parts, b._sum, b.offset, b.pitch, b.whole = self.parts, None, self.offset + start, self.pitch, self
+        b.shape, b.dtype, b.device = tuple(shape), self.dtype, self.device
         b.numel, b.stride, b.ndim, b.nbytes = _shape_info(b.shape)
         return b
 
     @property
     def pending(self) -> bool:
-        return self._sum is None
+        return self._sum is None and (self.whole is None or self.whole.pending)
 
     @property
     def ptr(self):
         if self._sum is None:
-            self._sum = self.parts.sum(0, keepdim=False).ptr
+            if self.whole is not None:                        # a piece: the whole is summed (once), the piece is a view of it
+                self._sum = self.whole.ptr + (self.offset - self.whole.offset)
+            else:
+                self._sum = self.parts.sum(0, keepdim=False).ptr
             self.parts = None
         return self._sum
 

@@ -2756,11 +2756,13 @@ def adam_multi_inplace_kernel() -> tuple[str, str, str]:
     addresses (p, g, m, v) per tensor, `sizes` the element counts, `first` the first block of each
     tensor and `owner` the tensor of every block; a block updates 1024 consecutive elements of its
     tensor (16-byte accesses: every address is 16-byte aligned, the n % 4 tail is done by the
-    tensor's first block).  Same arithmetic as the per-tensor kernel, so the same bits.
+    tensor's first block) -- or 64 of them when the gradient is a pending sum of more than 16 parts,
+    whose addition the block's threads then share.  Same arithmetic as the per-tensor kernel, so the same bits.
 
-    `rows` says how many rows of `size` floats a tensor's gradient pointer holds.  1: the gradient
-    itself.  More: its parts, whose sum over the rows is the gradient (the batch entries of a weight
-    gradient, the partial rows of an RMSNorm gain).  They are added up here, element by element, in
+    `rows_of` holds two numbers per tensor: how many parts its gradient pointer holds and how many floats
+    lie between one part and the next.  1 part: the gradient itself.  More: parts whose sum is the
+    gradient (the batch entries of a weight gradient -- for a third of a stacked weight one whole stacked
+    gradient apart -- or the partial rows of an RMSNorm gain).  They are added up here, element by element, in
     exactly the order reduce_cols_kernel adds a column of that many rows (thread rows 4 or 16 apart,
     four running sums each, joined pairwise, then the thread rows in order), so the update has the bits
     it would have had with the column-sum launch in between."""
@@ -2795,8 +2797,30 @@ template <int TY, typename T> static __device__ __forceinline__ T colsum(const f
     }
     return r;
 }
+// colsum<4> for up to 16 rows (the batch entries of a weight gradient, the partial rows of a gain): the same additions
+// in the same order, with every row's load issued before the first of them instead of four rounds of four
+template <typename T> static __device__ __forceinline__ T colsum16(const float* __restrict__ g, u32 rows, u32 n, u32 j) {
+    T t[16];
+    #pragma unroll
+    for (u32 l = 0; l < 16u; ++l) { zero_of(t[l]); if (l < rows) t[l] = ld_at(g, (u64)l * n, j, T()); }
+    T r; zero_of(r);
+    #pragma unroll
+    for (u32 ty = 0; ty < 4u; ++ty) {
+        T a0, a1, a2, a3; zero_of(a0); zero_of(a1); zero_of(a2); zero_of(a3);
+        if (ty + 12u < rows) { a0 = add2(a0, t[ty]); a1 = add2(a1, t[ty + 4u]); a2 = add2(a2, t[ty + 8u]); a3 = add2(a3, t[ty + 12u]); }
+        else {
+            #pragma unroll
+            for (u32 l = ty; l < 16u; l += 4u) if (l < rows) a0 = add2(a0, t[l]);
+        }
+        a0 = add2(a0, a1); a2 = add2(a2, a3); a0 = add2(a0, a2);
+        r = ty == 0u ? a0 : add2(r, a0);
+    }
+    return r;
+}
+// n: floats from one row to the next
 template <typename T> static __device__ __forceinline__ T grad_at(const float* __restrict__ g, u32 rows, u32 n, u32 j) {
     if (rows == 1u) return ld_at(g, 0, j, T());
+    if (rows <= 16u) return colsum16<T>(g, rows, n, j);
     return rows > 64u ? colsum<16, T>(g, rows, n, j) : colsum<4, T>(g, rows, n, j);
 }
 """
@@ -2810,13 +2834,49 @@ template <typename T> static __device__ __forceinline__ T grad_at(const float* _
     const float* __restrict__ g = reinterpret_cast<const float*>(ptrs[n_tensors + t]);
     float* m = reinterpret_cast<float*>(ptrs[2u * n_tensors + t]);
     float* v = reinterpret_cast<float*>(ptrs[3u * n_tensors + t]);
-    const u32 n = sizes[t], nv = n >> 2, rows = rows_of[t];
+    const u32 n = sizes[t], nv = n >> 2, rows = rows_of[2u * t], gp = rows_of[2u * t + 1u];       // parts of the gradient and their distance
+    if (rows > 16u && (n & 3u) == 0u) {{
+        // Many parts (the per-wavefront partial rows of an RMSNorm gain): a block takes 16 columns of 16 bytes and adds
+        // them up the way a 64 x 16 block of the column-sum kernel does -- thread row ty owns parts ty, ty + TY, ..
+        // in four running sums, joined pairwise; then the thread rows are added in order.
+        __shared__ float4 part[16][16];
+        const u32 ty = threadIdx.x >> 4, cx = threadIdx.x & 15u, col = lb * 16u + cx;
+        const u32 TY = rows > 64u ? 16u : 4u;
+        if (col < nv && ty < TY) {{
+            float4 a0, a1, a2, a3; zero_of(a0); zero_of(a1); zero_of(a2); zero_of(a3);
+            u32 l = ty;
+            for (; l + 3u * TY < rows; l += 4u * TY) {{
+                const float4 t0 = ld_at(g, (u64)l * gp, col, float4()), t1 = ld_at(g, (u64)(l + TY) * gp, col, float4());
+                const float4 t2 = ld_at(g, (u64)(l + 2u * TY) * gp, col, float4()), t3 = ld_at(g, (u64)(l + 3u * TY) * gp, col, float4());
+                a0 = add2(a0, t0); a1 = add2(a1, t1); a2 = add2(a2, t2); a3 = add2(a3, t3);
+            }}
+            for (; l < rows; l += TY) a0 = add2(a0, ld_at(g, (u64)l * gp, col, float4()));
+            a0 = add2(a0, a1); a2 = add2(a2, a3); a0 = add2(a0, a2);
+            part[ty][cx] = a0;
+        }}
+        __syncthreads();
+        if (ty == 0u && col < nv) {{
+            float4 g4 = part[0][cx];
+            for (u32 k = 1; k < TY; ++k) g4 = add2(g4, part[k][cx]);
+            const float4 p4 = reinterpret_cast<float4*>(p)[col];
+            const float4 m4 = reinterpret_cast<float4*>(m)[col], v4 = reinterpret_cast<float4*>(v)[col];
+            float4 po, mo, vo;
+            adam1(p4.x, g4.x, m4.x, v4.x, a, po.x, mo.x, vo.x);
+            adam1(p4.y, g4.y, m4.y, v4.y, a, po.y, mo.y, vo.y);
+            adam1(p4.z, g4.z, m4.z, v4.z, a, po.z, mo.z, vo.z);
+            adam1(p4.w, g4.w, m4.w, v4.w, a, po.w, mo.w, vo.w);
+            reinterpret_cast<float4*>(p)[col] = po;
+            reinterpret_cast<float4*>(m)[col] = mo;
+            reinterpret_cast<float4*>(v)[col] = vo;
+        }}
+        return;
+    }}
     const u32 i = lb * 256u + threadIdx.x;
     if (i < nv) {{
         float4 g4;
-        if ((n & 3u) == 0u) g4 = grad_at<float4>(g, rows, n, i);          // every row starts 16-byte aligned
-        else {{ g4.x = grad_at<float>(g, rows, n, 4u * i); g4.y = grad_at<float>(g, rows, n, 4u * i + 1u);
-               g4.z = grad_at<float>(g, rows, n, 4u * i + 2u); g4.w = grad_at<float>(g, rows, n, 4u * i + 3u); }}
+        if ((n & 3u) == 0u) g4 = grad_at<float4>(g, rows, gp, i);         // every part starts 16-byte aligned
+        else {{ g4.x = grad_at<float>(g, rows, gp, 4u * i); g4.y = grad_at<float>(g, rows, gp, 4u * i + 1u);
+               g4.z = grad_at<float>(g, rows, gp, 4u * i + 2u); g4.w = grad_at<float>(g, rows, gp, 4u * i + 3u); }}
         const float4 p4 = reinterpret_cast<float4*>(p)[i];
         const float4 m4 = reinterpret_cast<float4*>(m)[i], v4 = reinterpret_cast<float4*>(v)[i];
         float4 po, mo, vo;
@@ -2831,7 +2891,7 @@ template <typename T> static __device__ __forceinline__ T grad_at(const float* _
     if (lb == 0 && threadIdx.x < (n & 3u)) {{
         const u32 j = (nv << 2) + threadIdx.x;
         float po, mo, vo;
-        adam1(p[j], grad_at<float>(g, rows, n, j), m[j], v[j], a, po, mo, vo);
+        adam1(p[j], grad_at<float>(g, rows, gp, j), m[j], v[j], a, po, mo, vo);
         p[j] = po; m[j] = mo; v[j] = vo;
     }}
 }}

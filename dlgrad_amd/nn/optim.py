@@ -99,7 +99,7 @@ class Adam(Optimizer):
             quads = [(p.data, p.grad.data, self.m[id(p)].data, self.v[id(p)].data) for p in self.params
                      if p.grad is not None and p.numel]
             def base(b):                                 # a pending sum is handed over as its parts: asking for its ptr would run it
-                return b.parts.ptr.addr if getattr(b, "pending", False) else b.ptr.addr
+                return b.parts.ptr.addr + 4 * b.offset if getattr(b, "pending", False) else b.ptr.addr
             if all(not (base(b) & 15) for q in quads for b in q):
                 # every parameter in one launch; the address table is uploaded on the first step only
                 from dlgrad_amd.dispatch import dispatcher

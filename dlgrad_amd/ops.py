@@ -561,7 +561,10 @@ class SelfAttentionQKV(OP):
         g = self.qkv.causal_attention_qkv_bwd(self.p, upstream_grad, self.n_head, self.scale, self.y)     # (B, T, 3C)
         dx, dw = product_pair(("nn", g, self.w), ("tn", g, self.x))
         dw = unbroadcast(dw, self.w.shape)                                                        # (3C, C)
-        part = lambda i: Buffer(dw.ptr + i * C * C, (C, C), dw.device)                            # noqa: E731
+        if dw.__class__ is PartialSum:
+            part = lambda i: dw.piece(i * C * C, (C, C))                                          # noqa: E731  (stays pending)
+        else:
+            part = lambda i: Buffer(dw.ptr + i * C * C, (C, C), dw.device)                        # noqa: E731
         return dx, part(0), part(1), part(2)
 
 

@@ -1375,14 +1375,16 @@ class HIP:
         A gradient that is a pending sum (buffer.PartialSum) is taken as its parts: the kernel adds
         them up as it reads, in the order of the column-sum launch that would otherwise have run."""
         from dlgrad_amd.buffer import PartialSum
-        rows_of = []                                     # per tensor: how many rows of its size the gradient pointer holds
+        rows_of = []                                     # per tensor: how many parts the gradient pointer holds, and how far apart
         addrs = []
         for pb, gb, mb, vb in tensors:
             if gb.__class__ is PartialSum and gb.pending:
-                g_addr, rows = gb.parts.ptr.addr, gb.parts.shape[0]
+                g_addr, rows, pitch = gb.parts.ptr.addr + 4 * gb.offset, gb.parts.shape[0], gb.pitch
             else:
-                g_addr, rows = gb.ptr.addr, 1
-            rows_of.append(rows)
+                g_addr, rows, pitch = gb.ptr.addr, 1, 0
+            if pitch >= 2 ** 32 or pitch & 3 and not pb.numel & 3:
+                raise ValueError("adam_multi_inplace: parts of a pending gradient lie too far apart or break the 16-byte alignment")
+            rows_of += [rows, pitch]
             addrs += [pb.ptr.addr, g_addr, mb.ptr.addr, vb.ptr.addr]
         addrs = tuple(addrs)
         if any(a & 15 for a in addrs):
@@ -1391,11 +1393,13 @@ class HIP:
         if table is None or table["key"] != key:
             nt = len(tensors)
             sizes = np.array([q[0].numel for q in tensors], dtype=np.uint32)
-            nblk = np.maximum(1, (sizes.astype(np.int64) // 4 + 255) // 256)
+            # 256 threads take 256 16-byte items -- or 16 of them, sharing the addition of a gradient that is pending in many parts
+            per_block = np.array([16 if (r > 16 and not n & 3) else 256 for r, n in zip(rows_of[::2], sizes)], dtype=np.int64)
+            nblk = np.maximum(1, (sizes.astype(np.int64) // 4 + per_block - 1) // per_block)
             first = np.concatenate([[0], np.cumsum(nblk)[:-1]]).astype(np.uint32)
             owner = np.repeat(np.arange(nt, dtype=np.uint32), nblk)
             ptrs = np.array(addrs, dtype=np.uint64).reshape(nt, 4).T.reshape(-1)        # four rows: p, g, m, v
-            arrays = [np.ascontiguousarray(a).view(np.float32) for a in (ptrs, sizes, first, owner, np.array(rows_of, dtype=np.uint32))]     # raw bits
+            arrays = [np.ascontiguousarray(a).view(np.float32) for a in (ptrs, sizes, first, owner, np.array(rows_of, dtype=np.uint32))]     # raw bits; rows_of holds (parts, pitch) pairs
             reuse = (table is not None and not table["frozen"]
                      and [a.size for a in arrays] == [b.nbytes // 4 for b in table["bufs"]])
             bufs = table["bufs"] if reuse else [alloc(a.size) for a in arrays]

@@ -599,7 +599,8 @@ def test_adam_adds_up_pending_gradient_sums_with_the_bits_of_the_column_sum_laun
         pytest.skip("no HIP device")
     from dlgrad_amd.buffer import Buffer, PartialSum
     from dlgrad_amd.device import Device
-    cases = [((65, 128), 16), ((128,), 512), ((7,), 2), ((513, 3), 8), ((33, 20), 64), ((40, 25), 65), ((1024, 96), 200), ((6, 6), 1), ((129,), 3)]
+    cases = [((65, 128), 16), ((128,), 512), ((7,), 2), ((513, 3), 8), ((33, 20), 64), ((40, 25), 65), ((1024, 96), 200), ((6, 6), 1), ((129,), 3),
+             ((31, 4), 13), ((10,), 15), ((12, 8), 5), ((9, 4), 17)]
     rng = np.random.default_rng(21)
     values = [rng.standard_normal(shape).astype(np.float32) for shape, _ in cases]
     parts = [rng.standard_normal((rows, *shape)).astype(np.float32) for shape, rows in cases]
@@ -633,3 +634,42 @@ def test_adam_adds_up_pending_gradient_sums_with_the_bits_of_the_column_sum_laun
     if not hip.COMPILE_ONLY:
         for a, b in zip(results[True], results[False]):
             np.testing.assert_array_equal(a, b)
+
+
+@pytest.mark.gpu
+def test_pieces_of_a_pending_sum_stay_pending_for_the_one_launch_adam():
+    """The gradient of three stacked weights is one pending sum over the batch; each weight takes its third of
+    it (PartialSum.piece), which names the same parts at an offset, one whole gradient apart.  The one-launch Adam
+    reads the thirds in place: no column sum is launched, and the update has the bits of the update from the
+    summed gradient.  A piece that is read in any other way gives the matching slice of the sum."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    from dlgrad_amd.buffer import Buffer, PartialSum
+    from dlgrad_amd.device import Device
+    rng = np.random.default_rng(22)
+    for rows, n in ((16, 128 * 128), (5, 36), (40, 100)):
+        values = [rng.standard_normal((n,)).astype(np.float32) for _ in range(3)]
+        parts = rng.standard_normal((rows, 3 * n)).astype(np.float32)
+        results = {}
+        for pending in (True, False):
+            ps = [Tensor(v, requires_grad=True, device="hip") for v in values]
+            opt = nn.optim.Adam(ps, lr=1e-2, graph_safe=True)
+            b = Buffer.from_numpy(parts, Device.HIP)
+            whole = PartialSum.of(b, (3 * n,)) if pending else b.sum(0)
+            n0 = hip.launch_count
+            for i, p in enumerate(ps):
+                g = whole.piece(i * n, (n,)) if pending else Buffer(whole.ptr + i * n, (n,), Device.HIP)
+                p.grad = Tensor(g, device="hip")
+            opt.step()
+            if pending:
+                assert hip.launch_count - n0 == 2                      # the constants and the update
+                if not hip.COMPILE_ONLY:
+                    assert whole.pending and all(p.grad.data.pending for p in ps)
+                    want = b.sum(0).numpy()
+                    np.testing.assert_array_equal(ps[1].grad.numpy(), want[n:2 * n])
+                    assert not whole.pending and not ps[2].grad.data.pending
+                    np.testing.assert_array_equal(ps[2].grad.numpy(), want[2 * n:])
+            results[pending] = [p.numpy() for p in ps] + [opt.m[id(p)].numpy() for p in ps]
+        if not hip.COMPILE_ONLY:
+            for a, c in zip(results[True], results[False]):
+                np.testing.assert_array_equal(a, c)
