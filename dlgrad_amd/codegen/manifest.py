@@ -38,7 +38,7 @@ def merge(entries) -> None:
     """Adds (generator, params) pairs to kernels.json (sorted, de-duplicated)."""
     cur = {json.dumps([g, p]) for g, p in load()}
     cur |= {json.dumps([g, list(p)], default=list) for g, p in entries}
-    rows = sorted(json.loads(s) for s in cur)
+    rows = [json.loads(s) for s in sorted(cur)]            # by their text: parameters of one position may differ in type
     with open(PATH, "w") as f:
         f.write("[\n" + ",\n".join(json.dumps(r) for r in rows) + "\n]\n")
 
