@@ -1480,7 +1480,7 @@ class HIP:
             for path in (os.path.join(os.path.dirname(K.__file__), "matmul_tuned.json"), HIP._tuned_path()) if HIP.MATMUL_TABLE else ():
                 try:
                     with open(path) as f:
-                        table.update({k: v for k, v in json.load(f).items() if v in K.MATMUL_CONFIGS})
+                        table.update({k: v for k, v in json.load(f).items() if all(t in K.MATMUL_CONFIGS for t in v.split("+"))})
                 except (OSError, ValueError):
                     pass
             HIP._tuned = table
@@ -1591,11 +1591,16 @@ class HIP:
         return best
 
     @staticmethod
+    def _tile_key(M: int, N: int, Kd: int, batch: int, ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False) -> str:
+        """How the tile tables name a product."""
+        return f"{batch},{M},{N},{Kd}" + (",tn" if ta else ",nt" if tb else "") + (f",{tri}" if tri else "") + (",ld" if strided else "")
+
+    @staticmethod
     def _pick_tile(M: int, N: int, Kd: int, batch: int, veca: bool, vecb: bool, args: tuple,
                    ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False) -> str:
         if HIP.MATMUL_FORCE:
             return HIP.MATMUL_FORCE
-        key = f"{batch},{M},{N},{Kd}" + (",tn" if ta else ",nt" if tb else "") + (f",{tri}" if tri else "") + (",ld" if strided else "")
+        key = HIP._tile_key(M, N, Kd, batch, ta, tb, tri, strided)
         tile = HIP._tuned_table().get(key)
         if tile is not None:
             return tile
@@ -1741,13 +1746,20 @@ class HIP:
                 plan = False
             else:
                 cfgs, tails, grids, numels, has_e = [], [], [], [], []
+                # a pair that has been timed as a pair (the table's "pair:" entries) takes the two tiles that were fastest together,
+                # which need not be the ones that are fastest alone
+                pair_key = "pair:" + "|".join(HIP._tile_key(M, N, Kd, batch, ta, tb) + (f",{epi}" if epi else "")
+                                              for (_, _, ta, tb, epi, _), (M, N, Kd, _, batch, _, _, _) in zip(specs, parts))
+                together = None if HIP.MATMUL_FORCE else HIP._tuned_table().get(pair_key)
+                together = together.split("+") if together else None
                 for (x, y, ta, tb, epi, e), a, (M, N, Kd, nbc, batch, sa, sb, out_numel) in zip(specs, addrs, parts):
                     veca = (M if ta else Kd) % 4 == 0 and a[0] % 16 == 0
                     vecb = (Kd if tb else N) % 4 == 0 and a[1] % 16 == 0
                     if epi and e is not None and (a[2] % 16 or N % 4):
                         vecb = False
                     probe = alloc(out_numel)              # tiles are timed on a result of the real size
-                    tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, (a[0], a[1], probe.addr, M, N, Kd, nbc, *sa, *sb), ta, tb)
+                    tile = together[len(cfgs)] if together else HIP._pick_tile(
+                        M, N, Kd, batch, veca, vecb, (a[0], a[1], probe.addr, M, N, Kd, nbc, *sa, *sb), ta, tb)
                     bm, bn, _ = K.matmul_tile_shape(tile)
                     cfg = K.MATMUL_CONFIGS[tile]
                     cfgs.append((*cfg[:5], veca, vecb, ta, tb, "", False, epi, cfg[5] if len(cfg) > 5 else 32))
