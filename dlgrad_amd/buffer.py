@@ -281,14 +281,18 @@ class Buffer:
         kw = {"epi": epi, "e": e} if epi else {}
         return self._like(self._dispatch(BinaryOps.MATMUL, x=x, y=y, **self._tri(tri), **kw), out_shape)
 
-    def matmul_nt(self, other: "Buffer", tri: str = "", epi: str = "", e: "Buffer | None" = None) -> "Buffer":
-        """self (.., M, K) @ other(.., N, K)^T without materialising the transpose."""
+    def matmul_nt(self, other: "Buffer", tri: str = "", epi: str = "", e: "Buffer | None" = None,
+                  norm: tuple | None = None) -> "Buffer":
+        """self (.., M, K) @ other(.., N, K)^T without materialising the transpose.  norm (hip only, a single
+        row): (gain, eps) of an RMS normalisation applied to self on its way into the product, see HIP.matmul."""
         swapped = other.shape[:-2] + (other.shape[-1], other.shape[-2])
         p1, p2, out_shape = broadcast_shapes(self.shape, swapped)
         p2 = p2[:-2] + (p2[-1], p2[-2])
         x = self if self.shape == p1 else self._like(self.ptr, p1)
         y = other if other.shape == p2 else other._like(other.ptr, p2)
         kw = {"epi": epi, "e": e} if epi else {}
+        if norm is not None:
+            kw["norm"] = norm
         return self._like(self._dispatch(CustomOps.MATMUL_NT, x=x, y=y, **self._tri(tri), **kw), out_shape)
 
     def matmul_tn(self, other: "Buffer", tri: str = "") -> "Buffer":

@@ -2352,39 +2352,72 @@ MATMUL_TILE_MODEL = {
 # =====================================================================================
 
 @cache
-def row_matmul_nt_kernel(epi: str = "") -> tuple[str, str, str]:
+def row_matmul_nt_kernel(epi: str = "", norm_nval: int = 0) -> tuple[str, str, str]:
     """y[n] = sum_k x[k] * W[n][k] for one row x (K) and W stored (N, K): the linear layers of a
     decoding step, where an MFMA tile would hold one useful row in 16.  One wavefront per output:
     lane l multiplies the 16-byte items l, l + 64, ... of the row of W with the same items of x
     (K % 4 == 0, 16-byte aligned rows), four independent loads in flight, and the 64 partial sums are
-    added across the wavefront.  epi as in matmul_kernel ("add": + e[n], "relu", "gate": e[n] > 0)."""
+    added across the wavefront.  epi as in matmul_kernel ("add": + e[n], "relu", "gate": e[n] > 0).
+    norm_nval > 0: x is first RMS-normalised with the gain row g -- (x * r) * g with
+    r = 1 / sqrt(sum(x^2) / K + eps) -- by every wavefront for itself, the row (at most 64 * norm_nval
+    items) in registers: the statements of rmsnorm_fwd_kernel, so the values that enter the product
+    are the ones that kernel would have stored, and the launch between the two disappears."""
     assert epi in ("", "add", "relu", "gate")
-    name = f"row_matmul_nt{'_' + epi if epi else ''}"
+    name = f"row_matmul_nt{'_' + epi if epi else ''}{f'_rms{norm_nval}' if norm_nval else ''}"
     fin = {"": "acc", "add": "acc + e[n]", "relu": "(acc > 0.0f ? acc : 0.0f)", "gate": "(e[n] > 0.0f ? acc : 0.0f)"}[epi]
+    if norm_nval:
+        comps = (".x", ".y", ".z", ".w")
+        sq = " + ".join(f"v[k]{c} * v[k]{c}" for c in comps)
+        outs = "".join(f"            o{c} = (v[k]{c} * r) * g{c};\n" for c in comps)
+        body = f"""    float4 v[{norm_nval}];
+    float ss = 0.0f;
+    #pragma unroll
+    for (u32 k = 0; k < {norm_nval}u; ++k) {{
+        const u32 c = lane + k * 64u;
+        if (c < K4) {{ v[k] = x4[c]; ss += {sq}; }}
+    }}
+    ss = wave_sum(ss);
+    const float r = 1.0f / sqrtf(ss / (float)K + eps);
+    const float4* __restrict__ wv = reinterpret_cast<const float4*>(gain);
+    float acc = 0.0f;
+    #pragma unroll
+    for (u32 k = 0; k < {norm_nval}u; ++k) {{
+        const u32 c = lane + k * 64u;
+        if (c < K4) {{
+            const float4 g = wv[c];
+            float4 o;
+{outs}            acc = dot4(w4[c], o, acc);
+        }}
+    }}
+"""
+        extra, fmt = ", const float* __restrict__ gain, float eps", _fmt("P", "P", "P", "P", "I", "I", "P", "f")
+    else:
+        body = """    float acc = 0.0f;
+    u32 c = lane;
+    for (; c + 192u < K4; c += 256u) {
+        const float4 a0 = w4[c], a1 = w4[c + 64u], a2 = w4[c + 128u], a3 = w4[c + 192u];
+        const float4 b0 = x4[c], b1 = x4[c + 64u], b2 = x4[c + 128u], b3 = x4[c + 192u];
+        acc = dot4(a0, b0, acc); acc = dot4(a1, b1, acc); acc = dot4(a2, b2, acc); acc = dot4(a3, b3, acc);
+    }
+    for (; c < K4; c += 64u) acc = dot4(w4[c], x4[c], acc);
+"""
+        extra, fmt = "", _fmt("P", "P", "P", "P", "I", "I")
     src = f"""{PRELUDE}
 static __device__ __forceinline__ float dot4(float4 a, float4 b, float acc) {{
     acc = fmaf(a.x, b.x, acc); acc = fmaf(a.y, b.y, acc); acc = fmaf(a.z, b.z, acc); return fmaf(a.w, b.w, acc);
 }}
 extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ x,
-        const float* __restrict__ W, float* __restrict__ y, const float* __restrict__ e, u32 N, u32 K) {{
+        const float* __restrict__ W, float* __restrict__ y, const float* __restrict__ e, u32 N, u32 K{extra}) {{
     const u32 lane = threadIdx.x & 63u, n = blockIdx.x * 4u + (threadIdx.x >> 6);
     if (n >= N) return;
     const u32 K4 = K >> 2;
     const float4* __restrict__ w4 = reinterpret_cast<const float4*>(W + (u64)n * K);
     const float4* __restrict__ x4 = reinterpret_cast<const float4*>(x);
-    float acc = 0.0f;
-    u32 c = lane;
-    for (; c + 192u < K4; c += 256u) {{
-        const float4 a0 = w4[c], a1 = w4[c + 64u], a2 = w4[c + 128u], a3 = w4[c + 192u];
-        const float4 b0 = x4[c], b1 = x4[c + 64u], b2 = x4[c + 128u], b3 = x4[c + 192u];
-        acc = dot4(a0, b0, acc); acc = dot4(a1, b1, acc); acc = dot4(a2, b2, acc); acc = dot4(a3, b3, acc);
-    }}
-    for (; c < K4; c += 64u) acc = dot4(w4[c], x4[c], acc);
-    acc = wave_sum(acc);
+{body}    acc = wave_sum(acc);
     if (lane == 0u) y[n] = {fin};
 }}
 """
-    return src, name, _fmt("P", "P", "P", "P", "I", "I")
+    return src, name, fmt
 
 
 # =====================================================================================

@@ -136,23 +136,55 @@ def self_attention_qkv(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor, n_head: in
     return causal_self_attention(x.linear(wq, None), x.linear(wk, None), x.linear(wv, None), n_head, scale)
 
 
-def project_qkv_row(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor) -> tuple[Tensor, Tensor, Tensor]:
+def _row_norm(x: Tensor, w: Buffer, norm) -> tuple | None:
+    """(gain, eps) if the product of the single row x with w^T can RMS-normalise x on the way (hip device,
+    a norm with a gain, a row that fits the kernel), else None: the caller then applies the norm itself."""
+    if norm is None or norm.weight is None or not ops.FUSED or x.device is not Device.HIP or norm.weight.device is not Device.HIP:
+        return None
+    from dlgrad_amd.runtime.hip import HIP
+    return (norm.weight.data, norm.eps) if HIP.row_norm_fits(x.data, w, norm.weight.data) else None
+
+
+def project_qkv_row(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor, norm=None) -> tuple[Tensor, Tensor, Tensor]:
     """(x @ wq^T, x @ wk^T, x @ wv^T) for decoding.  When x is a single row and the weights are stacked
     in memory (stack_parameters), the hip device runs one product and the three results are the
-    thirds of its output row; such results carry no tape (inference only).  Otherwise three linears."""
+    thirds of its output row; such results carry no tape (inference only).  Otherwise three linears.
+    norm: an RMSNorm to apply to x first; in the one-product case it is applied inside the product."""
     if x.numel == x.shape[-1] and x.numel and ops.FUSED and ops.stacked(wq, wk, wv) and x.device is wq.device:
         C = wq.shape[0]
         w = Buffer(wq.data.ptr, (3 * C, wq.shape[1]), wq.device)
-        row = x.data.matmul_nt(w)
+        inside = _row_norm(x, w, norm)
+        row = x.data.matmul_nt(w, norm=inside) if inside else (x if norm is None else norm(x)).data.matmul_nt(w)
         shape = x.shape[:-1] + (C,)
         return tuple(Tensor(Buffer(row.ptr + i * C, shape, x.device), requires_grad=False) for i in range(3))
+    if norm is not None:
+        x = norm(x)
     return x.linear(wq, None), x.linear(wk, None), x.linear(wv, None)
 
 
-def mlp_relu(x: Tensor, w_fc: Tensor, w_proj: Tensor, residual: Tensor | None = None) -> Tensor:
+def norm_linear(x: Tensor, norm, weight: Tensor) -> Tensor:
+    """norm(x) @ weight^T.  For a single row on the hip device the normalisation happens inside the product
+    and the result carries no tape (decoding); otherwise the two ops."""
+    inside = _row_norm(x, weight.data, norm) if weight.ndim == 2 else None
+    if inside:
+        y = x.data.matmul_nt(weight.data, norm=inside)
+        return Tensor(y.reshape(x.shape[:-1] + (weight.shape[0],)), requires_grad=False)
+    return norm(x).linear(weight, None)
+
+
+def mlp_relu(x: Tensor, w_fc: Tensor, w_proj: Tensor, residual: Tensor | None = None, norm=None) -> Tensor:
     """relu(x @ w_fc^T) @ w_proj^T (+ residual): the bias-free feed-forward block of
     examples/gpt.py:69-78.  On the hip device one node whose ReLU, ReLU gradient and residual addition
-    happen as the products are stored (ops.MLPRelu); elsewhere the four ops."""
+    happen as the products are stored (ops.MLPRelu); elsewhere the four ops.
+    norm: an RMSNorm to apply to x first.  For a single row on the hip device it is applied inside the first
+    product, and the result then carries no tape (decoding)."""
+    if norm is not None:
+        inside = _row_norm(x, w_fc.data, norm) if (w_fc.ndim == 2 and w_proj.ndim == 2 and w_proj.device is x.device) else None
+        if inside and (residual is None or (residual.device is x.device and residual.shape == x.shape[:-1] + (w_proj.shape[0],))):
+            h = x.data.matmul_nt(w_fc.data, epi="relu", norm=inside)
+            y = h.matmul_nt(w_proj.data, epi="add", e=residual.data) if residual is not None else h.matmul_nt(w_proj.data)
+            return Tensor(y.reshape(x.shape[:-1] + (w_proj.shape[0],)), requires_grad=False)
+        x = norm(x)
     if ops.use_fused_epilogues(x, w_fc, w_proj) and (residual is None or (residual.device is x.device and residual.shape == x.shape[:-1] + (w_proj.shape[0],))):
         args = (x, w_fc, w_proj) if residual is None else (x, w_fc, w_proj, residual)
         return ops.MLPRelu.execute(*args)

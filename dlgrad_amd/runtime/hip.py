@@ -1611,7 +1611,7 @@ class HIP:
     @staticmethod
     @dispatcher.register(BinaryOps.MATMUL, Device.HIP)
     def matmul(x: Buffer, y: Buffer, ta: bool = False, tb: bool = False, tri: str = "", epi: str = "",
-               e: Buffer | None = None) -> DevicePtr:
+               e: Buffer | None = None, norm: tuple | None = None) -> DevicePtr:
         """x (.., M, K) @ y (.., K, N) for operands already padded to the same rank 2..4
         (buffer.py:231-243); batch dims of extent 1 broadcast through a zero stride as in
         cpu.py:519-532 and :553-559.  When y carries no batch at all the batch of x is
@@ -1620,9 +1620,22 @@ class HIP:
         tri: triangular structure of square (T x T) operands or outputs that the caller vouches
         for (K.matmul_kernel); the work it lets the kernel skip never changes a kept result.
         epi: "add" (result + e), "relu" (result where positive, else 0) or "gate" (result where e is
-        positive, else 0), applied as the result is stored; e has the shape of the result."""
+        positive, else 0), applied as the result is stored; e has the shape of the result.
+        norm: (gain, eps) -- x is a single row that is RMS-normalised with that gain row on its way into the
+        product (row_norm_fits says where this is provided): the RMSNorm launch in front of a linear layer
+        of a decoding step disappears, the values are those of the two launches."""
         xa, ya = x.ptr.addr, y.ptr.addr
         ea = 0 if e is None or e.ptr.__class__ is HostScalar else e.ptr.addr
+        if norm is not None:
+            if not HIP.row_norm_fits(x, y, norm[0]) or ta or not tb or tri:
+                raise ValueError(f"a normalising product is provided for one row against a transposed matrix, not {x.shape} x {y.shape}")
+            N, Kd = y.shape[-2:]
+            if epi not in ("", "add", "relu", "gate") or (epi in ("add", "gate") and (not ea or e.numel != N or ea & 15)):
+                raise ValueError(f"epilogue {epi!r} of a normalising product needs an aligned operand of {N} elements")
+            out = alloc(N)
+            k = kernel(K.row_matmul_nt_kernel, epi, K.rmsnorm_plan(Kd, 4))
+            launch(k, (N + 3) // 4, 256, xa, ya, out.addr, ea, N, Kd, _addr(norm[0]), float(norm[1]))
+            return out
         key = (x.shape, y.shape, ta, tb, tri, epi, None if e is None else e.shape, xa & 15, ya & 15, ea & 15,
                HIP.MATMUL_FORCE, HIP.ROW_MATMUL)
         plan = _matmul_plans.get(key)
@@ -1785,10 +1798,19 @@ class HIP:
         return outs
 
     @staticmethod
+    def row_norm_fits(x: Buffer, w: Buffer, gain: Buffer) -> bool:
+        """Whether the single-row product kernel takes x (one row of K) against w stored (N, K) and can RMS-normalise x
+        with the gain row on the way: the row fits a wavefront's registers and everything is read 16 bytes at a time."""
+        Kd = x.shape[-1] if x.ndim else 0
+        return (HIP.ROW_MATMUL and not HIP.MATMUL_FORCE and x.numel == Kd and Kd > 0 and Kd % 4 == 0 and w.ndim >= 2 and w.numel == w.shape[-2] * Kd
+                and w.shape[-1] == Kd and gain.numel == Kd and 0 < K.rmsnorm_plan(Kd, 4) <= 4
+                and not ((_addr(x) | _addr(w) | _addr(gain)) & 15))
+
+    @staticmethod
     @dispatcher.register(CustomOps.MATMUL_NT, Device.HIP)
-    def matmul_nt(x: Buffer, y: Buffer, tri: str = "", epi: str = "", e: Buffer | None = None) -> DevicePtr:
+    def matmul_nt(x: Buffer, y: Buffer, tri: str = "", epi: str = "", e: Buffer | None = None, norm: tuple | None = None) -> DevicePtr:
         """x (.., M, K) times the transpose of y (.., N, K), read in place."""
-        return HIP.matmul(x, y, tb=True, tri=tri, epi=epi, e=e)
+        return HIP.matmul(x, y, tb=True, tri=tri, epi=epi, e=e, norm=norm)
 
     @staticmethod
     @dispatcher.register(CustomOps.MATMUL_TN, Device.HIP)

@@ -87,9 +87,9 @@ class MLP:
         self.c_fc = nn.Linear(c.n_embd, 4 * c.n_embd, bias=False, device=c.device)
         self.c_proj = nn.Linear(4 * c.n_embd, c.n_embd, bias=False, device=c.device)
 
-    def __call__(self, x: Tensor, residual: Tensor | None = None) -> Tensor:
-        """c_proj(relu(c_fc(x))), plus the residual stream if given."""
-        return nn.mlp_relu(x, self.c_fc.weight, self.c_proj.weight, residual)
+    def __call__(self, x: Tensor, residual: Tensor | None = None, norm=None) -> Tensor:
+        """c_proj(relu(c_fc(x))), plus the residual stream if given; norm: the RMSNorm to apply to x first."""
+        return nn.mlp_relu(x, self.c_fc.weight, self.c_proj.weight, residual, norm)
 
 
 class Block:
@@ -247,9 +247,9 @@ class StaticDecoder:
         first[0, 0] = first_token
         self.seq.data.upload_(first)
 
-    def _attend(self, attn: CausalSelfAttention, x: Tensor, layer: int, hidden: Tensor, residual: Tensor) -> Tensor:
+    def _attend(self, attn: CausalSelfAttention, x: Tensor, norm, layer: int, hidden: Tensor, residual: Tensor) -> Tensor:
         T = self.model.config.block_size
-        q, k, v = nn.project_qkv_row(x, attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight)
+        q, k, v = nn.project_qkv_row(x, attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight, norm)
         self.cache.k[layer].data.row_store_(k.data, self.slot.data, also=(self.cache.v[layer].data, v.data))
         y = nn.cached_attention(q, self.cache.k[layer], self.cache.v[layer], T, attn.n_head, attn.scale, hidden)
         return attn.c_proj(y, residual)
@@ -269,10 +269,10 @@ class StaticDecoder:
         pos = slot + slot.clamp(min=0, max=1) if self.reference_positions else slot
         hidden = Tensor.arange((1, c.block_size), device=c.device) > slot                   # cache rows not written yet
         x = m.wte(self.tok) + m.wpe(pos)
-        for i, block in enumerate(m.blocks):
-            x = self._attend(block.attn, block.ln1(x), i, hidden, x)
-            x = block.mlp(block.ln2(x), x)
-        self._append(m.lm_head(m.ln_f(x)).reshape((1, c.vocab_size)).argmax(1))             # (1, 1)
+        for i, block in enumerate(m.blocks):                # each norm is applied by the product that consumes its row
+            x = self._attend(block.attn, x, block.ln1, i, hidden, x)
+            x = block.mlp(x, x, block.ln2)
+        self._append(nn.norm_linear(x, m.ln_f, m.lm_head.weight).reshape((1, c.vocab_size)).argmax(1))    # (1, 1)
 
     def step_window(self) -> None:
         """The step for a full window: tokens slot - block_size + 1 .. slot go through the whole model

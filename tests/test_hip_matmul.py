@@ -420,3 +420,48 @@ def test_large_products_do_not_travel_in_pairs():
         return
     np.testing.assert_array_equal(dx.numpy().view(np.uint32), gb.matmul(wb).numpy().view(np.uint32))
     np.testing.assert_array_equal(dw.numpy().view(np.uint32), gb.matmul_tn(xb).numpy().view(np.uint32))
+
+
+@pytest.mark.parametrize("K_,N,epi", [(128, 384, ""), (128, 512, "relu"), (128, 65, ""), (512, 128, "add"), (768, 7, ""), (1024, 260, "relu"),
+                                      (36, 20, "add")])
+def test_single_row_product_normalises_its_row_on_the_way(K_, N, epi):
+    """Decoding: RMSNorm followed by a linear layer on one row runs as one launch -- every wavefront of the
+    single-row product normalises the row for itself, with the statements of the RMSNorm kernel.  The result
+    must have the bits of the two launches, and be the float64 value to 2e-6 of the largest entry."""
+    require_gpu()
+    from dlgrad_amd import Tensor, nn
+    rng = np.random.default_rng(93)
+    x = rng.standard_normal((1, 1, K_), dtype=np.float32) * 3
+    w = rng.standard_normal((N, K_), dtype=np.float32) * K_ ** -0.5
+    gain = (1 + 0.1 * rng.standard_normal((1, K_))).astype(np.float32)
+    res = rng.standard_normal((1, 1, N), dtype=np.float32)
+    norm = nn.RMSNorm(K_, device="hip")
+    norm.weight = Tensor(gain, device="hip", requires_grad=True)
+    xt, wb, rb = Tensor(x, device="hip"), dev(w), dev(res)
+    assert hip.HIP.row_norm_fits(xt.data, wb, norm.weight.data)
+    kw = {"epi": epi, "e": rb if epi == "add" else None} if epi else {}
+    before = hip.launch_count
+    fused = xt.data.matmul_nt(wb, norm=(norm.weight.data, norm.eps), **kw)
+    assert hip.launch_count - before == 1
+    two = norm(xt).data.matmul_nt(wb, **kw)
+    if hip.COMPILE_ONLY:
+        return
+    np.testing.assert_array_equal(fused.numpy().view(np.uint32), two.numpy().view(np.uint32))
+    x64 = x.astype(np.float64)
+    y64 = (x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + norm.eps) * gain) @ w.T.astype(np.float64)
+    y64 = np.maximum(y64, 0) if epi == "relu" else y64 + res if epi == "add" else y64
+    assert np.abs(fused.numpy() - y64).max() <= 2e-6 * max(1.0, np.abs(y64).max())
+
+
+def test_rows_the_normalising_product_does_not_take():
+    require_gpu()
+    from dlgrad_amd.runtime.hip import HIP
+    g = lambda k: dev(np.ones((1, k), np.float32))                                      # noqa: E731
+    x = lambda *s: dev(np.ones(s, np.float32))                                          # noqa: E731
+    assert HIP.row_norm_fits(x(1, 1, 128), x(64, 128), g(128))
+    assert not HIP.row_norm_fits(x(1, 2, 128), x(64, 128), g(128))                      # two rows
+    assert not HIP.row_norm_fits(x(1, 1, 130), x(64, 130), g(130))                      # rows that are no whole 16-byte items
+    assert not HIP.row_norm_fits(x(1, 1, 2048), x(8, 2048), g(2048))                    # a row beyond the registers kept for it
+    assert not HIP.row_norm_fits(x(1, 1, 128), x(2, 64, 128), g(128))                   # a batch of matrices
+    with pytest.raises(ValueError):
+        x(1, 2, 128).matmul_nt(x(64, 128), norm=(g(128), 1e-6))
