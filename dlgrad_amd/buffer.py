@@ -293,6 +293,9 @@ class Buffer:
         kw = {"epi": epi, "e": e} if epi else {}
         if norm is not None:
             kw["norm"] = norm
+            if len(norm) > 2 and norm[2]:                 # also the normalised rows and their 1 / rms
+                out, yn, rinv = self._dispatch(CustomOps.MATMUL_NT, x=x, y=y, **self._tri(tri), **kw)
+                return self._like(out, out_shape), self._like(yn), self._like(rinv, (self.numel // max(self.shape[-1], 1),))
         return self._like(self._dispatch(CustomOps.MATMUL_NT, x=x, y=y, **self._tri(tri), **kw), out_shape)
 
     def matmul_tn(self, other: "Buffer", tri: str = "") -> "Buffer":

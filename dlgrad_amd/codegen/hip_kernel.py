@@ -1906,7 +1906,7 @@ MATMUL_TRI = ("", "out_lower", "a_lower", "at_lower")
 @cache
 def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb: bool,
                   ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False,
-                  epi: str = "", S: int = 32) -> tuple[str, str, str]:
+                  epi: str = "", S: int = 32, norm: bool = False) -> tuple[str, str, str]:
     """C[z] = op(A[z]) . op(B[z]), fp32, row-major, on the matrix cores (v_mfma_f32_32x32x2_f32, or
     v_mfma_f32_16x16x4_f32 for S = 16).
 
@@ -1955,6 +1955,13 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     strided: A, B and C have their own row pitches (lda, ldb, ldc, in floats) and C its own two batch
     strides, so operands and result can be matrices cut out of larger tensors -- the heads of a
     (B, T, h*d) projection are (T x d) matrices with pitch h*d, batch strides T*h*d and d.
+    norm: the rows of A are RMS-normalised on their way into the product -- (a * r) * gain with
+    r = 1 / sqrt(sum(a^2) / K + eps) per row -- for K <= BK, where a block's A tile holds whole rows:
+    once the tile is in LDS, each wavefront takes rows of it, a lane one 16-byte item, and rewrites them
+    with the statements of rmsnorm_fwd_kernel, so the product sees the values that kernel would have
+    stored.  The blocks of the first tile column also write the normalised rows to yn and r to rinv
+    (what the backward pass of the norm and of the product need) unless yn is null.  Arguments after
+    the others: gain, eps, yn, rinv.
     """
     BM, BN, T = S * MI * WM, S * NJ * WN, 64 * WM * WN
     NE = S * S // 64                                        # accumulator registers per MFMA tile
@@ -1963,6 +1970,9 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     name = (f"matmul_{BM}x{BN}x{BK}_w{WM}x{WN}_{'a4' if veca else 'a1'}{'b4' if vecb else 'b1'}"
             f"{'_tn' if ta else ''}{'_nt' if tb else ''}{'_' + tri if tri else ''}{'_ld' if strided else ''}{'_' + epi if epi else ''}{'_m16' if S == 16 else ''}")
     assert tri in MATMUL_TRI and not (tri == "a_lower" and ta) and not (tri == "at_lower" and not ta)
+    assert not norm or (veca and not ta and not tri and not strided and BK <= 256)
+    if norm:
+        name += "_rms"
     comp = ["x", "y", "z", "w"]
     vtype = {1: "float", 2: "float2", 3: "f3v", 4: "float4"}
 
@@ -2078,12 +2088,35 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     m0n0 = ("    const u32 m0 = ((tm + blockIdx.z) % tiles_m) * BM, n0 = tn * BN;" if tri
             else "    const u32 m0 = tm * BM, n0 = tn * BN;")
     skip_tile = "    if (n0 > m0 + BM - 1u) return;                    // the whole tile lies above the diagonal\n" if tri == "out_lower" else ""
+    norm_code = ""
+    if norm:
+        norm_code = f"""    {{   // every k of a row is in this tile (the launcher vouches for K <= BK): normalise the rows where they lie
+        const u32 K4 = g.K >> 2;
+        const bool keep = tn == 0u && yn != nullptr;          // one tile column writes what the backward pass needs
+        for (u32 rr = wave; rr < BM; rr += {WM * WN}u) {{
+            float4 av = make_float4(0.f, 0.f, 0.f, 0.f);
+            float ss = 0.0f;
+            if (lane < K4) {{ av = *reinterpret_cast<const float4*>(&As[0][rr][4u * lane]); ss += av.x * av.x + av.y * av.y + av.z * av.z + av.w * av.w; }}
+            ss = wave_sum(ss);
+            const float rs = 1.0f / sqrtf(ss / (float)g.K + eps);
+            if (lane < K4) {{
+                const float4 gn = reinterpret_cast<const float4*>(gain)[lane];
+                float4 o;
+                o.x = (av.x * rs) * gn.x; o.y = (av.y * rs) * gn.y; o.z = (av.z * rs) * gn.z; o.w = (av.w * rs) * gn.w;
+                *reinterpret_cast<float4*>(&As[0][rr][4u * lane]) = o;
+                if (keep && m0 + rr < g.M) reinterpret_cast<float4*>(yn + (u64)(m0 + rr) * g.K)[lane] = o;
+            }}
+            if (keep && lane == 0u && m0 + rr < g.M) rinv[m0 + rr] = rs;
+        }}
+    }}
+    __syncthreads();
+"""
     if tri in ("", "out_lower"):
-        kloop = """    const u32 nk = (g.K + BK - 1u) / BK;
+        kloop = f"""    const u32 nk = (g.K + BK - 1u) / BK;
     load_tiles(0u);
     stash_tiles(0u);
     __syncthreads();
-    for (u32 kt = 0; kt < nk; ++kt) {
+{norm_code}    for (u32 kt = 0; kt < nk; ++kt) {{
         const u32 buf = kt & 1u;"""
     else:
         krange = {"a_lower": "const u32 nk = (min(g.K, m0 + BM) + BK - 1u) / BK, kt0 = 0u;       // A is zero right of the diagonal",
@@ -2105,7 +2138,7 @@ struct MMArgs {{ u32 M, N, K, nbc, sa0, sa1, sb0, sb1; }};
 #define MI {MI}
 #define NJ {NJ}
 extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict__ A,
-        const float* __restrict__ B, float* __restrict__ C, MMArgs g) {{
+        const float* __restrict__ B, float* __restrict__ C, MMArgs g{", const float* __restrict__ E" if epi else ""}{", const float* __restrict__ gain, float eps, float* __restrict__ yn, float* __restrict__ rinv" if norm else ""}) {{
     {decl_a}
     {decl_b}
 
@@ -2169,8 +2202,7 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
     if epi:
         assert epi in ("add", "relu", "gate") and not strided
         macro = {"add": "((cv) + (ev))", "relu": "((cv) > 0.0f ? (cv) : 0.0f)", "gate": "((ev) > 0.0f ? (cv) : 0.0f)"}[epi]
-        edits = [("float* __restrict__ C, MMArgs g) {", "float* __restrict__ C, MMArgs g, const float* __restrict__ E) {"),
-                 ("C += (u64)blockIdx.z * g.M * g.N;", "C += (u64)blockIdx.z * g.M * g.N;\n    E += (u64)blockIdx.z * g.M * g.N;"),
+        edits = [("C += (u64)blockIdx.z * g.M * g.N;", "C += (u64)blockIdx.z * g.M * g.N;\n    E += (u64)blockIdx.z * g.M * g.N;"),
                  ("struct f3v {", f"#define EPI(cv, ev) {macro}\nstruct f3v {{")]
         if tb:
             edits.append(("crow[col] = acc[i][j][e];", "crow[col] = EPI(acc[i][j][e], ev[i][j][e]);"))
@@ -2210,7 +2242,7 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
         for was, now in edits:
             assert src.count(was) >= 1, was
             src = src.replace(was, now)
-        return src, name, _fmt("P", "P", "P", "8I", "P")
+        return src, name, _fmt("P", "P", "P", "8I", "P", *(("P", "f", "P", "P") if norm else ()))
     if strided:
         for was, now in (("struct MMArgs { u32 M, N, K, nbc, sa0, sa1, sb0, sb1; };",
                           "struct MMArgs { u32 M, N, K, nbc, sa0, sa1, sb0, sb1, lda, ldb, ldc, sc0, sc1; };"),
@@ -2223,7 +2255,7 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
             assert src.count(was) == 1, was
             src = src.replace(was, now)
         return src, name, _fmt("P", "P", "P", "13I")
-    return src, name, _fmt("P", "P", "P", "8I")
+    return src, name, _fmt("P", "P", "P", "8I", *(("P", "f", "P", "P") if norm else ()))
 
 
 @cache

@@ -1621,21 +1621,44 @@ class HIP:
         for (K.matmul_kernel); the work it lets the kernel skip never changes a kept result.
         epi: "add" (result + e), "relu" (result where positive, else 0) or "gate" (result where e is
         positive, else 0), applied as the result is stored; e has the shape of the result.
-        norm: (gain, eps) -- x is a single row that is RMS-normalised with that gain row on its way into the
-        product (row_norm_fits says where this is provided): the RMSNorm launch in front of a linear layer
-        of a decoding step disappears, the values are those of the two launches."""
+        norm: (gain, eps[, keep]) -- the rows of x are RMS-normalised with that gain row on their way into the
+        product (row_norm_fits / tile_norm_fits say where this is provided): the RMSNorm launch in front of a
+        linear layer disappears, the values are those of the two launches.  With keep the normalised rows and
+        the per-row 1 / rms are returned as well: (result, normalised x, rinv)."""
         xa, ya = x.ptr.addr, y.ptr.addr
         ea = 0 if e is None or e.ptr.__class__ is HostScalar else e.ptr.addr
         if norm is not None:
-            if not HIP.row_norm_fits(x, y, norm[0]) or ta or not tb or tri:
-                raise ValueError(f"a normalising product is provided for one row against a transposed matrix, not {x.shape} x {y.shape}")
-            N, Kd = y.shape[-2:]
-            if epi not in ("", "add", "relu", "gate") or (epi in ("add", "gate") and (not ea or e.numel != N or ea & 15)):
-                raise ValueError(f"epilogue {epi!r} of a normalising product needs an aligned operand of {N} elements")
-            out = alloc(N)
-            k = kernel(K.row_matmul_nt_kernel, epi, K.rmsnorm_plan(Kd, 4))
-            launch(k, (N + 3) // 4, 256, xa, ya, out.addr, ea, N, Kd, _addr(norm[0]), float(norm[1]))
-            return out
+            gain, eps, keep = norm[0], float(norm[1]), len(norm) > 2 and bool(norm[2])
+            if epi not in ("", "add", "relu", "gate") or ta or tri:
+                raise ValueError(f"a normalising product does not take epi={epi!r}, ta={ta}, tri={tri!r}")
+            if not keep and tb and HIP.row_norm_fits(x, y, gain):
+                N, Kd = y.shape[-2:]
+                if epi in ("add", "gate") and (not ea or e.numel != N or ea & 15):
+                    raise ValueError(f"epilogue {epi!r} of a normalising product needs an aligned operand of {N} elements")
+                out = alloc(N)
+                k = kernel(K.row_matmul_nt_kernel, epi, K.rmsnorm_plan(Kd, 4))
+                launch(k, (N + 3) // 4, 256, xa, ya, out.addr, ea, N, Kd, _addr(gain), eps)
+                return out
+            if not HIP.tile_norm_fits(x, y, gain, tb):
+                raise ValueError(f"a normalising product is not provided for {x.shape} x {y.shape}")
+            Kd = x.shape[-1]
+            M, N = x.numel // Kd, y.shape[-2] if tb else y.shape[-1]
+            if epi in ("add", "gate") and (not ea or e.numel != M * N):
+                raise ValueError(f"epilogue {epi!r} needs an operand shaped like the result ({M * N} elements)")
+            out = alloc(M * N)
+            yn, rinv = (alloc(M * Kd), alloc(M)) if keep else (None, None)
+            vecb = (Kd if tb else N) % 4 == 0 and not (ya & 15)
+            if epi and e is not None and (ea & 15 or N % 4):
+                vecb = False                                   # the epilogue reads e as it writes the result
+            tile = HIP.MATMUL_FORCE if K.MATMUL_CONFIGS.get(HIP.MATMUL_FORCE, (0,) * 5)[4] >= Kd else \
+                ("64x64m16k128" if N >= 256 and M >= 64 else "32x32m16k128")       # tiles whose k step holds a whole row
+            cfg = K.MATMUL_CONFIGS[tile]
+            bm, bn, threads = K.matmul_tile_shape(tile)
+            k = kernel(K.matmul_kernel, *cfg[:5], True, vecb, False, tb, "", False, epi, cfg[5] if len(cfg) > 5 else 32, True)
+            HIP.last_matmul_kernel = kernel_names.get(id(k))
+            tail = ((ea or out.addr,) if epi else ()) + (_addr(gain), eps, yn.addr if keep else 0, rinv.addr if keep else 0)
+            launch(k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, 1), threads, xa, ya, out.addr, M, N, Kd, 1, 0, 0, 0, 0, *tail)
+            return (out, yn, rinv) if keep else out
         key = (x.shape, y.shape, ta, tb, tri, epi, None if e is None else e.shape, xa & 15, ya & 15, ea & 15,
                HIP.MATMUL_FORCE, HIP.ROW_MATMUL)
         plan = _matmul_plans.get(key)
@@ -1805,6 +1828,16 @@ class HIP:
         return (HIP.ROW_MATMUL and not HIP.MATMUL_FORCE and x.numel == Kd and Kd > 0 and Kd % 4 == 0 and w.ndim >= 2 and w.numel == w.shape[-2] * Kd
                 and w.shape[-1] == Kd and gain.numel == Kd and 0 < K.rmsnorm_plan(Kd, 4) <= 4
                 and not ((_addr(x) | _addr(w) | _addr(gain)) & 15))
+
+    @staticmethod
+    def tile_norm_fits(x: Buffer, w: Buffer, gain: Buffer, tb: bool = True) -> bool:
+        """Whether the tile product can RMS-normalise the rows of x (.., K) on their way: K fits one k step of the
+        deepest tiles (so a block's tile of x holds whole rows), w is a single matrix -- (N, K) if tb else (K, N) --
+        and x and the gain row are read 16 bytes at a time."""
+        Kd = x.shape[-1] if x.ndim else 0
+        return (0 < Kd <= 128 and Kd % 4 == 0 and x.numel >= Kd and x.numel < 2 ** 31 and w.ndim >= 2 and w.numel == w.shape[-1] * w.shape[-2]
+                and (w.shape[-1] if tb else w.shape[-2]) == Kd and gain.numel == Kd and w.numel < 2 ** 31
+                and (x.numel // Kd) * (w.numel // Kd) < 2 ** 31 and not ((_addr(x) | _addr(gain)) & 15))
 
     @staticmethod
     @dispatcher.register(CustomOps.MATMUL_NT, Device.HIP)

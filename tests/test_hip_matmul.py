@@ -463,5 +463,46 @@ def test_rows_the_normalising_product_does_not_take():
     assert not HIP.row_norm_fits(x(1, 1, 130), x(64, 130), g(130))                      # rows that are no whole 16-byte items
     assert not HIP.row_norm_fits(x(1, 1, 2048), x(8, 2048), g(2048))                    # a row beyond the registers kept for it
     assert not HIP.row_norm_fits(x(1, 1, 128), x(2, 64, 128), g(128))                   # a batch of matrices
+    assert HIP.tile_norm_fits(x(1, 2, 128), x(64, 128), g(128))                         # several rows: the tile product takes them,
+    assert not HIP.tile_norm_fits(x(4, 256), x(64, 256), g(256))                        # up to 128 floats a row
+    assert not HIP.tile_norm_fits(x(4, 128), x(2, 64, 128), g(128))
     with pytest.raises(ValueError):
-        x(1, 2, 128).matmul_nt(x(64, 128), norm=(g(128), 1e-6))
+        x(1, 2, 130).matmul_nt(x(64, 130), norm=(g(130), 1e-6))
+
+
+@pytest.mark.parametrize("xs,N,epi,tile", [((16, 128, 128), 384, "", ""), ((16, 128, 128), 512, "relu", ""), ((1, 128, 128), 65, "", ""),
+                                           ((3, 50, 36), 20, "add", ""), ((2048, 128), 128, "", "64x64m16k128"), ((70, 64), 260, "relu", "32x32m16k128"),
+                                           ((1, 1, 128), 384, "", "32x32m16k128")])
+def test_tile_product_normalises_the_rows_of_its_left_operand(xs, N, epi, tile, monkeypatch):
+    """RMSNorm followed by a linear layer as one launch for rows of up to 128 floats: a block's tile of x holds whole
+    rows (one k step), which its wavefronts normalise in LDS with the statements of the RMSNorm kernel before the
+    matrix steps begin.  Result, normalised rows and 1 / rms must have the bits of the two launches."""
+    require_gpu()
+    from dlgrad_amd import Tensor, nn
+    from dlgrad_amd.runtime.hip import HIP
+    if tile:
+        monkeypatch.setattr(HIP, "MATMUL_FORCE", tile)
+    rng = np.random.default_rng(94)
+    Kd = xs[-1]
+    x = rng.standard_normal(xs, dtype=np.float32) * 2
+    w = rng.standard_normal((N, Kd), dtype=np.float32) * Kd ** -0.5
+    gain = (1 + 0.1 * rng.standard_normal((1, Kd))).astype(np.float32)
+    res = rng.standard_normal(xs[:-1] + (N,), dtype=np.float32)
+    xb, wb, gb, rb = dev(x), dev(w), dev(gain), dev(res)
+    assert HIP.tile_norm_fits(xb, wb, gb)
+    kw = {"epi": epi, "e": rb if epi == "add" else None} if epi else {}
+    before = hip.launch_count
+    out, yn, rinv = xb.matmul_nt(wb, norm=(gb, 1e-6, True), **kw)
+    assert hip.launch_count - before == 1 and "_rms" in (HIP.last_matmul_kernel or "_rms")
+    only = xb.matmul_nt(wb, norm=(gb, 1e-6), **kw) if x.size > Kd else out               # (a single row takes the row kernel)
+    y2, r2 = xb.rmsnorm(gb, 1e-6)
+    out2 = y2.matmul_nt(wb, **kw)
+    assert out.shape == out2.shape and yn.shape == y2.shape and rinv.shape == r2.shape
+    if hip.COMPILE_ONLY:
+        return
+    for name, a, b in (("result", out, out2), ("result alone", only, out2), ("normalised rows", yn, y2), ("1 / rms", rinv, r2)):
+        np.testing.assert_array_equal(a.numpy().view(np.uint32), b.numpy().view(np.uint32), err_msg=name)
+    x64 = x.astype(np.float64)
+    y64 = (x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + 1e-6) * gain) @ w.T.astype(np.float64)
+    y64 = np.maximum(y64, 0) if epi == "relu" else y64 + res if epi == "add" else y64
+    check_mm(out.numpy(), y64, "against float64")
