@@ -2093,7 +2093,8 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
         norm_code = f"""    {{   // every k of a row is in this tile (the launcher vouches for K <= BK): normalise the rows where they lie
         const u32 K4 = g.K >> 2;
         const bool keep = tn == 0u && yn != nullptr;          // one tile column writes what the backward pass needs
-        for (u32 rr = wave; rr < BM; rr += {WM * WN}u) {{
+        #pragma unroll
+        for (u32 rr = wave; rr < BM; rr += {WM * WN}u) {{           // (the rows of a wavefront are independent: their chains overlap)
             float4 av = make_float4(0.f, 0.f, 0.f, 0.f);
             float ss = 0.0f;
             if (lane < K4) {{ av = *reinterpret_cast<const float4*>(&As[0][rr][4u * lane]); ss += av.x * av.x + av.y * av.y + av.z * av.z + av.w * av.w; }}

@@ -126,13 +126,18 @@ def stack_parameters(tensors: list) -> None:
         t.data = part
 
 
-def self_attention_qkv(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor, n_head: int, scale: float) -> Tensor:
+def self_attention_qkv(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor, n_head: int, scale: float, norm=None) -> Tensor:
     """causal_self_attention(x @ wq^T, x @ wk^T, x @ wv^T, n_head, scale) for x (B, T, C) and three
     (C, C) weights: the projections and attention of examples/gpt.py:45-57.  When the weights are
     stacked in memory (stack_parameters) the hip device runs one projection and reads q, k, v out
-    of its result in place (ops.SelfAttentionQKV)."""
+    of its result in place (ops.SelfAttentionQKV).  norm: an RMSNorm to apply to x first; where the
+    one-projection form runs and the rows are short enough, that projection applies it."""
     if ops.use_fused_qkv_attention(x, wq, wk, wv, n_head):
-        return ops.SelfAttentionQKV.execute(x, wq, wk, wv, n_head=n_head, scale=scale)
+        if norm is not None and ops.tile_norm_applies(x, wq, norm):
+            return ops.SelfAttentionQKV.execute(x, wq, wk, wv, norm.weight, n_head=n_head, scale=scale, eps=norm.eps)
+        return ops.SelfAttentionQKV.execute(x if norm is None else norm(x), wq, wk, wv, n_head=n_head, scale=scale)
+    if norm is not None:
+        x = norm(x)
     return causal_self_attention(x.linear(wq, None), x.linear(wk, None), x.linear(wv, None), n_head, scale)
 
 
@@ -169,6 +174,8 @@ def norm_linear(x: Tensor, norm, weight: Tensor) -> Tensor:
     if inside:
         y = x.data.matmul_nt(weight.data, norm=inside)
         return Tensor(y.reshape(x.shape[:-1] + (weight.shape[0],)), requires_grad=False)
+    if ops.tile_norm_applies(x, weight, norm):
+        return ops.NormLinearNT.execute(x, weight, norm.weight, eps=norm.eps)
     return norm(x).linear(weight, None)
 
 
@@ -184,6 +191,8 @@ def mlp_relu(x: Tensor, w_fc: Tensor, w_proj: Tensor, residual: Tensor | None = 
             h = x.data.matmul_nt(w_fc.data, epi="relu", norm=inside)
             y = h.matmul_nt(w_proj.data, epi="add", e=residual.data) if residual is not None else h.matmul_nt(w_proj.data)
             return Tensor(y.reshape(x.shape[:-1] + (w_proj.shape[0],)), requires_grad=False)
+        if residual is x and ops.use_fused_epilogues(x, w_fc, w_proj) and w_proj.shape[0] == x.shape[-1] and ops.tile_norm_applies(x, w_fc, norm):
+            return ops.NormMLPRelu.execute(x, w_fc, w_proj, norm.weight, eps=norm.eps)       # x + mlp(norm(x)) as one node
         x = norm(x)
     if ops.use_fused_epilogues(x, w_fc, w_proj) and (residual is None or (residual.device is x.device and residual.shape == x.shape[:-1] + (w_proj.shape[0],))):
         args = (x, w_fc, w_proj) if residual is None else (x, w_fc, w_proj, residual)

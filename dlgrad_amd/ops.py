@@ -345,6 +345,54 @@ def product_pair(first: tuple, second: tuple) -> tuple:
     return tuple(out)
 
 
+def tile_norm_applies(x, w, norm) -> bool:
+    """Whether the product of the rows of x with w^T can apply the RMSNorm `norm` to x on the way (hip device, fused
+    kernels on, a norm with a gain row, rows of at most 128 floats)."""
+    if norm is None or norm.weight is None or not FUSED or x.device is not Device.HIP or norm.weight.device is not Device.HIP:
+        return False
+    from dlgrad_amd.runtime import hip
+    how = hip.HIP.NORM_IN_PRODUCT
+    if how == "0" or (how != "always" and hip.in_graph()):
+        return False
+    return w.ndim == 2 and hip.HIP.tile_norm_fits(x.data, w.data if hasattr(w, "data") else w, norm.weight.data)
+
+
+class _NormInFront:
+    """What the ops below share when an RMSNorm sits in front of their first product and is applied inside it:
+    they keep x, the gain, the normalised rows (the left operand of the weight gradient) and 1 / rms per row,
+    and finish their backward pass with the norm's own backward kernel, which -- like ops.RMSNorm -- can add
+    what x has collected so far as it stores dx."""
+
+    def _through_norm(self, dxn: Buffer, plus: Buffer | None) -> tuple:
+        return self.x.rmsnorm_bwd(self.gain, self.r, dxn, through_mean=not STRICT_REFERENCE, plus=plus)
+
+    def _plus(self, have: tuple) -> Buffer | None:
+        return have[0] if (have[0] is not None and have[0].shape == self.x.shape and have[0].device is self.x.device) else None
+
+
+class NormLinearNT(OP, _NormInFront):
+    """rmsnorm(x, gain) @ W^T for W stored (out, in): RMSNorm followed by LinearNT (the final norm and lm_head of
+    examples/gpt.py:100-101) with the normalisation done by the product kernel on its tile of x.  Same values as the
+    two nodes, one launch fewer forward."""
+
+    def forward(self, x: Buffer, w: Buffer, gain: Buffer, eps: float = 1e-6) -> Buffer:
+        self.x, self.w, self.gain = x, w, gain
+        out, self.xn, self.r = x.matmul_nt(w, norm=(gain, eps, True))
+        return out
+
+    def _grads(self, upstream_grad: Buffer, plus: Buffer | None) -> tuple:
+        dxn, dw = product_pair(("nn", upstream_grad, self.w), ("tn", upstream_grad, self.xn))
+        dx, dgain = self._through_norm(unbroadcast(dxn, self.x.shape), plus)
+        return dx, unbroadcast(dw, self.w.shape), dgain
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return self._grads(upstream_grad, None)
+
+    def backward_onto(self, upstream_grad: Buffer, have: tuple) -> tuple:
+        plus = self._plus(have)
+        return self._grads(upstream_grad, plus), ((0,) if plus is not None else ())
+
+
 class LinearNT(OP):
     """x @ W^T for W stored (out, in), the product inside Tensor.linear (tensor.py:549-563),
     with W read in place.  The reference builds it as Transpose -> MatMul, i.e. one permute
@@ -388,13 +436,42 @@ class MLPRelu(OP):
         self.gate = self.h                                  # positive where the ReLU let the value through
         return self.h.matmul_nt(w2, epi="add", e=r) if r is not None else self.h.matmul_nt(w2)
 
-    def backward(self, upstream_grad: Buffer) -> tuple:
+    def _products(self, upstream_grad: Buffer, left: Buffer) -> tuple:
+        """(gradient of the first product's left operand, dw1, dw2); `left` is that operand."""
         # each gradient of an input travels with the weight gradient that reads the same upstream tensor
         gh, dw2 = product_pair(("nn", upstream_grad, self.w2, "gate", self.gate),      # gradient before the ReLU
                                ("tn", upstream_grad, self.h))
-        dx, dw1 = product_pair(("nn", gh, self.w1), ("tn", gh, self.x))
-        dw2, dx, dw1 = unbroadcast(dw2, self.w2.shape), unbroadcast(dx, self.x.shape), unbroadcast(dw1, self.w1.shape)
+        dx, dw1 = product_pair(("nn", gh, self.w1), ("tn", gh, left))
+        return unbroadcast(dx, self.x.shape), unbroadcast(dw1, self.w1.shape), unbroadcast(dw2, self.w2.shape)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        dx, dw1, dw2 = self._products(upstream_grad, self.x)
         return (dx, dw1, dw2, upstream_grad) if self.has_r else (dx, dw1, dw2)
+
+
+class NormMLPRelu(MLPRelu, _NormInFront):
+    """x + MLPRelu(rmsnorm(x, gain)): the second half of a transformer block (examples/gpt.py:85) with the norm
+    applied inside the first product.  The residual is x itself, so on the way back its gradient -- the upstream
+    gradient -- is added by the norm's backward kernel as it stores dx, as it is when the nodes are separate."""
+
+    def forward(self, x: Buffer, w1: Buffer, w2: Buffer, gain: Buffer, eps: float = 1e-6) -> Buffer:
+        self.x, self.w1, self.w2, self.gain = x, w1, w2, gain
+        self.h, self.xn, self.r = x.matmul_nt(w1, epi="relu", norm=(gain, eps, True))
+        self.gate = self.h
+        return self.h.matmul_nt(w2, epi="add", e=x)
+
+    def _grads(self, upstream_grad: Buffer, have: Buffer | None) -> tuple:
+        dxn, dw1, dw2 = self._products(upstream_grad, self.xn)
+        plus = upstream_grad if have is None else have + upstream_grad
+        dx, dgain = self._through_norm(dxn, plus)
+        return dx, dw1, dw2, dgain
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return self._grads(upstream_grad, None)
+
+    def backward_onto(self, upstream_grad: Buffer, have: tuple) -> tuple:
+        plus = self._plus(have)
+        return self._grads(upstream_grad, plus), ((0,) if plus is not None else ())
 
 
 def use_fused_epilogues(x, *weights) -> bool:
@@ -548,24 +625,39 @@ class SelfAttentionQKV(OP):
     the weight gradients have the bits of the separate products; dx adds its 3C terms in one
     accumulator instead of three partial sums, so it differs from them by rounding."""
 
-    def forward(self, x: Buffer, wq: Buffer, wk: Buffer, wv: Buffer, n_head: int, scale: float) -> Buffer:
+    def forward(self, x: Buffer, wq: Buffer, wk: Buffer, wv: Buffer, gain: Buffer | None = None, n_head: int = 1,
+                scale: float = 1.0, eps: float = 1e-6) -> Buffer:
+        """gain: the gain row of an RMSNorm that sits in front of the projection and is applied inside it."""
         C = wq.shape[0]
-        self.x, self.n_head, self.scale = x, n_head, scale
+        self.x, self.n_head, self.scale, self.gain = x, n_head, scale, gain
         self.w = Buffer(wq.ptr, (3 * C, C), x.device)                    # the three matrices as one
-        self.qkv = x.matmul_nt(self.w)
+        if gain is None:
+            self.qkv, self.left = x.matmul_nt(self.w), x
+        else:
+            self.qkv, self.left, self.r = x.matmul_nt(self.w, norm=(gain, eps, True))
         self.y, self.p = self.qkv.causal_attention_qkv(n_head, scale)
         return self.y
 
-    def backward(self, upstream_grad: Buffer) -> tuple:
+    def _grads(self, upstream_grad: Buffer, plus: Buffer | None) -> tuple:
         C = self.w.shape[1]
         g = self.qkv.causal_attention_qkv_bwd(self.p, upstream_grad, self.n_head, self.scale, self.y)     # (B, T, 3C)
-        dx, dw = product_pair(("nn", g, self.w), ("tn", g, self.x))
+        dx, dw = product_pair(("nn", g, self.w), ("tn", g, self.left))
         dw = unbroadcast(dw, self.w.shape)                                                        # (3C, C)
         if dw.__class__ is PartialSum:
             part = lambda i: dw.piece(i * C * C, (C, C))                                          # noqa: E731  (stays pending)
         else:
             part = lambda i: Buffer(dw.ptr + i * C * C, (C, C), dw.device)                        # noqa: E731
-        return dx, part(0), part(1), part(2)
+        if self.gain is None:
+            return dx, part(0), part(1), part(2)
+        dx, dgain = _NormInFront._through_norm(self, dx, plus)
+        return dx, part(0), part(1), part(2), dgain
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        return self._grads(upstream_grad, None)
+
+    def backward_onto(self, upstream_grad: Buffer, have: tuple) -> tuple:
+        plus = _NormInFront._plus(self, have) if self.gain is not None else None
+        return self._grads(upstream_grad, plus), ((0,) if plus is not None else ())
 
 
 def use_fused_rmsnorm(x, weight) -> bool:

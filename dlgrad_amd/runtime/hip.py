@@ -262,6 +262,11 @@ def capturing() -> bool:
     return _capturing
 
 
+def in_graph() -> bool:
+    """Whether a Graph's arena is current: the step being issued is a warm-up for a capture, or is being captured."""
+    return _graph_depth > 0
+
+
 class Graph:
     """A whole step -- hundreds of launches -- recorded once and replayed as one submission.
 
@@ -1450,6 +1455,11 @@ class HIP:
     DECODE_FUSED = os.environ.get("DLGRAD_HIP_DECODE_FUSED", "1") != "0"    # "0": cached attention as product, softmax, product
     MATMUL_PAIRS = os.environ.get("DLGRAD_HIP_MATMUL_PAIRS", "1") != "0"       # "0": the two products of a linear layer's backward as two launches
     MATMUL_PAIR_MAX_FLOP = 1 << 30        # per product: beyond it a product fills the chip by itself
+    # An RMSNorm in front of a linear layer applied by the product's blocks: "1" where launches are issued one by one (a launch
+    # fewer: char-GPT eager step 1.49 -> 1.33 ms), not in steps that are captured (every column block of the product
+    # normalises its rows again, which costs a replayed step more than the node it saves: 0.635 -> 0.647 ms); "0" never,
+    # "always" also in captured steps
+    NORM_IN_PRODUCT = os.environ.get("DLGRAD_HIP_NORM_IN_PRODUCT", "1")
     CAUSAL_MASK_KNOWN = os.environ.get("DLGRAD_HIP_CAUSAL_MASK_KNOWN", "1") != "0"   # "0": the cached causal mask is read like any other mask
     CE_GRAD_ROWS = os.environ.get("DLGRAD_HIP_CE_GRAD_ROWS", "1") != "0"       # "0": the cross-entropy gradient as an element-wise launch
     ATTENTION_FUSED = os.environ.get("DLGRAD_HIP_ATTENTION_FUSED", "1") != "0"   # "0": short causal attention as products and softmax launches too

@@ -37,18 +37,18 @@ class CausalSelfAttention:
         nn.stack_parameters([self.q_proj.weight, self.k_proj.weight, self.v_proj.weight])
 
     def __call__(self, x: Tensor, cache: "KVCache | None" = None, layer: int = 0,
-                 residual: Tensor | None = None) -> Tensor:
+                 residual: Tensor | None = None, norm=None) -> Tensor:
         """Without a cache, or with an empty one: causal attention over the T positions of x
         (whose k/v projections are stored if a cache is given).  With a filled cache and
         T == 1: the new position attends to everything cached plus itself, no mask
-        (examples/gpt.py:44-66)."""
+        (examples/gpt.py:44-66).  norm: the RMSNorm to apply to x first (the projections apply it where they can)."""
         T = x.shape[1]
         if cache is None:
             # q, k, v projections, split into heads, ((q @ k^T) * scale).masked_fill(mask, -inf).softmax(dim=3) @ v,
             # merge the heads (examples/gpt.py:45-57): one node on the hip device
             return self.c_proj(nn.self_attention_qkv(x, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight,
-                                                     self.n_head, self.scale), residual)
-        q_lin, k_lin, v_lin = nn.project_qkv_row(x, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight)   # (B, T, C)
+                                                     self.n_head, self.scale, norm), residual)
+        q_lin, k_lin, v_lin = nn.project_qkv_row(x, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight, norm)   # (B, T, C)
         if cache.length > 0:
             assert T == 1, "incremental attention takes one new position"
             cache.write(layer, k_lin, v_lin, cache.length)
@@ -100,8 +100,8 @@ class Block:
         self.mlp = MLP(c)
 
     def __call__(self, x: Tensor, cache: KVCache | None = None, layer: int = 0) -> Tensor:
-        x = self.attn(self.ln1(x), cache, layer, residual=x)          # x + attention(norm(x))
-        return self.mlp(self.ln2(x), residual=x)                      # x + mlp(norm(x))
+        x = self.attn(x, cache, layer, residual=x, norm=self.ln1)     # x + attention(norm(x))
+        return self.mlp(x, residual=x, norm=self.ln2)                 # x + mlp(norm(x))
 
 
 _position_ids: dict = {}
@@ -131,7 +131,7 @@ class GPT:
         x = self.wte(idx) + self.wpe(_positions(T, idx.device))
         for block in self.blocks:
             x = block(x)
-        logits = self.lm_head(self.ln_f(x))
+        logits = nn.norm_linear(x, self.ln_f, self.lm_head.weight)
         if targets is None:
             return logits, None
         V = self.config.vocab_size

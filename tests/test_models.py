@@ -185,20 +185,24 @@ class ReluBranches:
 
         monkeypatch.setattr(ops.Relu, "forward", forward)
         monkeypatch.setattr(ops.Relu, "backward", backward)
-        fused0 = ops.MLPRelu.forward
+        def holds_its_relu(cls):                         # the feed-forward nodes hold their ReLU inside
+            fused0 = cls.forward
 
-        def fused_forward(node, *args):                 # the feed-forward node holds its ReLU inside
-            out = fused0(node, *args)
-            if not (hip.COMPILE_ONLY or record):
-                mask = node.h.numpy() > 0
-                want = tape.masks[tape.cursor]
-                tape.cursor += 1
-                tape.differing += int((mask != want).sum())
-                tape.total += mask.size
-                node.gate = Buffer.from_numpy(want.astype(np.float32), node.h.device)
-            return out
+            def fused_forward(node, *args, **kwargs):
+                out = fused0(node, *args, **kwargs)
+                if not (hip.COMPILE_ONLY or record):
+                    mask = node.h.numpy() > 0
+                    want = tape.masks[tape.cursor]
+                    tape.cursor += 1
+                    tape.differing += int((mask != want).sum())
+                    tape.total += mask.size
+                    node.gate = Buffer.from_numpy(want.astype(np.float32), node.h.device)
+                return out
 
-        monkeypatch.setattr(ops.MLPRelu, "forward", fused_forward)
+            monkeypatch.setattr(cls, "forward", fused_forward)
+
+        holds_its_relu(ops.MLPRelu)
+        holds_its_relu(ops.NormMLPRelu)
 
 
 @pytest.mark.gpu
@@ -673,3 +677,28 @@ def test_pieces_of_a_pending_sum_stay_pending_for_the_one_launch_adam():
         if not hip.COMPILE_ONLY:
             for a, c in zip(results[True], results[False]):
                 np.testing.assert_array_equal(a, c)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cfg", [TINY, C4], ids=["tiny", "char-gpt"])
+def test_norms_applied_inside_products_leave_every_bit_of_a_gpt_step(cfg, monkeypatch):
+    """Issued launch by launch, a step lets each RMSNorm be applied by the product that consumes its rows
+    (qkv projection, first feed-forward product, lm_head): 13 launches fewer on the char model.  The product's
+    blocks run the norm kernel's statements, the backward pass ends in the norm's own backward kernel, so
+    logits, loss, every gradient and every updated parameter must have the bits of the step with separate norms."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    runs = {}
+    for how in ("1", "0"):
+        monkeypatch.setattr(hip.HIP, "NORM_IN_PRODUCT", how)
+        n0 = hip.launch_count
+        _, logits, loss, grads, new = gpt_step("hip", cfg)
+        runs[how] = (hip.launch_count - n0, logits, loss, grads, new)
+    assert runs["0"][0] - runs["1"][0] == 2 * cfg["n_layer"] + 1
+    if hip.COMPILE_ONLY:
+        return
+    np.testing.assert_array_equal(runs["1"][1], runs["0"][1])
+    np.testing.assert_array_equal(runs["1"][2], runs["0"][2])
+    for k in runs["0"][3]:
+        np.testing.assert_array_equal(runs["1"][3][k], runs["0"][3][k], err_msg=f"grad {k}")
+        np.testing.assert_array_equal(runs["1"][4][k], runs["0"][4][k], err_msg=f"param {k}")
