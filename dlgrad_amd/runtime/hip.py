@@ -1370,6 +1370,34 @@ class HIP:
         launch(kernel(K.adam_inplace_kernel, vec), max(1, ((n + vec - 1) // vec + 255) // 256), 256,
                *addrs, n, _addr(consts))
 
+    _stage: dict = {"slots": [], "events": [], "next": 0}
+
+    @staticmethod
+    def _stage_upload(bufs: list, arrays: list) -> None:
+        """Uploads small host arrays into device buffers without waiting: they are copied into one of four page-locked
+        staging blocks and the copies are enqueued on the stream, in order with the launches around them.  A staging
+        block is reused only after the copies issued from it have finished (an event per block, normally long done)."""
+        st, l = HIP._stage, lib()
+        if st.get("lib") is not l:                           # a library that was shut down took its blocks and events with it
+            st.update(slots=[], events=[], next=0, lib=l)
+        need = sum(a.size for a in arrays)
+        i = st["next"]
+        st["next"] = (i + 1) % 4
+        if len(st["slots"]) <= i:
+            st["slots"].append(pinned_empty((max(need, 4096),)))
+            st["events"].append(l.event_create())
+        else:
+            l.event_sync(st["events"][i])
+            if st["slots"][i].size < need:
+                st["slots"][i] = pinned_empty((2 * need,))
+        slot, at = st["slots"][i], 0
+        for b, a in zip(bufs, arrays):
+            if a.size:
+                slot[at:at + a.size] = a.reshape(-1)
+                l.h2d_async(b.addr, slot[at:at + a.size].ctypes.data, a.nbytes)
+                at += a.size
+        l.event_record(st["events"][i])
+
     @staticmethod
     @dispatcher.register(CustomOps.ADAM_MULTI_INPLACE, Device.HIP)
     def adam_multi_inplace(tensors: list, consts: Buffer, table: dict | None) -> dict:
@@ -1417,8 +1445,10 @@ class HIP:
                 # a captured launch only records where the table is; its contents are written once the
                 # capture has ended, and never again: the graph replays with exactly these addresses
                 _after_capture.append(upload)
-            else:
+            elif _graph_depth or COMPILE_ONLY:
                 upload()
+            else:
+                HIP._stage_upload(bufs, arrays)                # an eager step: enqueued, the host does not wait
             table = {"key": key, "grid": int(nblk.sum()), "nt": nt, "bufs": bufs, "frozen": capturing()}
         if table["nt"]:
             b = table["bufs"]

@@ -225,6 +225,7 @@ def test_pinned_staging_uploads_without_a_wait_and_inside_a_captured_graph():
         pytest.skip("no HIP device")
     lib = hip.lib()
     rng = np.random.default_rng(8)
+    held = set(hip._pinned)                                       # (the runtime keeps a few small staging blocks of its own)
     stage = hip.pinned_empty((128, 784))
     assert stage.dtype == np.float32 and stage.shape == (128, 784) and hip._is_pinned(stage)
     stage[:] = rng.random((128, 784), dtype=np.float32)
@@ -248,7 +249,7 @@ def test_pinned_staging_uploads_without_a_wait_and_inside_a_captured_graph():
     del stage, x, y
     import gc
     gc.collect()
-    assert not hip._pinned                                        # the page-locked block went back
+    assert set(hip._pinned) == held                               # the page-locked block went back
 
 
 def _run_bench(*args):
