@@ -709,14 +709,18 @@ class CrossEntropy(OP):
             if HIP.ce_stats_fits(logits):
                 m, ls, row_loss = logits.ce_stats(target, negate=True)
                 self.logits, self.stats = logits, (m, ls)
-                return row_loss.sum()                       # = -(sum of the picked log-probs), bit for bit
+                return self._total(row_loss)                # = -(sum of the picked log-probs), bit for bit
             else:                                           # more than 2^31 elements
                 self.log_softmax, picked = logits.log_softmax_gather(target)
         else:
             shifted = logits - logits.max(dim=dim, keepdim=True)
             self.log_softmax = shifted - shifted.exp().sum(dim=dim, keepdim=True).log()
             picked = Buffer.ce_forward(self.log_softmax, self.target)
-        return -picked.sum()
+        return -self._total(picked)
+
+    @staticmethod
+    def _total(rows: Buffer) -> Buffer:
+        return rows.sum()
 
     def backward(self, upstream_grad: Buffer) -> tuple:
         if self.stats is not None:
@@ -726,6 +730,15 @@ class CrossEntropy(OP):
         probs = self.log_softmax.exp()
         Buffer.ce_backward(op=CustomOps.CE_BACKWARD, device=probs.device, x=probs, target=self.target)   # p - onehot
         return ((probs * upstream_grad) / self.N,)
+
+
+class CCrossEntropy(CrossEntropy):
+    """The mean-reduced form (ops.py:372-396): -MEAN of the picked log-probs, with CrossEntropy's backward
+    (which divides by the number of rows either way).  No Tensor method reaches it in the reference."""
+
+    @staticmethod
+    def _total(rows: Buffer) -> Buffer:
+        return rows.mean()                                  # (-s) / N and -(s / N) are the same bits
 
 
 class BCEWithLogitsLoss(OP):

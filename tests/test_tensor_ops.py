@@ -226,6 +226,22 @@ def test_cross_entropy_sum_forward_mean_backward(shape, device):
     close(a.grad.numpy(), ta.grad, atol=1e-6, rtol=1e-4)
 
 
+@pytest.mark.parametrize("shape", [(4, 7), (128, 100)])
+def test_cross_entropy_mean_forward(shape, device):
+    """CCrossEntropy (ops.py:372-396): the MEAN of the row losses, which is what torch's default
+    reduction gives, and the same gradient as CrossEntropy."""
+    from dlgrad_amd import ops
+    x = f32(*shape)
+    t = RNG.integers(0, shape[1], (shape[0], 1))
+    (a,), (ta,) = both((x,), device)
+    loss = ops.CCrossEntropy.execute(a, Tensor(t.astype(np.float32), device=device))
+    tl = torch.nn.functional.cross_entropy(ta, torch.tensor(t[:, 0]))
+    close(loss.numpy().reshape(()), tl.detach(), atol=1e-6, rtol=1e-4)
+    loss.backward()
+    tl.backward()
+    close(a.grad.numpy(), ta.grad, atol=1e-6, rtol=1e-4)
+
+
 @pytest.mark.parametrize("shape", [(4, 7), (1000, 1000)])
 def test_bce_with_logits_forward_backward(shape, device):
     """test/test_loss.py:39-65: mean of the numerically stable BCE-with-logits and its
