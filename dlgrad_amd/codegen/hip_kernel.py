@@ -994,7 +994,9 @@ def embedding_backward_ordered_kernel(stage: str, vec: int = 1, nt: bool = False
            meet in LDS, and each column is added in row order.  If idsegs says the id occurs in no
            other segment the sum is the final table row; otherwise it goes to partial[first
            position of the id in the segment], and that first position records the set of segments
-           in segmask (0 for every other position) and the id's first position in each of them.
+           in segmask (0 for every other position), looks up g, the id's first position of all (one
+           more round of ballots over the id's earliest segment), and enters itself in the list of
+           the id's first positions that is kept at g: firsts[g][rank of its segment], gfirst[i] = g.
          zero blocks: each owns 64 consecutive table rows and writes zeros to those whose idsegs
            entry is 0.  They are spread evenly among the sum blocks, so that the stream of zeros
            (bandwidth-bound) and the sums (latency-bound) run side by side.
@@ -1018,9 +1020,17 @@ def embedding_backward_ordered_kernel(stage: str, vec: int = 1, nt: bool = False
               if (nt and vec == 4) else f"zrow[c] = {zero};")
     if ivec == 4:
         # positions 4 * item .. 4 * item + 3 per thread; an item that sticks out past n is judged value by value
-        mscan = """    for (u32 t = threadIdx.x; 4u * t < n; t += 256u) {
-        if (4u * t + 3u < n) { const float4 q = reinterpret_cast<const float4*>(idx)[t]; MARK(q.x, 4u * t) MARK(q.y, 4u * t + 1u) MARK(q.z, 4u * t + 2u) MARK(q.w, 4u * t + 3u) }
-        else for (u32 p = 4u * t; p < n; ++p) MARK(idx[p], p)
+        # eight items per thread and round: their loads are all issued before the first comparison
+        mscan = """    for (u32 t0 = threadIdx.x; 4u * t0 < n; t0 += 2048u) {
+        float4 q[8];
+        #pragma unroll
+        for (u32 u = 0; u < 8u; ++u) { const u32 t = t0 + 256u * u; if (4u * t + 3u < n) q[u] = reinterpret_cast<const float4*>(idx)[t]; }
+        #pragma unroll
+        for (u32 u = 0; u < 8u; ++u) {
+            const u32 t = t0 + 256u * u;
+            if (4u * t + 3u < n) { MARK(q[u].x, 4u * t) MARK(q[u].y, 4u * t + 1u) MARK(q[u].z, 4u * t + 2u) MARK(q[u].w, 4u * t + 3u) }
+            else for (u32 p = 4u * t; p < n; ++p) MARK(idx[p], p)
+        }
     }"""
     else:
         mscan = """    for (u32 t = threadIdx.x; t < n; t += 256u) MARK(idx[t], t)"""
@@ -1043,8 +1053,9 @@ extern "C" __global__ __launch_bounds__(256) void {name}(u64* __restrict__ idseg
     if stage == "segments":
         body = f"""
 extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out,
-        float* __restrict__ partial, u64* __restrict__ segmask, u32* __restrict__ firsts, const u64* __restrict__ idsegs,
-        const float* __restrict__ g, const float* __restrict__ idx, u32 n, u32 W, u32 V, u32 n_zero_blocks, u32 every) {{
+        float* __restrict__ partial, u64* __restrict__ segmask, u32* __restrict__ firsts, u32* __restrict__ gfirst,
+        const u64* __restrict__ idsegs, const float* __restrict__ g, const float* __restrict__ idx, u32 n, u32 W, u32 V,
+        u32 n_zero_blocks, u32 every) {{
     __shared__ u32 lists[4][{EMB_SEGMENT}];
     __shared__ {VT} stage[4][{EMB_SEGMENT}];
     const u32 w = threadIdx.x >> 6, lane = threadIdx.x & 63u;
@@ -1089,20 +1100,26 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
     const u64 segs = idsegs[my];                                // the segments the id occurs in (this one among them)
     wave_lds_fence();
     const bool other = segs != (1ull << seg);
-    if (lane == 0u) segmask[i] = (r == 0u && other) ? segs : 0ull;
+    u64 mine = 0ull;                                            // what segmask[i] will hold
     if (r == 0u && other) {{                                     // the merge adds the partial rows of these first positions
         const u32 NS = (n + EMB_SEG - 1u) / EMB_SEG;
-        u32 k = 0;
-        for (u64 rest = segs; rest; rest &= rest - 1ull, ++k) {{
-            const u32 t0 = (u32)__builtin_ctzll(rest) * EMB_SEG;
+        const u32 tmin = (u32)__builtin_ctzll(segs);            // the id's earliest segment
+        u32 gf = i;                                             // the id's first position of all: this one, in that segment
+        if (tmin != seg) {{
+            const u32 t0 = tmin * EMB_SEG;
             u64 h2[EMB_NK];
             segment_hits(idx, my, t0, min(n, t0 + EMB_SEG), n, lane, h2);
-            u32 first = 0xFFFFFFFFu;
+            gf = 0xFFFFFFFFu;
             #pragma unroll
-            for (u32 j = EMB_NK; j-- > 0u;) if (h2[j]) first = t0 + 64u * j + (u32)__builtin_ctzll(h2[j]);
-            if (lane == 0u) firsts[(u64)i * NS + k] = first;
+            for (u32 j = EMB_NK; j-- > 0u;) if (h2[j]) gf = t0 + 64u * j + (u32)__builtin_ctzll(h2[j]);
+        }}
+        if (gf < n) {{                                           // (the mark launch saw the id there, so it is found)
+            mine = segs;
+            const u32 k = (u32)__popcll(segs & ((1ull << seg) - 1ull));        // this segment's rank among the id's
+            if (lane == 0u) {{ firsts[(u64)gf * NS + k] = i; gfirst[i] = gf; }}
         }}
     }}
+    if (lane == 0u) segmask[i] = mine;
     {VT}* __restrict__ dst = reinterpret_cast<{VT}*>(other ? partial + (u64)list[0] * W : out + (u64)my * W);
     const u32 c0 = r * Wv / m, c1 = (r + 1u) * Wv / m;        /* r < 512 and Wv < 2^22: no overflow */      // this wavefront's slice of the columns
     // The (row, column) items of the slice are spread over all 64 lanes, so every load of a pass
@@ -1139,22 +1156,25 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
     }}
 }}
 """
-        fmt = _fmt("P", "P", "P", "P", "P", "P", "P", "I", "I", "I", "I", "I")
+        fmt = _fmt("P", "P", "P", "P", "P", "P", "P", "P", "I", "I", "I", "I", "I")
     else:
         body = f"""
 extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out,
         const float* __restrict__ partial, const u64* __restrict__ segmask, const u32* __restrict__ firsts,
-        const float* __restrict__ idx, u32 n, u32 W, u32 V) {{
+        const u32* __restrict__ gfirst, const float* __restrict__ idx, u32 n, u32 W, u32 V) {{
     const u32 w = threadIdx.x >> 6, lane = threadIdx.x & 63u;
     const u32 i = blockIdx.x * 4u + w;                          // one wavefront per position
     if (i >= n) return;
     const u64 segs = segmask[i];
+    const float mine = idx[i];                                  // (read along with the mask: one trip to memory, not three)
+    const u32 gf = gfirst[i];                                   // (a position only where the mask is set; unused elsewhere)
     if (segs == 0ull) return;                                   // only the first positions of an id that spans segments work
-    const int my = (int)idx[i];
+    const int my = (int)mine;
     const u32 m = (u32)__popcll(segs);
     const u32 r = (u32)__popcll(segs & ((1ull << (i / EMB_SEG)) - 1ull));           // this segment's rank among them
-    // the id's first position in each of its segments, in segment order, as the first launch listed them
-    const u32* __restrict__ list = firsts + (u64)i * ((n + EMB_SEG - 1u) / EMB_SEG);
+    // the id's first position in each of its segments, in segment order: each of them entered itself in the
+    // list kept at the id's first position of all
+    const u32* __restrict__ list = firsts + (u64)gf * ((n + EMB_SEG - 1u) / EMB_SEG);
     const u32 Wv = W / {vec}u;
     {VT}* __restrict__ dst = reinterpret_cast<{VT}*>(out + (u64)my * W);
     const u32 c0 = r * Wv / m, c1 = (r + 1u) * Wv / m;        /* r < 512 and Wv < 2^22: no overflow */      // the first positions split the columns
@@ -1166,7 +1186,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
     }}
 }}
 """
-        fmt = _fmt("P", "P", "P", "P", "P", "I", "I", "I")
+        fmt = _fmt("P", "P", "P", "P", "P", "P", "I", "I", "I")
     return f"{PRELUDE}{_ORDERED_COMMON}{body}", name, fmt
 
 
@@ -1410,16 +1430,20 @@ extern "C" __global__ __launch_bounds__({threads}) void {name}(const float* __re
 
 
 @cache
-def ce_grad_rows_kernel(items: int, nt: bool, g_by_value: bool) -> tuple[str, str, str]:
+def ce_grad_rows_kernel(items: int, nt: bool, g_by_value: bool, pow2: bool = False) -> tuple[str, str, str]:
     """Gradient of the summed cross-entropy with respect to 2-D logits whose rows are multiples of
     four floats: out = ((exp((x - max) - logsum) - onehot(target)) * g) / n -- the four kernels of
     CrossEntropy.backward (ops.py:359-370) on a log-softmax rebuilt from the row statistics -- with a
     block per (row, run of 1024 * items columns): the row's three values are read once per block,
     no index is divided, and a thread has `items` 16-byte loads in flight before its first store.
     The same fp32 operations in the same order as the element-wise form of the expression.
-    nt: streaming loads and stores (tensors beyond the caches)."""
+    nt: streaming loads and stores (tensors beyond the caches).
+    pow2: n is a power of two and the caller passes 1 / n, itself a power of two, in its place: the
+    product with it is the quotient, bit for bit (both are the exact value, rounded once), and the
+    dozen instructions of an IEEE division per element, a third of the kernel's arithmetic, go."""
     assert items in (1, 2, 4)
-    name = f"ce_grad_rows_u{items}" + ("nt" if nt else "") + ("_v" if g_by_value else "_p")
+    name = f"ce_grad_rows_u{items}" + ("nt" if nt else "") + ("_v" if g_by_value else "_p") + ("_r" if pow2 else "")
+    by_n = "* n" if pow2 else "/ n"
     ld = "ld4_stream(reinterpret_cast<const float4*>(xr + c))" if nt else "*reinterpret_cast<const float4*>(xr + c)"
     st = ("{ const v4f ov = {o.x, o.y, o.z, o.w}; __builtin_nontemporal_store(ov, reinterpret_cast<v4f*>(orow + c)); }" if nt
           else "*reinterpret_cast<float4*>(orow + c) = o;")
@@ -1443,10 +1467,10 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
         const u32 c = c0 + 1024u * k;
         if (c < C) {{
             float4 o;
-            o.x = ((expf((v[k].x - m) - ls) - (c == t ? 1.0f : 0.0f)) * g) / n;
-            o.y = ((expf((v[k].y - m) - ls) - (c + 1u == t ? 1.0f : 0.0f)) * g) / n;
-            o.z = ((expf((v[k].z - m) - ls) - (c + 2u == t ? 1.0f : 0.0f)) * g) / n;
-            o.w = ((expf((v[k].w - m) - ls) - (c + 3u == t ? 1.0f : 0.0f)) * g) / n;
+            o.x = ((expf((v[k].x - m) - ls) - (c == t ? 1.0f : 0.0f)) * g) {by_n};
+            o.y = ((expf((v[k].y - m) - ls) - (c + 1u == t ? 1.0f : 0.0f)) * g) {by_n};
+            o.z = ((expf((v[k].z - m) - ls) - (c + 2u == t ? 1.0f : 0.0f)) * g) {by_n};
+            o.w = ((expf((v[k].w - m) - ls) - (c + 3u == t ? 1.0f : 0.0f)) * g) {by_n};
             {st}
         }}
     }}

@@ -1033,16 +1033,17 @@ class HIP:
                 # occurs, zeros elsewhere -- without a zero-fill pass and without atomics
                 NS = (n_idx + K.EMB_SEGMENT - 1) // K.EMB_SEGMENT
                 out, partial, segmask, firsts, idsegs = alloc(x.numel), alloc(n_idx * W), alloc(2 * n_idx), alloc(n_idx * NS), alloc(2 * V)
+                gfirst = alloc(n_idx)
                 vec = 4 if (W % 4 == 0 and not (_addr(upstream_grad) | out.addr | partial.addr) & 15) else 1
                 n_sum, n_zero = (n_idx + 3) // 4, (V + 63) // 64
                 every = max(1, (n_sum + n_zero) // n_zero)     # one zero block among every so many
                 launch(kernel(K.embedding_backward_ordered_kernel, "mark", 1, False, 4 if _addr(idx) % 16 == 0 else 1),
                        n_zero, 256, idsegs.addr, _addr(idx), n_idx, V)
                 launch(kernel(K.embedding_backward_ordered_kernel, "segments", vec, x.numel >= NT_STORE_MIN_ELEMENTS),
-                       n_sum + n_zero, 256, out.addr, partial.addr, segmask.addr, firsts.addr, idsegs.addr, _addr(upstream_grad),
-                       _addr(idx), n_idx, W, V, n_zero, every)
+                       n_sum + n_zero, 256, out.addr, partial.addr, segmask.addr, firsts.addr, gfirst.addr, idsegs.addr,
+                       _addr(upstream_grad), _addr(idx), n_idx, W, V, n_zero, every)
                 launch(kernel(K.embedding_backward_ordered_kernel, "merge", vec), n_sum, 256, out.addr, partial.addr,
-                       segmask.addr, firsts.addr, _addr(idx), n_idx, W, V)
+                       segmask.addr, firsts.addr, gfirst.addr, _addr(idx), n_idx, W, V)
                 return out
             out = alloc(x.numel, zero=True)                    # init_with_scalar(0), cpu.py:1031
             if n_idx:                                          # very long index lists: hardware fp32 atomics
@@ -1257,15 +1258,17 @@ class HIP:
         on the same values the stored tensor was made with), then the four kernels of
         CrossEntropy.backward (exp, in-place ce_backward, mul, div; ops.py:359-370) follow fused."""
         R, C = x.shape
-        items = 1 if C <= 1024 else 2 if C <= 2048 else 4
+        # a power of two divides exactly as its reciprocal multiplies (1 / n stays a normal number up to 2^126)
+        pow2 = 1.0 <= n <= 2.0 ** 126 and math.frexp(n)[0] == 0.5
+        items = 1 if C <= 1024 else 2 if (C <= 2048 or pow2) else 4     # (without the division two loads per thread go faster than four)
         runs = -(-C // (1024 * items))
         if HIP.CE_GRAD_ROWS and C % 4 == 0 and not (_addr(x) & 15) and 0 < R * runs < 2 ** 31 and x.numel < 2 ** 31:
             # a block per (row, run of columns): the row's statistics are read once per block and no index is divided
             by_value = upstream.is_host_scalar
-            k = kernel(K.ce_grad_rows_kernel, items, x.numel >= NT_STORE_MIN_ELEMENTS, by_value)
+            k = kernel(K.ce_grad_rows_kernel, items, x.numel >= NT_STORE_MIN_ELEMENTS, by_value, pow2)
             g = float(upstream.ptr.value) if by_value else _addr(upstream)
             return launch_out(k, R * runs, 256, field_offset(k[1].format, 5), x.numel, _addr(x), _addr(m), _addr(ls), _addr(target),
-                              g, 0, C, runs, float(n))
+                              g, 0, C, runs, 1.0 / n if pow2 else float(n))
         rows = [Buffer(b.ptr, (R, 1), Device.HIP) for b in (m, ls, target)]
         one = R == 1                                     # a single row collapses to a flat run: the column is i itself
         col = "i" if one else "(i % C)"
