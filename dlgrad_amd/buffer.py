@@ -541,6 +541,29 @@ class Buffer:
             dst2.row_store_(src2, idx)
         self._dispatch(CustomOps.ROW_STORE, dst=self, src=src, idx=idx, rows=rows, width=width)
 
+    # ---- the ends of a decoding step (hip) -------------------------------------------------------
+    def decode_qkv_row(self, w: "Buffer", gain: "Buffer", eps: float, kc: "Buffer", vc: "Buffer", slot: "Buffer") -> "Buffer":
+        """self: one row; w: the stacked (3C, K) q, k, v projection.  Returns q (C,) = the first third of
+        rmsnorm(self) @ w^T; the key and value thirds are written to row (int)slot of kc and vc."""
+        C = w.shape[-2] // 3
+        return Buffer.fresh(self._dispatch(CustomOps.DECODE_QKV_ROW, x=self, w=w, gain=gain, eps=eps, kc=kc, vc=vc, slot=slot),
+                            (C,), self.device)
+
+    @staticmethod
+    def decode_embed(wte: "Buffer", wpe: "Buffer", slot: "Buffer", T: int, tok: "Buffer | None" = None,
+                     seq: "Buffer | None" = None, refpos: bool = False):
+        """tok given: (x (1, 1, C), hidden (1, T)) = (wte[tok] + wpe[position of slot], arange(T) > slot).
+        seq given: x (1, T, C) = wte[last T tokens of seq up to slot] + wpe[0 .. T - 1]."""
+        C = wte.shape[1]
+        got = wte._dispatch(CustomOps.DECODE_EMBED, wte=wte, wpe=wpe, slot=slot, T=T, tok=tok, seq=seq, refpos=refpos)
+        if seq is not None:
+            return Buffer.fresh(got, (1, T, C), wte.device)
+        return Buffer.fresh(got[0], (1, 1, C), wte.device), Buffer.fresh(got[1], (1, T), wte.device)
+
+    def decode_next_(self, tok: "Buffer", slot: "Buffer", seq: "Buffer") -> None:
+        """self: the logits of the position just computed.  seq[slot + 1] = tok = argmax(self); slot += 1, in place."""
+        self._dispatch(CustomOps.DECODE_NEXT, logits=self, tok=tok, slot=slot, seq=seq)
+
     def sgd_step_(self, g: "Buffer", v: "Buffer | None", lr: float, momentum: float) -> None:
         """In-place SGD update of self (and of the velocity v when momentum is used)."""
         self._dispatch(CustomOps.SGD_STEP_INPLACE, p=self, g=g, v=v, lr=lr, momentum=momentum)

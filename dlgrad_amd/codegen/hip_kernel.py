@@ -2409,7 +2409,7 @@ MATMUL_TILE_MODEL = {
 # =====================================================================================
 
 @cache
-def row_matmul_nt_kernel(epi: str = "", norm_nval: int = 0) -> tuple[str, str, str]:
+def row_matmul_nt_kernel(epi: str = "", norm_nval: int = 0, kv: bool = False) -> tuple[str, str, str]:
     """y[n] = sum_k x[k] * W[n][k] for one row x (K) and W stored (N, K): the linear layers of a
     decoding step, where an MFMA tile would hold one useful row in 16.  One wavefront per output:
     lane l multiplies the 16-byte items l, l + 64, ... of the row of W with the same items of x
@@ -2418,9 +2418,14 @@ def row_matmul_nt_kernel(epi: str = "", norm_nval: int = 0) -> tuple[str, str, s
     norm_nval > 0: x is first RMS-normalised with the gain row g -- (x * r) * g with
     r = 1 / sqrt(sum(x^2) / K + eps) -- by every wavefront for itself, the row (at most 64 * norm_nval
     items) in registers: the statements of rmsnorm_fwd_kernel, so the values that enter the product
-    are the ones that kernel would have stored, and the launch between the two disappears."""
-    assert epi in ("", "add", "relu", "gate")
-    name = f"row_matmul_nt{'_' + epi if epi else ''}{f'_rms{norm_nval}' if norm_nval else ''}"
+    are the ones that kernel would have stored, and the launch between the two disappears.
+    kv (no epilogue): W is the stacked q, k, v projection (N = 3 * C3).  The first third of the outputs goes
+    to y as usual; the second and third are the new position's key and value and go straight to row
+    (int)slot[0] of the (rows, C3) stores kc and vc (nothing is stored for a row outside [0, rows), as
+    row_store_kernel has it): the launch that copied them there disappears.  Arguments after the others:
+    kc, vc, slot, C3, rows."""
+    assert epi in ("", "add", "relu", "gate") and not (kv and epi)
+    name = f"row_matmul_nt{'_' + epi if epi else ''}{f'_rms{norm_nval}' if norm_nval else ''}{'_kv' if kv else ''}"
     fin = {"": "acc", "add": "acc + e[n]", "relu": "(acc > 0.0f ? acc : 0.0f)", "gate": "(e[n] > 0.0f ? acc : 0.0f)"}[epi]
     if norm_nval:
         comps = (".x", ".y", ".z", ".w")
@@ -2459,6 +2464,20 @@ def row_matmul_nt_kernel(epi: str = "", norm_nval: int = 0) -> tuple[str, str, s
     for (; c < K4; c += 64u) acc = dot4(w4[c], x4[c], acc);
 """
         extra, fmt = "", _fmt("P", "P", "P", "P", "I", "I")
+    store = f"if (lane == 0u) y[n] = {fin};"
+    if kv:
+        extra += ", float* __restrict__ kc, float* __restrict__ vc, const float* __restrict__ slot, u32 C3, u32 rows"
+        fmt += "PPPII"
+        store = """if (lane == 0u) {
+        if (n < C3) y[n] = acc;
+        else {
+            const float fi = slot[0];
+            if (fi >= 0.0f && fi < (float)rows) {
+                const u32 third = n / C3;
+                (third == 1u ? kc : vc)[(u64)(u32)fi * C3 + (n - third * C3)] = acc;
+            }
+        }
+    }"""
     src = f"""{PRELUDE}
 static __device__ __forceinline__ float dot4(float4 a, float4 b, float acc) {{
     acc = fmaf(a.x, b.x, acc); acc = fmaf(a.y, b.y, acc); acc = fmaf(a.z, b.z, acc); return fmaf(a.w, b.w, acc);
@@ -2471,10 +2490,98 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
     const float4* __restrict__ w4 = reinterpret_cast<const float4*>(W + (u64)n * K);
     const float4* __restrict__ x4 = reinterpret_cast<const float4*>(x);
 {body}    acc = wave_sum(acc);
-    if (lane == 0u) y[n] = {fin};
+    {store}
 }}
 """
     return src, name, fmt
+
+
+# =====================================================================================
+# the ends of a decoding step: embedding of the token(s) to feed, choice of the next one
+# =====================================================================================
+
+@cache
+def decode_embed_kernel(window: bool) -> tuple[str, str, str]:
+    """The input of a decoding step, from device-resident state, in one launch.
+    window = False: x[0, :] = wte[tok] + wpe[pos] for the token tok[0] fed at index s = slot[0], with
+      pos = s, or s + clamp(s, 0, 1) when refpos (the reference numbers an incremental token one too
+      high, examples/gpt.py:199), and hidden[j] = (j > s) for the T cache rows: what the clamp, the add,
+      the comparison with arange, the two gathers and the add of the op-by-op step compute.
+    window = True: x[t, :] = wte[seq[s - (T - 1) + t]] + wpe[t] for t < T: the window of the last T
+      tokens out of the token buffer (rows, 1), embedded at positions 0 .. T - 1.
+    Rows are looked up as embedding_kernel does it -- offset (int)(id * W) formed in float, a row that
+    does not lie inside its table reads as zeros -- and the sum is the one fp32 addition of the add
+    kernel.  One wavefront per position."""
+    name = "decode_embed_window" if window else "decode_embed"
+    if window:
+        head = """    const u32 t = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (t >= T) return;
+    const float w = (float)t + (slot[0] - (float)(T - 1u));   // arange + (slot - (T - 1)), as the op-by-op step forms it
+    const int si = (int)(w * 1.0f);                             // the token buffer is a table of rows of one float
+    const float tok = (si < 0 || (u64)si + 1u > (u64)rows) ? 0.0f : seq[si];
+    const float pos = (float)t;
+    float* __restrict__ dst = x + (u64)t * C;
+"""
+        params = "const float* __restrict__ seq, const float* __restrict__ slot, float* __restrict__ x, u32 C, u32 V, u32 P, u32 T, u32 rows"
+        fmt = _fmt("P", "P", "P", "P", "P", "I", "I", "I", "I", "I")
+        tail = ""
+    else:
+        head = """    if (blockIdx.x != 0u || threadIdx.x >= 64u) {              // the other wavefronts write the mask of the cache rows
+        const u32 j = blockIdx.x * 256u + threadIdx.x - 64u;
+        if (j < T) hidden[j] = (float)j > slot[0] ? 1.0f : 0.0f;
+        return;
+    }
+    const float s = slot[0];
+    const float tok = tokp[0];
+    const float pos = refpos ? s + fminf(fmaxf(s, 0.0f), 1.0f) : s;
+    float* __restrict__ dst = x;
+"""
+        params = ("const float* __restrict__ tokp, const float* __restrict__ slot, float* __restrict__ x, float* __restrict__ hidden, "
+                  "u32 C, u32 V, u32 P, u32 T, u32 refpos")
+        fmt = _fmt("P", "P", "P", "P", "P", "P", "I", "I", "I", "I", "I")
+        tail = ""
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ wte, const float* __restrict__ wpe,
+        {params}) {{
+    const u32 lane = threadIdx.x & 63u;
+{head}    const int ti = (int)(tok * (float)C), pi = (int)(pos * (float)C);
+    const bool tok_ok = ti >= 0 && (u64)ti + C <= (u64)V * C, pos_ok = pi >= 0 && (u64)pi + C <= (u64)P * C;
+    for (u32 j = lane; j < C; j += 64u)
+        dst[j] = (tok_ok ? wte[(long long)ti + j] : 0.0f) + (pos_ok ? wpe[(long long)pi + j] : 0.0f);
+{tail}}}
+"""
+    return src, name, fmt
+
+
+@cache
+def decode_next_kernel() -> tuple[str, str, str]:
+    """The end of a decoding step in one launch: next = index of the first maximum of the V logits
+    (argmax_kernel's rule: strict '>' from (-FLT_MAX, 0)), then seq[s + 1] = next for s = slot[0] (skipped
+    when s + 1 lies outside the (rows, 1) token buffer), tok[0] = next and slot[0] = s + 1 -- what argmax,
+    add, row_store and two copies do in the op-by-op step.  One block."""
+    name = "decode_next"
+    src = f"""{PRELUDE}{_ARGMAX_PAIR}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ logits, float* __restrict__ tok,
+        float* __restrict__ slot, float* __restrict__ seq, u32 V, u32 rows) {{
+    __shared__ float sv[4];
+    __shared__ u32 si[4];
+    float best = NEG_FLT_MAX;
+    u32 bi = 0u;
+    for (u32 j = threadIdx.x; j < V; j += 256u) {{ const float v = logits[j]; if (v > best) {{ best = v; bi = j; }} }}
+    wave_argmax(best, bi);
+    if ((threadIdx.x & 63u) == 0u) {{ sv[threadIdx.x >> 6] = best; si[threadIdx.x >> 6] = bi; }}
+    __syncthreads();
+    if (threadIdx.x == 0u) {{
+        #pragma unroll
+        for (u32 w = 1; w < 4u; ++w) {{ const float ov = sv[w]; const u32 oi = si[w]; TAKE(best, bi, ov, oi) }}
+        const float nxt = (float)bi, ns = slot[0] + 1.0f;
+        if (ns >= 0.0f && ns < (float)rows) seq[(u32)ns] = nxt;
+        tok[0] = nxt;
+        slot[0] = ns;
+    }}
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "P", "I", "I")
 
 
 # =====================================================================================

@@ -167,6 +167,58 @@ def project_qkv_row(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor, norm=None) ->
     return x.linear(wq, None), x.linear(wk, None), x.linear(wv, None)
 
 
+def _decode_fused(*tensors: Tensor) -> bool:
+    if not ops.FUSED or any(t.device is not Device.HIP for t in tensors):
+        return False
+    from dlgrad_amd.runtime.hip import HIP
+    return HIP.DECODE_FUSED
+
+
+def decode_query_row(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor, norm, k_store: Tensor, v_store: Tensor,
+                     slot: Tensor) -> Tensor | None:
+    """Decoding on the hip device with stacked weights: the query projection (1, 1, C) of the single row
+    norm(x), while the key and value projections go straight to row (int)slot of the (rows, 1, C) stores --
+    project_qkv_row and the store of the two rows as one launch.  None where that is not provided
+    (the caller then does the two steps)."""
+    if norm is None or norm.weight is None or not _decode_fused(x, wq, k_store, v_store, slot, norm.weight) \
+            or not ops.stacked(wq, wk, wv) or x.numel != x.shape[-1]:
+        return None
+    from dlgrad_amd.runtime.hip import HIP
+    C = wq.shape[0]
+    w = Buffer(wq.data.ptr, (3 * C, wq.shape[1]), wq.device)
+    if k_store.numel != k_store.shape[0] * C or not HIP.decode_qkv_row_fits(x.data, w, norm.weight.data, k_store.data, v_store.data, slot.data):
+        return None
+    q = x.data.decode_qkv_row(w, norm.weight.data, norm.eps, k_store.data, v_store.data, slot.data)
+    return Tensor(q.reshape(x.shape[:-1] + (C,)), requires_grad=False)
+
+
+def decode_input(wte: Tensor, wpe: Tensor, tok: Tensor, slot: Tensor, T: int, reference_positions: bool):
+    """(x, hidden) for one decoding step on the hip device, in one launch: x (1, 1, C) = wte[tok] + wpe[pos]
+    with pos = slot (or slot + clamp(slot, 0, 1), the reference's numbering) and hidden (1, T) = arange(T) > slot,
+    the cache rows not written yet.  None where not provided."""
+    if not _decode_fused(wte, wpe, tok, slot) or wte.ndim != 2 or wpe.ndim != 2 or wte.shape[1] != wpe.shape[1]:
+        return None
+    x, hidden = Buffer.decode_embed(wte.data, wpe.data, slot.data, T, tok=tok.data, refpos=reference_positions)
+    return Tensor(x, requires_grad=False), Tensor(hidden, requires_grad=False)
+
+
+def decode_window_input(wte: Tensor, wpe: Tensor, seq: Tensor, slot: Tensor, T: int) -> Tensor | None:
+    """x (1, T, C) = wte[seq[slot - T + 1 .. slot]] + wpe[0 .. T - 1] on the hip device, in one launch: the
+    window of the last T tokens of the (rows, 1) token buffer, embedded.  None where not provided."""
+    if not _decode_fused(wte, wpe, seq, slot) or wte.ndim != 2 or wpe.ndim != 2 or wte.shape[1] != wpe.shape[1]:
+        return None
+    return Tensor(Buffer.decode_embed(wte.data, wpe.data, slot.data, T, seq=seq.data), requires_grad=False)
+
+
+def decode_append(logits: Tensor, tok: Tensor, slot: Tensor, seq: Tensor) -> bool:
+    """seq[slot + 1] = tok = argmax(logits); slot += 1 -- all in place, in one launch, on the hip device.
+    False where not provided (nothing done)."""
+    if not _decode_fused(logits, tok, slot, seq):
+        return False
+    logits.data.decode_next_(tok.data, slot.data, seq.data)
+    return True
+
+
 def norm_linear(x: Tensor, norm, weight: Tensor) -> Tensor:
     """norm(x) @ weight^T.  For a single row on the hip device the normalisation happens inside the product
     and the result carries no tape (decoding); otherwise the two ops."""

@@ -601,6 +601,55 @@ class HIP:
             launch(kernel(K.row_store_kernel, 2), ((width + 255) // 256, 2, 1), 256, _addr(dst), _addr(src), _addr(idx),
                    rows, width, _addr(dst2), _addr(src2))
 
+    # ---- the ends of a decoding step ---------------------------------------------------------------------------------
+    @staticmethod
+    def decode_qkv_row_fits(x: Buffer, w: Buffer, gain: Buffer, kc: Buffer, vc: Buffer, slot: Buffer) -> bool:
+        """One row x against the stacked (3C, K) projection w with the RMSNorm inside, key and value stores of rows of C."""
+        C = w.shape[-2] // 3 if w.ndim >= 2 else 0
+        return (HIP.DECODE_FUSED and C > 0 and w.shape[-2] == 3 * C and HIP.row_norm_fits(x, w, gain)
+                and kc.numel == vc.numel and kc.numel % C == 0 and kc.numel > 0 and slot.numel == 1 and not slot.is_host_scalar)
+
+    @staticmethod
+    @dispatcher.register(CustomOps.DECODE_QKV_ROW, Device.HIP)
+    def decode_qkv_row(x: Buffer, w: Buffer, gain: Buffer, eps: float, kc: Buffer, vc: Buffer, slot: Buffer) -> DevicePtr:
+        """q = (rmsnorm(x) @ w^T)[:C]; the other two thirds of that row go to row (int)slot of kc and vc."""
+        if not HIP.decode_qkv_row_fits(x, w, gain, kc, vc, slot):
+            raise ValueError(f"decode_qkv_row does not take {x.shape} x {w.shape} into {kc.shape}")
+        N, Kd = w.shape[-2:]
+        C = N // 3
+        out = alloc(C)
+        k = kernel(K.row_matmul_nt_kernel, "", K.rmsnorm_plan(Kd, 4), True)
+        launch(k, (N + 3) // 4, 256, _addr(x), _addr(w), out.addr, 0, N, Kd, _addr(gain), float(eps),
+               _addr(kc), _addr(vc), _addr(slot), C, kc.numel // C)
+        return out
+
+    @staticmethod
+    @dispatcher.register(CustomOps.DECODE_EMBED, Device.HIP)
+    def decode_embed(wte: Buffer, wpe: Buffer, slot: Buffer, T: int, tok: Buffer | None = None, seq: Buffer | None = None,
+                     refpos: bool = False):
+        """tok given: (x (C floats), hidden (T floats)) for the token tok[0] fed at index slot[0] against T cache rows.
+        seq given: x (T * C floats) for the window of the last T tokens of the (rows, 1) token buffer seq."""
+        V, C = wte.shape
+        P = wpe.shape[0]
+        if wpe.shape[1] != C or slot.numel != 1 or slot.is_host_scalar or (tok is None) == (seq is None) or T <= 0:
+            raise ValueError(f"decode_embed: tables {wte.shape}, {wpe.shape}, T={T}")
+        if seq is not None:
+            x = alloc(T * C)
+            launch(kernel(K.decode_embed_kernel, True), (T + 3) // 4, 256, _addr(wte), _addr(wpe), _addr(seq), _addr(slot), x.addr,
+                   C, V, P, T, seq.numel)
+            return x
+        x, hidden = alloc(C), alloc(T)
+        launch(kernel(K.decode_embed_kernel, False), (T + 64 + 255) // 256, 256, _addr(wte), _addr(wpe), _addr(tok), _addr(slot),
+               x.addr, hidden.addr, C, V, P, T, int(bool(refpos)))
+        return x, hidden
+
+    @staticmethod
+    @dispatcher.register(CustomOps.DECODE_NEXT, Device.HIP)
+    def decode_next(logits: Buffer, tok: Buffer, slot: Buffer, seq: Buffer) -> None:
+        if not logits.numel or tok.numel != 1 or slot.numel != 1 or tok.is_host_scalar or slot.is_host_scalar:
+            raise ValueError(f"decode_next: {logits.shape} logits, token {tok.shape}, index {slot.shape}")
+        launch(kernel(K.decode_next_kernel), 1, 256, _addr(logits), _addr(tok), _addr(slot), _addr(seq), logits.numel, seq.numel)
+
     @staticmethod
     @dispatcher.register(CustomOps.COPY_INTO, Device.HIP)
     def copy_into(dst: Buffer, src: Buffer) -> None:

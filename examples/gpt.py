@@ -249,12 +249,19 @@ class StaticDecoder:
 
     def _attend(self, attn: CausalSelfAttention, x: Tensor, norm, layer: int, hidden: Tensor, residual: Tensor) -> Tensor:
         T = self.model.config.block_size
-        q, k, v = nn.project_qkv_row(x, attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight, norm)
-        self.cache.k[layer].data.row_store_(k.data, self.slot.data, also=(self.cache.v[layer].data, v.data))
+        q = nn.decode_query_row(x, attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight, norm,
+                                self.cache.k[layer], self.cache.v[layer], self.slot)     # (k and v go straight to their cache rows)
+        if q is None:
+            q, k, v = nn.project_qkv_row(x, attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight, norm)
+            self.cache.k[layer].data.row_store_(k.data, self.slot.data, also=(self.cache.v[layer].data, v.data))
         y = nn.cached_attention(q, self.cache.k[layer], self.cache.v[layer], T, attn.n_head, attn.scale, hidden)
         return attn.c_proj(y, residual)
 
-    def _append(self, nxt: Tensor) -> None:
+    def _append(self, logits: Tensor) -> None:
+        """logits (1, V) of the newest position: its argmax becomes seq[slot + 1] and the next token; slot advances."""
+        if nn.decode_append(logits, self.tok, self.slot, self.seq):                     # one launch
+            return
+        nxt = logits.argmax(1)                                                          # (1, 1)
         nslot = self.slot + 1.0
         self.seq.data.row_store_(nxt.data, nslot.data)
         self.tok.data.copy_(nxt.data)
@@ -265,24 +272,34 @@ class StaticDecoder:
         token, and advances slot.  Reads and writes device memory only."""
         m, c = self.model, self.model.config
         slot = self.slot
-        # the reference numbers an incremental token one too high (examples/gpt.py:199); token 0 is a full forward there
-        pos = slot + slot.clamp(min=0, max=1) if self.reference_positions else slot
-        hidden = Tensor.arange((1, c.block_size), device=c.device) > slot                   # cache rows not written yet
-        x = m.wte(self.tok) + m.wpe(pos)
+        got = nn.decode_input(m.wte.weight, m.wpe.weight, self.tok, slot, c.block_size, self.reference_positions)
+        if got is not None:
+            x, hidden = got
+        else:
+            # the reference numbers an incremental token one too high (examples/gpt.py:199); token 0 is a full forward there
+            pos = slot + slot.clamp(min=0, max=1) if self.reference_positions else slot
+            hidden = Tensor.arange((1, c.block_size), device=c.device) > slot               # cache rows not written yet
+            x = m.wte(self.tok) + m.wpe(pos)
         for i, block in enumerate(m.blocks):                # each norm is applied by the product that consumes its row
             x = self._attend(block.attn, x, block.ln1, i, hidden, x)
             x = block.mlp(x, x, block.ln2)
-        self._append(nn.norm_linear(x, m.ln_f, m.lm_head.weight).reshape((1, c.vocab_size)).argmax(1))    # (1, 1)
+        self._append(nn.norm_linear(x, m.ln_f, m.lm_head.weight).reshape((1, c.vocab_size)))
 
     def step_window(self) -> None:
         """The step for a full window: tokens slot - block_size + 1 .. slot go through the whole model
         at positions 0 .. block_size - 1; the argmax of the last position becomes token slot + 1."""
         m, c = self.model, self.model.config
         T = c.block_size
-        where = Tensor.arange((1, T), device=c.device) + (self.slot - float(T - 1))        # indices into the token buffer
-        window = Tensor.embedding(self.seq, where).reshape((1, T))                          # the tokens themselves
-        logits, _ = m(window)
-        self._append(logits.reshape((T, c.vocab_size))[T - 1:T].argmax(1))
+        x = nn.decode_window_input(m.wte.weight, m.wpe.weight, self.seq, self.slot, T)     # window gathered and embedded in one launch
+        if x is None:
+            where = Tensor.arange((1, T), device=c.device) + (self.slot - float(T - 1))    # indices into the token buffer
+            window = Tensor.embedding(self.seq, where).reshape((1, T))                      # the tokens themselves
+            logits, _ = m(window)
+        else:
+            for block in m.blocks:
+                x = block(x)
+            logits = nn.norm_linear(x, m.ln_f, m.lm_head.weight)
+        self._append(logits.reshape((T, c.vocab_size))[T - 1:T])
 
     def capture(self) -> None:
         """hip only: records both steps into graphs (one warm-up run of each fixes every address first).

@@ -352,7 +352,7 @@ def test_decoding_step_replayed_as_a_graph_gives_the_eager_tokens(reference_posi
         return
     assert eager == want[0]
     dec.capture()
-    assert dec.graph.nodes > 20 and dec.window_graph.nodes > 20
+    assert dec.graph.nodes > 8 and dec.window_graph.nodes > 12       # (two layers: 5 launches each inside the window, 7 for a full window)
     assert dec.generate(0, 80) == want[0]
     assert dec.generate(9, 80) == want[9]
     assert dec.generate(0, 31) == want[0][:32]
@@ -384,6 +384,123 @@ def test_gpt_cached_decode_hip_vs_cpu_oracle(reference_positions):
     if not hip.COMPILE_ONLY:
         assert outs["hip"] == outs["cpu"]
         tensors_close(logits["hip"], logits["cpu"], "incremental logits", 1e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("reference_positions", [True, False])
+def test_the_ends_of_a_decoding_step_in_one_launch_each(reference_positions, monkeypatch):
+    """hip: the input of a step (token + position embedding, cache-row mask), the window of the last T tokens
+    embedded, and the end of a step (argmax appended, made the next token, index advanced) each run as one
+    launch; each must leave exactly the bits of the op-by-op composition it replaces, also for a token outside
+    the vocabulary, a full token buffer and logits with ties."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    rng = np.random.default_rng(12)
+    V, P, C, T, rows = 65, 32, 64, 32, 40
+    wte = Tensor(rng.standard_normal((V, C)).astype(np.float32), device="hip")
+    wpe = Tensor(rng.standard_normal((P, C)).astype(np.float32), device="hip")
+    for token, s in ((7.0, 0.0), (64.0, 5.0), (3.0, 31.0), (65.0, 4.0), (-1.0, 2.0)):
+        tok = Tensor(np.array([[token]], np.float32), device="hip")
+        slot = Tensor(np.array([[s]], np.float32), device="hip")
+        n0 = hip.launch_count
+        x, hidden = nn.decode_input(wte, wpe, tok, slot, T, reference_positions)
+        assert hip.launch_count - n0 == 1 and x.shape == (1, 1, C) and hidden.shape == (1, T)
+        pos = slot + slot.clamp(min=0, max=1) if reference_positions else slot
+        want_x = Tensor.embedding(wte, tok) + Tensor.embedding(wpe, pos)
+        want_hidden = Tensor.arange((1, T), device="hip") > slot
+        if not hip.COMPILE_ONLY:
+            np.testing.assert_array_equal(x.numpy().view(np.uint32), want_x.numpy().view(np.uint32))
+            np.testing.assert_array_equal(hidden.numpy(), want_hidden.numpy())
+    # the window of the last T tokens, also where it starts before the buffer (those read as token 0.0, as the gather has it)
+    seq_host = rng.integers(0, V, (rows, 1)).astype(np.float32)
+    seq_host[3] = 70.0                                              # a token outside the vocabulary: a row of zeros
+    seq = Tensor(seq_host, device="hip")
+    for s in (float(T - 1), 36.0, 39.0, 10.0):
+        slot = Tensor(np.array([[s]], np.float32), device="hip")
+        n0 = hip.launch_count
+        x = nn.decode_window_input(wte, wpe, seq, slot, T)
+        assert hip.launch_count - n0 == 1 and x.shape == (1, T, C)
+        where = Tensor.arange((1, T), device="hip") + (slot - float(T - 1))
+        window = Tensor.embedding(seq, where).reshape((1, T))
+        want = Tensor.embedding(wte, window) + Tensor.embedding(wpe, Tensor.arange((T,), device="hip"))
+        if not hip.COMPILE_ONLY:
+            np.testing.assert_array_equal(x.numpy().view(np.uint32), want.numpy().view(np.uint32))
+    # the end of a step
+    for case, s in (("plain", 4.0), ("ties", 0.0), ("full", float(rows - 1)), ("nan", 7.0), ("long", 2.0)):
+        n = 50304 if case == "long" else V
+        logits_host = rng.standard_normal((1, n)).astype(np.float32)
+        if case == "ties":
+            logits_host[0, [9, 30, 31]] = logits_host.max() + 1.0
+        if case == "nan":
+            logits_host[0, 5] = np.nan
+        if case == "long":
+            logits_host[0, [40000, 45000]] = 9.0
+        logits = Tensor(logits_host, device="hip")
+        got, want = {}, {}
+        for fused, res in ((True, got), (False, want)):
+            tok = Tensor(np.array([[1.0]], np.float32), device="hip")
+            slot = Tensor(np.array([[s]], np.float32), device="hip")
+            buf = Tensor(seq_host.copy(), device="hip")
+            n0 = hip.launch_count
+            if fused:
+                assert nn.decode_append(logits, tok, slot, buf) and hip.launch_count - n0 == 1
+            else:
+                nxt = logits.argmax(1)
+                nslot = slot + 1.0
+                buf.data.row_store_(nxt.data, nslot.data)
+                tok.data.copy_(nxt.data)
+                slot.data.copy_(nslot.data)
+            res.update(tok=tok.numpy(), slot=slot.numpy(), seq=buf.numpy())
+        if not hip.COMPILE_ONLY:
+            for k in want:
+                np.testing.assert_array_equal(got[k], want[k], err_msg=f"{case}: {k}")
+            if case == "ties":
+                assert got["tok"][0, 0] == 9.0
+            if case == "full":
+                np.testing.assert_array_equal(got["seq"], seq_host)          # nowhere to append: the buffer is untouched
+    monkeypatch.setattr(hip.HIP, "DECODE_FUSED", False)
+    assert nn.decode_input(wte, wpe, tok, slot, T, reference_positions) is None and not nn.decode_append(logits, tok, slot, seq)
+
+
+@pytest.mark.gpu
+def test_query_row_product_stores_key_and_value_in_their_cache_rows():
+    """hip, decoding with stacked weights: one launch normalises the row, multiplies it with the stacked projection,
+    returns the query third and writes the key and value thirds to row `slot` of their stores -- the bits of the
+    product followed by the store of the two rows; a slot outside the stores writes nothing."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    rng = np.random.default_rng(13)
+    C, rows = 64, 12
+    ws = [Tensor((rng.standard_normal((C, C)) * 0.2).astype(np.float32), device="hip") for _ in range(3)]
+    nn.stack_parameters(ws)
+    norm = nn.RMSNorm(C, device="hip")
+    norm.weight.data.upload_(rng.standard_normal(norm.weight.shape).astype(np.float32))
+    x = Tensor(rng.standard_normal((1, 1, C)).astype(np.float32), device="hip")
+    for s in (0.0, 7.0, 11.0, 12.0, -1.0):
+        slot = Tensor(np.array([[s]], np.float32), device="hip")
+        init = [rng.standard_normal((rows, 1, C)).astype(np.float32) for _ in range(2)]
+        fused = [Tensor(a.copy(), device="hip") for a in init]
+        plain = [Tensor(a.copy(), device="hip") for a in init]
+        n0 = hip.launch_count
+        q = nn.decode_query_row(x, *ws, norm, fused[0], fused[1], slot)
+        assert q is not None and hip.launch_count - n0 == 1 and q.shape == (1, 1, C)
+        q2, k2, v2 = nn.project_qkv_row(x, *ws, norm)
+        plain[0].data.row_store_(k2.data, slot.data, also=(plain[1].data, v2.data))
+        if hip.COMPILE_ONLY:
+            continue
+        np.testing.assert_array_equal(q.numpy().view(np.uint32), q2.numpy().view(np.uint32))
+        for f, p_, a in zip(fused, plain, init):
+            np.testing.assert_array_equal(f.numpy().view(np.uint32), p_.numpy().view(np.uint32))
+            if not 0 <= s < rows:
+                np.testing.assert_array_equal(f.numpy(), a)                  # nothing stored
+    # the rows not addressed are untouched: a fresh store, one fused call, all rows but `slot` unchanged
+    store_k = Tensor(np.zeros((rows, 1, C), np.float32), device="hip")
+    store_v = Tensor(np.ones((rows, 1, C), np.float32), device="hip")
+    nn.decode_query_row(x, *ws, norm, store_k, store_v, Tensor(np.array([[3.0]], np.float32), device="hip"))
+    if not hip.COMPILE_ONLY:
+        k_host, v_host = store_k.numpy(), store_v.numpy()
+        assert not np.delete(k_host, 3, axis=0).any() and (np.delete(v_host, 3, axis=0) == 1.0).all()
+        assert k_host[3].any() and (v_host[3] != 1.0).any()
 
 
 @pytest.mark.gpu
