@@ -1969,7 +1969,8 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     epi: what the epilogue does to each result c on its way to memory, with e the entry at the same place of a
     fourth operand E shaped like C: "add" stores c + e (a residual), "relu" stores max-like c > 0 ? c : 0,
     "gate" stores e > 0 ? c : 0 (the backward of a ReLU whose output is E).  One rounding each, as the
-    separate element-wise kernel would do.
+    separate element-wise kernel would do.  "bias": E is one row of N values, added to every row of C (the
+    bias of a linear layer, tensor.py:549-563: the Add node after the product, as the product is stored).
     S: edge of the MFMA tile.  A wavefront's share of one output element's k sum is a fixed chain of
     MFMA steps however small its tile, so a long-k product with few output tiles (2048 x 128 x 512: 64
     tiles of 64x64) is bound by that chain on a quarter of the SIMDs.  S = 16 gives every wavefront a
@@ -2225,10 +2226,12 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
 }}
 """
     if epi:
-        assert epi in ("add", "relu", "gate") and not strided
-        macro = {"add": "((cv) + (ev))", "relu": "((cv) > 0.0f ? (cv) : 0.0f)", "gate": "((ev) > 0.0f ? (cv) : 0.0f)"}[epi]
-        edits = [("C += (u64)blockIdx.z * g.M * g.N;", "C += (u64)blockIdx.z * g.M * g.N;\n    E += (u64)blockIdx.z * g.M * g.N;"),
-                 ("struct f3v {", f"#define EPI(cv, ev) {macro}\nstruct f3v {{")]
+        assert epi in ("add", "relu", "gate", "bias") and not strided
+        macro = {"add": "((cv) + (ev))", "relu": "((cv) > 0.0f ? (cv) : 0.0f)", "gate": "((ev) > 0.0f ? (cv) : 0.0f)",
+                 "bias": "((cv) + (ev))"}[epi]
+        edits = [("struct f3v {", f"#define EPI(cv, ev) {macro}\nstruct f3v {{")]
+        if epi != "bias":                               # (a bias row is the same for every batch entry)
+            edits.append(("C += (u64)blockIdx.z * g.M * g.N;", "C += (u64)blockIdx.z * g.M * g.N;\n    E += (u64)blockIdx.z * g.M * g.N;"))
         if tb:
             edits.append(("crow[col] = acc[i][j][e];", "crow[col] = EPI(acc[i][j][e], ev[i][j][e]);"))
         else:
@@ -2255,7 +2258,7 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
     for (int i = 0; i < MI; ++i)
         #pragma unroll
         for (int e = 0; e < {NE}; ++e) {{
-            const float* __restrict__ erow = E + (u64)min({row_expr}, g.M - 1u) * g.N;
+            const float* __restrict__ erow = {'E' if epi == 'bias' else f'E + (u64)min({row_expr}, g.M - 1u) * g.N'};
             {fetch}
         }}
 
@@ -3116,6 +3119,38 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* p, const float* 
 }}
 """
     return src, name, _fmt("P", "P", "P", "I", "f", "f")
+
+
+SGD_MULTI_MAX = 16
+
+
+@cache
+def sgd_multi_inplace_kernel(momentum: bool) -> tuple[str, str, str]:
+    """sgd_inplace_kernel for up to SGD_MULTI_MAX parameters in one launch.  Their addresses and sizes travel
+    in the kernel's argument block, so nothing is uploaded and a captured step replays with them; block b
+    works on the parameter whose first block is the last one not after b (unused entries hold the total).
+    Same statements, same roundings as the launch per parameter."""
+    name = f"sgd_multi_inplace{'_mom' if momentum else ''}"
+    M = SGD_MULTI_MAX
+    src = f"""{PRELUDE}
+struct SgdArgs {{ float* p[{M}]; const float* g[{M}]; float* v[{M}]; u32 first[{M}]; u32 n[{M}]; float lr, mu; }};
+extern "C" __global__ __launch_bounds__(256) void {name}(SgdArgs a) {{
+    #pragma clang fp contract(off)
+    float* p = a.p[0]; const float* g = a.g[0]; float* v = a.v[0];
+    u32 first = 0u, n = a.n[0];
+    #pragma unroll
+    for (u32 k = 1; k < {M}u; ++k)
+        if (blockIdx.x >= a.first[k]) {{ p = a.p[k]; g = a.g[k]; v = a.v[k]; first = a.first[k]; n = a.n[k]; }}
+    const u32 j = (blockIdx.x - first) * 256u + threadIdx.x;
+    if (j < n) {{
+        float upd = g[j];
+        {'{ const float t = v[j] * a.mu; upd = t + upd; v[j] = upd; }' if momentum else '(void)v;'}
+        const float t2 = upd * a.lr;
+        p[j] = p[j] - t2;
+    }}
+}}
+"""
+    return src, name, "@" + "P" * (3 * M) + "I" * (2 * M) + "ff"
 
 
 @cache

@@ -34,15 +34,28 @@ class Optimizer:
 
 class SGD(Optimizer):
     def __init__(self, params: list[Tensor], lr: float = 1e-3, momentum: float = 0.0,
-                 graph_safe: bool = False) -> None:
-        """graph_safe (hip only): parameters and velocities are updated in place, so a captured
-        step can be replayed.  Same arithmetic, same bits."""
+                 graph_safe: bool | None = None) -> None:
+        """graph_safe (hip only): parameters and velocities are updated in place -- sixteen parameters per
+        launch -- so a captured step can be replayed.  Same arithmetic, same bits.  None (the default) chooses
+        it whenever every parameter is on the hip device and the fused kernels are on; False keeps the
+        reference's expression, which rebinds `param.data` to a new buffer per update."""
         super().__init__(params, lr)
         self.momentum = momentum
+        if graph_safe is None:
+            graph_safe = bool(ops.FUSED and params and all(p.device is Device.HIP for p in params))
         self.graph_safe = graph_safe
         self.velocities = {id(p): Tensor.zeros_like(p) for p in params} if momentum else {}
 
     def step(self) -> None:
+        if self.graph_safe and ops.FUSED and self.params and all(p.device is Device.HIP for p in self.params):
+            # every parameter in one launch (sixteen at a time): same statements as the launch per parameter
+            from dlgrad_amd.runtime.hip import HIP
+            live = [p for p in self.params if p.grad is not None]
+            for p in live:
+                assert p.shape == p.grad.shape, f"The shape of the parameter {p.shape} and its grad {p.grad.shape} do not match"
+            HIP.sgd_multi_inplace([(p.data, p.grad.data, self.velocities[id(p)].data if self.momentum != 0 else None) for p in live],
+                                  self.lr, self.momentum)
+            return
         for p in self.params:
             if p.grad is None:
                 continue

@@ -406,8 +406,32 @@ class LinearNT(OP):
         return x.matmul_nt(w)
 
     def backward(self, upstream_grad: Buffer) -> tuple:
-        grad_x, grad_w = product_pair(("nn", upstream_grad, self.w), ("tn", upstream_grad, self.x))
-        return unbroadcast(grad_x, self.x.shape), unbroadcast(grad_w, self.w.shape)
+        return _linear_grads(self, upstream_grad)
+
+
+def _linear_grads(node: OP, upstream_grad: Buffer) -> tuple:
+    """(dX, dW) of x @ W^T for a node that kept x and w: one launch for the two products, or only the one that is asked for
+    (the input of a network's first layer wants no gradient)."""
+    if node.req_grad[0] and node.req_grad[1]:
+        grad_x, grad_w = product_pair(("nn", upstream_grad, node.w), ("tn", upstream_grad, node.x))
+        return unbroadcast(grad_x, node.x.shape), unbroadcast(grad_w, node.w.shape)
+    grad_x = unbroadcast(upstream_grad.matmul(node.w), node.x.shape) if node.req_grad[0] else None
+    grad_w = unbroadcast(upstream_grad.matmul_tn(node.x), node.w.shape) if node.req_grad[1] else None
+    return grad_x, grad_w
+
+
+class LinearNTBias(OP):
+    """x @ W^T + b with the bias row b (W's row count values) added as the product is stored: the Add node of
+    Tensor.linear (tensor.py:549-563) inside LinearNT, one kernel and one pass over the result fewer, same bits.
+    Backward: LinearNT's two products, and the column sum that Add's backward gives the bias."""
+
+    def forward(self, x: Buffer, w: Buffer, b: Buffer) -> Buffer:
+        self.x, self.w, self.b_shape = x, w, b.shape
+        return x.matmul_nt(w, epi="bias", e=b)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        grad_b = self.reduce_grad_for_broadcasting(upstream_grad, self.b_shape) if self.req_grad[2] else None    # as Add hands it to the bias
+        return (*_linear_grads(self, upstream_grad), grad_b)
 
 
 class LinearNTAdd(OP):

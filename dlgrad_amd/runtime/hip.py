@@ -1533,6 +1533,31 @@ class HIP:
         launch(kernel(K.sgd_inplace_kernel, v is not None), (n + 255) // 256, 256,
                _addr(p), _addr(g), _addr(v) if v is not None else 0, n, float(lr), float(momentum))
 
+    @staticmethod
+    def sgd_multi_inplace(triples: list, lr: float, momentum: float) -> None:
+        """The in-place SGD update of every (p, g, v) triple (v None without momentum) in launches of up to
+        K.SGD_MULTI_MAX parameters each; addresses and sizes travel as kernel arguments."""
+        M = K.SGD_MULTI_MAX
+        live = []
+        for p, g, v in triples:
+            if p.numel == 0:
+                continue
+            if g.numel != p.numel or (v is not None and v.numel != p.numel) or p.numel >= 2 ** 31:
+                raise ValueError(f"sgd_step_: parameter {p.shape}, gradient {g.shape}")
+            live.append((_addr(p), _addr(g), _addr(v) if v is not None else 0, p.numel))
+        k = kernel(K.sgd_multi_inplace_kernel, momentum != 0)
+        for at in range(0, len(live), M):
+            part = live[at:at + M]
+            blocks = [(n + 255) // 256 for *_, n in part]
+            first, total = [], 0
+            for b in blocks:
+                first.append(total)
+                total += b
+            pad = M - len(part)
+            launch(k, total, 256, *[q[0] for q in part], *[0] * pad, *[q[1] for q in part], *[0] * pad,
+                   *[q[2] for q in part], *[0] * pad, *first, *[total] * pad, *[q[3] for q in part], *[0] * pad,
+                   float(lr), float(momentum))
+
     ROW_MATMUL = os.environ.get("DLGRAD_HIP_ROW_MATMUL", "1") != "0"        # "0": one-row products on the MFMA tiles too
     DECODE_FUSED = os.environ.get("DLGRAD_HIP_DECODE_FUSED", "1") != "0"    # "0": cached attention as product, softmax, product
     MATMUL_PAIRS = os.environ.get("DLGRAD_HIP_MATMUL_PAIRS", "1") != "0"       # "0": the two products of a linear layer's backward as two launches
@@ -1773,15 +1798,21 @@ class HIP:
         out_numel = B0 * B1 * M * N
         out = alloc(out_numel)
         if epi:
-            if epi not in ("add", "relu", "gate") or tri:
+            if epi not in ("add", "relu", "gate", "bias") or tri:
                 raise ValueError(f"epilogue {epi!r} with tri={tri!r} is not provided")
-            if epi != "relu" and (e is None or e.is_host_scalar or e.numel != B0 * B1 * M * N):
+            if epi == "bias":
+                if e is None or e.is_host_scalar or e.numel != N:
+                    raise ValueError(f"epilogue 'bias' needs a row of {N} values")
+            elif epi != "relu" and (e is None or e.is_host_scalar or e.numel != B0 * B1 * M * N):
                 raise ValueError(f"epilogue {epi!r} needs an operand shaped like the result ({B0 * B1 * M * N} elements)")
         if B0 * B1 * M * N == 0:
             return out
         if Kd == 0:                                            # an empty sum: zeros, plus e for "add"
             if epi == "add":
                 lib().d2d(out.addr, _addr(e), 4 * B0 * B1 * M * N)
+            elif epi == "bias":
+                for r in range(B0 * B1 * M):
+                    lib().d2d(out.addr + 4 * r * N, _addr(e), 4 * N)
             else:
                 lib().fill_f32(out.addr, 0.0, B0 * B1 * M * N)
             return out
@@ -1799,7 +1830,7 @@ class HIP:
         if (M == 1 and batch == 1 and tb and not ta and not tri and HIP.ROW_MATMUL and not HIP.MATMUL_FORCE and Kd % 4 == 0
                 and not ((_addr(x) | _addr(y)) & 15) and (e is None or not e.is_host_scalar)):
             # one row against a transposed matrix (a linear layer while decoding): a wavefront per output
-            k = kernel(K.row_matmul_nt_kernel, epi)
+            k = kernel(K.row_matmul_nt_kernel, "add" if epi == "bias" else epi)      # (for a single row the bias is the residual)
             launch(k, (N + 3) // 4, 256, _addr(x), _addr(y), out.addr, _addr(e) if e is not None else 0, N, Kd)
             _matmul_plans[key] = (k, ((N + 3) // 4, 1, 1), (256, 1, 1), (N, Kd), N, 2, None)
             return out

@@ -242,6 +242,8 @@ class Tensor:
         """self @ weight.T + bias (tensor.py:549-563); weight is (out, in), so every call
         materialises the transpose, as there."""
         if ops.FUSED and self.device is Device.HIP and weight.ndim == 2 and self.ndim >= 2:
+            if bias is not None and bias.device is Device.HIP and bias.numel == weight.shape[0] and bias.shape[-1] == bias.numel:
+                return ops.LinearNTBias.execute(self, weight, bias)     # the addition happens as the product is stored
             out = ops.LinearNT.execute(self, weight)
         else:
             out = self @ weight.T

@@ -248,6 +248,9 @@ def test_epilogues_equal_the_separate_elementwise_kernels(shape_x, shape_y, nt):
     want_add = (plain + ed).numpy()
     want_relu = plain.relu().numpy()
     want_gate = (ed > 0.0).where(inp=plain, other=0.0).numpy()
+    bias = rng.standard_normal((1, plain.shape[-1]), dtype=np.float32)           # one row, added to every row of the product
+    bd = dev(bias)
+    want_bias = (plain + bd).numpy()
     small = min(plain.shape[-2:]) < 64
     tiles = [None] + [t for t in K.MATMUL_CONFIGS if not small or t in K.MATMUL_SMALL_TILES]
     for tile in tiles:
@@ -256,6 +259,7 @@ def test_epilogues_equal_the_separate_elementwise_kernels(shape_x, shape_y, nt):
             check(mm(epi="add", e=ed).numpy(), want_add, 0, f"add {tile}")
             check(mm(epi="relu").numpy(), want_relu, 0, f"relu {tile}")
             check(mm(epi="gate", e=ed).numpy(), want_gate, 0, f"gate {tile}")
+            check(mm(epi="bias", e=bd).numpy(), want_bias, 0, f"bias {tile}")
         finally:
             HIP.MATMUL_FORCE = prev
 
@@ -267,6 +271,8 @@ def test_epilogues_are_refused_without_a_fitting_operand():
         a.matmul(b, epi="add")                          # nothing to add
     with pytest.raises(ValueError):
         a.matmul(b, epi="gate", e=dev(f32(8, 4)))       # wrong size
+    with pytest.raises(ValueError):
+        a.matmul(b, epi="bias", e=dev(f32(8, 8)))       # a bias is one row
     with pytest.raises(ValueError):
         a.matmul(b, epi="square")                       # no such step
     with pytest.raises(ValueError):

@@ -599,6 +599,68 @@ def test_captured_graph_replays_match_eager_steps_bit_for_bit(monkeypatch):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(128, 784), (2, 784), (4, 9, 784), (130, 50)])
+def test_linear_layer_adds_its_bias_as_the_product_is_stored(shape, monkeypatch):
+    """hip: Tensor.linear with a bias is one launch forward (the Add node folded into the product's store) and
+    gives output, input gradient, weight gradient and bias gradient with the bits of the op-by-op form; an
+    input that wants no gradient gets none computed."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    from dlgrad_amd import ops
+    rng = np.random.default_rng(21)
+    n_out = 64 if shape[-1] == 784 else 10
+    xh, wh = rng.standard_normal(shape).astype(np.float32), (rng.standard_normal((n_out, shape[-1])) * 0.1).astype(np.float32)
+    bh, gh = rng.standard_normal((1, n_out)).astype(np.float32), rng.standard_normal(shape[:-1] + (n_out,)).astype(np.float32)
+    res = {}
+    for fused in (True, False):
+        monkeypatch.setattr(ops, "FUSED", fused)
+        x = Tensor(xh, device="hip", requires_grad=True)
+        w, b = Tensor(wh, device="hip", requires_grad=True), Tensor(bh, device="hip", requires_grad=True)
+        n0 = hip.launch_count
+        out = x.linear(w, b)
+        launches = hip.launch_count - n0
+        (out * Tensor(gh, device="hip")).sum().backward()
+        res[fused] = (launches, out.numpy(), x.grad.numpy(), w.grad.numpy(), b.grad.numpy())
+    assert res[True][0] == 1 and res[False][0] > 1
+    if not hip.COMPILE_ONLY:
+        for got, want, what in zip(res[True][1:], res[False][1:], ("out", "dx", "dw", "db")):
+            np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32), err_msg=what)
+    monkeypatch.setattr(ops, "FUSED", True)
+    x = Tensor(xh, device="hip")                                  # data: no gradient asked for
+    w, b = Tensor(wh, device="hip", requires_grad=True), Tensor(bh, device="hip", requires_grad=True)
+    x.linear(w, b).sum().backward()
+    assert x.grad is None and w.grad.shape == w.shape and b.grad.shape == b.shape
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("momentum", [0.0, 0.9])
+def test_in_place_sgd_updates_many_parameters_per_launch(momentum):
+    """hip: the in-place SGD takes up to sixteen parameters per launch; 37 of them (three launches), of sizes
+    around the block size, end with the bits of the out-of-place expression after three steps."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    rng = np.random.default_rng(22)
+    shapes = [(1,), (255,), (256,), (257,), (3, 100), (64, 784), (1, 64)] + [(int(n),) for n in rng.integers(1, 2000, 30)]
+    init = [rng.standard_normal(sh).astype(np.float32) for sh in shapes]
+    grads = [[rng.standard_normal(sh).astype(np.float32) for sh in shapes] for _ in range(3)]
+    res = {}
+    for graph_safe in (True, False):
+        ps = [Tensor(a.copy(), device="hip", requires_grad=True) for a in init]
+        opt = nn.optim.SGD(ps, lr=1e-2, momentum=momentum, graph_safe=graph_safe)
+        for step in range(3):
+            for p, g in zip(ps, grads[step]):
+                p.grad = Tensor(g, device="hip")
+            n0 = hip.launch_count
+            opt.step()
+            if graph_safe:
+                assert hip.launch_count - n0 == 3
+        res[graph_safe] = [p.numpy() for p in ps]
+    if not hip.COMPILE_ONLY:
+        for a, b in zip(res[True], res[False]):
+            np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("momentum", [0.0, 0.9])
 def test_captured_mlp_step_with_in_place_sgd_matches_eager_steps_bit_for_bit(momentum):
     """The 784-64-10 MLP step (test/test_forward_backward.py's shape) as a replayed graph with a new
