@@ -1091,8 +1091,9 @@ class HIP:
                 launch(kernel(K.embedding_backward_ordered_kernel, "segments", vec, x.numel >= NT_STORE_MIN_ELEMENTS),
                        n_sum + n_zero, 256, out.addr, partial.addr, segmask.addr, firsts.addr, gfirst.addr, idsegs.addr,
                        _addr(upstream_grad), _addr(idx), n_idx, W, V, n_zero, every)
-                launch(kernel(K.embedding_backward_ordered_kernel, "merge", vec), n_sum, 256, out.addr, partial.addr,
-                       segmask.addr, firsts.addr, gfirst.addr, _addr(idx), n_idx, W, V)
+                if NS > 1:                                     # (within one segment no id spans segments: nothing to merge)
+                    launch(kernel(K.embedding_backward_ordered_kernel, "merge", vec), n_sum, 256, out.addr, partial.addr,
+                           segmask.addr, firsts.addr, gfirst.addr, _addr(idx), n_idx, W, V)
                 return out
             out = alloc(x.numel, zero=True)                    # init_with_scalar(0), cpu.py:1031
             if n_idx:                                          # very long index lists: hardware fp32 atomics
