@@ -1190,6 +1190,63 @@ extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out
     return f"{PRELUDE}{_ORDERED_COMMON}{body}", name, fmt
 
 
+EMB_SMALL_MAX_N = 4096         # longest index list of the one-launch scatter-add: every row's wavefront reads all of it
+EMB_SMALL_MAX_WAVES = 4096     # (table rows) x (column chunks) it is used for: beyond that the three-launch form has more to offer
+
+
+@cache
+def embedding_backward_small_kernel(vec: int = 1) -> tuple[str, str, str]:
+    """Scatter-add into a small (V, W) table in one launch, in exactly the order of the reference's loop
+    (cpu_kernel.py:231-243: zero the table, then out[idx[i]] += g[i] for i = 0, 1, ...).
+    One wavefront per (table row, chunk of 64 * vec columns).  It reads the index list segment by segment
+    (512 positions, eight ballots), lists the positions that name its row in LDS, and adds their gradient
+    rows in index order, eight loads in flight; a row nobody names is written as zeros.  Every table element
+    is written once, nothing is zero-filled first, no atomics: the bits are those of the sequential loop
+    for every id, however its positions are spread.  Ids outside [0, V) take no part."""
+    name = f"embedding_scatter_small_v{vec}"
+    VT = "float4" if vec == 4 else "float"
+    zero = "make_float4(0.f, 0.f, 0.f, 0.f)" if vec == 4 else "0.0f"
+    add = ("acc.x += t[u].x; acc.y += t[u].y; acc.z += t[u].z; acc.w += t[u].w;" if vec == 4 else "acc += t[u];")
+    body = f"""
+extern "C" __global__ __launch_bounds__(256) void {name}(float* __restrict__ out, const float* __restrict__ g,
+        const float* __restrict__ idx, u32 n, u32 W, u32 V, u32 chunks) {{
+    __shared__ u32 lists[4][{EMB_SEGMENT}];
+    const u32 w = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    const u32 id = blockIdx.x * 4u + w;
+    const u32 v = id / chunks;
+    if (v >= V) return;
+    const u32 Wv = W / {vec}u;
+    const u32 c = (id - v * chunks) * 64u + lane;               // this lane's column item
+    const bool live = c < Wv;
+    u32* __restrict__ list = lists[w];
+    {VT} acc = {zero};
+    for (u32 s0 = 0; s0 < n; s0 += EMB_SEG) {{
+        u64 hit[EMB_NK];
+        segment_hits(idx, (int)v, s0, min(n, s0 + EMB_SEG), n, lane, hit);
+        u32 m = 0;
+        #pragma unroll
+        for (u32 k = 0; k < EMB_NK; ++k) {{
+            if ((hit[k] >> lane) & 1ull) list[m + (u32)__popcll(hit[k] & ((1ull << lane) - 1ull))] = s0 + 64u * k + lane;
+            m += (u32)__popcll(hit[k]);
+        }}
+        if (m == 0u) continue;                                  // (wave-uniform)
+        wave_lds_fence();
+        for (u32 q0 = 0; q0 < m; q0 += 8u) {{
+            {VT} t[8];
+            #pragma unroll
+            for (u32 u = 0; u < 8u; ++u)                        // loads past the end repeat the last row
+                t[u] = live ? reinterpret_cast<const {VT}*>(g + (u64)list[min(q0 + u, m - 1u)] * W)[c] : {zero};
+            #pragma unroll
+            for (u32 u = 0; u < 8u; ++u) if (q0 + u < m) {{ {add} }}
+        }}
+        wave_lds_fence();                                       // the next segment overwrites the list
+    }}
+    if (live) reinterpret_cast<{VT}*>(out + (u64)v * W)[c] = acc;
+}}
+"""
+    return f"{PRELUDE}{_ORDERED_COMMON}{body}", name, _fmt("P", "P", "P", "I", "I", "I", "I")
+
+
 @cache
 def ce_kernel(backward: bool) -> tuple[str, str, str]:
     """ce_forward: out[i] = x[(int)target[i] + stride0*i]; ce_backward: that element -= 1,

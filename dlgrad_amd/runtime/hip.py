@@ -1010,6 +1010,18 @@ class HIP:
 
     # ---- permute ---------------------------------------------------------------------------------------------
     @staticmethod
+    @dispatcher.register(UnaryOps.TRANSPOSE, Device.HIP)
+    def transpose(x: Buffer, dim0: int, dim1: int, out_stride: tuple | None = None, out_shape: tuple | None = None) -> DevicePtr:
+        """Materialised swap of two dims, under the name and keywords the reference's other runtimes register
+        (cpu_jit.py:316-317, metal.py:374-375; its live CPU runtime routes Buffer.transpose through PERMUTE,
+        buffer.py:292-297, as Buffer.transpose does here).  out_stride / out_shape follow from x and are not needed."""
+        nd = x.ndim
+        d0, d1 = dim0 % nd, dim1 % nd
+        order = list(range(nd))
+        order[d0], order[d1] = order[d1], order[d0]
+        return HIP.permute(x, tuple(order))
+
+    @staticmethod
     @dispatcher.register(UnaryOps.PERMUTE, Device.HIP)
     def permute(x: Buffer, order: tuple) -> DevicePtr:
         """Materialised permutation (cpu.py:333-368).  After merging dims that stay
@@ -1071,12 +1083,27 @@ class HIP:
 
     # ---- embedding and cross-entropy helpers ----------------------------------------------------------------------
     @staticmethod
+    def scatter_small_fits(V: int, W: int, n: int) -> bool:
+        """Whether the scatter-add into a (V, W) table from n indices goes out as the one-launch form: a list short
+        enough for every row's wavefront to read all of it, and few enough wavefronts."""
+        return (EMB_ORDERED and 0 < n <= K.EMB_SMALL_MAX_N and 0 < V and 0 < W
+                and V * (((W + 3) // 4 + 63) // 64) <= K.EMB_SMALL_MAX_WAVES and V * W < 2 ** 31)
+
+    @staticmethod
     @dispatcher.register(CustomOps.EMBEDDING, Device.HIP)
     def embedding(x: Buffer, idx: Buffer, out_numel: int, backward: bool = False,
                   upstream_grad: Buffer = None) -> DevicePtr:
         W, n_idx = x.shape[-1], idx.numel
         if backward:
             V = x.numel // W
+            if HIP.scatter_small_fits(V, W, n_idx):
+                # a small table and a short list: one launch, a wavefront per table row and 64 column items, the reference's order
+                out = alloc(x.numel)
+                vec = 4 if (W % 4 == 0 and not (_addr(upstream_grad) | out.addr) & 15) else 1
+                chunks = (W // vec + 63) // 64
+                launch(kernel(K.embedding_backward_small_kernel, vec), (V * chunks + 3) // 4, 256, out.addr, _addr(upstream_grad),
+                       _addr(idx), n_idx, W, V, chunks)
+                return out
             if n_idx and n_idx <= K.EMB_ORDERED_MAX and EMB_ORDERED and x.numel < 2 ** 31 and W <= 1 << 22:
                 # two launches write every element of the table exactly once -- sums in index order where an id
                 # occurs, zeros elsewhere -- without a zero-fill pass and without atomics

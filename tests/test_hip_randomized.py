@@ -148,7 +148,7 @@ def test_random_embedding_gathers_and_ordered_scatter_adds(seed):
     the gather is bit-exact, the scatter-add bit-exact against the float32 model of its summation
     order (index order inside segments of 512 positions, then the segment sums in order)."""
     require_gpu()
-    from tests.test_hip_reduce_layout import ordered_scatter_model
+    from tests.test_hip_reduce_layout import scatter_order_model
     rng = np.random.default_rng(5000 + seed)
     for _ in range(6):
         V = int(rng.choice([1, 3, 50, 700, 5000]))
@@ -164,7 +164,7 @@ def test_random_embedding_gathers_and_ordered_scatter_adds(seed):
         got = t.embedding(dev(ids), backward=True, upstream_grad=dev(g)).numpy()
         if hip.COMPILE_ONLY:
             continue
-        want = ordered_scatter_model(V, ids, g)
+        want = scatter_order_model(V, W, ids, g)
         assert (got.view(np.uint32) == want.view(np.uint32)).all(), f"scatter V{V} W{W} n{n} {kind}"
 
 

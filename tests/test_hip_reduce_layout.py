@@ -157,6 +157,11 @@ def test_transpose_helpers():
     check(dev(x).T.numpy(), x.T, 0, "T")
     x4 = f32(2, 3, 4, 5)
     check(dev(x4).transpose(1, 2).numpy(), x4.transpose(0, 2, 1, 3), 0, "transpose(1,2)")
+    # the op the reference's other runtimes register under UnaryOps.TRANSPOSE, with their keywords
+    from dlgrad_amd.dispatch import dispatcher
+    from dlgrad_amd.helpers import UnaryOps
+    got = dispatcher.dispatch(UnaryOps.TRANSPOSE, Device.HIP, x=dev(x4), out_stride=(60, 5, 15, 1), out_shape=(2, 4, 3, 5), dim0=1, dim1=2)
+    check(Buffer(got, (2, 4, 3, 5), Device.HIP).numpy(), x4.transpose(0, 2, 1, 3), 0, "UnaryOps.TRANSPOSE")
 
 
 @pytest.mark.parametrize("V,W,idx_shape", [(100, 32, (4, 16)), (65, 128, (16, 128)), (128, 128, (128,)),
@@ -218,16 +223,30 @@ def ordered_scatter_model(V, idx, g, segment=512):
     return out
 
 
+def scatter_order_model(V, W, idx, g):
+    """What the deterministic scatter-add must give, bit for bit: the sequential order of the reference's loop where
+    the one-launch form for small tables applies, the segment-wise order of the three-launch form elsewhere."""
+    n = int(np.asarray(idx).size)
+    return ordered_scatter_model(V, idx, g, segment=n if hip.HIP.scatter_small_fits(V, W, n) else 512)
+
+
+@pytest.mark.parametrize("small", [False, True])
 @pytest.mark.parametrize("W", [4, 7, 96, 2052])
 @pytest.mark.parametrize("pattern", ["same", "pairs", "span", "zipf", "hot"])
-def test_ordered_scatter_add_has_exactly_the_documented_summation_order(pattern, W):
+def test_ordered_scatter_add_has_exactly_the_documented_summation_order(pattern, W, small, monkeypatch):
     """Bit-exact against a float32 model of the order, for id patterns that exercise one id
     filling whole segments (its 512 wavefronts split the columns, most get none), adjacent
     pairs, ids that occur once in every segment (merge only), Zipf ids, and one hot id among
     unique ones; W = 7 takes the 4-byte kernels, W = 2052 needs two passes over a row.  Table
-    rows no index names come out as zeros although nothing zero-fills the table first."""
+    rows no index names come out as zeros although nothing zero-fills the table first.
+    small: the one-launch form for small tables (strictly the reference's sequential order); otherwise
+    the three-launch form, forced also where the one-launch form would apply."""
     require_gpu()
     V, n = 3000, 1536 + 77
+    if small and not hip.HIP.scatter_small_fits(V, W, n):
+        pytest.skip("too many wavefronts for the one-launch form")
+    if not small:
+        monkeypatch.setattr(hip.HIP, "scatter_small_fits", staticmethod(lambda V, W, n: False))
     rng = np.random.default_rng(W)
     ids = {"same": np.full(n, 5), "pairs": np.repeat(rng.permutation(V)[:(n + 1) // 2], 2)[:n],
            "span": np.tile(rng.permutation(V)[:512], 4)[:n], "zipf": np.minimum(rng.zipf(1.1, n) - 1, V - 1),
@@ -237,10 +256,14 @@ def test_ordered_scatter_add_has_exactly_the_documented_summation_order(pattern,
     poison = np.full((V, W), np.nan, np.float32)                  # whatever the output block held before must not show
     keep = [dev(poison) for _ in range(3)]
     del keep
+    n0 = hip.launch_count
     got = dev(f32(V, W)).embedding(dev(ids), backward=True, upstream_grad=dev(g)).numpy()
+    assert hip.launch_count - n0 == (1 if small else 3)
     if not hip.COMPILE_ONLY:
-        want = ordered_scatter_model(V, ids, g)
+        want = scatter_order_model(V, W, ids, g)
         np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+        if small:                                                 # the reference's loop, literally
+            np.testing.assert_array_equal(got.view(np.uint32), cref.embedding_backward((V, W), ids, g).view(np.uint32))
 
 
 @pytest.mark.parametrize("V,W,n", [(40, 2, 2000), (1, 1, 300), (70000, 4, 5), (130, 8, 32768), (64, 12, 40000)])
@@ -254,7 +277,7 @@ def test_scatter_add_on_narrow_tall_and_long_inputs(V, W, n):
     if hip.COMPILE_ONLY:
         return
     if n <= 32768:
-        want = ordered_scatter_model(V, idx, g)
+        want = scatter_order_model(V, W, idx, g)
         np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
     want = np.zeros((V, W))
     np.add.at(want, idx.astype(int), g.astype(np.float64))
