@@ -541,6 +541,11 @@ class Buffer:
             dst2.row_store_(src2, idx)
         self._dispatch(CustomOps.ROW_STORE, dst=self, src=src, idx=idx, rows=rows, width=width)
 
+    def embedding_sum(self, pos_table: "Buffer", idx: "Buffer", pos: "Buffer") -> "Buffer":
+        """self[idx] + pos_table[pos] for idx (B, T) and pos (T,): (B, T, W), one launch on the hip device."""
+        out = self._dispatch(CustomOps.EMBEDDING_SUM, tok_table=self, pos_table=pos_table, idx=idx, pos=pos)
+        return Buffer.fresh(out, tuple(idx.shape) + (self.shape[-1],), self.device)
+
     # ---- the ends of a decoding step (hip) -------------------------------------------------------
     def decode_qkv_row(self, w: "Buffer", gain: "Buffer", eps: float, kc: "Buffer", vc: "Buffer", slot: "Buffer") -> "Buffer":
         """self: one row; w: the stacked (3C, K) q, k, v projection.  Returns q (C,) = the first third of

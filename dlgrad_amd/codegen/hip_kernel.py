@@ -911,6 +911,38 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 
 
 @cache
+def embedding_sum_kernel() -> tuple[str, str, str]:
+    """out[i, :] = tok_table[idx[i]] + pos_table[pos[i % T]] for n = B * T positions: the token and position
+    embeddings of a transformer's input and their sum (examples/gpt.py:96-98: two gathers and a broadcast add)
+    in one launch.  Rows are looked up as embedding_kernel does it (offset (int)(id * W) formed in float, a row
+    outside its table reads as zeros) and the sum is the one fp32 addition of the add kernel: same bits.
+    One wavefront per position."""
+    name = "embedding_sum"
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ tok_table,
+        const float* __restrict__ pos_table, const float* __restrict__ idx, const float* __restrict__ pos,
+        float* __restrict__ out, u32 n, u32 T, u32 W, u32 tok_total, u32 pos_total, u32 aligned) {{
+    const u32 i = blockIdx.x * 4u + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    if (i >= n) return;
+    const int ti = (int)(idx[i] * (float)W), pi = (int)(pos[i % T] * (float)W);
+    const bool tok_ok = ti >= 0 && (u64)ti + W <= (u64)tok_total, pos_ok = pi >= 0 && (u64)pi + W <= (u64)pos_total;
+    const float* __restrict__ a = tok_table + (long long)(tok_ok ? ti : 0);
+    const float* __restrict__ b = pos_table + (long long)(pos_ok ? pi : 0);
+    float* __restrict__ dst = out + (u64)i * W;
+    if (aligned && tok_ok && pos_ok && ((ti | pi) & 3) == 0) {{
+        for (u32 v = lane; v < (W >> 2); v += 64u) {{
+            const float4 p = reinterpret_cast<const float4*>(a)[v], q = reinterpret_cast<const float4*>(b)[v];
+            reinterpret_cast<float4*>(dst)[v] = make_float4(p.x + q.x, p.y + q.y, p.z + q.z, p.w + q.w);
+        }}
+    }} else {{
+        for (u32 j = lane; j < W; j += 64u) dst[j] = (tok_ok ? a[j] : 0.0f) + (pos_ok ? b[j] : 0.0f);
+    }}
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "P", "P", "I", "I", "I", "I", "I", "I")
+
+
+@cache
 def embedding_backward_kernel() -> tuple[str, str, str]:
     """Scatter-add: out[(int)idx[i], j] += g[i, j] into a zeroed (V, W) table
     (cpu_kernel.py:231-243).  The row index is formed in integers; the reference forms

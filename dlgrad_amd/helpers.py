@@ -95,6 +95,7 @@ class CustomOps(_Op):
     ADAM_MULTI_INPLACE = auto()     # one launch for a whole parameter list (addresses in a device table)
     SGD_STEP_INPLACE = auto()       # p -= (momentum-filtered) g * lr where p is (graph replay)
     SET_VALUES = auto()             # a few floats given by value written into an existing buffer by a kernel (no transfer, no wait)
+    EMBEDDING_SUM = auto()          # token rows + position rows of a transformer's input: two gathers and their sum, one kernel
     DECODE_QKV_ROW = auto()         # q, k, v of one new position from the stacked projection, k and v stored into their cache rows
     DECODE_EMBED = auto()           # the input of a decoding step (token + position embedding, cache-row mask) from device-resident state
     DECODE_NEXT = auto()            # argmax of the logits, appended to the token buffer, made the next token; the index advanced

@@ -167,6 +167,17 @@ def project_qkv_row(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor, norm=None) ->
     return x.linear(wq, None), x.linear(wk, None), x.linear(wv, None)
 
 
+def embed_tokens(wte: "Embedding", wpe: "Embedding", idx: Tensor, pos: Tensor) -> Tensor:
+    """wte(idx) + wpe(pos) for token ids idx (B, T) and position ids pos (T,): the first line of a transformer's
+    forward (examples/gpt.py:96-98).  On the hip device one node and one launch, bit-identical to the three ops;
+    elsewhere the three ops."""
+    if ops.FUSED and idx.ndim == 2 and pos.ndim == 1 and pos.numel == idx.shape[1] and wte.weight.ndim == 2 \
+            and wpe.weight.ndim == 2 and wte.weight.shape[1] == wpe.weight.shape[1] \
+            and all(t.device is Device.HIP for t in (wte.weight, wpe.weight, idx, pos)):
+        return ops.EmbeddingSum.execute(wte.weight, wpe.weight, idx, pos)
+    return wte(idx) + wpe(pos)
+
+
 def _decode_fused(*tensors: Tensor) -> bool:
     if not ops.FUSED or any(t.device is not Device.HIP for t in tensors):
         return False

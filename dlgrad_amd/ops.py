@@ -786,6 +786,26 @@ class Embedding(OP):
         return (self.weight.embedding(self.idx, backward=True, upstream_grad=upstream_grad),)
 
 
+class EmbeddingSum(OP):
+    """tok_table[idx] + pos_table[pos] for idx (B, T) and pos (T,): the input of a transformer (examples/gpt.py:96-98:
+    two Embedding nodes and an Add) as one node and, on the hip device, one launch.  Backward: what those three
+    nodes do -- the scatter-add of the upstream rows into the token table, the sum over the batch that Add's
+    backward gives its broadcast operand, and the scatter-add of that into the position table."""
+
+    def forward(self, tok_table: Buffer, pos_table: Buffer, idx: Buffer, pos: Buffer) -> Buffer:
+        self.tok_table, self.pos_table, self.idx, self.pos = tok_table, pos_table, idx, pos
+        return tok_table.embedding_sum(pos_table, idx, pos)
+
+    def backward(self, upstream_grad: Buffer) -> tuple:
+        g_tok = g_pos = None
+        if self.req_grad[0]:
+            g_tok = self.tok_table.embedding(self.idx, backward=True, upstream_grad=upstream_grad)
+        if self.req_grad[1]:
+            rows = self.reduce_grad_for_broadcasting(upstream_grad, tuple(self.pos.shape) + (self.pos_table.shape[-1],))
+            g_pos = self.pos_table.embedding(self.pos, backward=True, upstream_grad=rows)
+        return g_tok, g_pos, None, None
+
+
 class Where(OP):
     def forward(self, cond: Buffer, inp: Buffer, other: Buffer) -> Buffer:
         self.cond = cond

@@ -1135,6 +1135,20 @@ class HIP:
         return out
 
     @staticmethod
+    @dispatcher.register(CustomOps.EMBEDDING_SUM, Device.HIP)
+    def embedding_sum(tok_table: Buffer, pos_table: Buffer, idx: Buffer, pos: Buffer) -> DevicePtr:
+        """out[i] = tok_table[idx[i]] + pos_table[pos[i % T]] for the idx.numel positions (T = pos.numel)."""
+        W, n, T = tok_table.shape[-1], idx.numel, pos.numel
+        if pos_table.shape[-1] != W or T == 0 or n % T or max(tok_table.numel, pos_table.numel, n * W) >= 2 ** 31:
+            raise ValueError(f"embedding_sum: tables {tok_table.shape}, {pos_table.shape}, {n} ids, {T} positions")
+        out = alloc(n * W)
+        if n:
+            aligned = int(W % 4 == 0 and not (_addr(tok_table) | _addr(pos_table) | out.addr) & 15)
+            launch(kernel(K.embedding_sum_kernel), (n + 3) // 4, 256, _addr(tok_table), _addr(pos_table), _addr(idx), _addr(pos),
+                   out.addr, n, T, W, tok_table.numel, pos_table.numel, aligned)
+        return out
+
+    @staticmethod
     @dispatcher.register(CustomOps.CE_FORWARD, Device.HIP)
     def ce_forward(x: Buffer, y: Buffer) -> DevicePtr:
         rows = x.shape[0]

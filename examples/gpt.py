@@ -128,7 +128,7 @@ class GPT:
     def __call__(self, idx: Tensor, targets: Tensor | None = None):
         """idx, targets: (B, T) token ids stored as fp32.  Returns (logits, loss)."""
         B, T = idx.shape
-        x = self.wte(idx) + self.wpe(_positions(T, idx.device))
+        x = nn.embed_tokens(self.wte, self.wpe, idx, _positions(T, idx.device))
         for block in self.blocks:
             x = block(x)
         logits = nn.norm_linear(x, self.ln_f, self.lm_head.weight)
