@@ -600,12 +600,13 @@ def test_captured_graph_replays_match_eager_steps_bit_for_bit(monkeypatch):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("V,P,C,B,T", [(65, 128, 128, 16, 128), (50, 9, 6, 3, 9), (300, 40, 64, 2, 33)])
-def test_token_and_position_embeddings_and_their_sum_in_one_launch(V, P, C, B, T):
+def test_token_and_position_embeddings_and_their_sum_in_one_launch(V, P, C, B, T, monkeypatch):
     """hip: nn.embed_tokens is one node and one launch; output and both table gradients have the bits of
     wte(idx) + wpe(pos) (two gathers, a broadcast add; backward: scatter-add, batch sum, scatter-add),
     also with ids outside their tables (rows of zeros, no gradient)."""
     if not (hip.available() or hip.COMPILE_ONLY):
         pytest.skip("no HIP device")
+    monkeypatch.setattr(hip, "EMB_ORDERED", True)      # (the atomic scatter-add adds in whatever order the hardware takes)
     rng = np.random.default_rng(V + T)
     ids = rng.integers(0, V, (B, T)).astype(np.float32)
     ids[0, 0], ids[B - 1, T - 1] = float(V), -1.0
