@@ -202,3 +202,70 @@ def test_random_masked_softmax_equals_its_chain(seed):
             continue
         assert (outs[0][0].view(np.uint32) == outs[1][0].view(np.uint32)).all(), f"forward {xs} {ms} {scale}"
         assert (outs[0][1].view(np.uint32) == outs[1][1].view(np.uint32)).all(), f"backward {xs} {ms} {scale}"
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_fused_launches_against_closed_forms(seed):
+    """The launches that fold several ops into one, on random shapes, against numpy closed forms with the same
+    roundings: token + position embedding (a gather, a gather, one fp32 add: bit-exact, ids outside their table
+    read as zeros, any row width and alignment); the bias a product adds as it stores (the product's own bits
+    plus one fp32 add); the end of a decoding step (first maximum; the token buffer's bound); the in-place SGD
+    for many parameters per launch (two or four roundings per element)."""
+    require_gpu()
+    from dlgrad_amd import Tensor, nn
+    rng = np.random.default_rng(7000 + seed)
+    for _ in range(4):
+        # ---- embedding sum
+        V, P = int(rng.choice([1, 7, 65, 300])), int(rng.choice([1, 9, 40]))
+        C = int(rng.choice([1, 3, 4, 6, 32, 100, 128]))
+        B, T = int(rng.choice([1, 2, 5])), int(rng.choice([1, 4, 9, 33]))
+        wte, wpe = rng.standard_normal((V, C), dtype=np.float32), rng.standard_normal((P, C), dtype=np.float32)
+        ids = rng.integers(-1, V + 1, (B, T)).astype(np.float32)
+        pos = rng.integers(-1, P + 1, (T,)).astype(np.float32)
+        tt, pt = (misaligned(wte), misaligned(wpe)) if rng.random() < 0.5 else (dev(wte), dev(wpe))
+        got = tt.embedding_sum(pt, dev(ids), dev(pos)).numpy()
+        tok_rows = np.where(((ids >= 0) & (ids < V))[..., None], wte[np.clip(ids, 0, V - 1).astype(int)], np.float32(0))
+        pos_rows = np.where(((pos >= 0) & (pos < P))[..., None], wpe[np.clip(pos, 0, P - 1).astype(int)], np.float32(0))
+        check(got, (tok_rows + pos_rows[None]).astype(np.float32), 0, f"embedding sum V{V} P{P} C{C} B{B} T{T}")
+        # ---- bias epilogue
+        M, Kd, N = int(rng.choice([1, 2, 31, 130])), int(rng.choice([4, 12, 64, 100])), int(rng.choice([1, 3, 10, 64, 130]))
+        x, w, b = rng.standard_normal((M, Kd), dtype=np.float32), rng.standard_normal((N, Kd), dtype=np.float32), rng.standard_normal((1, N), dtype=np.float32)
+        xd, wd = dev(x), dev(w)
+        plain = xd.matmul_nt(wd).numpy()
+        check(xd.matmul_nt(wd, epi="bias", e=dev(b)).numpy(), plain + b, 0, f"bias {M}x{Kd}x{N}")
+        # ---- the end of a decoding step
+        Vn, rows = int(rng.choice([2, 65, 1000, 5000])), int(rng.choice([1, 3, 40]))
+        logits = rng.standard_normal((1, Vn), dtype=np.float32)
+        if rng.random() < 0.5:
+            logits[0, rng.integers(0, Vn, 3)] = 9.0                  # ties: the first one wins
+        s = float(rng.integers(-1, rows + 1))
+        seq0 = rng.standard_normal((rows, 1), dtype=np.float32)
+        tok, slot, seq = (Tensor(a, device="hip") for a in (np.array([[5.0]], np.float32), np.array([[s]], np.float32), seq0.copy()))
+        assert nn.decode_append(Tensor(logits, device="hip"), tok, slot, seq)
+        if not hip.COMPILE_ONLY:
+            best = float(np.argmax(logits[0]))
+            want_seq = seq0.copy()
+            if 0 <= s + 1 < rows:
+                want_seq[int(s) + 1, 0] = best
+            assert tok.numpy()[0, 0] == best and slot.numpy()[0, 0] == s + 1, f"decode_next V{Vn} slot {s}"
+            np.testing.assert_array_equal(seq.numpy(), want_seq)
+        # ---- many parameters per SGD launch
+        count, mu, lr = int(rng.choice([1, 5, 16, 17, 33])), float(rng.choice([0.0, 0.9])), np.float32(0.05)
+        shapes = [(int(rng.integers(1, 700)),) for _ in range(count)]
+        ps = [rng.standard_normal(sh, dtype=np.float32) for sh in shapes]
+        gs = [rng.standard_normal(sh, dtype=np.float32) for sh in shapes]
+        params = [Tensor(p.copy(), device="hip", requires_grad=True) for p in ps]
+        opt = nn.optim.SGD(params, lr=float(lr), momentum=mu, graph_safe=True)
+        vs = [np.zeros_like(p) for p in ps]
+        for step in range(2):
+            for p, g in zip(params, gs):
+                p.grad = Tensor(g, device="hip")
+            opt.step()
+            for i, g in enumerate(gs):
+                upd = g
+                if mu:
+                    vs[i] = (vs[i] * np.float32(mu)).astype(np.float32) + g
+                    upd = vs[i]
+                ps[i] = ps[i] - (upd * lr).astype(np.float32)
+        for p, want in zip(params, ps):
+            check(p.numpy(), want, 0, f"sgd x{count} mu={mu}")
