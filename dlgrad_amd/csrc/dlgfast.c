@@ -165,7 +165,7 @@ static PyObject *fast_alloc(PyObject *self, PyObject *arg) {
     if (nbytes == (unsigned long long)-1 && PyErr_Occurred()) return NULL;
     void *p = NULL;
     int rc = p_alloc((size_t)nbytes, &p);
-    if (rc != 0) return raise_last(PyExc_MemoryError, rc);
+    if (rc != 0) return raise_last(rc == -9 ? PyExc_RuntimeError : PyExc_MemoryError, rc);   /* -9: refused inside a capture */
     return devptr_make((unsigned long long)(uintptr_t)p, nbytes, NULL);
 }
 
@@ -228,7 +228,7 @@ static PyObject *fast_launch_out(PyObject *self, PyObject *const *args, Py_ssize
     }
     void *p = NULL;
     int rc = p_alloc((size_t)nbytes, &p);
-    if (rc != 0) return raise_last(PyExc_MemoryError, rc);
+    if (rc != 0) return raise_last(rc == -9 ? PyExc_RuntimeError : PyExc_MemoryError, rc);   /* -9: refused inside a capture */
     PyObject *out = devptr_make((unsigned long long)(uintptr_t)p, nbytes, NULL);
     if (!out) {
         (void)p_free(p);

@@ -132,6 +132,14 @@ int alloc_locked(size_t nbytes, void **out) {
         it->second.pop_back();
         g_bytes_cached -= b;
     } else {
+        if (g_capturing) {                    // a device allocation (and the wait of its retry) is no part of a graph:
+            *out = nullptr;                   // the step being captured must find every block in its arena
+            char buf[256];
+            std::snprintf(buf, sizeof buf,
+                          "allocation of %zu bytes missed the arena during a capture: run the step once inside the "
+                          "arena first, with the same shapes", nbytes);
+            return fail_msg(-9, buf);
+        }
         void *p = nullptr;
         hipError_t e = hipMalloc(&p, b);
         if (e != hipSuccess) {                // give cached blocks back and retry once

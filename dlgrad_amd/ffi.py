@@ -179,11 +179,13 @@ class HipLib:
         fn = self._lib.dlg_hip_alloc_zero if zero else self._lib.dlg_hip_alloc
         if self._cffi is not None:
             ref, get = self._out(ctypes.c_void_p, "void *")
-            self._check(fn(nbytes, ref), MemoryError)
+            rc = fn(nbytes, ref)
+            self._check(rc, HipError if rc == -9 else MemoryError)      # -9: refused inside a capture
             return get()
         box = self._alloc_box                     # one reusable out-parameter: this runs per op
-        if fn(nbytes, self._alloc_ref) != 0:
-            self._check(-1, MemoryError)
+        rc = fn(nbytes, self._alloc_ref)
+        if rc != 0:
+            self._check(rc, HipError if rc == -9 else MemoryError)
         return box.value or 0
 
     def free(self, ptr: int) -> None:

@@ -141,6 +141,31 @@ def self_attention_qkv(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor, n_head: in
     return causal_self_attention(x.linear(wq, None), x.linear(wk, None), x.linear(wv, None), n_head, scale)
 
 
+_inference_depth = 0
+
+
+class inference:
+    """with nn.inference(): ... -- the caller states that nothing computed inside will be differentiated.
+    The single-row decoding forms of norm_linear, mlp_relu and project_qkv_row return results without a
+    tape; outside such a block they are taken only when no input asks for a gradient, so that a training
+    forward over a single row (a (1, 1) batch) keeps its graph."""
+
+    def __enter__(self):
+        global _inference_depth
+        _inference_depth += 1
+        return self
+
+    def __exit__(self, *exc):
+        global _inference_depth
+        _inference_depth -= 1
+        return False
+
+
+def _tape_free(*tensors) -> bool:
+    """May a result of these inputs go without a tape?  Inside nn.inference(), or when none of them requires a gradient."""
+    return _inference_depth > 0 or not any(t is not None and t.requires_grad for t in tensors)
+
+
 def _row_norm(x: Tensor, w: Buffer, norm) -> tuple | None:
     """(gain, eps) if the product of the single row x with w^T can RMS-normalise x on the way (hip device,
     a norm with a gain, a row that fits the kernel), else None: the caller then applies the norm itself."""
@@ -155,7 +180,8 @@ def project_qkv_row(x: Tensor, wq: Tensor, wk: Tensor, wv: Tensor, norm=None) ->
     in memory (stack_parameters), the hip device runs one product and the three results are the
     thirds of its output row; such results carry no tape (inference only).  Otherwise three linears.
     norm: an RMSNorm to apply to x first; in the one-product case it is applied inside the product."""
-    if x.numel == x.shape[-1] and x.numel and ops.FUSED and ops.stacked(wq, wk, wv) and x.device is wq.device:
+    if x.numel == x.shape[-1] and x.numel and ops.FUSED and ops.stacked(wq, wk, wv) and x.device is wq.device \
+            and _tape_free(x, wq, wk, wv, None if norm is None else norm.weight):
         C = wq.shape[0]
         w = Buffer(wq.data.ptr, (3 * C, wq.shape[1]), wq.device)
         inside = _row_norm(x, w, norm)
@@ -232,8 +258,9 @@ def decode_append(logits: Tensor, tok: Tensor, slot: Tensor, seq: Tensor) -> boo
 
 def norm_linear(x: Tensor, norm, weight: Tensor) -> Tensor:
     """norm(x) @ weight^T.  For a single row on the hip device the normalisation happens inside the product
-    and the result carries no tape (decoding); otherwise the two ops."""
-    inside = _row_norm(x, weight.data, norm) if weight.ndim == 2 else None
+    and the result carries no tape: taken inside nn.inference(), or when neither x nor the weight nor the gain
+    requires a gradient; otherwise the two ops (or their one-node form), which record the graph."""
+    inside = _row_norm(x, weight.data, norm) if (weight.ndim == 2 and _tape_free(x, weight, norm.weight)) else None
     if inside:
         y = x.data.matmul_nt(weight.data, norm=inside)
         return Tensor(y.reshape(x.shape[:-1] + (weight.shape[0],)), requires_grad=False)
@@ -247,9 +274,10 @@ def mlp_relu(x: Tensor, w_fc: Tensor, w_proj: Tensor, residual: Tensor | None = 
     examples/gpt.py:69-78.  On the hip device one node whose ReLU, ReLU gradient and residual addition
     happen as the products are stored (ops.MLPRelu); elsewhere the four ops.
     norm: an RMSNorm to apply to x first.  For a single row on the hip device it is applied inside the first
-    product, and the result then carries no tape (decoding)."""
+    product, and the result then carries no tape: taken inside nn.inference(), or when no input requires a gradient."""
     if norm is not None:
-        inside = _row_norm(x, w_fc.data, norm) if (w_fc.ndim == 2 and w_proj.ndim == 2 and w_proj.device is x.device) else None
+        inside = _row_norm(x, w_fc.data, norm) if (w_fc.ndim == 2 and w_proj.ndim == 2 and w_proj.device is x.device
+                                                   and _tape_free(x, w_fc, w_proj, residual, norm.weight)) else None
         if inside and (residual is None or (residual.device is x.device and residual.shape == x.shape[:-1] + (w_proj.shape[0],))):
             h = x.data.matmul_nt(w_fc.data, epi="relu", norm=inside)
             y = h.matmul_nt(w_proj.data, epi="add", e=residual.data) if residual is not None else h.matmul_nt(w_proj.data)

@@ -22,6 +22,7 @@ import json
 import math
 import os
 import struct
+import warnings
 
 import numpy as np
 
@@ -1622,6 +1623,7 @@ class HIP:
     MATMUL_TUNE_MIN_FLOP = 1 << 24
     _tuned: dict | None = None
     _tuned_new: dict = {}
+    _tune_warned = False                  # the first tile timing of a process says what it is doing
 
     MATMUL_TUNED_FILE = os.environ.get("DLGRAD_HIP_MATMUL_TUNED_FILE", os.path.join(CACHE_DIR, "matmul_tuned.json"))
     last_matmul_kernel: str | None = None      # name of the most recently launched product kernel (reported by the benchmark)
@@ -1708,6 +1710,13 @@ class HIP:
         global launch_count
         l = lib()
         count0 = launch_count
+        if not HIP._tune_warned and not COMPILE_ONLY:                # said once per process: the first step is slower, results are not
+            HIP._tune_warned = True
+            warnings.warn(f"dlgrad_amd: the matrix product {key} (batch,M,N,K) is in no tile table; timing every plausible tile "
+                          "on its operands now, once per shape and machine (about 10 ms for mid-sized products, up to 0.5 s at "
+                          "8192^3; the choice is stored in dlgrad_amd/_kcache/matmul_tuned.json and changes no result bit). "
+                          "DLGRAD_HIP_MATMUL_TUNE=0 switches the timing off; further shapes are timed without this message.",
+                          RuntimeWarning, stacklevel=2)
         best, best_ms = None, float("inf")
         e0, e1 = l.event_create(), l.event_create()
         for tile in HIP._tile_candidates(M, N, batch):

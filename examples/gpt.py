@@ -16,6 +16,18 @@ from dlgrad_amd import Tensor, nn
 from dlgrad_amd.helpers import STRICT_REFERENCE
 
 
+def _inference(fn):
+    """The decorated method differentiates nothing: it runs inside nn.inference(), where single-row
+    products may apply their norm on the way and return results without a tape."""
+    import functools
+
+    @functools.wraps(fn)
+    def run(*args, **kwargs):
+        with nn.inference():
+            return fn(*args, **kwargs)
+    return run
+
+
 class GPTConfig:
     def __init__(self, vocab_size: int = 65, block_size: int = 128, n_layer: int = 6, n_head: int = 4,
                  n_embd: int = 128, batch_size: int = 16, learning_rate: float = 1e-4, device: str = "hip") -> None:
@@ -145,6 +157,7 @@ class GPT:
             x = block(x, cache, i)
         return self.ln_f(x)
 
+    @_inference
     def prefill(self, idx: Tensor) -> tuple[Tensor, KVCache]:
         """Full forward over idx (B, T) that also fills a fresh cache; returns the logits of
         the last position as (B, 1, V) and the cache (the inference branch of
@@ -157,6 +170,7 @@ class GPT:
         last = x.reshape((T, C))[T - 1:T] if B == 1 else x.transpose(0, 1)[T - 1:T]
         return self.lm_head(last.reshape((B, 1, C))), cache
 
+    @_inference
     def forward_incremental(self, new_idx: Tensor, pos: Tensor, cache: KVCache) -> Tensor:
         """One new token per sequence: new_idx (B, 1), pos (1, 1) its position id; appends to
         the cache and returns logits (B, 1, V) (examples/gpt.py:114-136)."""
@@ -191,6 +205,7 @@ class GPT:
             n += 1
         return [int(v) for v in seq.numpy().reshape(-1)]
 
+    @_inference
     def generate_greedy(self, first_token: int, max_new_tokens: int) -> list[int]:
         """Greedy decode with full-context recompute per token, context cropped to
         block_size (the loop of examples/gpt.py:231-279 with argmax in place of sampling)."""
@@ -267,6 +282,7 @@ class StaticDecoder:
         self.tok.data.copy_(nxt.data)
         self.slot.data.copy_(nslot.data)
 
+    @_inference
     def step(self) -> None:
         """Feeds self.tok at index self.slot; leaves the argmax in seq[slot + 1] and as the next
         token, and advances slot.  Reads and writes device memory only."""
@@ -285,6 +301,7 @@ class StaticDecoder:
             x = block.mlp(x, x, block.ln2)
         self._append(nn.norm_linear(x, m.ln_f, m.lm_head.weight).reshape((1, c.vocab_size)))
 
+    @_inference
     def step_window(self) -> None:
         """The step for a full window: tokens slot - block_size + 1 .. slot go through the whole model
         at positions 0 .. block_size - 1; the argmax of the last position becomes token slot + 1."""

@@ -71,7 +71,11 @@ int dlg_hip_shutdown(void);
  * banks; such pointers stay 4 KiB aligned, and dlg_hip_free takes the
  * pointer that dlg_hip_alloc returned.
  * A NULL/failed allocation is an error return, which the Python side turns
- * into MemoryError exactly where the reference does (cpu.py:104,132,189).   */
+ * into MemoryError exactly where the reference does (cpu.py:104,132,189).
+ * While a capture is in progress (dlg_hip_graph_begin) an allocation that the
+ * current arena cannot serve from its returned blocks is refused with -9 (the
+ * Python side raises RuntimeError): hipMalloc, and the stream wait of its
+ * retry, are never issued under stream capture.                              */
 int dlg_hip_alloc(size_t nbytes, void **out);
 int dlg_hip_alloc_zero(size_t nbytes, void **out);
 int dlg_hip_fill_f32(void *dst, float value, size_t count);

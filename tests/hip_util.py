@@ -21,13 +21,15 @@ def dev(a) -> Buffer:
 
 
 def rel_err(got, want) -> float:
-    """max |got-want| / max(|want|, tiny) over elements; exact matches (incl. inf) count 0."""
+    """max |got-want| / max(|want|, tiny) over elements.  Exact matches (incl. equal infinities and
+    NaN on both sides) count 0; a NaN on one side only, or an infinity against anything else, is an
+    infinite error -- as with np.testing.assert_allclose, a lone NaN can never pass a tolerance."""
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
     same = (got == want) | (np.isnan(got) & np.isnan(want))
     with np.errstate(all="ignore"):
         e = np.abs(got - want) / np.maximum(np.abs(want), 1e-30)
-    e = np.where(same, 0.0, e)
-    return float(np.nanmax(e)) if e.size else 0.0
+    e = np.where(same, 0.0, np.where(np.isfinite(e), e, np.inf))
+    return float(np.max(e)) if e.size else 0.0
 
 
 def check(got, want, tol: float, what: str = "") -> None:

@@ -216,6 +216,41 @@ def test_capture_refuses_what_a_graph_cannot_replay():
 
 
 @pytest.mark.gpu
+def test_an_allocation_that_misses_the_arena_during_a_capture_is_refused_on_the_host():
+    """Under stream capture the allocator never reaches hipMalloc (nor the stream wait of its retry):
+    a capture whose body asks for a size that the warm-up pass did not leave in the arena ends with a
+    RuntimeError raised by the host, the capture is abandoned, and the device goes on working."""
+    from dlgrad_amd.runtime import hip
+    if not hip.available():
+        pytest.skip("no HIP device")
+    lib = hip.lib()
+    x = Buffer.from_numpy(np.ones((8, 8), np.float32), Device.HIP)
+    big = Buffer.from_numpy(np.ones((300, 300), np.float32), Device.HIP)
+    (big + big).numpy()                                           # its kernel is loaded before any capture
+    g = hip.Graph()
+    with g.arena():
+        y = x + x                                                 # the warm-up leaves one 256-byte block
+    del y
+    allocs = lib.pool_stats()[2]
+    with pytest.raises(RuntimeError, match="missed the arena during a capture"):
+        with g.capture():
+            z = big + big                                         # 360 000 bytes: no such block in the arena
+    assert not hip.capturing()
+    assert lib.pool_stats()[2] == allocs                          # no device allocation was made
+    with pytest.raises(RuntimeError, match="missed the arena during a capture"):
+        with g.capture():
+            y1 = x + x
+            y2 = x + x                                            # a second live block of a size the arena holds once
+    assert not hip.capturing()
+    np.testing.assert_array_equal((big + big).numpy(), np.full((300, 300), 2, np.float32))   # ordinary work goes on
+    with g.capture():                                             # and the same Graph can still capture what fits
+        y = x + x
+    g.replay()
+    np.testing.assert_array_equal(y.numpy(), np.full((8, 8), 2, np.float32))
+    g.close()
+
+
+@pytest.mark.gpu
 def test_pinned_staging_uploads_without_a_wait_and_inside_a_captured_graph():
     """A page-locked array is uploaded by an enqueued DMA; recorded into a graph, the copy
     re-reads the array on every replay, so a loop refills it between replays (after a sync)
@@ -393,3 +428,60 @@ def test_event_and_graph_handles_are_checked():
         lib.graph_launch(10 ** 9)
     lib.event_destroy(e0)
     assert hip.props()["name"], "the device name must not be empty"
+
+
+def test_tolerance_comparator_never_lets_a_lone_nan_or_infinity_pass():
+    """The helper every floating-point parity test rests on: a NaN or infinity on one side only is an
+    infinite error (np.testing.assert_allclose, the reference's comparator, behaves the same way);
+    NaN against NaN and equal infinities are matches."""
+    from tests.hip_util import check, rel_err
+    nan, inf = float("nan"), float("inf")
+    with pytest.raises(AssertionError):
+        check(np.array([1, nan, 3], np.float32), np.array([1, 2, 3], np.float32), 1e-6)
+    with pytest.raises(AssertionError):
+        check(np.array([1, 2, 3], np.float32), np.array([1, nan, 3], np.float32), 1e-6)
+    with pytest.raises(AssertionError):
+        check(np.array([1, inf, 3], np.float32), np.array([1, 2, 3], np.float32), 1e-6)
+    with pytest.raises(AssertionError):
+        check(np.array([1, inf, 3], np.float32), np.array([1, -inf, 3], np.float32), 1e-6)
+    with pytest.raises(AssertionError):
+        check(np.array([1, 2.001, 3], np.float32), np.array([1, 2, 3], np.float32), 1e-6)
+    assert rel_err(np.array([nan]), np.array([0.0])) == inf
+    check(np.array([1, nan, inf, -inf, 0], np.float32), np.array([1, nan, inf, -inf, 0], np.float32), 1e-6)
+    check(np.array([1, 2.0000001, 3], np.float32), np.array([1, 2, 3], np.float32), 1e-6)
+    check(np.zeros((0,), np.float32), np.zeros((0,), np.float32), 1e-6)
+
+
+def test_first_tile_timing_of_a_process_says_so_once(monkeypatch, tmp_path):
+    """A product shape that is in no tile table is timed with every plausible tile on first use, which makes
+    a user's first step many times slower: the first such timing of a process warns, naming the shape, the
+    cost and the switch; later ones stay silent.  (Host logic only: launches and events are stand-ins.)"""
+    import warnings
+    from dlgrad_amd.runtime.hip import HIP
+
+    class Events:
+        def event_create(self): return 1
+        def event_record(self, e): pass
+        def event_sync(self, e): pass
+        def event_elapsed_ms(self, a, b): return 1.0
+        def event_destroy(self, e): pass
+
+    monkeypatch.setattr(hip, "lib", lambda: Events())
+    monkeypatch.setattr(hip, "COMPILE_ONLY", False)
+    monkeypatch.setattr(HIP, "_launch_matmul", staticmethod(lambda *a, **k: None))
+    monkeypatch.setattr(HIP, "_tile_candidates", staticmethod(lambda M, N, batch: ["128x128x32_w2x2"]))
+    monkeypatch.setattr(HIP, "MATMUL_TUNED_FILE", str(tmp_path / "tuned.json"))
+    monkeypatch.setattr(HIP, "_tuned_new", {})
+    monkeypatch.setattr(HIP, "_tune_warned", False)
+    table = dict(HIP._tuned_table())
+    try:
+        with pytest.warns(RuntimeWarning, match=r"1,3000,1000,2000.*DLGRAD_HIP_MATMUL_TUNE=0"):
+            assert HIP._tune_tile("1,3000,1000,2000", True, True, 3000, 1000, 1, (), False, False) == "128x128x32_w2x2"
+        with warnings.catch_warnings():
+            warnings.simplefilter("error")                                # a second shape: timed without a word
+            assert HIP._tune_tile("1,3001,1000,2000", True, True, 3001, 1000, 1, (), False, False) == "128x128x32_w2x2"
+        import json
+        assert set(json.load(open(tmp_path / "tuned.json"))) == {"1,3000,1000,2000", "1,3001,1000,2000"}
+    finally:
+        HIP._tuned_table().clear()
+        HIP._tuned_table().update(table)

@@ -10,7 +10,7 @@ from dlgrad_amd.buffer import Buffer
 from dlgrad_amd.device import Device
 from oracle import cref
 from dlgrad_amd.runtime import hip
-from tests.hip_util import check, dev, require_gpu
+from tests.hip_util import check, dev, rel_err, require_gpu
 
 pytestmark = pytest.mark.gpu
 RNG = np.random.default_rng(11)
@@ -338,6 +338,7 @@ def test_c2_suite_at_16384x8192_matches_the_oracle(case):
     if tol == 0:
         assert np.array_equal(got, want), case
     else:
-        with np.errstate(all="ignore"):
-            err = np.abs(got.astype(np.float64) - want) / np.maximum(np.abs(want), 1e-30)
-        assert float(np.nanmax(np.where(got == want, 0.0, err))) <= tol, case
+        g, w = got.reshape(-1), want.reshape(-1)                # NaN-strict (rel_err), a slab at a time to bound float64 temporaries
+        step = 1 << 24
+        worst = max(rel_err(g[i:i + step], w[i:i + step]) for i in range(0, g.size, step))
+        assert worst <= tol, (case, worst)

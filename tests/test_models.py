@@ -77,11 +77,15 @@ def test_mlp_step_on_cpu_device_matches_torch():
         tensors_close(n, (t - 1e-3 * t.grad).detach().numpy(), "sgd")
 
 
-def torch_gpt_loss_and_grads(model: G.GPT, idx, tgt, dtype=torch.float32, details: dict | None = None):
+def torch_gpt_loss_and_grads(model: G.GPT, idx, tgt, dtype=torch.float32, details: dict | None = None, backward: bool = True):
     """Independent PyTorch statement of the examples/gpt.py graph.  details (a dict): receives the
-    logits and the ReLU branch taken per hidden unit, layer by layer."""
+    logits and the ReLU branch taken per hidden unit, layer by layer.  backward=False: the forward
+    pass alone, nothing kept for a backward pass (returns the loss and no gradients)."""
+    if not backward:
+        with torch.no_grad():
+            return torch_gpt_loss_and_grads(model, idx, tgt, dtype, details, backward=None)
     c = model.config
-    sd = {k: torch.tensor(v.numpy(), dtype=dtype, requires_grad=True) for k, v in nn.utils.get_state_dict(model).items()}
+    sd = {k: torch.tensor(v.numpy(), dtype=dtype, requires_grad=backward is True) for k, v in nn.utils.get_state_dict(model).items()}
 
     def rms(x, w):
         ms = (x ** 2).mean(-1, keepdim=True)
@@ -111,6 +115,8 @@ def torch_gpt_loss_and_grads(model: G.GPT, idx, tgt, dtype=torch.float32, detail
         details["logits"] = logits.detach().numpy()
     loss = torch.nn.functional.cross_entropy(logits.reshape(B * T, -1), torch.tensor(tgt).long().reshape(-1),
                                              reduction="sum")
+    if backward is None:
+        return loss.numpy(), {}
     (loss / (B * T)).backward()
     return loss.detach().numpy(), {k: v.grad.numpy() for k, v in sd.items()}
 
@@ -284,6 +290,154 @@ def test_scaled_gpt_step_hip_vs_float64(monkeypatch):
     for k in g64:
         tensors_close(g_forced[k], g64[k], f"grad {k}")
     assert worst_free <= 5e-3                                     # a differing gate moves gradients by ~1e-3 of their scale
+
+
+C5_FULL = dict(vocab_size=50304, block_size=1024, n_layer=12, n_head=12, n_embd=768, batch_size=8)
+
+
+@pytest.mark.gpu
+def test_scaled_gpt_full_depth_forward_hip_vs_float64():
+    """BASELINE config 5 at its own depth and batch: all twelve layers, batch 8 x 1024 Zipf(1.1) token ids,
+    weights N(0, 0.02) from seed 0 -- the model, ids and targets that bench.py's scaled-GPT leg times (same
+    seeds) -- forward on the hip device against the float64 PyTorch statement of the graph run on the host
+    cores (forward only; the pattern of the reference's test/test_gpt.py:44-205).  The summed loss to 1e-5,
+    every logit to 1e-4 of the largest.  The loss per token printed here is the one bench.py reports as
+    gpt_scaled_c5.loss_per_token_first_forward."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    cfg = C5_FULL
+    rng = np.random.default_rng(7)
+    ids = np.minimum(rng.zipf(1.1, (2, cfg["batch_size"], cfg["block_size"])) - 1, cfg["vocab_size"] - 1).astype(np.float32)
+    model = G.GPT(G.GPTConfig(device="hip", **cfg))
+    G.init_weights_(model, 0)
+    logits, loss = model(Tensor(ids[0], device="hip"), Tensor(ids[1], device="hip"))
+    if hip.COMPILE_ONLY:
+        return
+    l_hip, lg_hip = float(loss.numpy()), logits.numpy()
+    del logits, loss
+    details: dict = {}
+    torch.manual_seed(0)
+    l64, _ = torch_gpt_loss_and_grads(model, ids[0], ids[1], torch.float64, details, backward=False)
+    del model
+    lg64 = details["logits"]
+    tokens = cfg["batch_size"] * cfg["block_size"]
+    print(f"scaled GPT, 12 layers, batch 8: loss per token {l_hip / tokens:.6f} on hip, {float(l64) / tokens:.6f} in float64")
+    assert abs(l_hip - float(l64)) <= 1e-5 * abs(float(l64)), (l_hip, float(l64))
+    assert lg_hip.shape == lg64.shape and np.isfinite(lg_hip).all()
+    scale = float(np.abs(lg64).max())
+    worst = max(float(np.abs(lg_hip[b] - lg64[b]).max()) for b in range(lg64.shape[0])) / scale     # a batch row at a time
+    print(f"largest logit error {worst:.2e} of the largest logit ({scale:.3f})")
+    assert worst <= 1e-4
+    rows = np.random.default_rng(0).integers(0, tokens, 64)                                 # and a row sample element by element
+    tensors_close(lg_hip.reshape(tokens, -1)[rows], lg64.reshape(tokens, -1)[rows], "sampled logit rows")
+
+
+def decode_with_logits(model: G.GPT, first_token: int, n_new: int, reference_positions: bool):
+    """The control flow of GPT.generate_greedy_cached (the reference's generate, examples/gpt.py:169-226,
+    greedy), keeping the logits every token was chosen from: (ids, [logits (V,) per new token])."""
+    c = model.config
+    ids, rows, start, cache = [int(first_token)], [], 0, None
+    for _ in range(n_new):
+        n = len(ids)
+        if n - start >= c.block_size:
+            start, cache = n - c.block_size, None
+        if cache is None:
+            logits, cache = model.prefill(Tensor(np.asarray(ids[start:], np.float32).reshape(1, n - start), device=c.device))
+        else:
+            length = n - start
+            pos = Tensor(np.array([[length if reference_positions else length - 1]], np.float32), device=c.device)
+            logits = model.forward_incremental(Tensor(np.array([[ids[-1]]], np.float32), device=c.device), pos, cache)
+        row = logits.numpy().reshape(-1)
+        rows.append(row)
+        ids.append(int(np.argmax(row)))
+    return ids, rows
+
+
+def same_ids_or_a_near_tie(got: list, want: list, want_rows: list, what: str) -> int:
+    """Token for token equal -- or, at the first token that differs, the oracle's two candidates must be
+    tied to within 1e-4 of its largest logit (printed): from there on the sequences are different
+    contexts and nothing more can be compared.  Returns the number of tokens that were compared."""
+    assert len(got) == len(want), what
+    for t in range(1, len(want)):
+        if got[t] != want[t]:
+            row = want_rows[t - 1]
+            gap = float(row[want[t]] - row[got[t]])
+            print(f"{what}: token {t} is {got[t]} where the oracle has {want[t]}; the oracle's logits for the two differ by "
+                  f"{gap:.3e}, its largest logit is {float(np.abs(row).max()):.3e}; {t} of {len(want) - 1} tokens compared")
+            assert 0 <= gap <= 1e-4 * float(np.abs(row).max()), f"{what}: token {t} differs and the oracle's logits are not tied"
+            return t
+    return len(want) - 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("reference_positions", [True, False])
+def test_char_gpt_decodes_256_tokens_like_the_cpu_oracle(reference_positions):
+    """BASELINE config 4's decode on the model it names: 6 layers, 4 heads, width 128, window 128, weights
+    N(0, 0.02) from seed 0 (the model bench.py times), 256 greedy tokens from id 0.  The oracle is the
+    reference's loop on the C restatement's cpu device (key/value cache while the window fills, a full forward
+    over the last 128 tokens per token after that).  Against it, on the hip device: the same loop with the
+    device-resident cache, the two fixed-shape steps issued eagerly, and the same two steps captured and
+    replayed (what bench.py's tokens/s is measured on); with each token at its own position also the
+    full-recompute loop.  With weights this small the logits of a step lie close together, so a token that
+    differs is accepted only where the oracle's own top two logits are tied to 1e-4 of its largest -- and
+    is printed, never silent."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    n_new = 256
+    models = {}
+    for dev in ("cpu", "hip"):
+        models[dev] = G.GPT(G.GPTConfig(device=dev, **C4))
+        G.init_weights_(models[dev], 0)
+    hip_model = models["hip"]
+    runs = {"device-resident cache loop": hip_model.generate_greedy_cached(0, n_new, reference_positions=reference_positions)}
+    dec = G.StaticDecoder(hip_model, reference_positions=reference_positions, capacity=n_new + 1)
+    runs["fixed-shape steps, eager"] = dec.generate(0, n_new)
+    if not hip.COMPILE_ONLY:
+        dec.capture()
+        runs["fixed-shape steps, replayed graphs"] = dec.generate(0, n_new)
+    dec.close()
+    if not reference_positions:
+        runs["full recompute loop"] = hip_model.generate_greedy(0, n_new)
+    if hip.COMPILE_ONLY:
+        return
+    want, want_rows = decode_with_logits(models["cpu"], 0, n_new, reference_positions)
+    assert want == models["cpu"].generate_greedy_cached(0, n_new, reference_positions=reference_positions)
+    assert len(set(want)) > 1, "a constant sequence would compare nothing"
+    gaps = sorted(float(np.sort(r)[-1] - np.sort(r)[-2]) / float(np.abs(r).max()) for r in want_rows)
+    print(f"oracle ids {want[:12]}...; smallest top-2 logit gaps relative to the largest logit: {[f'{g:.2e}' for g in gaps[:3]]}")
+    for what, got in runs.items():
+        compared = same_ids_or_a_near_tie(got, want, want_rows, what)
+        assert compared >= 1
+    assert runs["fixed-shape steps, replayed graphs"] == runs["fixed-shape steps, eager"]      # bit-identical steps
+
+
+@pytest.mark.gpu
+def test_a_training_forward_over_a_single_row_keeps_its_tape():
+    """idx of shape (1, 1) with targets: every product of the step has a single row, which is the shape
+    the decoding forms serve without a tape.  Outside nn.inference() they must not be taken when a
+    gradient is wanted: loss and every gradient as on the cpu device."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    out = {}
+    for dev in ("cpu", "hip"):
+        model = G.GPT(G.GPTConfig(device=dev, **dict(TINY, n_embd=64)))
+        G.init_weights_(model, 5, std=0.2)
+        logits, loss = model(Tensor(np.array([[7]], np.float32), device=dev), Tensor(np.array([[3]], np.float32), device=dev))
+        assert logits.requires_grad and loss.requires_grad
+        loss.backward()
+        sd = nn.utils.get_state_dict(model)
+        assert all(p.grad is not None for k, p in sd.items() if not k.startswith("wpe")), "a parameter got no gradient"
+        out[dev] = (loss.numpy(), {k: p.grad.numpy() for k, p in sd.items() if p.grad is not None})
+        with nn.inference():
+            no_tape, _ = model(Tensor(np.array([[7]], np.float32), device=dev))
+        if not hip.COMPILE_ONLY:
+            tensors_close(no_tape.numpy(), logits.numpy(), "inference logits", 1e-5)
+    if hip.COMPILE_ONLY:
+        return
+    tensors_close(out["hip"][0], out["cpu"][0], "loss")
+    assert out["hip"][1].keys() == out["cpu"][1].keys()
+    for k in out["cpu"][1]:
+        tensors_close(out["hip"][1][k], out["cpu"][1][k], f"grad {k}")
 
 
 @pytest.mark.gpu
