@@ -569,6 +569,11 @@ class Buffer:
         """self: the logits of the position just computed.  seq[slot + 1] = tok = argmax(self); slot += 1, in place."""
         self._dispatch(CustomOps.DECODE_NEXT, logits=self, tok=tok, slot=slot, seq=seq)
 
+    def decode_sample_(self, u: "Buffer", tok: "Buffer", slot: "Buffer", seq: "Buffer", temperature: float) -> None:
+        """self: the logits of the position just computed.  seq[slot + 1] = tok = the token that u[slot] draws from
+        softmax(self / temperature) by inversion; slot += 1, in place."""
+        self._dispatch(CustomOps.DECODE_SAMPLE, logits=self, u=u, tok=tok, slot=slot, seq=seq, temperature=temperature)
+
     def sgd_step_(self, g: "Buffer", v: "Buffer | None", lr: float, momentum: float) -> None:
         """In-place SGD update of self (and of the velocity v when momentum is used)."""
         self._dispatch(CustomOps.SGD_STEP_INPLACE, p=self, g=g, v=v, lr=lr, momentum=momentum)

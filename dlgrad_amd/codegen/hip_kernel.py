@@ -2676,6 +2676,81 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
     return src, name, _fmt("P", "P", "P", "P", "I", "I")
 
 
+@cache
+def decode_sample_kernel() -> tuple[str, str, str]:
+    """The end of a *sampling* decoding step in one launch: the next token is drawn from
+    softmax(logits / temperature) by inversion, as np.random.choice(V, p=probs) draws it
+    (examples/gpt.py:215-221, :259-260): next = the first index whose running sum of the
+    probabilities exceeds the uniform number.  The uniform number is u[s] for s = slot[0], the
+    index of the token just fed -- a device array filled beforehand, so a captured step draws a
+    new number on every replay.  Then, as decode_next: seq[s + 1] = next (skipped outside the
+    (rows, 1) token buffer), tok[0] = next, slot[0] = s + 1.
+
+    One block.  Thread t owns the contiguous run [t * ceil(V / 256), ...) of the vocabulary:
+    e_j = exp(x_j / temperature - max) is summed over the run in index order, the runs are joined
+    by a scan over the 256 threads, and the thread whose run contains the target u * total walks
+    it again to find the index.  The sums are fp32 in a fixed order: the same logits and the
+    same u always give the same token.  If rounding leaves u * total at or above every running
+    sum, the last index of non-zero probability is taken."""
+    name = "decode_sample"
+    src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ logits, const float* __restrict__ u,
+        float* __restrict__ tok, float* __restrict__ slot, float* __restrict__ seq, u32 V, u32 rows, u32 n_u,
+        float temperature) {{
+    __shared__ float swave[4];
+    __shared__ float sruns[4];
+    __shared__ u32 sfound[4];
+    const u32 t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    const u32 run = (V + 255u) / 256u;
+    const u32 j0 = min(t * run, V), j1 = min(j0 + run, V);
+    float m = NEG_FLT_MAX;
+    for (u32 j = j0; j < j1; ++j) m = fmaxf(m, logits[j] / temperature);
+    m = wave_max(m);
+    if (lane == 0u) swave[w] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(swave[0], swave[1]), fmaxf(swave[2], swave[3]));
+    float own = 0.0f;
+    for (u32 j = j0; j < j1; ++j) own += expf(logits[j] / temperature - m);
+    float upto = own;                                   // inclusive scan over the lanes of the wavefront
+    #pragma unroll
+    for (u32 d = 1; d < 64u; d <<= 1) {{
+        const float o = __shfl_up(upto, d, WAVE);
+        if (lane >= d) upto += o;
+    }}
+    if (lane == 63u) sruns[w] = upto;
+    __syncthreads();
+    float before = 0.0f;
+    for (u32 k = 0; k < w; ++k) before += sruns[k];
+    const float total = ((sruns[0] + sruns[1]) + sruns[2]) + sruns[3];
+    const float sf = slot[0];
+    const u32 ui = (sf >= 0.0f && sf < (float)n_u) ? (u32)sf : 0u;
+    const float target = u[ui] * total;
+    float sum = before + (upto - own);                  // everything in front of this thread's run
+    u32 found = V;
+    for (u32 j = j0; j < j1; ++j) {{
+        sum += expf(logits[j] / temperature - m);
+        if (sum > target) {{ found = j; break; }}
+    }}
+    #pragma unroll
+    for (u32 d = 32; d >= 1u; d >>= 1) found = min(found, (u32)__shfl_xor((int)found, (int)d, WAVE));
+    if (lane == 0u) sfound[w] = found;
+    __syncthreads();
+    if (t == 0u) {{
+        found = min(min(sfound[0], sfound[1]), min(sfound[2], sfound[3]));
+        if (found >= V) {{                               // rounding left the target beyond every running sum: the last token that can be drawn
+            found = V - 1u;
+            while (found > 0u && !(expf(logits[found] / temperature - m) > 0.0f)) --found;
+        }}
+        const float nxt = (float)found, ns = sf + 1.0f;
+        if (ns >= 0.0f && ns < (float)rows) seq[(u32)ns] = nxt;
+        tok[0] = nxt;
+        slot[0] = ns;
+    }}
+}}
+"""
+    return src, name, _fmt("P", "P", "P", "P", "P", "I", "I", "I", "f")
+
+
 # =====================================================================================
 # attention for one new position (decoding)
 # =====================================================================================

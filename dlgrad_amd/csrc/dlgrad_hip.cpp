@@ -68,6 +68,8 @@ unsigned g_colour = 0;
 std::map<uint64_t, std::map<size_t, std::vector<void *>>> g_free;   // arena -> bucket -> cached blocks
 std::unordered_map<void *, Block> g_live;                            // block -> bucket, arena
 std::map<uint64_t, bool> g_arena_alive;                              // arenas that still exist
+struct Usage { size_t live = 0, peak = 0; };                         // blocks of one bucket of one arena: in use now, most at once
+std::map<uint64_t, std::map<size_t, Usage>> g_usage;                 // arena (never 0) -> bucket -> usage
 uint64_t g_arena = 0, g_next_arena = 1;
 uint64_t g_bytes_in_use = 0, g_bytes_cached = 0, g_device_allocs = 0;
 std::atomic<bool> g_capturing{false};                            // read by calls that refuse to run inside a capture
@@ -162,6 +164,10 @@ int alloc_locked(size_t nbytes, void **out) {
     if (stagger) *out = static_cast<char *>(base) + (g_colour++ % kColours) * kStagger;
     g_live[*out] = Block{b, g_arena, base};
     g_bytes_in_use += b;
+    if (g_arena != 0) {
+        Usage &u = g_usage[g_arena][b];
+        if (++u.live > u.peak) u.peak = u.live;
+    }
     return 0;
 }
 
@@ -299,6 +305,13 @@ int dlg_hip_free(void *ptr) {
     Block blk = it->second;
     g_live.erase(it);
     g_bytes_in_use -= blk.bucket;
+    if (blk.arena != 0) {
+        auto ua = g_usage.find(blk.arena);
+        if (ua != g_usage.end()) {
+            auto ub = ua->second.find(blk.bucket);
+            if (ub != ua->second.end() && ub->second.live) --ub->second.live;
+        }
+    }
     if (blk.arena != 0 && !g_arena_alive[blk.arena]) {      // its graph is gone: give the memory back
         (void)hipFree(blk.base);
         return 0;
@@ -598,6 +611,32 @@ int dlg_hip_arena_set(uint64_t arena) {
     return 0;
 }
 
+int dlg_hip_arena_reserve(uint64_t arena) {
+    NEED_INIT();
+    if (g_capturing) return fail_msg(-9, "dlg_hip_arena_reserve allocates device memory and cannot run inside a capture");
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (arena == 0 || !g_arena_alive[arena]) return fail_msg(-30, "no such arena");
+    // A pass that repeats what the arena has seen needs, per bucket, as many blocks at once as the most that
+    // were ever in use together; blocks of the earlier pass that are still held do not come back for it.
+    for (auto &kv : g_usage[arena]) {
+        std::vector<void *> &cached = g_free[arena][kv.first];
+        while (cached.size() < kv.second.peak) {
+            void *p = nullptr;
+            hipError_t e = hipMalloc(&p, kv.first);
+            if (e != hipSuccess || !p) {
+                (void)hipGetLastError();
+                char buf[160];
+                std::snprintf(buf, sizeof buf, "Failed to reserve %zu bytes of device memory for an arena", kv.first);
+                return fail_msg(-3, buf);
+            }
+            ++g_device_allocs;
+            cached.push_back(p);
+            g_bytes_cached += kv.first;
+        }
+    }
+    return 0;
+}
+
 int dlg_hip_arena_destroy(uint64_t arena) {
     NEED_INIT();
     if (arena == 0) return fail_msg(-30, "the default pool cannot be destroyed");
@@ -605,6 +644,7 @@ int dlg_hip_arena_destroy(uint64_t arena) {
     std::lock_guard<std::mutex> lk(g_mu);
     if (g_arena == arena) g_arena = 0;
     g_arena_alive[arena] = false;
+    g_usage.erase(arena);
     trim_arena_locked(arena);
     return 0;
 }

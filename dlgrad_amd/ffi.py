@@ -50,6 +50,7 @@ _SIGS = {
                                               _c.c_void_p]),
     "dlg_hip_arena_create": (_c.c_int, [_c.POINTER(_c.c_uint64)]),
     "dlg_hip_arena_set": (_c.c_int, [_c.c_uint64]),
+    "dlg_hip_arena_reserve": (_c.c_int, [_c.c_uint64]),
     "dlg_hip_arena_destroy": (_c.c_int, [_c.c_uint64]),
     "dlg_hip_graph_begin": (_c.c_int, []),
     "dlg_hip_graph_end": (_c.c_int, [_c.POINTER(_c.c_uint64), _c.POINTER(_c.c_uint64)]),
@@ -294,6 +295,10 @@ class HipLib:
 
     def arena_set(self, arena: int) -> None:
         self._check(self._lib.dlg_hip_arena_set(arena))
+
+    def arena_reserve(self, arena: int) -> None:
+        rc = self._lib.dlg_hip_arena_reserve(arena)
+        self._check(rc, MemoryError if rc == -3 else HipError)
 
     def arena_destroy(self, arena: int) -> None:
         self._check(self._lib.dlg_hip_arena_destroy(arena))

@@ -99,6 +99,7 @@ class CustomOps(_Op):
     DECODE_QKV_ROW = auto()         # q, k, v of one new position from the stacked projection, k and v stored into their cache rows
     DECODE_EMBED = auto()           # the input of a decoding step (token + position embedding, cache-row mask) from device-resident state
     DECODE_NEXT = auto()            # argmax of the logits, appended to the token buffer, made the next token; the index advanced
+    DECODE_SAMPLE = auto()          # the same with the token drawn from softmax(logits / temperature) by a given uniform number
     RMSNORM = auto()                # (x * rsqrt(mean(x^2) + eps)) * w over the last axis, one kernel
     RMSNORM_BWD = auto()            # its backward: dx in one kernel, dw by partial rows + a column sum
 
@@ -227,3 +228,18 @@ CACHE_DIR = os.environ.get(
 # `pow` arguments, dlgrad/runtime/cpu.py:252 and :500) are reproduced when this is
 # on, which is the default because parity is judged against that behaviour.
 STRICT_REFERENCE = os.environ.get("DLGRAD_STRICT_REFERENCE", "1") != "0"
+
+
+def sample_from_logits(logits, u: float, temperature: float = 1.0) -> int:
+    """The token np.random.choice(V, p=softmax(logits / temperature)) returns when its uniform draw is u:
+    the host-side sampling of examples/gpt.py:209-221 and :258-266 (numpy on the downloaded logits) with
+    the random number made explicit.  choice() inverts the cumulative sum of p, taken in float64 and
+    divided by its last entry: the first index whose entry exceeds u."""
+    import numpy as np
+    x = np.asarray(logits, dtype=np.float32).reshape(-1) / np.float32(temperature)
+    x = x - np.max(x)
+    e = np.exp(x)
+    p = e / e.sum()
+    cdf = np.cumsum(p.astype(np.float64))
+    cdf /= cdf[-1]
+    return min(int(np.searchsorted(cdf, float(u), side="right")), x.size - 1)

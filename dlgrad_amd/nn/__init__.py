@@ -256,6 +256,16 @@ def decode_append(logits: Tensor, tok: Tensor, slot: Tensor, seq: Tensor) -> boo
     return True
 
 
+def decode_sample(logits: Tensor, u: Tensor, tok: Tensor, slot: Tensor, seq: Tensor, temperature: float) -> bool:
+    """seq[slot + 1] = tok = the token drawn from softmax(logits / temperature) by the uniform number u[slot]
+    (inversion of the running sum, as np.random.choice does); slot += 1 -- in place, in one launch, on the hip
+    device.  False where not provided (nothing done)."""
+    if not _decode_fused(logits, u, tok, slot, seq):
+        return False
+    logits.data.decode_sample_(u.data, tok.data, slot.data, seq.data, temperature)
+    return True
+
+
 def norm_linear(x: Tensor, norm, weight: Tensor) -> Tensor:
     """norm(x) @ weight^T.  For a single row on the hip device the normalisation happens inside the product
     and the result carries no tape: taken inside nn.inference(), or when neither x nor the weight nor the gain

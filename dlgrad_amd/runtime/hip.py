@@ -308,6 +308,7 @@ class Graph:
             self._enter()
             try:
                 yield self
+                self._lib.arena_reserve(self.arena_id)     # blocks for a repeat of this pass, also while its results are held
             finally:
                 self._leave()
         return cm()
@@ -650,6 +651,16 @@ class HIP:
         if not logits.numel or tok.numel != 1 or slot.numel != 1 or tok.is_host_scalar or slot.is_host_scalar:
             raise ValueError(f"decode_next: {logits.shape} logits, token {tok.shape}, index {slot.shape}")
         launch(kernel(K.decode_next_kernel), 1, 256, _addr(logits), _addr(tok), _addr(slot), _addr(seq), logits.numel, seq.numel)
+
+    @staticmethod
+    @dispatcher.register(CustomOps.DECODE_SAMPLE, Device.HIP)
+    def decode_sample(logits: Buffer, u: Buffer, tok: Buffer, slot: Buffer, seq: Buffer, temperature: float) -> None:
+        if not logits.numel or not u.numel or tok.numel != 1 or slot.numel != 1 or tok.is_host_scalar or slot.is_host_scalar \
+                or u.is_host_scalar or not float(temperature) > 0.0:
+            raise ValueError(f"decode_sample: {logits.shape} logits, {u.shape} uniform numbers, token {tok.shape}, "
+                             f"index {slot.shape}, temperature {temperature}")
+        launch(kernel(K.decode_sample_kernel), 1, 256, _addr(logits), _addr(u), _addr(tok), _addr(slot), _addr(seq),
+               logits.numel, seq.numel, u.numel, float(temperature))
 
     @staticmethod
     @dispatcher.register(CustomOps.COPY_INTO, Device.HIP)

@@ -13,7 +13,7 @@ from __future__ import annotations
 import numpy as np
 
 from dlgrad_amd import Tensor, nn
-from dlgrad_amd.helpers import STRICT_REFERENCE
+from dlgrad_amd.helpers import STRICT_REFERENCE, sample_from_logits
 
 
 def _inference(fn):
@@ -179,10 +179,25 @@ class GPT:
         cache.length += 1
         return self.lm_head(x)
 
+    def generate(self, first_token: int, max_new_tokens: int, temperature: float = 1.0, u=None,
+                 reference_positions: bool = STRICT_REFERENCE) -> list[int]:
+        """The reference's generate (examples/gpt.py:169-226) with its sampling: the key/value-cache loop of
+        generate_greedy_cached, each token drawn on the host from softmax(logits / temperature) of the
+        downloaded logits (np.random.choice there; helpers.sample_from_logits here, which is choice() with
+        its uniform draw given).  u: max_new_tokens uniform numbers in [0, 1), one per token (a tensor or an
+        array); drawn from the device's seeded generator (dlgrad_amd.manual_seed) when None."""
+        if u is None:
+            u = Tensor.uniform((max(max_new_tokens, 1),), device=self.config.device)
+        u = np.asarray(u.numpy() if isinstance(u, Tensor) else u, dtype=np.float32).reshape(-1)
+        if u.size < max_new_tokens or not temperature > 0:
+            raise ValueError("generate: one uniform number per new token and a positive temperature are needed")
+        return self.generate_greedy_cached(first_token, max_new_tokens, reference_positions, (float(temperature), u))
+
     def generate_greedy_cached(self, first_token: int, max_new_tokens: int,
-                               reference_positions: bool = STRICT_REFERENCE) -> list[int]:
+                               reference_positions: bool = STRICT_REFERENCE, sampling: tuple | None = None) -> list[int]:
         """The control flow of the reference's generate (examples/gpt.py:169-226) with argmax in
-        place of sampling: a full forward when there is no cache, one-token steps after it,
+        place of sampling (sampling = (temperature, uniform numbers): drawn on the host instead, see
+        generate): a full forward when there is no cache, one-token steps after it,
         and -- as there -- no sliding: once the sequence has reached block_size the cache is
         dropped and every further token is a full forward over the last block_size tokens.
         reference_positions reproduces its position id for an incremental token, the sequence
@@ -200,7 +215,11 @@ class GPT:
                 length = n - start
                 pos = Tensor.full((1, 1), float(length if reference_positions else length - 1), device=c.device)
                 logits = self.forward_incremental(seq[n - 1:n], pos, cache)
-            nxt = logits.reshape((1, c.vocab_size)).argmax(1)                           # (1, 1), on the device
+            if sampling is None:
+                nxt = logits.reshape((1, c.vocab_size)).argmax(1)                       # (1, 1), on the device
+            else:
+                drawn = sample_from_logits(logits.numpy(), sampling[1][n - 1], sampling[0])
+                nxt = Tensor(np.array([[drawn]], np.float32), device=c.device)
             seq[n:n + 1].data.copy_(nxt.data)
             n += 1
         return [int(v) for v in seq.numpy().reshape(-1)]
@@ -244,18 +263,38 @@ class StaticDecoder:
     Same tokens as generate_greedy_cached (the probabilities differ only in the order of the
     softmax sums) and, with reference_positions=False, as full recompute (generate_greedy)."""
 
-    def __init__(self, model: GPT, reference_positions: bool = STRICT_REFERENCE, capacity: int | None = None) -> None:
+    def __init__(self, model: GPT, reference_positions: bool = STRICT_REFERENCE, capacity: int | None = None,
+                 temperature: float | None = None) -> None:
+        """temperature: None decodes greedily; a positive number draws every token from
+        softmax(logits / temperature) as the reference's generate does (examples/gpt.py:209-221, :258-266),
+        with the uniform numbers of the device's seeded generator (dlgrad_amd.manual_seed), one per token,
+        made before the first step (reset) and kept on the device: on the hip device the draw is the last
+        launch of the step, so a captured step samples too."""
         c = model.config
+        if temperature is not None and not temperature > 0:
+            raise ValueError("temperature must be positive")
+        self.temperature = None if temperature is None else float(temperature)
         self.model, self.reference_positions = model, reference_positions
         self.capacity = int(capacity) if capacity is not None else 2 * c.block_size + 1     # tokens the buffer holds
         self.cache = KVCache(c, 1)
         self.tok = Tensor.full((1, 1), 0.0, device=c.device)          # token to feed
         self.slot = Tensor.full((1, 1), 0.0, device=c.device)         # its index = cache row to write
         self.seq = Tensor.full((max(self.capacity, c.block_size + 1), 1), 0.0, device=c.device)
+        self.u = Tensor.full((self.seq.shape[0],), 0.0, device=c.device) if self.temperature is not None else None
         self.graph = None
         self.window_graph = None
 
-    def reset(self, first_token: int) -> None:
+    def reset(self, first_token: int, u=None) -> None:
+        """u: the uniform numbers of a sampling decoder, one per token index (a tensor or an array of at least
+        as many as will be generated); None draws capacity new ones from the device's generator."""
+        if self.u is not None:                                      # in place: captured steps keep reading this address
+            if u is None:
+                self.u.data.copy_(Tensor.uniform(self.u.shape, device=self.u.device).data)
+            else:
+                given = np.asarray(u.numpy() if isinstance(u, Tensor) else u, dtype=np.float32).reshape(-1)
+                full = np.zeros(self.u.shape, np.float32)
+                full[:min(given.size, full.size)] = given[:full.size]
+                self.u.data.upload_(full)
         self.tok.data.upload_(np.array([[first_token]], np.float32))
         self.slot.data.upload_(np.zeros((1, 1), np.float32))
         first = np.zeros(self.seq.shape, np.float32)
@@ -273,10 +312,19 @@ class StaticDecoder:
         return attn.c_proj(y, residual)
 
     def _append(self, logits: Tensor) -> None:
-        """logits (1, V) of the newest position: its argmax becomes seq[slot + 1] and the next token; slot advances."""
-        if nn.decode_append(logits, self.tok, self.slot, self.seq):                     # one launch
+        """logits (1, V) of the newest position: its argmax -- or, for a sampling decoder, the token that u[slot] draws
+        from softmax(logits / temperature) -- becomes seq[slot + 1] and the next token; slot advances."""
+        if self.temperature is not None:
+            if nn.decode_sample(logits, self.u, self.tok, self.slot, self.seq, self.temperature):     # one launch
+                return
+            # elsewhere as the reference does it: on the host, from the downloaded logits
+            s = int(self.slot.numpy()[0, 0])
+            drawn = sample_from_logits(logits.numpy(), self.u.numpy().reshape(-1)[s], self.temperature)
+            nxt = Tensor(np.array([[drawn]], np.float32), device=logits.device)
+        elif nn.decode_append(logits, self.tok, self.slot, self.seq):                   # one launch
             return
-        nxt = logits.argmax(1)                                                          # (1, 1)
+        else:
+            nxt = logits.argmax(1)                                                      # (1, 1)
         nslot = self.slot + 1.0
         self.seq.data.row_store_(nxt.data, nslot.data)
         self.tok.data.copy_(nxt.data)
@@ -337,11 +385,12 @@ class StaticDecoder:
             with self.window_graph.capture():
                 self.step_window()
 
-    def generate(self, first_token: int, max_new_tokens: int) -> list[int]:
+    def generate(self, first_token: int, max_new_tokens: int, u=None) -> list[int]:
+        """u: for a sampling decoder, the uniform number per token (see reset)."""
         c = self.model.config
         if not 0 <= max_new_tokens <= self.capacity - 1:
             raise ValueError(f"this decoder holds {self.capacity} tokens: at most {self.capacity - 1} new ones")
-        self.reset(first_token)
+        self.reset(first_token, u)
         for t in range(max_new_tokens):
             if t < c.block_size - 1:                      # t + 1 tokens so far: still inside the window
                 self.graph.replay() if self.graph is not None else self.step()

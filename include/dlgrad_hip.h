@@ -173,6 +173,12 @@ int dlg_hip_reduce_full_static(uint64_t k_stage, uint64_t k_fold, const void *x,
  * calls fail while capturing); dlg_hip_graph_launch replays it on the same stream.                                                                */
 int dlg_hip_arena_create(uint64_t *arena);
 int dlg_hip_arena_set(uint64_t arena);            /* 0 = the ordinary pool */
+/* Tops the arena's returned blocks up, size class by size class, to the largest number of blocks
+ * of that class that were ever in use at once: after it, a pass that repeats the allocations the
+ * arena has seen finds every block without a device allocation, also while results of the earlier
+ * pass are still held.  Called between the warm-up pass and the capture, because an allocation that
+ * misses the arena during a capture is refused (dlg_hip_alloc).  Fails inside a capture.           */
+int dlg_hip_arena_reserve(uint64_t arena);
 int dlg_hip_arena_destroy(uint64_t arena);
 int dlg_hip_graph_begin(void);
 int dlg_hip_graph_end(uint64_t *graph, uint64_t *n_nodes);   /* graph == NULL abandons the capture */

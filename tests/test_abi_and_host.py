@@ -229,8 +229,16 @@ def test_an_allocation_that_misses_the_arena_during_a_capture_is_refused_on_the_
     (big + big).numpy()                                           # its kernel is loaded before any capture
     g = hip.Graph()
     with g.arena():
-        y = x + x                                                 # the warm-up leaves one 256-byte block
-    del y
+        y = x + x                                                 # the warm-up uses one 256-byte block at a time
+    allocs_warm = lib.pool_stats()[2]
+    with g.capture():                                             # ... and a repeat of it finds its block although y is still held
+        y_again = x + x
+    assert lib.pool_stats()[2] == allocs_warm
+    g.close()
+    g = hip.Graph()
+    with g.arena():
+        y = x + x
+    del y, y_again
     allocs = lib.pool_stats()[2]
     with pytest.raises(RuntimeError, match="missed the arena during a capture"):
         with g.capture():
@@ -240,8 +248,10 @@ def test_an_allocation_that_misses_the_arena_during_a_capture_is_refused_on_the_
     with pytest.raises(RuntimeError, match="missed the arena during a capture"):
         with g.capture():
             y1 = x + x
-            y2 = x + x                                            # a second live block of a size the arena holds once
+            y2 = x + x
+            y3 = x + x                                            # three blocks at once of a size the arena holds twice
     assert not hip.capturing()
+    del y1, y2                                                    # (back to the arena)
     np.testing.assert_array_equal((big + big).numpy(), np.full((300, 300), 2, np.float32))   # ordinary work goes on
     with g.capture():                                             # and the same Graph can still capture what fits
         y = x + x

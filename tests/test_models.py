@@ -81,7 +81,7 @@ def torch_gpt_loss_and_grads(model: G.GPT, idx, tgt, dtype=torch.float32, detail
     """Independent PyTorch statement of the examples/gpt.py graph.  details (a dict): receives the
     logits and the ReLU branch taken per hidden unit, layer by layer.  backward=False: the forward
     pass alone, nothing kept for a backward pass (returns the loss and no gradients)."""
-    if not backward:
+    if backward is False:
         with torch.no_grad():
             return torch_gpt_loss_and_grads(model, idx, tgt, dtype, details, backward=None)
     c = model.config
@@ -409,6 +409,143 @@ def test_char_gpt_decodes_256_tokens_like_the_cpu_oracle(reference_positions):
         compared = same_ids_or_a_near_tie(got, want, want_rows, what)
         assert compared >= 1
     assert runs["fixed-shape steps, replayed graphs"] == runs["fixed-shape steps, eager"]      # bit-identical steps
+
+
+def test_host_sampling_is_numpy_choice_with_its_uniform_draw_made_explicit():
+    """helpers.sample_from_logits(logits, u, temperature) against the call the reference makes,
+    np.random.choice(V, p=softmax(logits / temperature)) (examples/gpt.py:209-221, :258-266), on a legacy
+    RandomState whose next uniform draw is known to be u: the same token, for flat and for peaked rows."""
+    rng = np.random.default_rng(0)
+    for case in range(300):
+        V = int(rng.integers(2, 200))
+        logits = (rng.standard_normal(V) * rng.choice([0.02, 1.0, 8.0])).astype(np.float32)
+        temperature = float(rng.choice([0.7, 1.0, 1.3]))
+        x = logits / np.float32(temperature)
+        x = x - np.max(x)
+        p = np.exp(x) / np.sum(np.exp(x))
+        seed = int(rng.integers(0, 2 ** 31))
+        u = np.random.RandomState(seed).random_sample()
+        assert helpers.sample_from_logits(logits, u, temperature) == np.random.RandomState(seed).choice(V, p=p), case
+    assert helpers.sample_from_logits(np.array([0.0, 0.0], np.float32), 0.4999) == 0
+    assert helpers.sample_from_logits(np.array([0.0, 0.0], np.float32), 0.5) == 1
+    assert helpers.sample_from_logits(np.array([0.0, -np.inf, 0.0], np.float32), 0.75) == 2      # a token of probability 0 is never drawn
+
+
+def test_sampling_decoder_reproduces_the_sampling_loop_on_the_cpu_oracle():
+    """StaticDecoder(temperature=...) -- fixed-shape steps, the uniform numbers held in a tensor -- draws the
+    tokens of GPT.generate (the reference's loop, sampling on the host) when both are given the same numbers,
+    inside the window and beyond it; other numbers give another sequence; greedy decoders are unchanged."""
+    import dlgrad_amd
+    model = G.GPT(G.GPTConfig(device="cpu", **dict(TINY, n_embd=32, block_size=12)))
+    G.init_weights_(model, 3, std=0.5)
+    u = np.random.default_rng(5).random(31).astype(np.float32)
+    want = model.generate(3, 30, temperature=0.7, u=u)
+    assert len(want) == 31 and want != model.generate_greedy_cached(3, 30)
+    dec = G.StaticDecoder(model, capacity=31, temperature=0.7)
+    assert dec.generate(3, 30, u=u) == want
+    assert dec.generate(3, 12, u=u) == want[:13]
+    assert dec.generate(3, 30, u=np.roll(u, 1)) != want
+    oracle.cpu_runtime.CPU.manual_seed(11)
+    a = dec.generate(3, 30)                                       # numbers from the device's own seeded generator
+    oracle.cpu_runtime.CPU.manual_seed(11)
+    assert dec.generate(3, 30) == a and a != dec.generate(3, 30)
+    with pytest.raises(ValueError):
+        G.StaticDecoder(model, temperature=0.0)
+
+
+def sampled_like_the_oracle(got: list, want: list, want_rows: list, u, temperature: float, what: str) -> int:
+    """Token for token equal -- or, at the first token that differs, the uniform number must lie within 1e-5
+    of the oracle's own boundary between the two tokens (printed): the running sums are added in different
+    orders, and from there on the sequences are different contexts.  Returns the number of tokens compared."""
+    assert len(got) == len(want), what
+    for t in range(1, len(want)):
+        if got[t] != want[t]:
+            x = np.asarray(want_rows[t - 1], np.float32) / np.float32(temperature)
+            e = np.exp((x - x.max()).astype(np.float64))
+            cdf = np.cumsum(e) / e.sum()
+            lo, hi = (0.0 if got[t] == 0 else cdf[got[t] - 1]), cdf[got[t]]
+            dist = max(lo - float(u[t - 1]), float(u[t - 1]) - hi, 0.0)
+            print(f"{what}: token {t} is {got[t]} where the oracle draws {want[t]}; u = {float(u[t - 1]):.8f} lies {dist:.2e} outside "
+                  f"the oracle's interval [{lo:.8f}, {hi:.8f}) of that token; {t} of {len(want) - 1} tokens compared")
+            assert dist <= 1e-5, f"{what}: token {t} differs and u is not at the boundary"
+            return t
+    return len(want) - 1
+
+
+@pytest.mark.gpu
+def test_sampling_on_the_device_draws_the_tokens_of_the_cpu_oracle():
+    """hip: the one-launch draw (decode_sample: softmax(logits / temperature), running sum, first index beyond
+    u * total) against numpy's choice() arithmetic on the same logits and the same uniform number, row by
+    row for vocabularies from 2 to 50304; then the char-GPT of BASELINE config 4 sampling 200 tokens at
+    temperature 0.7 -- fixed-shape steps eager and as replayed graphs -- against the reference's loop
+    (cache, host-side sampling) on the C restatement's cpu device with the same numbers.  A draw may differ
+    only where u sits on the boundary between two tokens (1e-5), and says so."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    rng = np.random.default_rng(21)
+    checked = boundary = 0
+    for V in (2, 3, 64, 65, 255, 256, 257, 1000, 50304):
+        for trial in range(6):
+            logits = (rng.standard_normal((1, V)) * rng.choice([0.02, 1.0, 6.0])).astype(np.float32)
+            if trial == 5 and V > 3:
+                logits[0, 1::2] = -np.inf                          # tokens that must never be drawn
+            temperature = float(rng.choice([0.7, 1.0, 1.6]))
+            n_u = 5
+            us = rng.random(n_u).astype(np.float32)
+            if trial == 0:
+                us[:2] = (0.0, np.nextafter(np.float32(1), np.float32(0)))
+            lg, ut = Tensor(logits, device="hip"), Tensor(us, device="hip")
+            for s in range(n_u):
+                tok, slot = Tensor(np.array([[9]], np.float32), device="hip"), Tensor(np.array([[s]], np.float32), device="hip")
+                seq = Tensor(np.zeros((n_u + 1, 1), np.float32), device="hip")
+                assert nn.decode_sample(lg, ut, tok, slot, seq, temperature)
+                if hip.COMPILE_ONLY:
+                    continue
+                got, want = int(tok.numpy()[0, 0]), helpers.sample_from_logits(logits, us[s], temperature)
+                assert slot.numpy()[0, 0] == s + 1 and seq.numpy()[s + 1, 0] == got and np.count_nonzero(seq.numpy()) <= 1
+                assert np.isfinite(logits[0, got]), "a token of probability 0 was drawn"
+                checked += 1
+                if got != want:
+                    boundary += 1
+                    sampled_like_the_oracle([0, got], [0, want], [logits[0]], [us[s]], temperature, f"V={V} u={us[s]}")
+    models = {}
+    for dev in ("cpu", "hip"):
+        models[dev] = G.GPT(G.GPTConfig(device=dev, **C4))
+        G.init_weights_(models[dev], 0)
+    n_new, temperature = 200, 0.7
+    u = np.random.default_rng(8).random(n_new + 1).astype(np.float32)
+    dec = G.StaticDecoder(models["hip"], capacity=n_new + 1, temperature=temperature)
+    runs = {"fixed-shape sampling steps, eager": dec.generate(0, n_new, u=u)}
+    if hip.COMPILE_ONLY:
+        return
+    dec.capture()
+    nodes_sampling = dec.graph.nodes
+    runs["fixed-shape sampling steps, replayed graphs"] = dec.generate(0, n_new, u=u)
+    other = dec.generate(0, n_new, u=np.roll(u, 3))                                  # the replayed graphs read the new numbers
+    dec.close()
+    greedy = G.StaticDecoder(models["hip"], capacity=n_new + 1)
+    greedy.capture()
+    assert nodes_sampling == greedy.graph.nodes                                       # the draw replaces the argmax launch
+    greedy.close()
+    want_rows: list = []
+    cpu = models["cpu"]
+    real_sample = helpers.sample_from_logits
+    import examples.gpt as gpt_module
+
+    def recording(logits, uval, temp):
+        want_rows.append(np.array(logits, np.float32).reshape(-1))
+        return real_sample(logits, uval, temp)
+
+    gpt_module.sample_from_logits = recording
+    try:
+        want = cpu.generate(0, n_new, temperature=temperature, u=u)
+    finally:
+        gpt_module.sample_from_logits = real_sample
+    assert len(set(want)) > 20 and other != runs["fixed-shape sampling steps, replayed graphs"]
+    for what, got in runs.items():
+        assert sampled_like_the_oracle(got, want, want_rows, u, temperature, what) >= 1
+    assert runs["fixed-shape sampling steps, replayed graphs"] == runs["fixed-shape sampling steps, eager"]
+    print(f"decode_sample: {checked} single draws compared with numpy's choice arithmetic, {boundary} on a boundary")
 
 
 @pytest.mark.gpu
