@@ -2019,7 +2019,7 @@ MATMUL_TRI = ("", "out_lower", "a_lower", "at_lower")
 @cache
 def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb: bool,
                   ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False,
-                  epi: str = "", S: int = 32, norm: bool = False) -> tuple[str, str, str]:
+                  epi: str = "", S: int = 32, norm: bool = False, splitk: bool = False) -> tuple[str, str, str]:
     """C[z] = op(A[z]) . op(B[z]), fp32, row-major, on the matrix cores (v_mfma_f32_32x32x2_f32, or
     v_mfma_f32_16x16x4_f32 for S = 16).
 
@@ -2076,8 +2076,18 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     stored.  The blocks of the first tile column also write the normalised rows to yn and r to rinv
     (what the backward pass of the norm and of the product need) unless yn is null.  Arguments after
     the others: gain, eps, yn, rinv.
+    splitk: the k sum is cut into gridDim.y slices of kchunk (a multiple of BK) and block (x, y, z) adds slice y
+    of tile x: a product with few output tiles and a long k (the weight gradient of a linear layer is a handful
+    of tiles with k = the number of tokens) then fills the chip.  Each block writes its partial tile to slab
+    (z * gridDim.y + y) of a workspace W of gridDim.z * gridDim.y * M * N floats instead of C, and a column-sum
+    launch over the slabs finishes the product.  An output element is then a sum of per-slice sums: not the
+    bits of the unsplit kernel (each slice still adds its k in that kernel's order), within the 1e-4 that
+    products are held to.  (Folding the slabs in the same launch, by the block that finishes a tile last, was
+    measured and dropped: the device-wide fence in front of the arrival counter cost 50 us per launch.)
+    Arguments after the others: W, kchunk.
     """
     BM, BN, T = S * MI * WM, S * NJ * WN, 64 * WM * WN
+    assert isinstance(splitk, bool) and not (splitk and (tri or strided or epi or norm))
     NE = S * S // 64                                        # accumulator registers per MFMA tile
     assert BK % 8 == 0 and MI in (1, 2, 3, 4) and NJ in (1, 2, 3, 4) and S in (16, 32) and T <= 1024
     assert matmul_lds_bytes(WM, WN, MI, NJ, BK, ta, tb, S) <= MATMUL_LDS_LIMIT
@@ -2087,6 +2097,8 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     assert not norm or (veca and not ta and not tri and not strided and BK <= 256)
     if norm:
         name += "_rms"
+    if splitk:
+        name += "_sk"
     comp = ["x", "y", "z", "w"]
     vtype = {1: "float", 2: "float2", 3: "f3v", 4: "float4"}
 
@@ -2107,12 +2119,12 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
             idx = f"const u32 {x}_q = tid % {Q}u, {x}_r = tid / {Q}u;"
             where = f"const u32 row = {base} + {x}_r + p * {rpp}u, k = k0 + 4u * {x}_q;"
             if vec:
-                ld_code = (f"r{x}[p] = (row < g.{ext} && k < g.K) ? *reinterpret_cast<const float4*>({X} + (u64)row * g.K + k)\n"
+                ld_code = (f"r{x}[p] = (row < g.{ext} && k < KEND) ? *reinterpret_cast<const float4*>({X} + (u64)row * g.K + k)\n"
                            f"                                         : make_float4(0.f, 0.f, 0.f, 0.f);")
             else:
                 ld_code = (f"const float* __restrict__ s = {X} + (u64)row * g.K + k;\n"
                            f"            const bool ok = row < g.{ext};\n" +
-                           "".join(f"            r{x}[p].{c} = (ok && k + {n}u < g.K) ? s[{n}] : 0.f;\n" for n, c in enumerate(comp)))
+                           "".join(f"            r{x}[p].{c} = (ok && k + {n}u < KEND) ? s[{n}] : 0.f;\n" for n, c in enumerate(comp)))
             st = f"{guard}*reinterpret_cast<float4*>(&{X}s[buf][{x}_r + p * {rpp}u][4u * {x}_q]) = r{x}[p];"
             decl = f"__shared__ __attribute__((aligned(16))) float {X}s[2][{R}][{BK + 4}];"
         else:
@@ -2124,11 +2136,11 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
             idx = f"const u32 {x}_q = tid % {Q}u, {x}_r = tid / {Q}u;"
             where = f"const u32 k = k0 + {x}_r + p * {rpp}u, col = {base} + 4u * {x}_q;"
             if vec:
-                ld_code = (f"r{x}[p] = (k < g.K && col < g.{ext}) ? *reinterpret_cast<const float4*>({X} + (u64)k * g.{ext} + col)\n"
+                ld_code = (f"r{x}[p] = (k < KEND && col < g.{ext}) ? *reinterpret_cast<const float4*>({X} + (u64)k * g.{ext} + col)\n"
                            f"                                         : make_float4(0.f, 0.f, 0.f, 0.f);")
             else:
                 ld_code = (f"const float* __restrict__ s = {X} + (u64)k * g.{ext} + col;\n"
-                           f"            const bool ok = k < g.K;\n" +
+                           f"            const bool ok = k < KEND;\n" +
                            "".join(f"            r{x}[p].{c} = (ok && col + {n}u < g.{ext}) ? s[{n}] : 0.f;\n" for n, c in enumerate(comp)))
             st = f"{guard}*reinterpret_cast<float4*>(&{X}s[buf][{x}_r + p * {rpp}u][4u * {x}_q]) = r{x}[p];"
             decl = f"__shared__ __attribute__((aligned(16))) float {X}s[2][{BK}][{R}];"
@@ -2226,7 +2238,14 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     }}
     __syncthreads();
 """
-    if tri in ("", "out_lower"):
+    if splitk:
+        kloop = f"""    const u32 nk = (kend + BK - 1u) / BK, kt0 = kbeg / BK;                 // this block's slice of k
+    load_tiles(kt0 * BK);
+    stash_tiles(0u);
+    __syncthreads();
+    for (u32 kt = kt0; kt < nk; ++kt) {{
+        const u32 buf = (kt - kt0) & 1u;"""
+    elif tri in ("", "out_lower"):
         kloop = f"""    const u32 nk = (g.K + BK - 1u) / BK;
     load_tiles(0u);
     stash_tiles(0u);
@@ -2242,6 +2261,12 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     __syncthreads();
     for (u32 kt = kt0; kt < nk; ++kt) {{
         const u32 buf = (kt - kt0) & 1u;"""
+    split_head = split_tail = ""
+    if splitk:
+        split_head = """    const u32 kbeg = blockIdx.y * kchunk, kend = min(g.K, kbeg + kchunk);
+    const u64 slab_elts = (u64)g.M * g.N;
+    float* __restrict__ slab = W + ((u64)blockIdx.z * gridDim.y + blockIdx.y) * slab_elts;
+"""
     f4v_typedef = "" if S == 32 else "\ntypedef float f4v __attribute__((ext_vector_type(4)));"
     src = f"""{PRELUDE}
 typedef float f16v __attribute__((ext_vector_type(16)));{f4v_typedef}
@@ -2252,8 +2277,9 @@ struct MMArgs {{ u32 M, N, K, nbc, sa0, sa1, sb0, sb1; }};
 #define BK {BK}u
 #define MI {MI}
 #define NJ {NJ}
+#define KEND {"kend" if splitk else "g.K"}
 extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict__ A,
-        const float* __restrict__ B, float* __restrict__ C, MMArgs g{", const float* __restrict__ E" if epi else ""}{", const float* __restrict__ gain, float eps, float* __restrict__ yn, float* __restrict__ rinv" if norm else ""}) {{
+        const float* __restrict__ B, float* __restrict__ C, MMArgs g{", const float* __restrict__ E" if epi else ""}{", const float* __restrict__ gain, float eps, float* __restrict__ yn, float* __restrict__ rinv" if norm else ""}{", float* __restrict__ W, u32 kchunk" if splitk else ""}) {{
     {decl_a}
     {decl_b}
 
@@ -2272,7 +2298,7 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
     A += (u64)zb * g.sa0 + (u64)zc * g.sa1;
     B += (u64)zb * g.sb0 + (u64)zc * g.sb1;
     C += (u64)blockIdx.z * g.M * g.N;
-
+{split_head}
     const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const u32 r = lane & {S - 1}u, h = lane >> {5 if S == 32 else 4};
     const u32 wm0 = (wave / {WN}u) * {S * MI}u, wn0 = (wave % {WN}u) * {S * NJ}u;
@@ -2308,11 +2334,11 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
         for (int e = 0; e < {NE}; ++e) {{
             const u32 row = {row_expr};
             if (row < g.M) {{
-                float* __restrict__ crow = C + (u64)row * g.N;
+                float* __restrict__ crow = {"slab" if splitk else "C"} + (u64)row * g.N;
 {store}
             }}
         }}
-}}
+{split_tail}}}
 """
     if epi:
         assert epi in ("add", "relu", "gate", "bias") and not strided
@@ -2372,7 +2398,7 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
             assert src.count(was) == 1, was
             src = src.replace(was, now)
         return src, name, _fmt("P", "P", "P", "13I")
-    return src, name, _fmt("P", "P", "P", "8I", *(("P", "f", "P", "P") if norm else ()))
+    return src, name, _fmt("P", "P", "P", "8I", *(("P", "f", "P", "P") if norm else ()), *(("P", "I") if splitk else ()))
 
 
 @cache

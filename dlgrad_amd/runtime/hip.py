@@ -255,6 +255,7 @@ def _upload(dst_addr: int, a: np.ndarray) -> None:
 
 # ---- captured graphs ------------------------------------------------------------------------
 _graph_depth = 0       # > 0 while a Graph's arena is current (warm-up or capture)
+_current_arena = 0     # its id (0: the ordinary pool)
 _after_capture: list = []   # host work a captured step deferred until its capture has ended (table uploads)
 _capturing = False
 
@@ -289,15 +290,15 @@ class Graph:
         self.handle, self.nodes = 0, 0
 
     def _enter(self) -> None:
-        global _graph_depth
+        global _graph_depth, _current_arena
         if _graph_depth:
             raise RuntimeError("graph arenas do not nest")
         self._lib.arena_set(self.arena_id)
-        _graph_depth = 1
+        _graph_depth, _current_arena = 1, self.arena_id
 
     def _leave(self) -> None:
-        global _graph_depth
-        _graph_depth = 0
+        global _graph_depth, _current_arena
+        _graph_depth, _current_arena = 0, 0
         self._lib.arena_set(0)
 
     def arena(self):
@@ -1630,6 +1631,7 @@ class HIP:
     # "1": a shape met for the first time (and large enough to matter) is timed once with every
     # plausible tile and the fastest is remembered; "0": shipped table, then the model
     MATMUL_TUNE = os.environ.get("DLGRAD_HIP_MATMUL_TUNE", "1") != "0"
+    MATMUL_SPLITK = os.environ.get("DLGRAD_HIP_MATMUL_SPLITK", "1") != "0"  # "0": never cut the k sum of a product into slices
     MATMUL_TABLE = os.environ.get("DLGRAD_HIP_MATMUL_TABLE", "1") != "0"    # "0": ignore the measured tables (model, or first-use timing, only)
     MATMUL_TUNE_MIN_FLOP = 1 << 24
     _tuned: dict | None = None
@@ -1652,7 +1654,7 @@ class HIP:
             for path in (os.path.join(os.path.dirname(K.__file__), "matmul_tuned.json"), HIP._tuned_path()) if HIP.MATMUL_TABLE else ():
                 try:
                     with open(path) as f:
-                        table.update({k: v for k, v in json.load(f).items() if all(t in K.MATMUL_CONFIGS for t in v.split("+"))})
+                        table.update({k: v for k, v in json.load(f).items() if all(HIP._valid_tile(t) for t in v.split("+"))})
                 except (OSError, ValueError):
                     pass
             HIP._tuned = table
@@ -1683,11 +1685,31 @@ class HIP:
             best = "64x64k64"                       # few blocks, long K: the deep-K form of the same tile
         return best
 
+    SPLITK_BASES = ("128x128", "128x64", "64x64k64", "64x64m16")      # tiles whose split-k forms are timed
+
     @staticmethod
-    def _tile_candidates(M: int, N: int, batch: int) -> list[str]:
+    def _splitk_eligible(M: int, N: int, Kd: int, batch: int) -> bool:
+        """Few output tiles (128 x 128 tiles for at most half the CUs; for all of them when k is at least 2048)
+        and a k long enough to cut.  Measured on (768 x 8192)^T (8192 x 768): 60 -> 86 TFLOP/s, on the 3072-wide
+        one 81 -> 100, on (128 x 2048)(2048 x 512) 11 -> 23; squares (512^3, 1024^3) gain nothing."""
+        tiles = -(-M // 128) * -(-N // 128) * batch
+        return HIP.MATMUL_SPLITK and ((Kd >= 512 and tiles <= 128) or (Kd >= 2048 and tiles <= 256))
+
+    @staticmethod
+    def _tile_candidates(M: int, N: int, batch: int, Kd: int = 0, split: bool = False) -> list[str]:
         """Tiles worth timing: none much larger than the output, and the two smallest only
-        where the output is small enough for them to have a chance."""
+        where the output is small enough for them to have a chance.  split: also the split-k forms of a
+        few tiles, 2 to 16 slices of at least 128 k each."""
         out = []
+        if split:
+            for base in HIP.SPLITK_BASES:
+                bm, bn, _ = K.matmul_tile_shape(base)
+                if bm > max(32, 2 * M) or bn > max(32, 2 * N):
+                    continue
+                tiles = -(-M // bm) * -(-N // bn) * batch
+                for slices in (2, 4, 8, 16):
+                    if Kd // slices >= 128 and tiles * slices <= 2048 and HIP._split_plan(f"{base}/{slices}", Kd)[0] == slices:
+                        out.append(f"{base}/{slices}")
         for name in K.MATMUL_CONFIGS:
             bm, bn, _ = K.matmul_tile_shape(name)
             if bm > max(32, 2 * M) or bn > max(32, 2 * N):
@@ -1698,18 +1720,55 @@ class HIP:
         return out
 
     @staticmethod
+    def _split_of(tile: str) -> tuple[str, int]:
+        """"128x128/4" -> ("128x128", 4): the k sum cut into 4 slices, a block per (tile, slice), the partial tiles
+        added up by a column-sum launch.  A plain tile name: (tile, 1)."""
+        base, _, sk = tile.partition("/")
+        return (base, int(sk)) if sk else (base, 1)
+
+    @staticmethod
+    def _valid_tile(tile: str) -> bool:
+        try:
+            base, slices = HIP._split_of(tile)
+        except ValueError:
+            return False
+        return base in K.MATMUL_CONFIGS and 1 <= slices <= 64
+
+    @staticmethod
+    def _split_plan(tile: str, Kd: int) -> tuple[int, int]:
+        """(slices, kchunk) actually launched: kchunk a multiple of the tile's k step, no empty slice."""
+        base, slices = HIP._split_of(tile)
+        bk = K.MATMUL_CONFIGS[base][4]
+        kchunk = -(-(-(-Kd // slices)) // bk) * bk
+        return -(-Kd // kchunk), kchunk
+
+    @staticmethod
     def _launch_matmul(tile: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple,
                        ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False, epi: str = "") -> None:
+        if "/" in tile:
+            if tri or strided or epi:
+                raise ValueError(f"a split-k tile ({tile}) takes no triangular, strided or epilogue form")
+            Kd = args[5]
+            k, grid, threads = HIP._matmul_kernel(tile, veca, vecb, M, N, batch, ta, tb, Kd=Kd)
+            HIP.last_matmul_kernel = kernel_names.get(id(k))
+            ws = alloc(batch * grid[1] * M * N)                        # one slab per slice (handed back as soon as both launches are issued)
+            launch(k, grid, threads, *args, ws.addr, HIP._split_plan(tile, Kd)[1])
+            HIP._reduce_cols("sum", ws.addr, batch, grid[1], M * N, 1.0, args[2])
+            return
         k, grid, threads = HIP._matmul_kernel(tile, veca, vecb, M, N, batch, ta, tb, tri, strided, epi)
         HIP.last_matmul_kernel = kernel_names.get(id(k))
         launch(k, grid, threads, *args)
 
     @staticmethod
     def _matmul_kernel(tile: str, veca: bool, vecb: bool, M: int, N: int, batch: int, ta: bool = False, tb: bool = False,
-                       tri: str = "", strided: bool = False, epi: str = "") -> tuple:
-        """(loaded kernel, grid, threads per block) of one product."""
-        bm, bn, threads = K.matmul_tile_shape(tile)
-        cfg = K.MATMUL_CONFIGS[tile]                           # (WM, WN, MI, NJ, BK) and, for the 16-wide MFMA tiles, 16
+                       tri: str = "", strided: bool = False, epi: str = "", Kd: int = 0) -> tuple:
+        """(loaded kernel, grid, threads per block) of one product (Kd: needed for a split-k tile only)."""
+        base, slices = HIP._split_of(tile)
+        bm, bn, threads = K.matmul_tile_shape(base)
+        cfg = K.MATMUL_CONFIGS[base]                           # (WM, WN, MI, NJ, BK) and, for the 16-wide MFMA tiles, 16
+        if slices > 1:
+            k = kernel(K.matmul_kernel, *cfg[:5], veca, vecb, ta, tb, "", False, "", cfg[5] if len(cfg) > 5 else 32, False, True)
+            return k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), HIP._split_plan(tile, Kd)[0], batch), threads
         k = kernel(K.matmul_kernel, *cfg[:5], veca, vecb, ta, tb, tri, strided, epi, *cfg[5:])
         return k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch), threads
 
@@ -1725,12 +1784,13 @@ class HIP:
             HIP._tune_warned = True
             warnings.warn(f"dlgrad_amd: the matrix product {key} (batch,M,N,K) is in no tile table; timing every plausible tile "
                           "on its operands now, once per shape and machine (about 10 ms for mid-sized products, up to 0.5 s at "
-                          "8192^3; the choice is stored in dlgrad_amd/_kcache/matmul_tuned.json and changes no result bit). "
+                          "8192^3; the choice is stored in dlgrad_amd/_kcache/matmul_tuned.json; no tile changes a result bit except the split-k "
+                          "forms, which add the same terms slice by slice). "
                           "DLGRAD_HIP_MATMUL_TUNE=0 switches the timing off; further shapes are timed without this message.",
                           RuntimeWarning, stacklevel=2)
         best, best_ms = None, float("inf")
         e0, e1 = l.event_create(), l.event_create()
-        for tile in HIP._tile_candidates(M, N, batch):
+        for tile in HIP._tile_candidates(M, N, batch, args[5], key.endswith(",sk")):
             HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri, strided)   # loads the code object
             if COMPILE_ONLY:
                 continue
@@ -1776,14 +1836,24 @@ class HIP:
 
     @staticmethod
     def _pick_tile(M: int, N: int, Kd: int, batch: int, veca: bool, vecb: bool, args: tuple,
-                   ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False) -> str:
+                   ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False, split_ok: bool = False) -> str:
+        """split_ok: the caller can take a split-k tile (a plain product: no epilogue, structure or pitch).  Such
+        products have table entries of their own (key + ",sk"), since the other forms of the same shape cannot
+        use what was found for them."""
         if HIP.MATMUL_FORCE:
-            return HIP.MATMUL_FORCE
+            return HIP.MATMUL_FORCE if split_ok else HIP._split_of(HIP.MATMUL_FORCE)[0]
         key = HIP._tile_key(M, N, Kd, batch, ta, tb, tri, strided)
+        tune = HIP.MATMUL_TUNE and not capturing() and 2 * M * N * Kd * batch >= HIP.MATMUL_TUNE_MIN_FLOP
+        if split_ok and not tri and not strided and HIP._splitk_eligible(M, N, Kd, batch):
+            tile = HIP._tuned_table().get(key + ",sk")
+            if tile is not None:
+                return tile
+            if tune:
+                return HIP._tune_tile(key + ",sk", veca, vecb, M, N, batch, args, ta, tb)
         tile = HIP._tuned_table().get(key)
         if tile is not None:
-            return tile
-        if HIP.MATMUL_TUNE and not capturing() and 2 * M * N * Kd * batch >= HIP.MATMUL_TUNE_MIN_FLOP:
+            return HIP._split_of(tile)[0]
+        if tune:
             return HIP._tune_tile(key, veca, vecb, M, N, batch, args, ta, tb, tri, strided)
         return HIP._model_tile(M, N, batch, Kd)
 
@@ -1839,10 +1909,14 @@ class HIP:
             launch(k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, 1), threads, xa, ya, out.addr, M, N, Kd, 1, 0, 0, 0, 0, *tail)
             return (out, yn, rinv) if keep else out
         key = (x.shape, y.shape, ta, tb, tri, epi, None if e is None else e.shape, xa & 15, ya & 15, ea & 15,
-               HIP.MATMUL_FORCE, HIP.ROW_MATMUL)
+               HIP.MATMUL_FORCE, HIP.ROW_MATMUL, HIP.MATMUL_SPLITK)
         plan = _matmul_plans.get(key)
         if plan is not None:                                   # a shape seen before: pack the addresses and go
             k, grid, threads, tail, out_numel, e_at, name = plan
+            if e_at == 3:                                      # a split-k tile: a workspace and a second launch
+                out = alloc(out_numel)
+                HIP._launch_matmul(k, *grid, (xa, ya, out.addr, *tail), *threads)
+                return out
             if e_at == 0:                                      # (x, y, out, sizes and strides)
                 HIP.last_matmul_kernel = name
                 return launch_out(k, grid, threads, 16, out_numel, xa, ya, 0, *tail)
@@ -1905,14 +1979,17 @@ class HIP:
         if epi and e is not None and (_addr(e) % 16 or N % 4):
             vecb = False                                       # the epilogue reads e as it writes the result
         args = (_addr(x), _addr(y), out.addr, M, N, Kd, nbc, *sa, *sb)
-        tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, args, ta, tb, tri)
+        tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, args, ta, tb, tri, split_ok=not epi and not tri)
         if epi:
             HIP._launch_matmul(tile, veca, vecb, M, N, batch, (*args, out.addr if e is None else _addr(e)), ta, tb, "", False, epi)
         else:
             HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri)
         if not capturing():                                    # (while capturing, a shape met for the first time is not timed)
-            k, grid, threads = HIP._matmul_kernel(tile, veca, vecb, M, N, batch, ta, tb, "" if epi else tri, False, epi)
-            _matmul_plans[key] = (k, grid, threads, args[3:], out_numel, 1 if epi else 0, HIP.last_matmul_kernel)
+            if "/" in tile:
+                _matmul_plans[key] = (tile, (veca, vecb, M, N, batch), (ta, tb), args[3:], out_numel, 3, HIP.last_matmul_kernel)
+            else:
+                k, grid, threads = HIP._matmul_kernel(tile, veca, vecb, M, N, batch, ta, tb, "" if epi else tri, False, epi)
+                _matmul_plans[key] = (k, grid, threads, args[3:], out_numel, 1 if epi else 0, HIP.last_matmul_kernel)
         return out
 
     @staticmethod

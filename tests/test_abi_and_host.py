@@ -479,17 +479,17 @@ def test_first_tile_timing_of_a_process_says_so_once(monkeypatch, tmp_path):
     monkeypatch.setattr(hip, "lib", lambda: Events())
     monkeypatch.setattr(hip, "COMPILE_ONLY", False)
     monkeypatch.setattr(HIP, "_launch_matmul", staticmethod(lambda *a, **k: None))
-    monkeypatch.setattr(HIP, "_tile_candidates", staticmethod(lambda M, N, batch: ["128x128x32_w2x2"]))
+    monkeypatch.setattr(HIP, "_tile_candidates", staticmethod(lambda M, N, batch, Kd=0, split=False: ["128x128x32_w2x2"]))
     monkeypatch.setattr(HIP, "MATMUL_TUNED_FILE", str(tmp_path / "tuned.json"))
     monkeypatch.setattr(HIP, "_tuned_new", {})
     monkeypatch.setattr(HIP, "_tune_warned", False)
     table = dict(HIP._tuned_table())
     try:
         with pytest.warns(RuntimeWarning, match=r"1,3000,1000,2000.*DLGRAD_HIP_MATMUL_TUNE=0"):
-            assert HIP._tune_tile("1,3000,1000,2000", True, True, 3000, 1000, 1, (), False, False) == "128x128x32_w2x2"
+            assert HIP._tune_tile("1,3000,1000,2000", True, True, 3000, 1000, 1, (0, 0, 0, 3000, 1000, 2000), False, False) == "128x128x32_w2x2"
         with warnings.catch_warnings():
             warnings.simplefilter("error")                                # a second shape: timed without a word
-            assert HIP._tune_tile("1,3001,1000,2000", True, True, 3001, 1000, 1, (), False, False) == "128x128x32_w2x2"
+            assert HIP._tune_tile("1,3001,1000,2000", True, True, 3001, 1000, 1, (0, 0, 0, 3001, 1000, 2000), False, False) == "128x128x32_w2x2"
         import json
         assert set(json.load(open(tmp_path / "tuned.json"))) == {"1,3000,1000,2000", "1,3001,1000,2000"}
     finally:

@@ -144,8 +144,8 @@ def test_first_use_of_a_large_shape_times_the_tiles_and_remembers_the_winner(mon
     check_mm(got, x.astype(np.float64) @ y, "tuned shape")
     if H.COMPILE_ONLY:
         return
-    key = f"1,{M},{N},{Kd}"
-    assert HIP._tuned[key] in __import__("dlgrad_amd.codegen.hip_kernel", fromlist=["x"]).MATMUL_CONFIGS
+    key = f"1,{M},{N},{Kd},sk"                          # few tiles, k >= 512: timed with the split-k forms too, under a key of its own
+    assert HIP._valid_tile(HIP._tuned[key]) and HIP._split_of(HIP._tuned[key])[0] in __import__("dlgrad_amd.codegen.hip_kernel", fromlist=["x"]).MATMUL_CONFIGS
     import json
     assert json.load(open(tmp_path / "matmul_tuned.json"))[key] == HIP._tuned[key]
     small = (dev(f32(64, 64)) @ dev(f32(64, 64))).numpy()         # below the threshold: the model picks, nothing is stored
@@ -196,7 +196,7 @@ def test_every_tile_configuration_transposed(tile, monkeypatch):
 
 
 @pytest.mark.parametrize("T,d,batch", [(128, 32, (2, 3)), (1024, 64, (2,)), (100, 20, (3,)), (257, 64, ()), (64, 8, (1, 2))])
-def test_triangular_hints_skip_work_without_changing_a_bit(T, d, batch):
+def test_triangular_hints_skip_work_without_changing_a_bit(T, d, batch, monkeypatch):
     """tri = out_lower / a_lower / at_lower tell the product kernel which tiles or which part of
     the k range a triangular operand or a masked consumer makes irrelevant.  With operands that
     really have that structure every kept entry must equal the plain product bit for bit, for
@@ -204,6 +204,7 @@ def test_triangular_hints_skip_work_without_changing_a_bit(T, d, batch):
     require_gpu()
     from dlgrad_amd.codegen import hip_kernel as K
     from dlgrad_amd.runtime.hip import HIP
+    monkeypatch.setattr(HIP, "MATMUL_SPLITK", False)     # the plain products compared with are the unsplit kernel's (a split-k tile adds slice sums)
     rng = np.random.default_rng(T + d)
     low = np.tril(rng.standard_normal(batch + (T, T), dtype=np.float32))          # zero above the diagonal
     x = rng.standard_normal(batch + (T, d), dtype=np.float32)
@@ -512,3 +513,35 @@ def test_tile_product_normalises_the_rows_of_its_left_operand(xs, N, epi, tile, 
     y64 = (x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + 1e-6) * gain) @ w.T.astype(np.float64)
     y64 = np.maximum(y64, 0) if epi == "relu" else y64 + res if epi == "add" else y64
     check_mm(out.numpy(), y64, "against float64")
+
+
+@pytest.mark.parametrize("tile", ["128x128/4", "64x64k64/8", "64x64m16/3", "128x64/2", "64x64k64/16"])
+def test_split_k_products_add_their_slices_in_a_fixed_order(tile, monkeypatch):
+    """The k sum cut into slices, one block per (tile, slice), the partial tiles added up by a column-sum
+    launch: NN, TN and NT forms, edge tiles, a k that the slices do not divide, batches -- against float64 at
+    the product bar of 1e-4 (the bits are not those of the unsplit kernel: an element is now a sum of
+    per-slice sums), and the same bits on a repeat."""
+    require_gpu()
+    from dlgrad_amd.runtime.hip import HIP
+    monkeypatch.setattr(HIP, "MATMUL_FORCE", tile)
+    for (M, Kd, N), batch in (((512, 512, 512), ()), ((200, 1030, 136), ()), ((96, 2048, 520), ()), ((130, 700, 70), (3,)),
+                              ((64, 4096, 64), (2, 2)), ((1024, 1024, 1024), ())):
+        a, b = f32(*batch, M, Kd), f32(*batch, Kd, N, scale=Kd ** -0.5)
+        da, db = dev(a), dev(b)
+        first = da.matmul(db).numpy()
+        if not hip.COMPILE_ONLY:
+            assert HIP.last_matmul_kernel.endswith("_sk"), HIP.last_matmul_kernel
+        check_mm(first, a.astype(np.float64) @ b.astype(np.float64), f"{tile} {batch}{(M, Kd, N)}")
+        again = da.matmul(db).numpy()
+        if not hip.COMPILE_ONLY:
+            np.testing.assert_array_equal(again, first, err_msg=f"{tile} {(M, Kd, N)} repeated")
+        if not batch:
+            at, bt = dev(np.ascontiguousarray(a.T)), dev(np.ascontiguousarray(b.T))
+            check_mm(at.matmul_tn(db).numpy(), a.astype(np.float64) @ b.astype(np.float64), f"{tile} TN {(M, Kd, N)}")
+            check_mm(da.matmul_nt(bt).numpy(), a.astype(np.float64) @ b.astype(np.float64), f"{tile} NT {(M, Kd, N)}")
+    # an epilogue cannot be split: the forced tile falls back to its unsplit form and the bits are the unsplit kernel's
+    a, b, e = f32(128, 512), f32(512, 128, scale=512 ** -0.5), f32(128, 128)
+    fused = dev(a).matmul(dev(b), epi="add", e=dev(e)).numpy()
+    monkeypatch.setattr(HIP, "MATMUL_FORCE", tile.split("/")[0])
+    if not hip.COMPILE_ONLY:
+        np.testing.assert_array_equal(fused, ((dev(a) @ dev(b)) + dev(e)).numpy())

@@ -573,8 +573,17 @@ def test_a_training_forward_over_a_single_row_keeps_its_tape():
         return
     tensors_close(out["hip"][0], out["cpu"][0], "loss")
     assert out["hip"][1].keys() == out["cpu"][1].keys()
-    for k in out["cpu"][1]:
-        tensors_close(out["hip"][1][k], out["cpu"][1][k], f"grad {k}")
+    # with one position the softmax of the attention is the constant 1: the q and k projections get a gradient that is
+    # exactly 0 in the loops and rounding noise (1e-7 of the model's largest gradient) in the one-launch attention, so
+    # every tensor is held to 1e-4 of its own largest entry or of a hundredth of the largest gradient of the model,
+    # whichever is larger
+    largest = max(float(np.abs(g).max()) for g in out["cpu"][1].values())
+    assert largest > 0
+    for k, want in out["cpu"][1].items():
+        got = out["hip"][1][k]
+        assert np.isfinite(got).all(), k
+        err = float(np.abs(got.astype(np.float64) - want).max()) / max(float(np.abs(want).max()), 1e-2 * largest)
+        assert err <= 1e-4, f"grad {k}: {err:.3e}"
 
 
 @pytest.mark.gpu
