@@ -406,12 +406,19 @@ class Buffer:
         """self is a masked_softmax output; returns the gradient of its input."""
         return self._like(self._dispatch(CustomOps.MASKED_SOFTMAX_BWD, y=self, g=upstream, mask=mask, scale=scale))
 
+    @staticmethod
+    def _attention_kept(p, B: int, n_head: int, T: int) -> tuple:
+        """Shape of what a causal attention keeps for its backward pass: the probabilities (B, n_head, T, T), or the
+        log-sum-exp of every score row (B, n_head, T) where the runtime's kernels never store the probabilities."""
+        nbytes = getattr(p, "nbytes", None)
+        return (B, n_head, T) if nbytes is not None and nbytes < 4 * B * n_head * T * T else (B, n_head, T, T)
+
     def causal_attention(self, k: "Buffer", v: "Buffer", n_head: int, scale: float) -> tuple["Buffer", "Buffer"]:
         """self, k, v: (B, T, C) projections with C = n_head * d.  Returns the context (B, T, C) and the
         attention probabilities (B, n_head, T, T); the heads are read and written in place."""
         B, T, _ = self.shape
         y, p = self._dispatch(CustomOps.CAUSAL_ATTENTION, q=self, k=k, v=v, n_head=n_head, scale=scale)
-        return self._like(y), self._like(p, (B, n_head, T, T))
+        return self._like(y), self._like(p, self._attention_kept(p, B, n_head, T))
 
     def causal_attention_bwd(self, k: "Buffer", v: "Buffer", p: "Buffer", dy: "Buffer", n_head: int,
                              scale: float, y: "Buffer | None" = None) -> tuple["Buffer", "Buffer", "Buffer"]:
@@ -424,7 +431,7 @@ class Buffer:
         probabilities (B, n_head, T, T)."""
         B, T, C3 = self.shape
         y, p = self._dispatch(CustomOps.CAUSAL_ATTENTION_QKV, qkv=self, n_head=n_head, scale=scale)
-        return self._like(y, (B, T, C3 // 3)), self._like(p, (B, n_head, T, T))
+        return self._like(y, (B, T, C3 // 3)), self._like(p, self._attention_kept(p, B, n_head, T))
 
     def causal_attention_qkv_bwd(self, p: "Buffer", dy: "Buffer", n_head: int, scale: float, y: "Buffer | None" = None) -> "Buffer":
         """Gradient of causal_attention_qkv with respect to self, same (B, T, 3C) layout."""

@@ -3140,6 +3140,297 @@ extern "C" __global__ __launch_bounds__(512) void attention_small_bwd(const floa
     return f"{PRELUDE}{WAVE_LDS_FENCE}{common}{body}", name, fmt
 
 
+ATTN_FLASH_D = 64          # widest head the streaming attention kernels take (zero-padded to 32 or 64 columns in LDS)
+
+
+@cache
+def attention_flash_kernel(stage: str, DP: int, blocks_per_cu: int = 1) -> tuple[str, str, str]:
+    """Causal self-attention for long sequences without the (T x T) probabilities in memory
+    (examples/gpt.py:50-55 runs product, scale, mask, softmax, product and keeps four T x T tensors
+    per head for the backward pass).  Heads of width d <= DP (DP = 32 or 64, d % 4 == 0) are read where
+    they lie inside (B, T, pitch) tensors, zero-padded to DP columns on the chip.
+
+    All products run on v_mfma_f32_32x32x2_f32 (lane l feeds A[l % 32][l / 32] and B[l / 32][l % 32]; entry e
+    of a lane's accumulator is row 8 (e / 4) + 4 (l / 32) + e % 4, column l % 32).  The kernels are arranged so
+    that the tile a wavefront has just computed is, entry for entry, the B operand of its next product: the
+    sixteen rows a lane holds are exactly the k values it feeds in sixteen steps, in the order k = 8 (s / 4) +
+    4 h + s % 4 for step s, and the A operand is read from LDS in the same order.  Nothing is transposed
+    and no score passes through LDS.
+
+      "fwd"    a block of four wavefronts per (sequence, head, 128 queries), a wavefront per 32 queries, which it
+               holds in registers as the B operand of S^T = K Q^T.  The keys and values stream through LDS 64 at a
+               time (double-buffered, the next tile in flight in registers).  In S^T a lane holds one query's
+               scores against 32 of the 64 keys (the lane 32 further on holds the other 32), so the running
+               maximum and sum of the online softmax are register operations and one exchange.  The
+               probabilities exp(s * scale - m) feed O^T += V^T P^T; the accumulator is rescaled by
+               exp(m_old - m_new) per tile and divided by the sum at the end.  Besides the context
+               y (B, T, y_pitch) the kernel writes lse = m + log(sum) per (sequence, head, query).
+      "delta"  delta = rowsum(dy * y) per (sequence, head, query) (equal to rowsum(dP * P), since y = P v).
+      "bwd"    a block per (sequence, head, 128 keys), a wavefront per 32 keys, whose key and value rows it holds
+               in registers as B operands.  Queries stream through LDS 64 at a time with their dy rows, lse and
+               delta: S = Q K^T again, P = exp(S * scale - lse), dP = dy V^T, dS = P (dP - delta) scale; then
+               dV^T += dy^T P and dK^T += Q^T dS with P and dS as B operands straight from the accumulators.
+               dS is written to ds (B, n_head, T, T) for the product dQ = dS K that follows (a plain
+               lower-triangular product); query tiles above the diagonal inside the block's aligned group of
+               256 are written as zeros, because that product reads whole tiles along the diagonal.
+    Against the chain: 7 tile products per (query tile, key tile) pair instead of 6, and two passes over
+    one T x T tensor per head instead of eleven over four; the sums are added in another order (2e-6 of the
+    largest entry against float64)."""
+    assert stage in ("fwd", "delta", "bwd") and DP in (32, 64) and blocks_per_cu in (1, 2)
+    name = f"attention_flash_{stage}" + (f"_d{DP}" if stage != "delta" else "") + ("_o2" if blocks_per_cu == 2 else "")
+    bounds = "256, 2" if blocks_per_cu == 2 else "256"           # "256, 2": registers held to what lets two blocks share a CU
+    NB, ND, LP = DP // 8, DP // 32, DP + 4          # groups of 8 columns, 32-column tiles, LDS row pitch
+    if stage == "delta":
+        src = f"""{PRELUDE}
+extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict__ dy, const float* __restrict__ y,
+        float* __restrict__ delta, u32 rows, u32 T, u32 d, u32 y_pitch, u32 n_head) {{
+    // sixteen lanes per (sequence, position, head): 16-byte items 0 .. 15 of the head's row
+    const u32 item = blockIdx.x * 16u + (threadIdx.x >> 4), sub = threadIdx.x & 15u;
+    float part = 0.0f;
+    const bool live = item < rows;
+    const u32 hd = live ? item % n_head : 0u, bt = live ? item / n_head : 0u;     // bt = b * T + t
+    if (live && 4u * sub < d) {{
+        const u64 at = (u64)bt * y_pitch + (u64)hd * d + 4u * sub;
+        const float4 g = *reinterpret_cast<const float4*>(dy + at), o = *reinterpret_cast<const float4*>(y + at);
+        part = (g.x * o.x + g.y * o.y) + (g.z * o.z + g.w * o.w);
+    }}
+    part += dpp_f<DPP_XOR1>(part);
+    part += dpp_f<DPP_XOR2>(part);
+    part += dpp_f<DPP_HALF_MIRROR>(part);
+    part += dpp_f<DPP_MIRROR>(part);
+    if (live && sub == 0u) delta[((u64)(bt / T) * n_head + hd) * T + bt % T] = part;
+}}
+"""
+        return src, name, _fmt("P", "P", "P", "I", "I", "I", "I", "I")
+    common = f"""
+typedef float f16v __attribute__((ext_vector_type(16)));
+#define DP {DP}u
+#define NB {NB}u
+#define ND {ND}u
+#define LP {LP}u
+#define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0)
+#define ROW_OF(e, h) (8u * ((e) >> 2) + 4u * (h) + ((e) & 3u))
+// e^x for x <= 0 as one multiplication and the hardware's 2^x (1 ulp): its argument is off by at most |x| 2^-24 log2(e), so a
+// probability e^x is off by that fraction of itself -- 2e-6 of 4e-9 at x = -20, one rounding at x = 0
+static __device__ __forceinline__ float exp_neg(float x) {{ return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }}
+// 16-byte item `it` of rows [row0, ..) of a head: row row0 + it / (DP / 4), columns 4 (it % (DP / 4)) ..; zeros outside [0, T) x [0, d)
+static __device__ __forceinline__ float4 head_item(const float* __restrict__ src, u32 it, u32 row0, u32 T, u32 d, u32 pitch) {{
+    const u32 row = row0 + it / (DP / 4u), c4 = (it % (DP / 4u)) << 2;
+    return (row < T && c4 < d) ? *reinterpret_cast<const float4*>(src + (u64)row * pitch + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
+}}
+static __device__ __forceinline__ void put_item(float* __restrict__ tile, u32 it, const float4 v) {{
+    *reinterpret_cast<float4*>(tile + (it / (DP / 4u)) * LP + ((it % (DP / 4u)) << 2)) = v;
+}}
+// the rows a lane holds as B operand: row `row` of a head, columns 8 blk + 4 h .. + 3 for blk = 0 .. NB - 1
+static __device__ __forceinline__ void own_row(float4 (&reg)[{NB}], const float* __restrict__ src, u32 row, u32 h, u32 T, u32 d, u32 pitch) {{
+    #pragma unroll
+    for (u32 blk = 0; blk < NB; ++blk) {{
+        const u32 c4 = 8u * blk + 4u * h;
+        reg[blk] = (row < T && c4 < d) ? *reinterpret_cast<const float4*>(src + (u64)row * pitch + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }}
+}}
+// acc += X Y^T for the 32 rows of X at `xs` (LDS, [row][LP]) and the 32 rows of Y that the lanes hold in `reg`
+static __device__ __forceinline__ void rows_times_own(f16v& acc, const float* __restrict__ xs, const float4 (&reg)[{NB}], u32 r, u32 h) {{
+    #pragma unroll
+    for (u32 blk = 0; blk < NB; ++blk) {{
+        const float4 a = *reinterpret_cast<const float4*>(xs + r * LP + 8u * blk + 4u * h);
+        acc = MFMA(a.x, reg[blk].x, acc); acc = MFMA(a.y, reg[blk].y, acc);
+        acc = MFMA(a.z, reg[blk].z, acc); acc = MFMA(a.w, reg[blk].w, acc);
+    }}
+}}
+// acc (32 columns c0 .. of X^T, by the lanes' 32 columns) += X^T B, for the 32 rows of X at `xs` and B = the tile a lane holds in `b`
+static __device__ __forceinline__ void cols_times_tile(f16v& acc, const float* __restrict__ xs, u32 c0, const f16v& b, u32 r, u32 h) {{
+    #pragma unroll
+    for (u32 st = 0; st < 16u; ++st) acc = MFMA(xs[ROW_OF(st, h) * LP + c0 + r], b[st], acc);
+}}
+"""
+    if stage == "fwd":
+        body = f"""
+extern "C" __global__ __launch_bounds__({bounds}) void {name}(const float* __restrict__ q, const float* __restrict__ k,
+        const float* __restrict__ v, float* __restrict__ y, float* __restrict__ lse,
+        u32 T, u32 d, u32 pitch, u32 y_pitch, u32 n_head, u32 nq, float scale) {{
+    __shared__ __attribute__((aligned(16))) float Ks[2][64u * LP], Vs[2][64u * LP];
+    // the query tiles with the most keys first
+    const u32 bh = blockIdx.x % (gridDim.x / nq), qi = nq - 1u - blockIdx.x / (gridDim.x / nq), b = bh / n_head, hd = bh % n_head;
+    const u32 t = threadIdx.x, w = t >> 6, lane = t & 63u, r = lane & 31u, h = lane >> 5;
+    const u64 in_off = (u64)b * T * pitch + (u64)hd * d;
+    const u32 q0 = 128u * qi + 32u * w, query = q0 + r;                  // this wavefront's queries; this lane's
+    const u32 n_kv = (min(T, 128u * qi + 128u) + 63u) / 64u;             // key tiles at or below the block's last query
+    float4 qreg[{NB}];
+    own_row(qreg, q + in_off, query, h, T, d, pitch);
+    f16v o[{ND}];
+    #pragma unroll
+    for (u32 dt = 0; dt < ND; ++dt) {{ _Pragma("unroll") for (int z = 0; z < 16; ++z) o[dt][z] = 0.0f; }}
+    float m_run = -__builtin_inff(), l_run = 0.0f;
+    constexpr u32 NI = 64u * (DP / 4u) / 256u;                           // 16-byte items per thread and tile
+    float4 kn[NI], vn[NI];
+    auto fetch = [&](u32 j) {{
+        #pragma unroll
+        for (u32 n = 0; n < NI; ++n) {{
+            kn[n] = head_item(k + in_off, t + 256u * n, 64u * j, T, d, pitch);
+            vn[n] = head_item(v + in_off, t + 256u * n, 64u * j, T, d, pitch);
+        }}
+    }};
+    auto stash = [&](u32 buf) {{
+        #pragma unroll
+        for (u32 n = 0; n < NI; ++n) {{ put_item(Ks[buf], t + 256u * n, kn[n]); put_item(Vs[buf], t + 256u * n, vn[n]); }}
+    }};
+    fetch(0u);
+    stash(0u);
+    __syncthreads();
+    for (u32 j = 0; j < n_kv; ++j) {{
+        const u32 buf = j & 1u, kv0 = 64u * j;
+        if (j + 1u < n_kv) fetch(j + 1u);
+        if (kv0 <= q0 + 31u) {{                                          // some key of the tile is visible to some query of the wavefront
+            f16v s[2];
+            #pragma unroll
+            for (u32 kt = 0; kt < 2u; ++kt) {{
+                _Pragma("unroll") for (int z = 0; z < 16; ++z) s[kt][z] = 0.0f;
+                rows_times_own(s[kt], Ks[buf] + 32u * kt * LP, qreg, r, h);          // S^T: keys by queries
+            }}
+            const bool diagonal = kv0 + 63u > q0;                        // some key of the tile lies beyond some query
+            float mx = -__builtin_inff();
+            #pragma unroll
+            for (u32 kt = 0; kt < 2u; ++kt)
+                #pragma unroll
+                for (u32 e = 0; e < 16u; ++e) {{
+                    float x = s[kt][e] * scale;
+                    if (diagonal && kv0 + 32u * kt + ROW_OF(e, h) > query) x = -__builtin_inff();
+                    s[kt][e] = x;
+                    mx = fmaxf(mx, x);
+                }}
+            mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+            const float m_new = fmaxf(m_run, mx);                        // finite: key 0 is visible to every query
+            const float alpha = exp_neg(m_run - m_new);
+            float part = 0.0f;
+            #pragma unroll
+            for (u32 kt = 0; kt < 2u; ++kt)
+                #pragma unroll
+                for (u32 e = 0; e < 16u; ++e) {{ const float pe = exp_neg(s[kt][e] - m_new); s[kt][e] = pe; part += pe; }}
+            l_run = l_run * alpha + part;
+            m_run = m_new;
+            #pragma unroll
+            for (u32 dt = 0; dt < ND; ++dt) {{
+                _Pragma("unroll") for (int z = 0; z < 16; ++z) o[dt][z] *= alpha;
+                #pragma unroll
+                for (u32 kt = 0; kt < 2u; ++kt) cols_times_tile(o[dt], Vs[buf] + 32u * kt * LP, 32u * dt, s[kt], r, h);    // O^T += V^T P^T
+            }}
+        }}
+        if (j + 1u < n_kv) stash(buf ^ 1u);
+        __syncthreads();
+    }}
+    const float l = l_run + __shfl_xor(l_run, 32, WAVE);
+    if (query < T) {{
+        if (h == 0u) lse[(u64)bh * T + query] = m_run + logf(l);
+        float* __restrict__ yrow = y + (u64)b * T * y_pitch + (u64)query * y_pitch + (u64)hd * d;
+        #pragma unroll
+        for (u32 dt = 0; dt < ND; ++dt)
+            #pragma unroll
+            for (u32 g = 0; g < 4u; ++g) {{
+                const u32 col = 32u * dt + 8u * g + 4u * h;
+                if (col < d) *reinterpret_cast<float4*>(yrow + col) =
+                    make_float4(o[dt][4u * g] / l, o[dt][4u * g + 1u] / l, o[dt][4u * g + 2u] / l, o[dt][4u * g + 3u] / l);
+            }}
+    }}
+}}
+"""
+        fmt = _fmt("P", "P", "P", "P", "P", "I", "I", "I", "I", "I", "I", "f")
+    else:
+        body = f"""
+extern "C" __global__ __launch_bounds__({bounds}) void {name}(const float* __restrict__ q, const float* __restrict__ k,
+        const float* __restrict__ v, const float* __restrict__ dy, const float* __restrict__ lse, const float* __restrict__ delta,
+        float* __restrict__ ds, float* __restrict__ dk, float* __restrict__ dv,
+        u32 T, u32 d, u32 pitch, u32 y_pitch, u32 g_pitch, u32 n_head, u32 nk, float scale) {{
+    __shared__ __attribute__((aligned(16))) float Qs[2][64u * LP], Gs[2][64u * LP], Ls[2][64], Ds[2][64];
+    // the key tiles with the most queries first
+    const u32 bh = blockIdx.x % (gridDim.x / nk), ki = blockIdx.x / (gridDim.x / nk), b = bh / n_head, hd = bh % n_head;
+    const u32 t = threadIdx.x, w = t >> 6, lane = t & 63u, r = lane & 31u, h = lane >> 5;
+    const u64 in_off = (u64)b * T * pitch + (u64)hd * d, y_off = (u64)b * T * y_pitch + (u64)hd * d;
+    const u32 k0 = 128u * ki + 32u * w, key = k0 + r;                    // this wavefront's keys; this lane's
+    const u32 j0 = (128u * ki / 256u) * 4u, nq = (T + 63u) / 64u;         // query tiles from the start of the aligned group of 256
+    float4 kreg[{NB}], vreg[{NB}];
+    own_row(kreg, k + in_off, key, h, T, d, pitch);
+    own_row(vreg, v + in_off, key, h, T, d, pitch);
+    f16v gk[{ND}], gv[{ND}];
+    #pragma unroll
+    for (u32 dt = 0; dt < ND; ++dt) {{ _Pragma("unroll") for (int z = 0; z < 16; ++z) {{ gk[dt][z] = 0.0f; gv[dt][z] = 0.0f; }} }}
+    constexpr u32 NI = 64u * (DP / 4u) / 256u;
+    float4 qn[NI], gn[NI];
+    float ln = 0.0f, dn = 0.0f;
+    const float* __restrict__ lrow = lse + (u64)bh * T;
+    const float* __restrict__ drow = delta + (u64)bh * T;
+    float* __restrict__ dsout = ds + (u64)bh * T * T;
+    auto fetch = [&](u32 j) {{
+        #pragma unroll
+        for (u32 n = 0; n < NI; ++n) {{
+            qn[n] = head_item(q + in_off, t + 256u * n, 64u * j, T, d, pitch);
+            gn[n] = head_item(dy + y_off, t + 256u * n, 64u * j, T, d, y_pitch);
+        }}
+        if (t < 64u) {{ const u32 row = 64u * j + t; ln = row < T ? lrow[row] : __builtin_inff(); dn = row < T ? drow[row] : 0.0f; }}
+    }};
+    auto stash = [&](u32 buf) {{
+        #pragma unroll
+        for (u32 n = 0; n < NI; ++n) {{ put_item(Qs[buf], t + 256u * n, qn[n]); put_item(Gs[buf], t + 256u * n, gn[n]); }}
+        if (t < 64u) {{ Ls[buf][t] = ln; Ds[buf][t] = dn; }}
+    }};
+    fetch(j0);
+    stash(0u);
+    __syncthreads();
+    for (u32 j = j0; j < nq; ++j) {{
+        const u32 buf = (j - j0) & 1u, qt0 = 64u * j;
+        if (j + 1u < nq) fetch(j + 1u);
+        #pragma unroll
+        for (u32 qt = 0; qt < 2u; ++qt) {{
+            const u32 row0 = qt0 + 32u * qt;                             // first query of this 32 x 32 tile
+            f16v p, dsv;
+            _Pragma("unroll") for (int z = 0; z < 16; ++z) {{ p[z] = 0.0f; dsv[z] = 0.0f; }}
+            const bool live = row0 + 31u >= k0;                           // some query of the tile sees some key of the wavefront
+            if (live) {{
+                rows_times_own(p, Qs[buf] + 32u * qt * LP, kreg, r, h);              // S: queries by keys
+                rows_times_own(dsv, Gs[buf] + 32u * qt * LP, vreg, r, h);            // dP = dy V^T
+                #pragma unroll
+                for (u32 e = 0; e < 16u; ++e) {{
+                    const u32 lr = 32u * qt + ROW_OF(e, h);
+                    const float pe = (key > qt0 + lr) ? 0.0f : exp_neg(p[e] * scale - Ls[buf][lr]);     // (rows beyond T: lse = +inf)
+                    p[e] = pe;
+                    dsv[e] = (pe * (dsv[e] - Ds[buf][lr])) * scale;
+                }}
+                #pragma unroll
+                for (u32 dt = 0; dt < ND; ++dt) {{
+                    cols_times_tile(gv[dt], Gs[buf] + 32u * qt * LP, 32u * dt, p, r, h);       // dV^T += dy^T P
+                    cols_times_tile(gk[dt], Qs[buf] + 32u * qt * LP, 32u * dt, dsv, r, h);     // dK^T += Q^T dS
+                }}
+            }}
+            if (key < T) {{
+                #pragma unroll
+                for (u32 e = 0; e < 16u; ++e) {{
+                    const u32 row = row0 + ROW_OF(e, h);
+                    if (row < T) dsout[(u64)row * T + key] = dsv[e];
+                }}
+            }}
+        }}
+        if (j + 1u < nq) stash(buf ^ 1u);
+        __syncthreads();
+    }}
+    if (key < T) {{
+        const u64 g_off = (u64)b * T * g_pitch + (u64)key * g_pitch + (u64)hd * d;
+        #pragma unroll
+        for (u32 dt = 0; dt < ND; ++dt)
+            #pragma unroll
+            for (u32 g = 0; g < 4u; ++g) {{
+                const u32 col = 32u * dt + 8u * g + 4u * h;
+                if (col < d) {{
+                    *reinterpret_cast<float4*>(dk + g_off + col) = make_float4(gk[dt][4u * g], gk[dt][4u * g + 1u], gk[dt][4u * g + 2u], gk[dt][4u * g + 3u]);
+                    *reinterpret_cast<float4*>(dv + g_off + col) = make_float4(gv[dt][4u * g], gv[dt][4u * g + 1u], gv[dt][4u * g + 2u], gv[dt][4u * g + 3u]);
+                }}
+            }}
+    }}
+}}
+"""
+        fmt = _fmt("P", "P", "P", "P", "P", "P", "P", "P", "P", "I", "I", "I", "I", "I", "I", "I", "f")
+    return f"{PRELUDE}{common}{body}", name, fmt
+
+
 @cache
 def adam_multi_inplace_kernel() -> tuple[str, str, str]:
     """adam_inplace_kernel for a whole parameter list in one launch.  `ptrs` holds four rows of

@@ -1624,6 +1624,10 @@ class HIP:
     NORM_IN_PRODUCT = os.environ.get("DLGRAD_HIP_NORM_IN_PRODUCT", "1")
     CAUSAL_MASK_KNOWN = os.environ.get("DLGRAD_HIP_CAUSAL_MASK_KNOWN", "1") != "0"   # "0": the cached causal mask is read like any other mask
     CE_GRAD_ROWS = os.environ.get("DLGRAD_HIP_CE_GRAD_ROWS", "1") != "0"       # "0": the cross-entropy gradient as an element-wise launch
+    # registers of the streaming attention backward held to 256 so that two blocks share a CU (312 and one block otherwise):
+    # 392 -> 334 us per layer at (8, 12, 1024, 64)
+    FLASH_BWD_BLOCKS_PER_CU = int(os.environ.get("DLGRAD_HIP_FLASH_BWD_BLOCKS_PER_CU", "2"))
+    ATTENTION_FLASH = os.environ.get("DLGRAD_HIP_ATTENTION_FLASH", "1") != "0"   # "0": long causal attention as products and softmax launches over stored T x T tensors
     ATTENTION_FUSED = os.environ.get("DLGRAD_HIP_ATTENTION_FUSED", "1") != "0"   # "0": short causal attention as products and softmax launches too
 
     # ---- matmul ----------------------------------------------------------------------------------------------------------
@@ -2115,12 +2119,14 @@ class HIP:
 
     @staticmethod
     def _gemm_strided(A: tuple, B: tuple, C: tuple, M: int, N: int, Kd: int, B0: int, B1: int,
-                      ta: bool = False, tb: bool = False, tri: str = "") -> None:
+                      ta: bool = False, tb: bool = False, tri: str = "", rows_group: int = 0) -> None:
         """C[b0, b1] = op(A[b0, b1]) . op(B[b0, b1]) for matrices cut out of larger tensors: every
         operand is (address, row pitch, stride of b0, stride of b1) in floats.  Same kernel, same
-        order of additions as the contiguous product of the same logical matrices."""
+        order of additions as the contiguous product of the same logical matrices.
+        rows_group: with tri, the structured operand holds defined values only inside aligned groups of that
+        many rows along the diagonal, so the tile's rows must divide it."""
         (aa, lda, sa0, sa1), (ba, ldb, sb0, sb1), (ca, ldc, sc0, sc1) = A, B, C
-        key = (A[1:], B[1:], C[1:], M, N, Kd, B0, B1, ta, tb, tri, aa & 15, ba & 15, ca & 15, HIP.MATMUL_FORCE)
+        key = (A[1:], B[1:], C[1:], M, N, Kd, B0, B1, ta, tb, tri, aa & 15, ba & 15, ca & 15, HIP.MATMUL_FORCE, rows_group)
         plan = _gemm_plans.get(key)
         if plan is not None:
             k, grid, threads, tail = plan
@@ -2134,6 +2140,8 @@ class HIP:
         args = (aa, ba, ca, M, N, Kd, B1, sa0, sa1, sb0, sb1, lda, ldb, ldc, sc0, sc1)
         batch = B0 * B1
         tile = HIP._pick_tile(M, N, Kd, batch, veca, vecb, args, ta, tb, tri, True)
+        if rows_group and rows_group % K.matmul_tile_shape(tile)[0]:
+            tile = "64x64k64"                                  # the caller's operand is only defined in aligned groups of rows_group rows
         HIP._launch_matmul(tile, veca, vecb, M, N, batch, args, ta, tb, tri, True)
         if not capturing():
             _gemm_plans[key] = (*HIP._matmul_kernel(tile, veca, vecb, M, N, batch, ta, tb, tri, True), args[3:])
@@ -2151,11 +2159,18 @@ class HIP:
                 and 0 < heads < 2 ** 29 and not any(a & 15 for a in read_addrs) and not any(q & 3 for q in read_pitches))
 
     @staticmethod
+    def _flash_fits(T: int, d: int, heads: int, addrs: tuple, pitches: tuple) -> bool:
+        """Whether the streaming attention kernels take the case (any T; heads of up to 64 columns, 16-byte accesses)."""
+        return (HIP.ATTENTION_FLASH and T > 0 and 0 < d <= K.ATTN_FLASH_D and d % 4 == 0 and T < 2 ** 20
+                and 0 < heads * ((T + 127) // 128) < 2 ** 31 and not any(a & 15 for a in addrs) and not any(q & 3 for q in pitches))
+
+    @staticmethod
     def _attend(qa: int, ka: int, va: int, pitch: int, ya: int, y_pitch: int, Bn: int, T: int, n_head: int, d: int,
                 scale: float) -> DevicePtr:
         """Causal attention over heads that lie at addresses qa, ka, va with row pitch `pitch` (batch
-        stride T * pitch, head stride d); the context goes to ya with pitch y_pitch.  Returns the
-        probabilities (Bn, n_head, T, T)."""
+        stride T * pitch, head stride d); the context goes to ya with pitch y_pitch.  Returns what the
+        backward pass needs besides its inputs: the probabilities (Bn, n_head, T, T), or -- from the
+        streaming kernels, which never store them -- the log-sum-exp of every score row (Bn, n_head, T)."""
         from dlgrad_amd.ops import causal_mask
         if HIP._attention_fits(T, d, Bn * n_head, (qa, ka, va), (pitch,)):
             # one block per (sequence, head, 32 rows): scores, softmax and context without leaving the chip
@@ -2164,6 +2179,13 @@ class HIP:
             launch(kernel(K.attention_small_kernel, "fwd"), Bn * n_head * nt, 512, qa, ka, va, ya, p.addr, T, d, pitch, y_pitch,
                    n_head, nt, float(scale))
             return p
+        if HIP._flash_fits(T, d, Bn * n_head, (qa, ka, va, ya), (pitch, y_pitch)):
+            # one block per (sequence, head, 128 queries): keys and values stream past, online softmax, no T x T tensor
+            lse = alloc(Bn * n_head * T)
+            nq = (T + 127) // 128
+            launch(kernel(K.attention_flash_kernel, "fwd", 32 if d <= 32 else 64), Bn * n_head * nq, 256, qa, ka, va, ya, lse.addr,
+                   T, d, pitch, y_pitch, n_head, nq, float(scale))
+            return lse
         raw = alloc(Bn * n_head * T * T)
         dense = lambda addr: (addr, T, n_head * T * T, T * T)                       # noqa: E731
         HIP._gemm_strided(HIP._heads(qa, T, pitch, d), HIP._heads(ka, T, pitch, d), dense(raw.addr), T, T, d, Bn, n_head,
@@ -2183,6 +2205,20 @@ class HIP:
             nt = (T + 31) // 32
             launch(kernel(K.attention_small_kernel, "bwd"), Bn * n_head * nt, 512, qa, ka, va, _addr(p), ya, dya, dqa, dka, dva,
                    T, d, pitch, dy_pitch, g_pitch, n_head, nt, float(scale))
+            return
+        if p.numel == Bn * n_head * T and (T > 1 or HIP._flash_fits(T, d, Bn * n_head, (qa, ka, va), (pitch,))):
+            # p is the log-sum-exp per score row (the streaming forward): probabilities are recomputed tile by tile
+            if ya is None or not HIP._flash_fits(T, d, Bn * n_head, (qa, ka, va, dya, ya, dka, dva), (pitch, dy_pitch, g_pitch)):
+                raise ValueError("the streaming attention backward needs the forward context and 16-byte aligned heads")
+            delta = alloc(Bn * n_head * T)
+            rows = Bn * T * n_head
+            launch(kernel(K.attention_flash_kernel, "delta", 32), (rows + 15) // 16, 256, dya, ya, delta.addr, rows, T, d, dy_pitch, n_head)
+            ds = alloc(Bn * n_head * T * T)
+            nk = (T + 127) // 128
+            launch(kernel(K.attention_flash_kernel, "bwd", 32 if d <= 32 else 64, HIP.FLASH_BWD_BLOCKS_PER_CU), Bn * n_head * nk, 256, qa, ka, va, dya, _addr(p),
+                   delta.addr, ds.addr, dka, dva, T, d, pitch, dy_pitch, g_pitch, n_head, nk, float(scale))
+            HIP._gemm_strided((ds.addr, T, n_head * T * T, T * T), HIP._heads(ka, T, pitch, d), HIP._heads(dqa, T, g_pitch, d),
+                              T, d, T, Bn, n_head, tri="a_lower", rows_group=256)
             return
         dense = lambda addr: (addr, T, n_head * T * T, T * T)                       # noqa: E731
         dp = alloc(p.numel)

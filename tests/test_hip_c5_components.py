@@ -301,7 +301,8 @@ def test_attention_on_the_projections_equals_split_attend_merge(B, T, h, d, monk
     transpose -> reshape, including head sizes that force 4-byte accesses."""
     require_gpu()
     from dlgrad_amd import nn, ops
-    monkeypatch.setattr(hip.HIP, "ATTENTION_FUSED", False)       # the one-launch kernels for short sequences add in another order
+    monkeypatch.setattr(hip.HIP, "ATTENTION_FUSED", False)       # the one-launch kernels for short sequences add in another order,
+    monkeypatch.setattr(hip.HIP, "ATTENTION_FLASH", False)       # and so do the streaming kernels for long ones
     rng = np.random.default_rng(72)
     C = h * d
     q, k, v, g = (rng.standard_normal((B, T, C), dtype=np.float32) for _ in range(4))
@@ -392,6 +393,72 @@ def test_short_attention_in_one_launch_per_pass(B, T, h, d, stacked, monkeypatch
         return
     assert p.shape == (B, h, T, T) and not np.triu(p, 1).any() and np.isfinite(p).all()
     assert np.abs(p.sum(-1, dtype=np.float64) - 1).max() <= 1e-5
+    for name, a, w, c in zip(("y", "dq", "dk", "dv"), got, want, chain):
+        assert np.isfinite(a).all(), name
+        bound = 2e-6 * max(1.0, np.abs(w).max())
+        assert np.abs(a - w).max() <= bound, f"{name}: {np.abs(a - w).max():.3g} > {bound:.3g}"
+        assert np.abs(c - w).max() <= bound, f"chain {name}"
+
+
+@pytest.mark.parametrize("B,T,h,d", [(1, 1024, 12, 64), (2, 257, 1, 64), (3, 100, 2, 20), (2, 384, 3, 48), (1, 130, 2, 32), (2, 129, 5, 4),
+                                     (1, 640, 2, 64), (1, 1, 2, 64), (1, 777, 1, 36)])
+@pytest.mark.parametrize("stacked", [False, True])
+def test_streaming_attention_against_float64(B, T, h, d, stacked, monkeypatch):
+    """Sequences beyond the one-launch kernels (or heads wider than 32): keys and values stream past
+    128 queries per block with an online softmax, and the backward pass recomputes the probabilities
+    from the kept log-sum-exp per row -- no T x T tensor is kept, the forward is one launch, the backward a
+    row-sum launch, the key-side launch that also writes dS, and the product dQ = dS K.  Context and all
+    three gradients against float64 at 2e-6 of the largest entry, for ragged T and head widths that are
+    padded on the chip, from separate (B, T, C) projections and from one interleaved (B, T, 3C) one, with
+    free memory full of NaN (nothing unwritten is read); the kept statistics against float64 too.  The chain
+    of products and softmax launches over stored T x T tensors (DLGRAD_HIP_ATTENTION_FLASH=0) meets the
+    same bound; the two add in different orders, so their bits are not compared."""
+    require_gpu()
+    from dlgrad_amd.buffer import Buffer
+    from dlgrad_amd.device import Device
+    monkeypatch.setattr(hip.HIP, "ATTENTION_FUSED", False)               # (shapes the one-launch kernels would take go to the streaming ones)
+    rng = np.random.default_rng(75 + T)
+    C = h * d
+    q, k, v, g = (rng.standard_normal((B, T, C), dtype=np.float32) for _ in range(4))
+    scale = d ** -0.5
+    want = None if hip.COMPILE_ONLY else attention_float64(q, k, v, g, h, scale)
+    poison = [Buffer.from_numpy(np.full(n, np.nan, np.float32), Device.HIP) for n in (B * h * T * T, 3 * B * T * C, B * T * C, B * h * T)]
+    hip.lib().sync()
+    del poison
+
+    def run():
+        if stacked:
+            qkv = Buffer.from_numpy(np.ascontiguousarray(np.concatenate([q, k, v], axis=2)), Device.HIP)
+            before = hip.launch_count
+            y, p = qkv.causal_attention_qkv(h, scale)
+            dg = qkv.causal_attention_qkv_bwd(p, Buffer.from_numpy(g, Device.HIP), h, scale, y)
+            launches = hip.launch_count - before
+            if hip.COMPILE_ONLY:
+                return launches, None, None
+            dg = dg.numpy()
+            return launches, [y.numpy(), dg[:, :, :C], dg[:, :, C:2 * C], dg[:, :, 2 * C:]], p.numpy()
+        bufs = [Buffer.from_numpy(a, Device.HIP) for a in (q, k, v, g)]
+        before = hip.launch_count
+        y, p = bufs[0].causal_attention(bufs[1], bufs[2], h, scale)
+        grads = bufs[0].causal_attention_bwd(bufs[1], bufs[2], p, bufs[3], h, scale, y)
+        launches = hip.launch_count - before
+        if hip.COMPILE_ONLY:
+            return launches, None, None
+        return launches, [y.numpy()] + [a.numpy() for a in grads], p.numpy()
+
+    launches, got, lse = run()
+    assert launches == 4, launches
+    monkeypatch.setattr(hip.HIP, "ATTENTION_FLASH", False)
+    chain_launches, chain, p = run()
+    assert chain_launches > 4
+    if hip.COMPILE_ONLY:
+        return
+    assert lse.size == B * h * T and (lse.shape == (B, h, T) or T == 1) and p.shape == (B, h, T, T)    # (for T = 1 the two shapes hold as many numbers)
+    lse = lse.reshape(B, h, T)
+    s64 = np.einsum("bthd,bshd->bhts", q.reshape(B, T, h, d).astype(np.float64), k.reshape(B, T, h, d).astype(np.float64)) * scale
+    s64 = np.where(np.tril(np.ones((T, T), bool)), s64, -np.inf)
+    want_lse = np.log(np.exp(s64 - s64.max(-1, keepdims=True)).sum(-1)) + s64.max(-1)
+    assert np.abs(lse - want_lse).max() <= 2e-6 * max(1.0, np.abs(want_lse).max())
     for name, a, w, c in zip(("y", "dq", "dk", "dv"), got, want, chain):
         assert np.isfinite(a).all(), name
         bound = 2e-6 * max(1.0, np.abs(w).max())
