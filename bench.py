@@ -293,7 +293,8 @@ def run_c5(steps: int, warmup: int) -> dict:
             ("embedding_scatter_add", lambda: table.embedding(idx, backward=True, upstream_grad=g),
              4 * V * W + 4 * n * W + 4 * n),
             ("softmax_98304x1024", lambda: att.softmax(1), 8 * att.numel),
-            # items above the diagonal are exact zeros and are not read: half of each input row moves
+            # items above the diagonal are exact zeros and are not read: half of each input row moves; the mask is the cached causal
+            # mask, whose bits the kernel computes from the indices instead of reading them (6 and 8 B per element, not 8 and 12)
             ("scaled_causal_softmax_(8,12,1024,1024)", lambda: att4.masked_softmax(causal, 0.125), 6 * att.numel),
             ("scaled_causal_softmax_backward", lambda: probs.masked_softmax_bwd(att4, causal, 0.125), 8 * att.numel),
             # forward: one read of the logits, (max, log-sum) and the picked log-prob per row; backward: logits in, gradient out
@@ -473,7 +474,7 @@ def run_gpt_large(steps: int = 2) -> dict:
     lib.sync()
     t_inf = time.perf_counter() - t0
     del logits
-    times, loss = [], None
+    times, loss, first_loss = [], None, None
     for _ in range(steps + 1):
         t0 = time.perf_counter()
         opt.zero_grad()
@@ -482,6 +483,8 @@ def run_gpt_large(steps: int = 2) -> dict:
         opt.step()
         lib.sync()
         times.append(time.perf_counter() - t0)
+        if first_loss is None:
+            first_loss = float(loss.numpy()) / tokens             # the loss of the seeded weights: what the float64 parity test holds
     n_params = sum(p.numel for p in params)
     in_use, cached, _ = lib.pool_stats()
     step_s = sum(times[1:]) / steps                               # the first step (kernel loading, tile timing) is warm-up
@@ -490,7 +493,9 @@ def run_gpt_large(steps: int = 2) -> dict:
             "train_step_ms": round(step_s * 1e3, 2), "train_tokens_per_s": round(tokens / step_s, 1),
             "train_TFLOPs_est": round(6 * (n_params - c.vocab_size * c.n_embd - c.block_size * c.n_embd) * tokens
                                       / step_s / 1e12, 2),
+            "loss_per_token_first_forward": round(first_loss, 6),
             "loss_per_token": round(float(loss.numpy()) / tokens, 4),
+            "attention": "streaming kernels (no T x T tensor kept)" if hip.HIP.ATTENTION_FLASH else "products and softmax over stored T x T tensors",
             "pool_GiB": round((in_use + cached) / 2 ** 30, 1)}
 
 
@@ -538,7 +543,35 @@ def run_decode(n_tokens: int = 256) -> dict:
                              "tokens_inside_window": GPT_C4["block_size"] - 1,
                              "tokens_by_full_window_steps": n_tokens - GPT_C4["block_size"] + 1,
                              "same_ids_as_full_recompute": ids3 == ids}
+    out["positions"] = ("reference_positions=False: every token at its own position, which makes the cached and the captured steps "
+                        "comparable with full recompute; the library default follows helpers.STRICT_REFERENCE (the reference numbers an "
+                        "incremental token one too high), timed below")
     dec.close()
+    # the same captured steps with the reference's position ids (the strict default), checked against its cache loop
+    strict = G.StaticDecoder(model, reference_positions=True, capacity=n_tokens + 1)
+    if not hip.COMPILE_ONLY:
+        strict.capture()
+    strict.generate(0, 8)
+    hip.lib().sync()
+    t0 = time.perf_counter()
+    ids4 = strict.generate(0, n_tokens)
+    dt = time.perf_counter() - t0
+    out["reference_positions_true"] = {"ms_per_token": round(dt / n_tokens * 1e3, 3), "tokens_per_s": round(n_tokens / dt, 1),
+                                       "same_ids_as_cached_loop": ids4 == model.generate_greedy_cached(0, n_tokens, reference_positions=True)}
+    strict.close()
+    # sampling (temperature 0.7, as the reference's generate_endless): the draw is the last launch of each captured step
+    sampler = G.StaticDecoder(model, reference_positions=False, capacity=n_tokens + 1, temperature=0.7)
+    if not hip.COMPILE_ONLY:
+        sampler.capture()
+    u = np.random.default_rng(8).random(n_tokens + 1).astype(np.float32)
+    sampler.generate(0, 8, u=u)
+    hip.lib().sync()
+    t0 = time.perf_counter()
+    ids5 = sampler.generate(0, n_tokens, u=u)
+    dt = time.perf_counter() - t0
+    out["sampling_temperature_0.7"] = {"ms_per_token": round(dt / n_tokens * 1e3, 3), "tokens_per_s": round(n_tokens / dt, 1),
+                                        "distinct_tokens": len(set(ids5)), "graph_nodes": sampler.graph.nodes if sampler.graph else 0}
+    sampler.close()
     return out
 
 

@@ -89,6 +89,9 @@ _HOST_UNARY = {
 }
 
 
+_frozen: dict = {}      # id(ptr) -> ptr of allocations that the in-place methods refuse to write (Buffer.freeze)
+
+
 class Buffer:
     """shape / numel / stride / ndim / dtype / device / nbytes are attributes of the Buffer itself;
     `metadata` (the reference keeps them in a separate BufferMetadata object, buffer.py:24-32, and
@@ -530,10 +533,22 @@ class Buffer:
         """In-place Adam update of self, m and v with the constants held in device memory."""
         self._dispatch(CustomOps.ADAM_STEP_INPLACE, p=self, g=g, m=m, v=v, consts=consts)
 
+    def freeze(self) -> "Buffer":
+        """Marks this Buffer's allocation read-only for the in-place methods (upload_, copy_, row_store_,
+        set_values_): for constants that kernels are allowed to recompute instead of reading -- the cached causal
+        mask, whose bits the softmax kernels derive from the indices once they recognise its allocation."""
+        _frozen[id(self.ptr)] = self.ptr                # (the pointer object is kept, so its id cannot be reused)
+        return self
+
+    def _writable(self, what: str) -> None:
+        if id(self.ptr) in _frozen:
+            raise ValueError(f"{what}: this Buffer is a read-only constant (kernels may compute its values instead of reading them)")
+
     def row_store_(self, src: "Buffer", idx: "Buffer", also: "tuple[Buffer, Buffer] | None" = None) -> None:
         """self[(int)idx, :] = src, rows being the leading dim of self; idx is a one-element
         Buffer on the same device, read where the kernel runs.  also = (dst2, src2): the same for a
         second destination of the same shape (one launch on the hip device)."""
+        self._writable("row_store_")
         rows = self.shape[0]
         width = self.numel // max(rows, 1)
         if src.numel != width or idx.numel != 1 or idx.is_host_scalar:
@@ -588,10 +603,12 @@ class Buffer:
     def set_values_(self, values: tuple) -> None:
         """Writes up to eight floats, given by value, into the first elements of this Buffer with a kernel
         launch (hip): nothing is transferred and the host does not wait."""
+        self._writable("set_values_")
         self._dispatch(CustomOps.SET_VALUES, dst=self, values=tuple(values))
 
     def upload_(self, arr: np.ndarray) -> None:
         """Overwrites this Buffer's memory with `arr` (same element count); the address stays."""
+        self._writable("upload_")
         if arr.size != self.numel:
             raise ValueError(f"Buffer size mismatch! Expected {self.numel} elements, got {arr.size}")
         self._dispatch(BufferOps.CREATE, data=arr, into=self)
@@ -599,6 +616,7 @@ class Buffer:
     def copy_(self, src: "Buffer") -> None:
         """Overwrites this Buffer's memory with the elements of `src` (same count, same
         device) without leaving the device; the address stays."""
+        self._writable("copy_")
         if src.numel != self.numel or src.device is not self.device:
             raise ValueError(f"copy_: {src.shape} on {src.device} into {self.shape} on {self.device}")
         self._dispatch(CustomOps.COPY_INTO, dst=self, src=src)
@@ -680,6 +698,15 @@ class Buffer:
 # Sums over a leading dim that the hip runtime can leave pending (see PartialSum)
 PENDING_SUMS = True
 PENDING_SUM_MAX_ROWS = 512          # what one column-sum launch folds; the pending form must mean exactly that launch
+# A pending sum keeps all its parts alive until somebody reads it -- rows times the memory of the value, for every weight of
+# a model until the optimizer step.  Beyond this many bytes of parts held at once, further sums run at once (one launch each,
+# their parts freed) instead of staying pending.
+PENDING_SUM_BUDGET_BYTES = int(__import__("os").environ.get("DLGRAD_HIP_PENDING_SUM_BYTES", str(8 << 30)))
+_pending_bytes = [0]
+
+
+def _pending_release(nbytes: int) -> None:
+    _pending_bytes[0] -= nbytes
 
 
 class PartialSum(Buffer):
@@ -692,7 +719,7 @@ class PartialSum(Buffer):
     the gradient, in the very order the column-sum kernel uses, so the separate launch per weight (a
     quarter of the launches of a char-GPT step) disappears and the bits stay.  Every other reader --
     numpy(), another op, a per-tensor optimizer -- touches `ptr`, which runs the sum then, once."""
-    __slots__ = ("parts", "_sum", "offset", "pitch", "whole")
+    __slots__ = ("parts", "_sum", "offset", "pitch", "whole", "_held")
 
     @staticmethod
     def of(parts: Buffer, shape: tuple) -> Buffer:
@@ -700,11 +727,15 @@ class PartialSum(Buffer):
         sums do not apply (another device, too many rows, nothing to add)."""
         rows = parts.shape[0] if parts.ndim else 0
         if (not PENDING_SUMS or parts.device is not Device.HIP or parts.__class__ is PartialSum or not 1 < rows <= PENDING_SUM_MAX_ROWS
-                or parts.numel != rows * prod_(shape) or parts.numel == 0):
+                or parts.numel != rows * prod_(shape) or parts.numel == 0
+                or _pending_bytes[0] + parts.nbytes > PENDING_SUM_BUDGET_BYTES):
             out = parts.sum(0, keepdim=False)
             return out if out.shape == tuple(shape) else out.reshape(shape)
+        import weakref
         b = _new_buffer(PartialSum)
         b.parts, b._sum, b.offset, b.whole = parts, None, 0, None
+        _pending_bytes[0] += parts.nbytes
+        b._held = weakref.finalize(b, _pending_release, parts.nbytes)      # given back when the sum runs or the object goes
         b.shape, b.dtype, b.device = tuple(shape), parts.dtype, parts.device
         b.numel, b.stride, b.ndim, b.nbytes = _shape_info(b.shape)
         b.pitch = b.numel                                  # floats from one part to the next
@@ -717,7 +748,7 @@ class PartialSum(Buffer):
         if self._sum is not None:
             return Buffer(self._sum + start, shape, self.device)
         b = _new_buffer(PartialSum)
-        b.parts, b._sum, b.offset, b.pitch, b.whole = self.parts, None, self.offset + start, self.pitch, self
+        b.parts, b._sum, b.offset, b.pitch, b.whole, b._held = self.parts, None, self.offset + start, self.pitch, self, None
         b.shape, b.dtype, b.device = tuple(shape), self.dtype, self.device
         b.numel, b.stride, b.ndim, b.nbytes = _shape_info(b.shape)
         return b
@@ -733,9 +764,15 @@ class PartialSum(Buffer):
                 self._sum = self.whole.ptr + (self.offset - self.whole.offset)
             else:
                 self._sum = self.parts.sum(0, keepdim=False).ptr
-            self.parts = None
+            self._drop_parts()
         return self._sum
+
+    def _drop_parts(self) -> None:
+        self.parts = None
+        if self._held is not None:
+            self._held()                                      # (a finalizer runs once: the bytes leave the budget here)
 
     @ptr.setter
     def ptr(self, value) -> None:
-        self._sum, self.parts = value, None
+        self._sum = value
+        self._drop_parts()

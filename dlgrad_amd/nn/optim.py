@@ -41,6 +41,7 @@ class SGD(Optimizer):
         reference's expression, which rebinds `param.data` to a new buffer per update."""
         super().__init__(params, lr)
         self.momentum = momentum
+        self._auto = graph_safe is None       # chosen here: step() follows ops.FUSED if that is switched later
         if graph_safe is None:
             graph_safe = bool(ops.FUSED and params and all(p.device is Device.HIP for p in params))
         self.graph_safe = graph_safe
@@ -60,7 +61,7 @@ class SGD(Optimizer):
             if p.grad is None:
                 continue
             assert p.shape == p.grad.shape, f"The shape of the parameter {p.shape} and its grad {p.grad.shape} do not match"
-            if self.graph_safe:
+            if self.graph_safe and (ops.FUSED or not self._auto):
                 v = self.velocities[id(p)].data if self.momentum != 0 else None
                 p.data.sgd_step_(p.grad.data, v, self.lr, self.momentum)
                 continue
@@ -87,6 +88,7 @@ class Adam(Optimizer):
         self.m = {id(p): Tensor.zeros_like(p) for p in params}
         self.v = {id(p): Tensor.zeros_like(p) for p in params}
         self.t = 0
+        self._auto = graph_safe is None       # chosen here: step() follows ops.FUSED if that is switched later
         if graph_safe is None:
             graph_safe = bool(ops.FUSED and params and all(p.device is Device.HIP for p in params))
         self.graph_safe = graph_safe
@@ -105,7 +107,7 @@ class Adam(Optimizer):
         self.consts.data.set_values_(self._consts())
 
     def step(self) -> None:
-        if self.graph_safe:
+        if self.graph_safe and (ops.FUSED or not self._auto):     # (the default follows the switch: with the fused kernels off, the reference's expressions)
             from dlgrad_amd.runtime import hip
             if not hip.capturing():
                 self.advance()

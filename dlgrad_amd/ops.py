@@ -552,7 +552,7 @@ def causal_mask(T: int, device) -> Buffer:
     key = (T, device)
     if key not in _causal_masks:
         allowed = Buffer.arange((1, T), device) <= Buffer.arange((T, 1), device)
-        _causal_masks[key] = allowed == 0.0
+        _causal_masks[key] = (allowed == 0.0).freeze()      # read-only: the hip softmax kernels compute these bits instead of reading them
     return _causal_masks[key]
 
 

@@ -509,7 +509,23 @@ class _MapPlan:
                            (n + 1023) // 1024, tail, None, None]
 
 
-_map_plans: dict = {}
+PLAN_CACHE_ENTRIES = 8192
+
+
+class _PlanCache(dict):
+    """A launch-plan table that cannot grow without bound: a workload whose shapes change on every call (a decoding
+    loop whose cache grows by a row per token) would otherwise leave an entry per shape for ever.  Lookups are plain
+    dictionary lookups; storing into a full table first drops the older half (insertion order)."""
+    __slots__ = ()
+
+    def __setitem__(self, key, value) -> None:
+        if len(self) >= PLAN_CACHE_ENTRIES and key not in self:
+            for old in list(self)[:PLAN_CACHE_ENTRIES // 2]:
+                del self[old]
+        dict.__setitem__(self, key, value)
+
+
+_map_plans: dict = _PlanCache()
 EMB_ORDERED = os.environ.get("DLGRAD_HIP_EMB_ORDERED", "1") != "0"     # 0: fp32 atomics for every size
 NT_STORE_MIN_ELEMENTS = int(os.environ.get("DLGRAD_HIP_NT_MIN", str(1 << 25)))   # 128 MiB of fp32
 
@@ -552,15 +568,15 @@ def _map(tag: str, expr: str, operands: list[Buffer], out_shape: tuple, svals: t
 
 
 _U64 = (1 << 64) - 1
-_gemm_plans: dict = {}             # the same for products of matrices cut out of larger tensors
-_pair_plans: dict = {}             # the same for two products that travel as one launch
-_matmul_plans: dict = {}           # (shapes, flags, alignment bits) -> (kernel, grid, threads, fixed arguments, ...) of a product seen before
+_gemm_plans: dict = _PlanCache()   # the same for products of matrices cut out of larger tensors
+_pair_plans: dict = _PlanCache()   # the same for two products that travel as one launch
+_matmul_plans: dict = _PlanCache() # (shapes, flags, alignment bits) -> (kernel, grid, threads, fixed arguments, ...) of a product seen before
 # short rows of an even length: "direct" = a thread per row with 8-byte loads straight from memory (7.2 us for
 # 1 000 000 x 10 against 8.1 for "staged", 256 rows per block through LDS, which remains the form for odd lengths)
 ARGMAX_SHORT_ROWS = os.environ.get("DLGRAD_HIP_ARGMAX_SHORT_ROWS", "direct")
 ARGMAX_COL_UNROLL = 8              # rows in flight per thread of the column argmax (8192 x 8192: 50.2 us with 4, 49.5 with 8)
 ARGMAX_COL_BLOCKS = 512            # blocks of 64 x 16 threads the column argmax aims for; more only lengthen the fold
-_permute_plans: dict = {}
+_permute_plans: dict = _PlanCache()
 PERMUTE_DIAG = os.environ.get("DLGRAD_HIP_PERMUTE_DIAG", "1") != "0"     # diagonal tile order for power-of-two pitches
 
 
@@ -759,7 +775,7 @@ class HIP:
     def _binary_entry(op: str):
         """The dispatch-table entry of one binary op: after the first call for a pair of shapes the launch
         plan is found with one dictionary lookup on (shape, shape) and nothing else is recomputed."""
-        expr, plans = K.BINARY_EXPR[op], {}
+        expr, plans = K.BINARY_EXPR[op], _PlanCache()
 
         def run(x: Buffer, y: Buffer) -> DevicePtr:
             xp, yp = x.ptr, y.ptr
@@ -810,7 +826,7 @@ class HIP:
     def _unary_entry(tag: str):
         """The dispatch-table entry of one parameterless unary op: one dictionary lookup on the shape finds the
         launch plan of a call seen before."""
-        expr, plans = K.UNARY_EXPR[tag], {}
+        expr, plans = K.UNARY_EXPR[tag], _PlanCache()
 
         def run(x: Buffer) -> DevicePtr:
             plan = plans.get(x.shape)

@@ -292,6 +292,7 @@ def test_scaled_gpt_step_hip_vs_float64(monkeypatch):
     assert worst_free <= 5e-3                                     # a differing gate moves gradients by ~1e-3 of their scale
 
 
+C5_LOSS_PER_TOKEN = 11.071584      # float64 loss per token of the seeded scaled GPT on its seeded Zipf batch (bench.py: loss_per_token_first_forward)
 C5_FULL = dict(vocab_size=50304, block_size=1024, n_layer=12, n_head=12, n_embd=768, batch_size=8)
 
 
@@ -323,6 +324,7 @@ def test_scaled_gpt_full_depth_forward_hip_vs_float64():
     tokens = cfg["batch_size"] * cfg["block_size"]
     print(f"scaled GPT, 12 layers, batch 8: loss per token {l_hip / tokens:.6f} on hip, {float(l64) / tokens:.6f} in float64")
     assert abs(l_hip - float(l64)) <= 1e-5 * abs(float(l64)), (l_hip, float(l64))
+    assert abs(float(l64) / tokens - C5_LOSS_PER_TOKEN) <= 1e-5 * C5_LOSS_PER_TOKEN     # the figure bench.py prints for these seeds
     assert lg_hip.shape == lg64.shape and np.isfinite(lg_hip).all()
     scale = float(np.abs(lg64).max())
     worst = max(float(np.abs(lg_hip[b] - lg64[b]).max()) for b in range(lg64.shape[0])) / scale     # a batch row at a time
@@ -1151,6 +1153,37 @@ def test_adam_adds_up_pending_gradient_sums_with_the_bits_of_the_column_sum_laun
     if not hip.COMPILE_ONLY:
         for a, b in zip(results[True], results[False]):
             np.testing.assert_array_equal(a, b)
+
+
+@pytest.mark.gpu
+def test_pending_sums_keep_within_their_byte_budget(monkeypatch):
+    """A pending sum keeps its parts alive (rows times the value's memory).  The parts held by all pending sums
+    together are counted: a sum that would take them past the budget runs at once instead, and the count falls
+    back when a pending sum is read, replaced or dropped."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    import gc
+    from dlgrad_amd import buffer as B
+    from dlgrad_amd.device import Device
+    gc.collect()
+    held0 = B._pending_bytes[0]
+    monkeypatch.setattr(B, "PENDING_SUM_BUDGET_BYTES", held0 + 3 * 4 * 8 * 100)        # room for three sets of 8 x 100 floats
+    parts = np.random.default_rng(0).standard_normal((8, 100)).astype(np.float32)
+    sums = [B.PartialSum.of(B.Buffer.from_numpy(parts, Device.HIP), (100,)) for _ in range(5)]
+    assert [s.__class__ is B.PartialSum and s.pending for s in sums] == [True, True, True, False, False]
+    assert B._pending_bytes[0] == held0 + 3 * parts.nbytes
+    if not hip.COMPILE_ONLY:
+        want = B.Buffer.from_numpy(parts, Device.HIP).sum(0).numpy()
+        for s in sums:
+            np.testing.assert_array_equal(s.numpy(), want)          # reading runs the pending ones: same launch, same bits
+        assert B._pending_bytes[0] == held0 and not any(getattr(s, "pending", False) for s in sums)
+    del sums
+    gc.collect()
+    sums = [B.PartialSum.of(B.Buffer.from_numpy(parts, Device.HIP), (100,)) for _ in range(2)]
+    assert B._pending_bytes[0] == held0 + 2 * parts.nbytes
+    del sums
+    gc.collect()
+    assert B._pending_bytes[0] == held0                             # dropped unread: given back as well
 
 
 @pytest.mark.gpu

@@ -306,3 +306,24 @@ def test_dropout_edges_and_tril(device):
     close(a.dropout(0.0).numpy(), a.numpy(), atol=0, rtol=0)
     close(Tensor.tril(a, 0.0).numpy(), np.tril(a.numpy()), atol=0, rtol=0)
     close(Tensor.tril(a, 1.0).numpy(), np.tril(a.numpy(), 1), atol=0, rtol=0)
+
+
+def test_the_cached_causal_mask_is_read_only():
+    """ops.causal_mask hands out one cached (T, T) Buffer per size and device; the hip softmax kernels recognise
+    its allocation and compute its bits from the indices instead of reading them, so writing into it in place
+    would silently change nothing they see: the in-place methods refuse."""
+    import oracle.cpu_runtime  # noqa: F401
+    from dlgrad_amd import ops
+    from dlgrad_amd.buffer import Buffer
+    from dlgrad_amd.device import Device
+    m = ops.causal_mask(5, Device.CPU)
+    np.testing.assert_array_equal(m.numpy(), np.triu(np.ones((5, 5), np.float32), 1))
+    with pytest.raises(ValueError, match="read-only"):
+        m.upload_(np.zeros((5, 5), np.float32))
+    with pytest.raises(ValueError, match="read-only"):
+        m.copy_(Buffer.from_numpy(np.zeros((5, 5), np.float32), Device.CPU))
+    with pytest.raises(ValueError, match="read-only"):
+        m.row_store_(Buffer.from_numpy(np.zeros((5,), np.float32), Device.CPU), Buffer.from_numpy(np.zeros((1,), np.float32), Device.CPU))
+    other = Buffer.from_numpy(np.ones((5, 5), np.float32), Device.CPU)
+    other.upload_(np.zeros((5, 5), np.float32))                   # ordinary buffers are written as before
+    assert not other.numpy().any()
