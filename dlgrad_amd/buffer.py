@@ -705,9 +705,6 @@ PENDING_SUM_BUDGET_BYTES = int(__import__("os").environ.get("DLGRAD_HIP_PENDING_
 _pending_bytes = [0]
 
 
-def _pending_release(nbytes: int) -> None:
-    _pending_bytes[0] -= nbytes
-
 
 class PartialSum(Buffer):
     """A Buffer whose value is `parts.sum(0)` -- the sum over the leading dim of a (rows, *shape)
@@ -731,11 +728,10 @@ class PartialSum(Buffer):
                 or _pending_bytes[0] + parts.nbytes > PENDING_SUM_BUDGET_BYTES):
             out = parts.sum(0, keepdim=False)
             return out if out.shape == tuple(shape) else out.reshape(shape)
-        import weakref
         b = _new_buffer(PartialSum)
         b.parts, b._sum, b.offset, b.whole = parts, None, 0, None
         _pending_bytes[0] += parts.nbytes
-        b._held = weakref.finalize(b, _pending_release, parts.nbytes)      # given back when the sum runs or the object goes
+        b._held = parts.nbytes                             # given back when the sum runs or the object goes (__del__)
         b.shape, b.dtype, b.device = tuple(shape), parts.dtype, parts.device
         b.numel, b.stride, b.ndim, b.nbytes = _shape_info(b.shape)
         b.pitch = b.numel                                  # floats from one part to the next
@@ -748,7 +744,7 @@ class PartialSum(Buffer):
         if self._sum is not None:
             return Buffer(self._sum + start, shape, self.device)
         b = _new_buffer(PartialSum)
-        b.parts, b._sum, b.offset, b.pitch, b.whole, b._held = self.parts, None, self.offset + start, self.pitch, self, None
+        b.parts, b._sum, b.offset, b.pitch, b.whole, b._held = self.parts, None, self.offset + start, self.pitch, self, 0
         b.shape, b.dtype, b.device = tuple(shape), self.dtype, self.device
         b.numel, b.stride, b.ndim, b.nbytes = _shape_info(b.shape)
         return b
@@ -769,8 +765,14 @@ class PartialSum(Buffer):
 
     def _drop_parts(self) -> None:
         self.parts = None
-        if self._held is not None:
-            self._held()                                      # (a finalizer runs once: the bytes leave the budget here)
+        if self._held:
+            _pending_bytes[0] -= self._held                   # the bytes leave the budget here, once
+            self._held = 0
+
+    def __del__(self) -> None:
+        held = getattr(self, "_held", 0)
+        if held:
+            _pending_bytes[0] -= held
 
     @ptr.setter
     def ptr(self, value) -> None:

@@ -3163,7 +3163,9 @@ def attention_flash_kernel(stage: str, DP: int, blocks_per_cu: int = 1) -> tuple
                scores against 32 of the 64 keys (the lane 32 further on holds the other 32), so the running
                maximum and sum of the online softmax are register operations and one exchange.  The
                probabilities exp(s * scale - m) feed O^T += V^T P^T; the accumulator is rescaled by
-               exp(m_old - m_new) per tile and divided by the sum at the end.  Besides the context
+               exp(m_old - m_new) whenever a maximum moved and divided by the sum at the end.  The scores are kept in
+               units of log2 (scale * log2 e is multiplied into the query registers once), so a probability is one
+               subtraction and one hardware 2^x (1 ulp).  Besides the context
                y (B, T, y_pitch) the kernel writes lse = m + log(sum) per (sequence, head, query).
       "delta"  delta = rowsum(dy * y) per (sequence, head, query) (equal to rowsum(dP * P), since y = P v).
       "bwd"    a block per (sequence, head, 128 keys), a wavefront per 32 keys, whose key and value rows it holds
@@ -3210,9 +3212,6 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 #define LP {LP}u
 #define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0)
 #define ROW_OF(e, h) (8u * ((e) >> 2) + 4u * (h) + ((e) & 3u))
-// e^x for x <= 0 as one multiplication and the hardware's 2^x (1 ulp): its argument is off by at most |x| 2^-24 log2(e), so a
-// probability e^x is off by that fraction of itself -- 2e-6 of 4e-9 at x = -20, one rounding at x = 0
-static __device__ __forceinline__ float exp_neg(float x) {{ return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }}
 // 16-byte item `it` of rows [row0, ..) of a head: row row0 + it / (DP / 4), columns 4 (it % (DP / 4)) ..; zeros outside [0, T) x [0, d)
 static __device__ __forceinline__ float4 head_item(const float* __restrict__ src, u32 it, u32 row0, u32 T, u32 d, u32 pitch) {{
     const u32 row = row0 + it / (DP / 4u), c4 = (it % (DP / 4u)) << 2;
@@ -3258,6 +3257,9 @@ extern "C" __global__ __launch_bounds__({bounds}) void {name}(const float* __res
     const u32 n_kv = (min(T, 128u * qi + 128u) + 63u) / 64u;             // key tiles at or below the block's last query
     float4 qreg[{NB}];
     own_row(qreg, q + in_off, query, h, T, d, pitch);
+    const float s2 = scale * 1.44269504088896340736f;                    // scores are kept in units of log2: exp(x) = 2^(x log2 e)
+    #pragma unroll
+    for (u32 blk = 0; blk < NB; ++blk) {{ qreg[blk].x *= s2; qreg[blk].y *= s2; qreg[blk].z *= s2; qreg[blk].w *= s2; }}
     f16v o[{ND}];
     #pragma unroll
     for (u32 dt = 0; dt < ND; ++dt) {{ _Pragma("unroll") for (int z = 0; z < 16; ++z) o[dt][z] = 0.0f; }}
@@ -3288,40 +3290,43 @@ extern "C" __global__ __launch_bounds__({bounds}) void {name}(const float* __res
                 _Pragma("unroll") for (int z = 0; z < 16; ++z) s[kt][z] = 0.0f;
                 rows_times_own(s[kt], Ks[buf] + 32u * kt * LP, qreg, r, h);          // S^T: keys by queries
             }}
-            const bool diagonal = kv0 + 63u > q0;                        // some key of the tile lies beyond some query
+            if (kv0 + 63u > q0) {{                                       // some key of the tile lies beyond some query: the causal mask
+                #pragma unroll
+                for (u32 kt = 0; kt < 2u; ++kt)
+                    #pragma unroll
+                    for (u32 e = 0; e < 16u; ++e) if (kv0 + 32u * kt + ROW_OF(e, h) > query) s[kt][e] = -__builtin_inff();
+            }}
             float mx = -__builtin_inff();
             #pragma unroll
             for (u32 kt = 0; kt < 2u; ++kt)
                 #pragma unroll
-                for (u32 e = 0; e < 16u; ++e) {{
-                    float x = s[kt][e] * scale;
-                    if (diagonal && kv0 + 32u * kt + ROW_OF(e, h) > query) x = -__builtin_inff();
-                    s[kt][e] = x;
-                    mx = fmaxf(mx, x);
-                }}
+                for (u32 e = 0; e < 16u; ++e) mx = fmaxf(mx, s[kt][e]);
             mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
             const float m_new = fmaxf(m_run, mx);                        // finite: key 0 is visible to every query
-            const float alpha = exp_neg(m_run - m_new);
             float part = 0.0f;
             #pragma unroll
             for (u32 kt = 0; kt < 2u; ++kt)
                 #pragma unroll
-                for (u32 e = 0; e < 16u; ++e) {{ const float pe = exp_neg(s[kt][e] - m_new); s[kt][e] = pe; part += pe; }}
-            l_run = l_run * alpha + part;
-            m_run = m_new;
+                for (u32 e = 0; e < 16u; ++e) {{ const float pe = __builtin_amdgcn_exp2f(s[kt][e] - m_new); s[kt][e] = pe; part += pe; }}
+            if (__any(m_new != m_run)) {{                                // (a maximum that stays is the rule after the first few tiles)
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                l_run *= alpha;
+                #pragma unroll
+                for (u32 dt = 0; dt < ND; ++dt) {{ _Pragma("unroll") for (int z = 0; z < 16; ++z) o[dt][z] *= alpha; }}
+                m_run = m_new;
+            }}
+            l_run += part;
             #pragma unroll
-            for (u32 dt = 0; dt < ND; ++dt) {{
-                _Pragma("unroll") for (int z = 0; z < 16; ++z) o[dt][z] *= alpha;
+            for (u32 dt = 0; dt < ND; ++dt)
                 #pragma unroll
                 for (u32 kt = 0; kt < 2u; ++kt) cols_times_tile(o[dt], Vs[buf] + 32u * kt * LP, 32u * dt, s[kt], r, h);    // O^T += V^T P^T
-            }}
         }}
         if (j + 1u < n_kv) stash(buf ^ 1u);
         __syncthreads();
     }}
     const float l = l_run + __shfl_xor(l_run, 32, WAVE);
     if (query < T) {{
-        if (h == 0u) lse[(u64)bh * T + query] = m_run + logf(l);
+        if (h == 0u) lse[(u64)bh * T + query] = (m_run + log2f(l)) * 0.69314718055994530942f;
         float* __restrict__ yrow = y + (u64)b * T * y_pitch + (u64)query * y_pitch + (u64)hd * d;
         #pragma unroll
         for (u32 dt = 0; dt < ND; ++dt)
@@ -3351,6 +3356,9 @@ extern "C" __global__ __launch_bounds__({bounds}) void {name}(const float* __res
     float4 kreg[{NB}], vreg[{NB}];
     own_row(kreg, k + in_off, key, h, T, d, pitch);
     own_row(vreg, v + in_off, key, h, T, d, pitch);
+    const float s2 = scale * 1.44269504088896340736f;                    // scores in units of log2, as in the forward pass
+    #pragma unroll
+    for (u32 blk = 0; blk < NB; ++blk) {{ kreg[blk].x *= s2; kreg[blk].y *= s2; kreg[blk].z *= s2; kreg[blk].w *= s2; }}
     f16v gk[{ND}], gv[{ND}];
     #pragma unroll
     for (u32 dt = 0; dt < ND; ++dt) {{ _Pragma("unroll") for (int z = 0; z < 16; ++z) {{ gk[dt][z] = 0.0f; gv[dt][z] = 0.0f; }} }}
@@ -3366,7 +3374,7 @@ extern "C" __global__ __launch_bounds__({bounds}) void {name}(const float* __res
             qn[n] = head_item(q + in_off, t + 256u * n, 64u * j, T, d, pitch);
             gn[n] = head_item(dy + y_off, t + 256u * n, 64u * j, T, d, y_pitch);
         }}
-        if (t < 64u) {{ const u32 row = 64u * j + t; ln = row < T ? lrow[row] : __builtin_inff(); dn = row < T ? drow[row] : 0.0f; }}
+        if (t < 64u) {{ const u32 row = 64u * j + t; ln = row < T ? lrow[row] * 1.44269504088896340736f : __builtin_inff(); dn = row < T ? drow[row] : 0.0f; }}
     }};
     auto stash = [&](u32 buf) {{
         #pragma unroll
@@ -3391,9 +3399,13 @@ extern "C" __global__ __launch_bounds__({bounds}) void {name}(const float* __res
                 #pragma unroll
                 for (u32 e = 0; e < 16u; ++e) {{
                     const u32 lr = 32u * qt + ROW_OF(e, h);
-                    const float pe = (key > qt0 + lr) ? 0.0f : exp_neg(p[e] * scale - Ls[buf][lr]);     // (rows beyond T: lse = +inf)
+                    const float pe = __builtin_amdgcn_exp2f(p[e] - Ls[buf][lr]);                        // (rows beyond T: lse = +inf)
                     p[e] = pe;
                     dsv[e] = (pe * (dsv[e] - Ds[buf][lr])) * scale;
+                }}
+                if (k0 + 31u > row0) {{                                   // the tile straddles the diagonal: nothing above it
+                    #pragma unroll
+                    for (u32 e = 0; e < 16u; ++e) if (key > row0 + ROW_OF(e, h)) {{ p[e] = 0.0f; dsv[e] = 0.0f; }}
                 }}
                 #pragma unroll
                 for (u32 dt = 0; dt < ND; ++dt) {{

@@ -575,7 +575,10 @@ _matmul_plans: dict = _PlanCache() # (shapes, flags, alignment bits) -> (kernel,
 # 1 000 000 x 10 against 8.1 for "staged", 256 rows per block through LDS, which remains the form for odd lengths)
 ARGMAX_SHORT_ROWS = os.environ.get("DLGRAD_HIP_ARGMAX_SHORT_ROWS", "direct")
 ARGMAX_COL_UNROLL = 8              # rows in flight per thread of the column argmax (8192 x 8192: 50.2 us with 4, 49.5 with 8)
-ARGMAX_COL_BLOCKS = 512            # blocks of 64 x 16 threads the column argmax aims for; more only lengthen the fold
+# blocks of 64 x 16 threads the first stage of a tall column reduction aims for (16384 x 8192 over axis 0: 88.5 us with 8192,
+# 83.6 us = 6.4 TB/s with 2048 -- row chunks of 256 and a quarter of the partials -- 85.8 us with 512)
+REDUCE_COL_BLOCKS = int(os.environ.get("DLGRAD_HIP_REDUCE_COL_BLOCKS", "2048"))
+ARGMAX_COL_BLOCKS = 1024           # blocks of 64 x 16 threads the column argmax aims for (8192 x 8192: 65.6 us with 128, 51.5 with 256 or 512, 49.8 with 1024, 57.8 with 2048)
 _permute_plans: dict = _PlanCache()
 PERMUTE_DIAG = os.environ.get("DLGRAD_HIP_PERMUTE_DIAG", "1") != "0"     # diagonal tile order for power-of-two pitches
 
@@ -926,7 +929,7 @@ class HIP:
         ty = 16 if L > 64 else 4
         nt = vec == 4 and O * L * I >= NT_STORE_MIN_ELEMENTS
         k = kernel(K.reduce_cols_kernel, kop, vec, ty, nt)
-        chunks = 1 if L <= 512 else max(1, min(8192 // max(1, bx * O), L // 64))
+        chunks = 1 if L <= 512 else max(1, min(REDUCE_COL_BLOCKS // max(1, bx * O), L // 64))
         if chunks == 1:
             launch(k, (bx, 1, O), (64, ty, 1), x_addr, out_addr, L, I, L, float(divisor))
             return
