@@ -315,6 +315,39 @@ def run_c5(steps: int, warmup: int) -> dict:
             for name, _, b in work}
 
 
+def run_attention(steps: int, warmup: int) -> dict:
+    """Causal self-attention of the scaled GPT, (8, 12, 1024, 64) read from one interleaved (8, 1024, 3 * 768) projection:
+    forward, and backward (row sums, the key-side launch that writes dS, and the product dQ = dS K).  Matrix-core bound:
+    flops are those of the causal half -- 2 products forward, 5 backward (S is recomputed) of T^2 / 2 * d * 2 each per
+    head -- and the figure is against the fp32 MFMA peak.  DLGRAD_HIP_ATTENTION_FLASH=0 times the chain over stored
+    T x T tensors instead."""
+    _, _, Buffer, Device, hip = _imports()
+    lib = hip.lib()
+    rng = np.random.default_rng(9)
+    B, T, h, d = 8, 1024, 12, 64
+    C = h * d
+    qkv = Buffer.from_numpy(rng.standard_normal((B, T, 3 * C), dtype=np.float32), Device.HIP)
+    g = Buffer.from_numpy(rng.standard_normal((B, T, C), dtype=np.float32), Device.HIP)
+    scale = d ** -0.5
+    y, kept = qkv.causal_attention_qkv(h, scale)
+    per_product = B * h * T * T * d                                   # 2 * (T^2 / 2) * d flops per head
+    work = [("causal_attention_forward_(8,12,1024,64)", lambda: qkv.causal_attention_qkv(h, scale), 2 * per_product),
+            ("causal_attention_backward_(8,12,1024,64)", lambda: qkv.causal_attention_qkv_bwd(kept, g, h, scale, y), 5 * per_product)]
+    timer = EventTimer(lib)
+    for _ in range(warmup):
+        for _, f, _ in work:
+            f()
+    for _ in range(steps):
+        for name, f, _ in work:
+            timer.run(name, f)
+    lib.sync()
+    per = timer.collect()
+    return {name: {"ms": round(float(np.mean(per[name])), 4), "TFLOPs": round(fl / float(np.mean(per[name])) / 1e9, 1),
+                   "frac_mfma_fp32": round(fl / float(np.mean(per[name])) / 1e9 / MFMA_FP32_PEAK_TFLOPS, 3),
+                   "kept_for_backward_MiB": round(kept.nbytes / 2 ** 20, 1)}
+            for name, _, fl in work}
+
+
 def run_layout_and_select(steps: int, warmup: int) -> dict:
     """The kernel classes the C2 suite does not touch, at sizes beyond the caches: transposes
     and head permutes (8 B/elt), argmax (4 B/elt + 4 B/output), comparisons, clamp, pow,
@@ -792,6 +825,7 @@ def main() -> None:
             extra["mlp_784_64_10_step"] = {k: round(v, 3) for k, v in run_mlp(50, 5).items()}
             extra["mlp_784_64_10_step_hipgraph"] = {k: round(v, 3) for k, v in run_mlp_graph(200, 10).items()}
             extra["c5_components"] = run_c5(max(3, min(args.steps, 10)), 2)
+            extra["c5_attention"] = run_attention(max(3, min(args.steps, 10)), 2)
             extra["layout_and_select"] = run_layout_and_select(max(3, min(args.steps, 10)), 2)
             extra["host_device_transfers"] = run_transfers()
             extra["gpt_scaled_c5"] = run_gpt_large(2)
@@ -847,7 +881,7 @@ def main() -> None:
                "roofline": {"bound": "hbm", "achieved": comp[worst]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                             "frac": comp[worst]["GBps"] / HBM_PEAK_GBS, "traffic": None, "kernel": worst,
                             "avg_launch_ms": comp[worst]["ms"]},
-               "per_op": comp}
+               "per_op": comp, "attention": run_attention(args.steps, args.warmup)}
     else:
         r = run_mlp(args.steps, args.warmup)
         out = {"metric": "MLP 784-64-10 step samples/s (1 GPU)", "value": r["samples_per_s"], "unit": "samples/s",
