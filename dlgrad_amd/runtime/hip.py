@@ -1943,7 +1943,7 @@ class HIP:
             launch(k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, 1), threads, xa, ya, out.addr, M, N, Kd, 1, 0, 0, 0, 0, *tail)
             return (out, yn, rinv) if keep else out
         key = (x.shape, y.shape, ta, tb, tri, epi, None if e is None else e.shape, xa & 15, ya & 15, ea & 15,
-               HIP.MATMUL_FORCE, HIP.ROW_MATMUL, HIP.MATMUL_SPLITK)
+               HIP.MATMUL_FORCE, HIP.ROW_MATMUL, HIP.MATMUL_SPLITK, HIP.MATMUL_EXACT)
         plan = _matmul_plans.get(key)
         if plan is not None:                                   # a shape seen before: pack the addresses and go
             k, grid, threads, tail, out_numel, e_at, name = plan
@@ -2157,7 +2157,7 @@ class HIP:
         rows_group: with tri, the structured operand holds defined values only inside aligned groups of that
         many rows along the diagonal, so the tile's rows must divide it."""
         (aa, lda, sa0, sa1), (ba, ldb, sb0, sb1), (ca, ldc, sc0, sc1) = A, B, C
-        key = (A[1:], B[1:], C[1:], M, N, Kd, B0, B1, ta, tb, tri, aa & 15, ba & 15, ca & 15, HIP.MATMUL_FORCE, rows_group)
+        key = (A[1:], B[1:], C[1:], M, N, Kd, B0, B1, ta, tb, tri, aa & 15, ba & 15, ca & 15, HIP.MATMUL_FORCE, rows_group, HIP.MATMUL_EXACT)
         plan = _gemm_plans.get(key)
         if plan is not None:
             k, grid, threads, tail = plan

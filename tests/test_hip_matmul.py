@@ -127,6 +127,37 @@ def test_every_tile_gives_the_same_bits(monkeypatch):
         check(got, first, 0, f"{tile} vs 64x64")
 
 
+def test_whole_tile_form_gives_the_bits_of_the_guarded_form(monkeypatch):
+    """A product cut into whole tiles runs the form of the kernel whose k loop carries no bounds tests: same loads, same
+    products in the same order, so the same bits as the guarded form -- for every tile, with the operands as stored,
+    transposed in place, and with a step on the accumulator as it is stored.  The shapes are two tiles by three with
+    three or more k steps, so first, middle and last steps of the loop are all there."""
+    require_gpu()
+    from dlgrad_amd.codegen import hip_kernel as K
+    from dlgrad_amd.runtime.hip import HIP
+    monkeypatch.setattr(HIP, "MATMUL_SPLITK", False)
+    rng = np.random.default_rng(11)
+    for tile, cfg in K.MATMUL_CONFIGS.items():
+        bm, bn, _ = K.matmul_tile_shape(tile)
+        M, N, Kd = 2 * bm, 3 * bn, max(3 * cfg[4], 192)
+        x, y = rng.standard_normal((M, Kd), dtype=np.float32), rng.standard_normal((Kd, N), dtype=np.float32) * np.float32(Kd ** -0.5)
+        e = rng.standard_normal((M, N), dtype=np.float32)
+        xd, yd, ytd, xtd, ed = dev(x), dev(y), dev(np.ascontiguousarray(y.T)), dev(np.ascontiguousarray(x.T)), dev(e)
+        monkeypatch.setattr(HIP, "MATMUL_FORCE", tile)
+        runs = {"nn": lambda: xd.matmul(yd), "nt": lambda: xd.matmul_nt(ytd), "tn": lambda: xtd.matmul_tn(yd),
+                "nn add": lambda: xd.matmul(yd, epi="add", e=ed), "nt relu": lambda: xd.matmul_nt(ytd, epi="relu"),
+                "nn gate": lambda: xd.matmul(yd, epi="gate", e=ed)}
+        for what, run in runs.items():
+            monkeypatch.setattr(HIP, "MATMUL_EXACT", False)
+            want = run().numpy()
+            guarded = HIP.last_matmul_kernel
+            monkeypatch.setattr(HIP, "MATMUL_EXACT", True)
+            got = run().numpy()
+            assert guarded and not guarded.endswith("_x") and HIP.last_matmul_kernel == guarded + "_x", (tile, what, guarded, HIP.last_matmul_kernel)
+            check(got, want, 0, f"{tile} {what}: whole-tile form vs guarded form")
+        check_mm(xd.matmul(yd).numpy(), x.astype(np.float64) @ y, f"{tile} whole-tile form")
+
+
 def test_first_use_of_a_large_shape_times_the_tiles_and_remembers_the_winner(monkeypatch, tmp_path):
     require_gpu()
     from dlgrad_amd.runtime import hip as H
