@@ -2017,9 +2017,19 @@ MATMUL_TRI = ("", "out_lower", "a_lower", "at_lower")
 
 
 @cache
+def matmul_groups_fit(WM: int, WN: int, MI: int, NJ: int, BK: int, ta: bool, tb: bool, S: int, G: int) -> bool:
+    """Whether a block of G k-groups of this tile exists: at most 1024 threads, and LDS for G sets of operand buffers plus
+    the groups' partial tiles where those do not fit into A's buffers."""
+    BM, BN = S * MI * WM, S * NJ * WN
+    red_in_a = (G - 1) * BM * BN <= 2 * G * (BK * BM if ta else BM * (BK + 4))
+    return (G * 64 * WM * WN <= 1024 and
+            G * matmul_lds_bytes(WM, WN, MI, NJ, BK, ta, tb, S) + (0 if red_in_a else (G - 1) * 4 * BM * BN) <= MATMUL_LDS_LIMIT)
+
+
 def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb: bool,
                   ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False,
-                  epi: str = "", S: int = 32, norm: bool = False, splitk: bool = False, exact: bool = False) -> tuple[str, str, str]:
+                  epi: str = "", S: int = 32, norm: bool = False, splitk: bool = False, exact: bool = False,
+                  kgroups: int = 1, deep: bool = False) -> tuple[str, str, str]:
     """C[z] = op(A[z]) . op(B[z]), fp32, row-major, on the matrix cores (v_mfma_f32_32x32x2_f32, or
     v_mfma_f32_16x16x4_f32 for S = 16).
 
@@ -2092,12 +2102,32 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     fetch in front of the MFMA run (left alone, the compiler sinks the loads to their use and waits for them there).
     Same loads, same products: same bits; 4096^3 118.6 -> 133.4 TFLOP/s, 2048^3 101.0 -> 108.5, 1024^3 75.8 -> 82.6,
     8192^3 135.3 -> 137.3 in one run.
+    kgroups: G > 1 cuts the k sum into G slices *inside a block*: the block has G times the wavefronts, group q of them runs
+    the whole k loop of the tile over k in [q * kchunk, (q + 1) * kchunk) with LDS buffers of its own, and at the end the
+    groups' partial tiles meet in LDS and group 0 adds them in group order and stores.  For an output of few tiles this puts
+    G wavefronts on every SIMD of the CUs that have a block, so one group's LDS and memory latency is covered by another's
+    MFMA run -- what a second launch over slabs cannot give a product that already has a block on every CU.  All groups take
+    the same number of k steps (they share the barriers); steps beyond K read zeros.  The sum is added in a fixed order of its
+    own (slice by slice), like the split-k form.  Arguments after the others: kchunk (a multiple of BK).
+    deep: the k loop as a software pipeline two steps deep.  The tiles of step t + 2 are fetched during step t into a second
+    set of registers, and the LDS stores of the tiles of step t + 1 are issued between the MFMA steps of the second half of
+    step t instead of behind them (the fetches, with their address arithmetic and bounds tests, between those of the first
+    half; the LDS reads of each group of 8 k one group ahead of its MFMA steps).  A wavefront issues in order: whatever
+    follows a run of dependent MFMA steps waits for the run, but an instruction placed between two of them is issued while
+    the first one executes.  Scheduling fences pin the order.  Measured beforehand by taking parts of the step away: at
+    4096^3 the fetches' latency cost 7 % of the launch and the LDS stores 5 %, at 1024^3 11 % each; with this form 1024^3
+    24.2 -> 20.6 us, 2048^3 152.8 -> 136.4, 4096^3 1047 -> 998, 512^3 7.7 -> 6.7, (768 x 1024)^T (1024 x 3072) 56.7 -> 49.5.
+    The step past the last one fetches the last tiles again instead of branching.  Same loads, same MFMA steps in the same
+    order: same bits.
     """
     BM, BN, T = S * MI * WM, S * NJ * WN, 64 * WM * WN
+    G = kgroups
     assert isinstance(splitk, bool) and not (splitk and (tri or strided or epi or norm))
+    assert G in (1, 2, 3, 4, 8, 16) and not (G > 1 and (splitk or tri or strided or epi or norm))
     NE = S * S // 64                                        # accumulator registers per MFMA tile
-    assert BK % 8 == 0 and MI in (1, 2, 3, 4) and NJ in (1, 2, 3, 4) and S in (16, 32) and T <= 1024
-    assert matmul_lds_bytes(WM, WN, MI, NJ, BK, ta, tb, S) <= MATMUL_LDS_LIMIT
+    assert BK % 8 == 0 and MI in (1, 2, 3, 4) and NJ in (1, 2, 3, 4) and S in (16, 32) and G * T <= 1024
+    red_in_a = (G - 1) * BM * BN <= 2 * G * (BK * BM if ta else BM * (BK + 4))       # the partial tiles of the groups reuse A's LDS buffers if they fit
+    assert matmul_groups_fit(WM, WN, MI, NJ, BK, ta, tb, S, G)
     name = (f"matmul_{BM}x{BN}x{BK}_w{WM}x{WN}_{'a4' if veca else 'a1'}{'b4' if vecb else 'b1'}"
             f"{'_tn' if ta else ''}{'_nt' if tb else ''}{'_' + tri if tri else ''}{'_ld' if strided else ''}{'_' + epi if epi else ''}{'_m16' if S == 16 else ''}")
     assert tri in MATMUL_TRI and not (tri == "a_lower" and ta) and not (tri == "at_lower" and not ta)
@@ -2106,6 +2136,11 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
         name += "_rms"
     if splitk:
         name += "_sk"
+    if G > 1:
+        name += f"_g{G}"
+    if deep:
+        assert not norm
+        name += "_d"
     if exact:
         assert veca and vecb and not norm
         name += "_x"
@@ -2137,7 +2172,7 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
                            f"            const bool ok = row < g.{ext};\n" +
                            "".join(f"            r{x}[p].{c} = (ok && k + {n}u < KEND) ? s[{n}] : 0.f;\n" for n, c in enumerate(comp)))
             st = f"{guard}*reinterpret_cast<float4*>(&{X}s[buf][{x}_r + p * {rpp}u][4u * {x}_q]) = r{x}[p];"
-            decl = f"__shared__ __attribute__((aligned(16))) float {X}s[2][{R}][{BK + 4}];"
+            decl = f"__shared__ __attribute__((aligned(16))) float {X}s[{2 * G}][{R}][{BK + 4}];"
         else:
             Q = R // 4
             assert T >= Q
@@ -2155,7 +2190,7 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
                            f"            const bool ok = k < KEND;\n" +
                            "".join(f"            r{x}[p].{c} = (ok && col + {n}u < g.{ext}) ? s[{n}] : 0.f;\n" for n, c in enumerate(comp)))
             st = f"{guard}*reinterpret_cast<float4*>(&{X}s[buf][{x}_r + p * {rpp}u][4u * {x}_q]) = r{x}[p];"
-            decl = f"__shared__ __attribute__((aligned(16))) float {X}s[2][{BK}][{R}];"
+            decl = f"__shared__ __attribute__((aligned(16))) float {X}s[{2 * G}][{BK}][{R}];"
         load = f"""        #pragma unroll
         for (u32 p = 0; p < {P}u; ++p) {{
             {where}
@@ -2166,10 +2201,15 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
         for (u32 p = 0; p < {P}u; ++p)
             {st}
 """
-        return decl, idx, P, load, stash
+        def ld_piece(rs: int, pi: int, k0: str) -> str:           # pass pi of the fetch into register set rs
+            return f"            {{ const u32 p = {pi}u, k0 = {k0}; {where} {ld_code} }}\n".replace(f"r{x}[p]", f"r{x}{rs}[p]")
 
-    decl_a, idx_a, PA, load_a, stash_a = loader("A", not ta, "M", BM, "M", "M", "m0", veca)
-    decl_b, idx_b, PB, load_b, stash_b = loader("B", tb, "N", BN, "N", "N", "n0", vecb)
+        def st_piece(rs: int, pi: int, buf: str) -> str:          # pass pi of register set rs into LDS buffer buf
+            return f"            {{ const u32 p = {pi}u, buf = {buf}; {st} }}\n".replace(f"r{x}[p]", f"r{x}{rs}[p]")
+        return decl, idx, P, load, stash, ld_piece, st_piece
+
+    decl_a, idx_a, PA, load_a, stash_a, ld_piece_a, st_piece_a = loader("A", not ta, "M", BM, "M", "M", "m0", veca)
+    decl_b, idx_b, PB, load_b, stash_b, ld_piece_b, st_piece_b = loader("B", tb, "N", BN, "N", "N", "n0", vecb)
 
     # ---- the multiply: one group of 8 k per iteration, four 32x32x2 (two 16x16x4) MFMA steps
     pre = ""
@@ -2198,6 +2238,80 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
                 mfma += (f"              acc[{i_}][{j_}] = __builtin_amdgcn_mfma_f32_{'32x32x2' if S == 32 else '16x16x4'}f32("
                          f"{ai}, {bj}, acc[{i_}][{j_}], 0, 0, 0);\n")
         mfma += "            }\n"
+
+    if deep:
+        NSTEP = 4 if S == 32 else 2
+        hk = "h" if S == 32 else "(h & 1u)"
+
+        def krow_at(kb: str, st_: int) -> str:
+            return f"{kb} + 4u * h + {st_}u" if S == 32 else f"{kb} + 4u * (h & 1u) + (h >> 1) + {2 * st_}u"
+
+        def reads(P: str, kb: str) -> str:
+            out = ""
+            if not ta:
+                out += "".join(f"                fa[{P}][{i}] = *reinterpret_cast<const float4*>(&As[buf][wm0 + {S}u * {i} + r][{kb} + 4u * {hk}]);\n" for i in range(MI))
+            if tb:
+                out += "".join(f"                fb[{P}][{j}] = *reinterpret_cast<const float4*>(&Bs[buf][wn0 + {S}u * {j} + r][{kb} + 4u * {hk}]);\n" for j in range(NJ))
+            for st_ in range(NSTEP):
+                if ta:
+                    out += f"                fav[{P}][{st_}] = *reinterpret_cast<const {vtype[MI]}*>(&As[buf][{krow_at(kb, st_)}][wm0 + {MI}u * r]);\n"
+                if not tb:
+                    out += f"                fbv[{P}][{st_}] = *reinterpret_cast<const {vtype[NJ]}*>(&Bs[buf][{krow_at(kb, st_)}][wn0 + {NJ}u * r]);\n"
+            return out
+
+        steps, step_lines = "", []
+        for st_ in range(NSTEP):
+            pick = (lambda v: f"{v}.{comp[st_]}") if S == 32 else (lambda v: f"((h >> 1) ? {v}.{comp[2 * st_ + 1]} : {v}.{comp[2 * st_]})")
+            for i_ in range(MI):
+                ai = ((f"fav[P][{st_}]" if MI == 1 else f"fav[P][{st_}].{comp[i_]}") if ta else pick(f"fa[P][{i_}]"))
+                for j_ in range(NJ):
+                    bj = (pick(f"fb[P][{j_}]") if tb else (f"fbv[P][{st_}]" if NJ == 1 else f"fbv[P][{st_}].{comp[j_]}"))
+                    step_lines.append(f"            acc[{i_}][{j_}] = __builtin_amdgcn_mfma_f32_{'32x32x2' if S == 32 else '16x16x4'}f32("
+                                      f"{ai}, {bj}, acc[{i_}][{j_}], 0, 0, 0);\n")
+        steps = "".join(step_lines)
+        frag_decl = (("" if ta else f"        float4 fa[2][{MI}];\n") + (f"        float4 fb[2][{NJ}];\n" if tb else "") +
+                     (f"        {vtype[MI]} fav[2][{NSTEP}];\n" if ta else "") + ("" if tb else f"        {vtype[NJ]} fbv[2][{NSTEP}];\n"))
+    mfma_run = f"""        #pragma unroll
+        for (u32 kb = 0; kb < BK; kb += 8u) {{
+{mfma}        }}"""
+
+    def deep_step(cb: int, ls: int, ss: int, k0: str) -> str:
+        """One k step of the deep form: MFMA steps on LDS buffer cb; the fetch of the tiles at k0 into register set ls is spread
+        over the first half of the MFMA steps, the LDS stores of register set ss into buffer cb ^ 1 over the second half."""
+        FENCE = "            __builtin_amdgcn_sched_barrier(0);\n"
+        groups = BK // 8
+        half = max(1, groups // 2)
+        fetch = [ld_piece_a(ls, p_, k0) for p_ in range(PA)] + [ld_piece_b(ls, p_, k0) for p_ in range(PB)]
+        lds = (lambda b_: f"gb + {b_}u") if G > 1 else (lambda b_: f"{b_}u")          # (a k-group has its own pair of buffers)
+        store = [st_piece_a(ss, p_, lds(cb ^ 1)) for p_ in range(PA)] + [st_piece_b(ss, p_, lds(cb ^ 1)) for p_ in range(PB)]
+
+        def spread(lines: list, extras: list) -> str:
+            # an extra after every n-th MFMA step, the first one behind the first step (which is then executing)
+            if not extras:
+                return "".join(lines)
+            n = max(1, len(lines) // len(extras))
+            out, e = "", 0
+            for at, line in enumerate(lines):
+                out += line
+                if at % n == 0 and e < len(extras):
+                    out += FENCE + extras[e] + FENCE
+                    e += 1
+            return out + "".join(FENCE + x for x in extras[e:])
+        code = f"        {{   // MFMA steps on buffer {cb}; fetch into register set {ls}; register set {ss} into buffer {cb ^ 1}\n            const u32 buf = {lds(cb)};\n"
+        code += reads("0", "0u")
+        first = [(g_, l_) for g_ in range(half) for l_ in step_lines]
+        second = [(g_, l_) for g_ in range(half, groups) for l_ in step_lines]
+        for part, extras in ((first, fetch), (second, store)):
+            # the lines of a group carry the operand set of the group; the reads of the next group go in front of the group's first step
+            lines = []
+            for at, (g_, l_) in enumerate(part):
+                head = ""
+                if at % len(step_lines) == 0 and g_ + 1 < groups:
+                    head = reads(f"{(g_ + 1) & 1}", f"{8 * (g_ + 1)}u") + FENCE
+                lines.append(head + l_.replace("[P]", f"[{g_ & 1}]"))
+            code += spread(lines, extras)
+        return code + "        }\n"
+
 
     # ---- epilogue: accumulator e of tile (i, j) belongs to operand-row index 8*(e/4) + 4*h + e%4
     # (4*h + e for the 16-wide tile) of A's tile i and operand-row index lane%S of B's tile j
@@ -2250,7 +2364,15 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     }}
     __syncthreads();
 """
-    if splitk:
+    if G > 1:
+        kloop = f"""    const u32 kt0 = kbeg / BK, nk = kt0 + kchunk / BK;         // every group takes the same number of steps: they share the barriers
+    const u32 gb = 2u * grp;                                      // this group's pair of LDS buffers
+    load_tiles(kt0 * BK);
+    stash_tiles(gb);
+    __syncthreads();
+    for (u32 kt = kt0; kt < nk; ++kt) {{
+        const u32 buf = gb + ((kt - kt0) & 1u);"""
+    elif splitk:
         kloop = f"""    const u32 nk = (kend + BK - 1u) / BK, kt0 = kbeg / BK;                 // this block's slice of k
     load_tiles(kt0 * BK);
     stash_tiles(0u);
@@ -2273,28 +2395,73 @@ def matmul_kernel(WM: int, WN: int, MI: int, NJ: int, BK: int, veca: bool, vecb:
     __syncthreads();
     for (u32 kt = kt0; kt < nk; ++kt) {{
         const u32 buf = (kt - kt0) & 1u;"""
+    if deep:
+        if G > 1:
+            krange = "const u32 kt0 = kbeg / BK, nk = kt0 + kchunk / BK, gb = 2u * grp;      // every group takes the same number of steps: they share the barriers"
+        elif splitk:
+            krange = "const u32 nk = (kend + BK - 1u) / BK, kt0 = kbeg / BK;                 // this block's slice of k"
+        elif tri in ("", "out_lower"):
+            krange = "const u32 nk = (g.K + BK - 1u) / BK, kt0 = 0u;"
+        else:
+            krange = {"a_lower": "const u32 nk = (min(g.K, m0 + BM) + BK - 1u) / BK, kt0 = 0u;       // A is zero right of the diagonal",
+                      "at_lower": "const u32 nk = (g.K + BK - 1u) / BK, kt0 = m0 / BK;                 // the stored A is zero above the diagonal"}[tri]
+        all_fetch = lambda rs, k0: "".join(ld_piece_a(rs, p_, k0) for p_ in range(PA)) + "".join(ld_piece_b(rs, p_, k0) for p_ in range(PB))
+        all_store = lambda rs, buf: "".join(st_piece_a(rs, p_, buf) for p_ in range(PA)) + "".join(st_piece_b(rs, p_, buf) for p_ in range(PB))
+        kloop = f"""    {krange}
+    float4 ra0[{PA}], rb0[{PB}], ra1[{PA}], rb1[{PB}];           // two sets of registers for tiles on their way to LDS
+{frag_decl}    {{
+{all_fetch(0, "kt0 * BK")}{all_store(0, "gb" if G > 1 else "0u")}{all_fetch(1, "min(kt0 + 1u, nk - 1u) * BK")}    }}
+    __syncthreads();
+    for (u32 kt = kt0; ; kt += 2u) {{
+{deep_step(0, 0, 1, "min(kt + 2u, nk - 1u) * BK")}        __syncthreads();
+        if (kt + 1u >= nk) break;
+{deep_step(1, 1, 0, "min(kt + 3u, nk - 1u) * BK")}        __syncthreads();
+        if (kt + 2u >= nk) break;"""
     split_head = split_tail = ""
     if splitk:
         split_head = """    const u32 kbeg = blockIdx.y * kchunk, kend = min(g.K, kbeg + kchunk);
     const u64 slab_elts = (u64)g.M * g.N;
     float* __restrict__ slab = W + ((u64)blockIdx.z * gridDim.y + blockIdx.y) * slab_elts;
 """
-    if exact:
+    if deep:
+        loop_body = ""
+    elif exact:
         # one straight run of code per k step: fetch, fence, MFMA run, LDS stores of what was fetched
         loop_body = f"""        load_tiles(min(kt + 1u, nk - 1u) * BK);
         __builtin_amdgcn_sched_barrier(0);
-        #pragma unroll
-        for (u32 kb = 0; kb < BK; kb += 8u) {{
-{mfma}        }}
+{mfma_run}
         stash_tiles(buf ^ 1u);
         __syncthreads();"""
     else:
         loop_body = f"""        if (kt + 1u < nk) load_tiles((kt + 1u) * BK);
-        #pragma unroll
-        for (u32 kb = 0; kb < BK; kb += 8u) {{
-{mfma}        }}
+{mfma_run}
         if (kt + 1u < nk) stash_tiles(buf ^ 1u);
         __syncthreads();"""
+    group_head = group_join = ""
+    if G > 1:
+        group_head = "    const u32 kbeg = grp * kchunk, kend = min(g.K, kbeg + kchunk);            // this group's slice of k\n"
+        group_join = f"""    // the groups' partial tiles meet in LDS (entry-major: a wavefront writes 64 consecutive floats); group 0 adds them in group order
+    {f"float (*Red)[{MI * NJ * NE}][{T}] = reinterpret_cast<float (*)[{MI * NJ * NE}][{T}]>(&As[0][0][0]);      // (behind the last barrier of the k loop nobody reads the tiles any more)" if red_in_a else f"__shared__ float Red[{G - 1}][{MI * NJ * NE}][{T}];"}
+    if (grp != 0u) {{
+        #pragma unroll
+        for (int i = 0; i < MI; ++i)
+            #pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                #pragma unroll
+                for (int e = 0; e < {NE}; ++e) Red[grp - 1u][(i * NJ + j) * {NE} + e][tid] = acc[i][j][e];
+    }}
+    __syncthreads();
+    if (grp != 0u) return;
+    #pragma unroll
+    for (int q = 0; q < {G - 1}; ++q)
+        #pragma unroll
+        for (int i = 0; i < MI; ++i)
+            #pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                #pragma unroll
+                for (int e = 0; e < {NE}; ++e) acc[i][j][e] += Red[q][(i * NJ + j) * {NE} + e][tid];
+
+"""
     f4v_typedef = "" if S == 32 else "\ntypedef float f4v __attribute__((ext_vector_type(4)));"
     src = f"""{PRELUDE}
 typedef float f16v __attribute__((ext_vector_type(16)));{f4v_typedef}
@@ -2305,9 +2472,9 @@ struct MMArgs {{ u32 M, N, K, nbc, sa0, sa1, sb0, sb1; }};
 #define BK {BK}u
 #define MI {MI}
 #define NJ {NJ}
-#define KEND {"kend" if splitk else "g.K"}
-extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict__ A,
-        const float* __restrict__ B, float* __restrict__ C, MMArgs g{", const float* __restrict__ E" if epi else ""}{", const float* __restrict__ gain, float eps, float* __restrict__ yn, float* __restrict__ rinv" if norm else ""}{", float* __restrict__ W, u32 kchunk" if splitk else ""}) {{
+#define KEND {"kend" if splitk or G > 1 else "g.K"}
+extern "C" __global__ __launch_bounds__({G * T}) void {name}(const float* __restrict__ A,
+        const float* __restrict__ B, float* __restrict__ C, MMArgs g{", const float* __restrict__ E" if epi else ""}{", const float* __restrict__ gain, float eps, float* __restrict__ yn, float* __restrict__ rinv" if norm else ""}{", float* __restrict__ W, u32 kchunk" if splitk else ""}{", u32 kchunk" if G > 1 else ""}) {{
     {decl_a}
     {decl_b}
 
@@ -2327,8 +2494,8 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
     B += (u64)zb * g.sb0 + (u64)zc * g.sb1;
     C += (u64)blockIdx.z * g.M * g.N;
 {split_head}
-    const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const u32 r = lane & {S - 1}u, h = lane >> {5 if S == 32 else 4};
+    {f"const u32 grp = threadIdx.x / {T}u, tid = threadIdx.x % {T}u" if G > 1 else "const u32 tid = threadIdx.x"}, lane = tid & 63u, wave = tid >> 6;
+{group_head}    const u32 r = lane & {S - 1}u, h = lane >> {5 if S == 32 else 4};
     const u32 wm0 = (wave / {WN}u) * {S * MI}u, wn0 = (wave % {WN}u) * {S * NJ}u;
     {idx_a}
     {idx_b}
@@ -2351,7 +2518,7 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
 {loop_body}
     }}
 
-    #pragma unroll
+{group_join}    #pragma unroll
     for (int i = 0; i < MI; ++i)
         #pragma unroll
         for (int e = 0; e < {NE}; ++e) {{
@@ -2418,10 +2585,10 @@ extern "C" __global__ __launch_bounds__({T}) void {name}(const float* __restrict
                           "B + (u64)row * g.ldb + k" if tb else "B + (u64)k * g.ldb + col"),
                          ("C += (u64)blockIdx.z * g.M * g.N;", "C += (u64)zb * g.sc0 + (u64)zc * g.sc1;"),
                          ("C + (u64)row * g.N;", "C + (u64)row * g.ldc;")):
-            assert src.count(was) == 1, was
+            assert src.count(was) >= 1, was                       # (the deep form names each operand address once per fetch pass)
             src = src.replace(was, now)
         return src, name, _fmt("P", "P", "P", "13I")
-    return src, name, _fmt("P", "P", "P", "8I", *(("P", "f", "P", "P") if norm else ()), *(("P", "I") if splitk else ()))
+    return src, name, _fmt("P", "P", "P", "8I", *(("P", "f", "P", "P") if norm else ()), *(("P", "I") if splitk else ()), *(("I",) if G > 1 else ()))
 
 
 @cache
@@ -2443,9 +2610,9 @@ def matmul_pair_kernel(first: tuple, second: tuple) -> tuple[str, str, str]:
     parts = []
     for tag, a in (("p0", first), ("p1", second)):
         WM, WN, MI, NJ, BK, veca, vecb, ta, tb, tri, strided, epi, S, *rest = a
-        exact = bool(rest and rest[0])
+        exact, deep = bool(rest and rest[0]), bool(len(rest) > 1 and rest[1])
         assert not tri and not strided
-        src, name, fmt = matmul_kernel(WM, WN, MI, NJ, BK, veca, vecb, ta, tb, tri, strided, epi, S, False, False, exact)
+        src, name, fmt = matmul_kernel(WM, WN, MI, NJ, BK, veca, vecb, ta, tb, tri, strided, epi, S, False, False, exact, 1, deep)
         assert src.startswith(PRELUDE)
         body = src[len(PRELUDE):]
         body, n = re.subn(r'extern "C" __global__ __launch_bounds__\(\d+\) void \w+\(',
@@ -2515,6 +2682,7 @@ MATMUL_CONFIGS = {
     "128x64w8": (4, 2, 1, 1, 32),       # one block and only its own waves can overlap loads with MFMA (2048^3: 115
     "64x128w8": (2, 4, 1, 1, 32),       # against 97 TFLOP/s for four waves of 64x64); the eight-wave halves for narrow outputs
     "64x64": (2, 2, 1, 1, 16),
+    "64x64k32": (2, 2, 1, 1, 32),
     "64x64k64": (2, 2, 1, 1, 64),       # same tile, K walked 64 at a time: fewer barriers when one block per CU
     "32x32": (1, 1, 1, 1, 16),          # has nobody to overlap with (1024^3: 73 against 62 TFLOP/s)
     # sixth entry 16: wavefronts of 16x16 (v_mfma_f32_16x16x4_f32) for small outputs with a long k, where the
@@ -2528,7 +2696,7 @@ MATMUL_CONFIGS = {
     "32x32m16k128": (2, 2, 1, 1, 128, 16),
     "32x32m16k64": (2, 2, 1, 1, 64, 16),
 }
-MATMUL_SMALL_TILES = ("64x64", "64x64k64", "32x32", "64x64m16", "64x32m16", "32x32m16", "64x64m16k128", "32x32m16k128", "32x32m16k64")
+MATMUL_SMALL_TILES = ("64x64", "64x64k32", "64x64k64", "32x32", "64x64m16", "64x32m16", "32x32m16", "64x64m16k128", "32x32m16k128", "32x32m16k64")
 
 
 def matmul_tile_shape(tile: str) -> tuple[int, int, int]:

@@ -1710,6 +1710,8 @@ class HIP:
         return best
 
     SPLITK_BASES = ("128x128", "128x64", "64x64k64", "64x64m16")      # tiles whose split-k forms are timed
+    KGROUP_BASES = ("128x128", "128x64", "64x64", "64x64k32", "64x64k64", "32x32", "32x32m16", "64x64m16")     # tiles whose k-group forms are timed
+    MATMUL_KGROUPS = os.environ.get("DLGRAD_HIP_MATMUL_KGROUPS", "1") != "0"    # "0": no product cuts k among the wavefronts of a block
 
     @staticmethod
     def _splitk_eligible(M: int, N: int, Kd: int, batch: int) -> bool:
@@ -1734,6 +1736,13 @@ class HIP:
                 for slices in (2, 4, 8, 16):
                     if Kd // slices >= 128 and tiles * slices <= 2048 and HIP._split_plan(f"{base}/{slices}", Kd)[0] == slices:
                         out.append(f"{base}/{slices}")
+            for base in HIP.KGROUP_BASES if HIP.MATMUL_KGROUPS else ():
+                bm, bn, _ = K.matmul_tile_shape(base)
+                if bm > max(32, 2 * M) or bn > max(32, 2 * N) or -(-M // bm) * -(-N // bn) * batch > 1024:
+                    continue
+                for groups in (2, 4, 8):
+                    if Kd // groups >= 64 and HIP._valid_tile(f"{base}*{groups}") and HIP._group_plan(f"{base}*{groups}", Kd)[0] == groups:
+                        out.append(f"{base}*{groups}")
         for name in K.MATMUL_CONFIGS:
             bm, bn, _ = K.matmul_tile_shape(name)
             if bm > max(32, 2 * M) or bn > max(32, 2 * N):
@@ -1746,17 +1755,30 @@ class HIP:
     @staticmethod
     def _split_of(tile: str) -> tuple[str, int]:
         """"128x128/4" -> ("128x128", 4): the k sum cut into 4 slices, a block per (tile, slice), the partial tiles
-        added up by a column-sum launch.  A plain tile name: (tile, 1)."""
+        added up by a column-sum launch.  A plain tile name: (tile, 1).  "64x64*2" (k cut among two groups of wavefronts
+        inside each block, see _groups_of) -> ("64x64", 1)."""
         base, _, sk = tile.partition("/")
-        return (base, int(sk)) if sk else (base, 1)
+        return (base.partition("*")[0], int(sk)) if sk else (base.partition("*")[0], 1)
+
+    @staticmethod
+    def _groups_of(tile: str) -> int:
+        """"64x64*2" -> 2: every block has two groups of the tile's wavefronts, each with half of k (K.matmul_kernel, kgroups)."""
+        _, _, g = tile.partition("*")
+        return int(g) if g else 1
 
     @staticmethod
     def _valid_tile(tile: str) -> bool:
         try:
             base, slices = HIP._split_of(tile)
+            groups = HIP._groups_of(tile)
         except ValueError:
             return False
-        return base in K.MATMUL_CONFIGS and 1 <= slices <= 64
+        if base not in K.MATMUL_CONFIGS or not 1 <= slices <= 64 or (groups > 1 and (slices > 1 or groups not in (2, 3, 4, 8, 16))):
+            return False
+        cfg = K.MATMUL_CONFIGS[base]
+        # (a group form must fit whichever operand is read transposed)
+        return groups == 1 or all(K.matmul_groups_fit(*cfg[:5], ta, tb, cfg[5] if len(cfg) > 5 else 32, groups)
+                                  for ta, tb in ((False, False), (True, False), (False, True)))
 
     @staticmethod
     def _split_plan(tile: str, Kd: int) -> tuple[int, int]:
@@ -1767,8 +1789,27 @@ class HIP:
         return -(-Kd // kchunk), kchunk
 
     @staticmethod
+    def _group_plan(tile: str, Kd: int) -> tuple[int, int]:
+        """(groups, kchunk) of a k-group tile as launched: every group the same number of whole k steps (a group whose slice lies
+        beyond k reads zeros); a k of fewer steps than groups were asked for gets fewer groups, down to 1 (the plain tile)."""
+        base, groups = HIP._split_of(tile)[0], HIP._groups_of(tile)
+        bk = K.MATMUL_CONFIGS[base][4]
+        steps = -(-Kd // bk)
+        if steps < groups:
+            groups = max((g for g in (1, 2, 3, 4, 8, 16) if g <= steps), default=1)
+        return groups, -(-steps // groups) * bk
+
+    @staticmethod
     def _launch_matmul(tile: str, veca: bool, vecb: bool, M: int, N: int, batch: int, args: tuple,
                        ta: bool = False, tb: bool = False, tri: str = "", strided: bool = False, epi: str = "") -> None:
+        if "*" in tile:
+            if tri or strided or epi:
+                raise ValueError(f"a k-group tile ({tile}) takes no triangular, strided or epilogue form")
+            k, grid, threads = HIP._matmul_kernel(tile, veca, vecb, M, N, batch, ta, tb, Kd=args[5])
+            HIP.last_matmul_kernel = kernel_names.get(id(k))
+            groups, kchunk = HIP._group_plan(tile, args[5])
+            launch(k, grid, threads, *args, *((kchunk,) if groups > 1 else ()))
+            return
         if "/" in tile:
             if tri or strided or epi:
                 raise ValueError(f"a split-k tile ({tile}) takes no triangular, strided or epilogue form")
@@ -1792,12 +1833,28 @@ class HIP:
         cfg = K.MATMUL_CONFIGS[base]                           # (WM, WN, MI, NJ, BK) and, for the 16-wide MFMA tiles, 16
         S = cfg[5] if len(cfg) > 5 else 32
         exact = HIP._whole_tiles(base, veca, vecb, M, N, Kd)
+        groups = HIP._groups_of(tile)
+        if groups > 1:
+            groups, kchunk = HIP._group_plan(tile, Kd)
+        if groups > 1:
+            if tri or strided or epi or not K.matmul_groups_fit(*cfg[:5], ta, tb, S, groups):
+                raise ValueError(f"tile {tile} does not fit this product (k = {Kd})")
+            k = kernel(K.matmul_kernel, *cfg[:5], veca, vecb, ta, tb, "", False, "", S, False, False, exact and Kd == groups * kchunk, groups, HIP._deep_form(base))
+            return k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch), groups * threads
         if slices > 1:
             n_slices, kchunk = HIP._split_plan(tile, Kd)
-            k = kernel(K.matmul_kernel, *cfg[:5], veca, vecb, ta, tb, "", False, "", S, False, True, exact and Kd % kchunk == 0)
+            k = kernel(K.matmul_kernel, *cfg[:5], veca, vecb, ta, tb, "", False, "", S, False, True, exact and Kd % kchunk == 0, 1, HIP._deep_form(base))
             return k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), n_slices, batch), threads
-        k = kernel(K.matmul_kernel, *cfg[:5], veca, vecb, ta, tb, tri, strided, epi, S, False, False, exact)
+        k = kernel(K.matmul_kernel, *cfg[:5], veca, vecb, ta, tb, tri, strided, epi, S, False, False, exact, 1, HIP._deep_form(base))
         return k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, batch), threads
+
+    MATMUL_DEEP = os.environ.get("DLGRAD_HIP_MATMUL_DEEP", "1") != "0"      # "0": product kernels fetch one k step ahead and store to LDS behind the MFMA run
+
+    @staticmethod
+    def _deep_form(tile: str) -> bool:
+        """Whether products of this tile run the k loop that fetches two steps ahead and issues its fetches and LDS stores between
+        the MFMA steps (K.matmul_kernel, deep): same bits, 4 to 17 % faster on every shape measured."""
+        return HIP.MATMUL_DEEP
 
     @staticmethod
     def _whole_tiles(tile: str, veca: bool, vecb: bool, M: int, N: int, Kd: int) -> bool:
@@ -1943,7 +2000,7 @@ class HIP:
             launch(k, (((M + bm - 1) // bm) * ((N + bn - 1) // bn), 1, 1), threads, xa, ya, out.addr, M, N, Kd, 1, 0, 0, 0, 0, *tail)
             return (out, yn, rinv) if keep else out
         key = (x.shape, y.shape, ta, tb, tri, epi, None if e is None else e.shape, xa & 15, ya & 15, ea & 15,
-               HIP.MATMUL_FORCE, HIP.ROW_MATMUL, HIP.MATMUL_SPLITK, HIP.MATMUL_EXACT)
+               HIP.MATMUL_FORCE, HIP.ROW_MATMUL, HIP.MATMUL_SPLITK, HIP.MATMUL_EXACT, HIP.MATMUL_KGROUPS, HIP.MATMUL_DEEP)
         plan = _matmul_plans.get(key)
         if plan is not None:                                   # a shape seen before: pack the addresses and go
             k, grid, threads, tail, out_numel, e_at, name = plan
@@ -2021,6 +2078,10 @@ class HIP:
         if not capturing():                                    # (while capturing, a shape met for the first time is not timed)
             if "/" in tile:
                 _matmul_plans[key] = (tile, (veca, vecb, M, N, batch), (ta, tb), args[3:], out_numel, 3, HIP.last_matmul_kernel)
+            elif "*" in tile:
+                k, grid, threads = HIP._matmul_kernel(tile, veca, vecb, M, N, batch, ta, tb, Kd=Kd)
+                groups, kchunk = HIP._group_plan(tile, Kd)
+                _matmul_plans[key] = (k, grid, threads, (*args[3:], *((kchunk,) if groups > 1 else ())), out_numel, 0, HIP.last_matmul_kernel)
             else:
                 k, grid, threads = HIP._matmul_kernel(tile, veca, vecb, M, N, batch, ta, tb, "" if epi else tri, False, epi, Kd)
                 _matmul_plans[key] = (k, grid, threads, args[3:], out_numel, 1 if epi else 0, HIP.last_matmul_kernel)
@@ -2068,7 +2129,7 @@ class HIP:
         addrs = tuple((x.ptr.addr, y.ptr.addr, 0 if e is None or e.ptr.__class__ is HostScalar else e.ptr.addr)
                       for x, y, _, _, _, e in specs)
         key = tuple((x.shape, y.shape, ta, tb, epi, None if e is None else e.shape, a[0] & 15, a[1] & 15, a[2] & 15)
-                    for (x, y, ta, tb, epi, e), a in zip(specs, addrs)) + (HIP.MATMUL_FORCE,)
+                    for (x, y, ta, tb, epi, e), a in zip(specs, addrs)) + (HIP.MATMUL_FORCE, HIP.MATMUL_EXACT, HIP.MATMUL_DEEP)
         plan = _pair_plans.get(key)
         if plan is None:
             parts = [HIP._pair_part(*sp) for sp in specs]
@@ -2095,7 +2156,7 @@ class HIP:
                     bm, bn, _ = K.matmul_tile_shape(tile)
                     cfg = K.MATMUL_CONFIGS[tile]
                     cfgs.append((*cfg[:5], veca, vecb, ta, tb, "", False, epi, cfg[5] if len(cfg) > 5 else 32,
-                                 HIP._whole_tiles(tile, veca, vecb, M, N, Kd)))
+                                 HIP._whole_tiles(tile, veca, vecb, M, N, Kd), HIP._deep_form(tile)))
                     tails.append((M, N, Kd, nbc, *sa, *sb))
                     grids.append((((M + bm - 1) // bm) * ((N + bn - 1) // bn), batch))
                     numels.append(out_numel)
@@ -2157,7 +2218,7 @@ class HIP:
         rows_group: with tri, the structured operand holds defined values only inside aligned groups of that
         many rows along the diagonal, so the tile's rows must divide it."""
         (aa, lda, sa0, sa1), (ba, ldb, sb0, sb1), (ca, ldc, sc0, sc1) = A, B, C
-        key = (A[1:], B[1:], C[1:], M, N, Kd, B0, B1, ta, tb, tri, aa & 15, ba & 15, ca & 15, HIP.MATMUL_FORCE, rows_group, HIP.MATMUL_EXACT)
+        key = (A[1:], B[1:], C[1:], M, N, Kd, B0, B1, ta, tb, tri, aa & 15, ba & 15, ca & 15, HIP.MATMUL_FORCE, rows_group, HIP.MATMUL_EXACT, HIP.MATMUL_DEEP)
         plan = _gemm_plans.get(key)
         if plan is not None:
             k, grid, threads, tail = plan

@@ -410,12 +410,16 @@ PAIR_CASES = [
 
 
 @pytest.mark.parametrize("gs,ws,xs,epi", PAIR_CASES)
-def test_two_products_in_one_launch_keep_their_bits(gs, ws, xs, epi):
+def test_two_products_in_one_launch_keep_their_bits(gs, ws, xs, epi, monkeypatch):
     """dX = G W (optionally with an epilogue) and dW = G^T X of a linear layer go out as one launch of two
     tile grids.  Each block runs the product kernel's own code on the block index it would have had, so both
-    results must equal those of the separate launches bit for bit, and the pair must be one launch."""
+    results must equal those of the separate launches bit for bit, and the pair must be one launch.  (The separate
+    launches are held to the tiles that add k in one piece: a product alone may otherwise be given a tile that cuts k
+    into slices, which a pair never is.)"""
     require_gpu()
     from dlgrad_amd.buffer import Buffer
+    from dlgrad_amd.runtime.hip import HIP
+    monkeypatch.setattr(HIP, "MATMUL_SPLITK", False)
     rng = np.random.default_rng(91)
     g, w, x = (rng.standard_normal(s, dtype=np.float32) for s in (gs, ws, xs))
     gate = rng.standard_normal(gs[:-1] + ws[-1:], dtype=np.float32)
@@ -561,7 +565,7 @@ def test_split_k_products_add_their_slices_in_a_fixed_order(tile, monkeypatch):
         da, db = dev(a), dev(b)
         first = da.matmul(db).numpy()
         if not hip.COMPILE_ONLY:
-            assert HIP.last_matmul_kernel.endswith(("_sk", "_sk_x")), HIP.last_matmul_kernel    # (_x: whole tiles, no conditional part in the k loop)
+            assert "_sk" in HIP.last_matmul_kernel.split("_w")[1], HIP.last_matmul_kernel    # (then _d: the deep k loop; _x: whole tiles, no bounds tests)
         check_mm(first, a.astype(np.float64) @ b.astype(np.float64), f"{tile} {batch}{(M, Kd, N)}")
         again = da.matmul(db).numpy()
         if not hip.COMPILE_ONLY:
@@ -576,3 +580,86 @@ def test_split_k_products_add_their_slices_in_a_fixed_order(tile, monkeypatch):
     monkeypatch.setattr(HIP, "MATMUL_FORCE", tile.split("/")[0])
     if not hip.COMPILE_ONLY:
         np.testing.assert_array_equal(fused, ((dev(a) @ dev(b)) + dev(e)).numpy())
+
+
+@pytest.mark.parametrize("tile", ["64x64k64*2", "64x64k32*4", "32x32m16*4", "32x32*8", "128x128*2", "64x64*3"])
+def test_k_group_products_add_their_slices_in_a_fixed_order(tile, monkeypatch):
+    """The k sum cut among groups of wavefronts inside every block, the partial tiles joined through LDS in group
+    order: NN, TN and NT forms, edge tiles, a k that the groups do not divide (the last group's extra steps read
+    zeros), batches -- against float64 at the product bar of 1e-4, and the same bits on a repeat."""
+    require_gpu()
+    from dlgrad_amd.runtime.hip import HIP
+    monkeypatch.setattr(HIP, "MATMUL_FORCE", tile)
+    for (M, Kd, N), batch in (((512, 512, 512), ()), ((200, 1030, 136), ()), ((96, 2048, 520), ()), ((130, 700, 70), (3,)),
+                              ((64, 4096, 64), (2, 2)), ((1024, 1024, 1024), ()), ((64, 96, 64), ())):
+        a, b = f32(*batch, M, Kd), f32(*batch, Kd, N, scale=Kd ** -0.5)
+        da, db = dev(a), dev(b)
+        first = da.matmul(db).numpy()
+        if not hip.COMPILE_ONLY:
+            assert f"_g{HIP._group_plan(tile, Kd)[0]}" in HIP.last_matmul_kernel, HIP.last_matmul_kernel
+        check_mm(first, a.astype(np.float64) @ b.astype(np.float64), f"{tile} {batch}{(M, Kd, N)}")
+        again = da.matmul(db).numpy()
+        if not hip.COMPILE_ONLY:
+            np.testing.assert_array_equal(again, first, err_msg=f"{tile} {(M, Kd, N)} repeated")
+        if not batch:
+            at, bt = dev(np.ascontiguousarray(a.T)), dev(np.ascontiguousarray(b.T))
+            check_mm(at.matmul_tn(db).numpy(), a.astype(np.float64) @ b.astype(np.float64), f"{tile} TN {(M, Kd, N)}")
+            check_mm(da.matmul_nt(bt).numpy(), a.astype(np.float64) @ b.astype(np.float64), f"{tile} NT {(M, Kd, N)}")
+    # an epilogue takes no k-group tile: the forced tile falls back to its plain form and the bits are the plain kernel's
+    a, b, e = f32(128, 512), f32(512, 128, scale=512 ** -0.5), f32(128, 128)
+    fused = dev(a).matmul(dev(b), epi="add", e=dev(e)).numpy()
+    monkeypatch.setattr(HIP, "MATMUL_FORCE", tile.split("*")[0])
+    if not hip.COMPILE_ONLY:
+        np.testing.assert_array_equal(fused, ((dev(a) @ dev(b)) + dev(e)).numpy())
+
+
+def test_two_step_deep_k_loop_gives_the_bits_of_the_plain_loop(monkeypatch):
+    """The k loop that fetches two steps ahead and issues its fetches and LDS stores between the MFMA steps performs the
+    loads and MFMA steps of the plain loop in the same order: same bits, for every tile -- on a shape with edge tiles
+    and a ragged k (the guarded form), on whole tiles (the form without bounds tests), with one, two and three k steps,
+    as stored and transposed in place, with epilogues, triangular structure, split k and k groups."""
+    require_gpu()
+    from dlgrad_amd.codegen import hip_kernel as K
+    from dlgrad_amd.runtime.hip import HIP
+    rng = np.random.default_rng(12)
+
+    def both(run, what):
+        monkeypatch.setattr(HIP, "MATMUL_DEEP", False)
+        want = run().numpy()
+        plain = HIP.last_matmul_kernel
+        monkeypatch.setattr(HIP, "MATMUL_DEEP", True)
+        got = run().numpy()
+        if not hip.COMPILE_ONLY:
+            assert plain and "_d" not in plain.split("_w")[1] and "_d" in HIP.last_matmul_kernel.split("_w")[1], (what, plain, HIP.last_matmul_kernel)
+        check(got, want, 0, f"{what}: deep loop vs plain loop")
+
+    for tile, cfg in K.MATMUL_CONFIGS.items():
+        bm, bn, _ = K.matmul_tile_shape(tile)
+        monkeypatch.setattr(HIP, "MATMUL_FORCE", tile)
+        for M, N, Kd in ((200, 196, 328), (2 * bm, 2 * bn, 3 * cfg[4]), (bm, bn, cfg[4]), (bm + 4, bn, 2 * cfg[4] + 8)):
+            x, y = rng.standard_normal((M, Kd), dtype=np.float32), rng.standard_normal((Kd, N), dtype=np.float32) * np.float32(Kd ** -0.5)
+            e = rng.standard_normal((M, N), dtype=np.float32)
+            xd, yd, ytd, xtd, ed = dev(x), dev(y), dev(np.ascontiguousarray(y.T)), dev(np.ascontiguousarray(x.T)), dev(e)
+            both(lambda: xd.matmul(yd), f"{tile} {(M, N, Kd)} nn")
+            both(lambda: xd.matmul_nt(ytd), f"{tile} {(M, N, Kd)} nt")
+            both(lambda: xtd.matmul_tn(yd), f"{tile} {(M, N, Kd)} tn")
+            both(lambda: xd.matmul(yd, epi="add", e=ed), f"{tile} {(M, N, Kd)} nn add")
+            both(lambda: xd.matmul_nt(ytd, epi="gate", e=ed), f"{tile} {(M, N, Kd)} nt gate")
+        T = 2 * max(bm, bn) + 8
+        q, kk = rng.standard_normal((2, T, 64), dtype=np.float32), rng.standard_normal((2, T, 64), dtype=np.float32)
+        low = np.tril(rng.standard_normal((2, T, T), dtype=np.float32))
+        qd, kd, lowd = dev(q), dev(kk), dev(low)
+        both(lambda: qd.matmul_nt(kd, tri="out_lower"), f"{tile} out_lower")
+        both(lambda: lowd.matmul(kd, tri="a_lower"), f"{tile} a_lower")
+        both(lambda: lowd.matmul_tn(kd, tri="at_lower"), f"{tile} at_lower")
+    x, y = rng.standard_normal((200, 1030), dtype=np.float32), rng.standard_normal((1030, 136), dtype=np.float32)
+    xd, yd = dev(x), dev(y)
+    for tile in ("128x128/4", "64x64k64/8", "64x64k64*2", "32x32m16*4", "64x64k32*4"):
+        monkeypatch.setattr(HIP, "MATMUL_FORCE", tile)
+        both(lambda: xd.matmul(yd), f"{tile} ragged")
+    x, y = rng.standard_normal((256, 1024), dtype=np.float32), rng.standard_normal((1024, 256), dtype=np.float32)
+    xd, yd = dev(x), dev(y)
+    for tile in ("128x128/4", "64x64k64/8", "64x64k64*2", "32x32m16*4", "64x64k32*4"):
+        monkeypatch.setattr(HIP, "MATMUL_FORCE", tile)
+        both(lambda: xd.matmul(yd), f"{tile} whole tiles")
+
