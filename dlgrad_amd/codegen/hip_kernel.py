@@ -2671,7 +2671,9 @@ extern "C" __global__ __launch_bounds__({threads}) void {name}({params[0]},
 # Every tile accumulates k in the same order, so the choice never changes a result bit.
 MATMUL_CONFIGS = {
     "256x256": (4, 2, 2, 4, 16),
+    "256x256k32": (4, 2, 2, 4, 32),     # the same tiles with k walked 32 at a time: half the barriers, one block per CU
     "256x128": (4, 1, 2, 4, 16),
+    "256x128k32": (4, 1, 2, 4, 32),
     "128x256": (4, 2, 1, 4, 32),
     "192x192": (2, 2, 3, 3, 16),
     "128x192": (4, 2, 1, 3, 32),

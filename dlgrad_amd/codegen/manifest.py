@@ -27,19 +27,19 @@ def _tuplify(v):
     return tuple(_tuplify(x) for x in v) if isinstance(v, list) else v
 
 
-def load() -> list[tuple[str, tuple]]:
-    if not os.path.exists(PATH):
+def load(path: str = PATH) -> list[tuple[str, tuple]]:
+    if not os.path.exists(path):
         return []
-    with open(PATH) as f:
+    with open(path) as f:
         return [(g, _tuplify(p)) for g, p in json.load(f)]
 
 
-def merge(entries) -> None:
-    """Adds (generator, params) pairs to kernels.json (sorted, de-duplicated)."""
-    cur = {json.dumps([g, p]) for g, p in load()}
+def merge(entries, path: str = PATH) -> None:
+    """Adds (generator, params) pairs to the list at `path` (kernels.json unless told otherwise; sorted, de-duplicated)."""
+    cur = {json.dumps([g, p]) for g, p in load(path)}
     cur |= {json.dumps([g, list(p)], default=list) for g, p in entries}
     rows = [json.loads(s) for s in sorted(cur)]            # by their text: parameters of one position may differ in type
-    with open(PATH, "w") as f:
+    with open(path, "w") as f:
         f.write("[\n" + ",\n".join(json.dumps(r) for r in rows) + "\n]\n")
 
 

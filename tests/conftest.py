@@ -61,3 +61,8 @@ def default_switches(monkeypatch):
     monkeypatch.setattr(HIP, "MATMUL_FORCE", None)
     monkeypatch.setattr(HIP, "ROW_MATMUL", True)
     monkeypatch.setattr(HIP, "DECODE_FUSED", True)
+    # Tiles come from the committed table and the model, not from timings taken on this machine: which tile wins a
+    # timing differs from machine to machine, and among the candidates of a few-tile product are the forms that cut k
+    # into slices, which change result bits -- a test that compares two routes bit for bit must not depend on that.
+    # The tests of the timing itself switch it on.
+    monkeypatch.setattr(HIP, "MATMUL_TUNE", False)
