@@ -248,7 +248,7 @@ C5_SHAPED = dict(vocab_size=50304, block_size=1024, n_layer=2, n_head=12, n_embd
 
 @pytest.mark.gpu
 def test_scaled_gpt_step_hip_vs_float64(monkeypatch):
-    """The scaled GPT (BASELINE config 5) end to end at its real width, vocabulary and sequence length --
+    """The scaled GPT (vocabulary 50304, window 1024, width 768, 12 heads) end to end at its real width, vocabulary and sequence length --
     two of its twelve layers, batch 2, Zipf(1.1) token ids -- forward and backward on the hip device against
     an independent float64 PyTorch statement of the same graph (the pattern of the reference's
     test/test_gpt.py:44-205; the C restatement's naive loops would need minutes for the 50304-wide head).
@@ -298,7 +298,7 @@ C5_FULL = dict(vocab_size=50304, block_size=1024, n_layer=12, n_head=12, n_embd=
 
 @pytest.mark.gpu
 def test_scaled_gpt_full_depth_forward_hip_vs_float64():
-    """BASELINE config 5 at its own depth and batch: all twelve layers, batch 8 x 1024 Zipf(1.1) token ids,
+    """The scaled GPT at its own depth and batch: all twelve layers, batch 8 x 1024 Zipf(1.1) token ids,
     weights N(0, 0.02) from seed 0 -- the model, ids and targets that bench.py's scaled-GPT leg times (same
     seeds) -- forward on the hip device against the float64 PyTorch statement of the graph run on the host
     cores (forward only; the pattern of the reference's test/test_gpt.py:44-205).  The summed loss to 1e-5,
@@ -374,7 +374,7 @@ def same_ids_or_a_near_tie(got: list, want: list, want_rows: list, what: str) ->
 @pytest.mark.gpu
 @pytest.mark.parametrize("reference_positions", [True, False])
 def test_char_gpt_decodes_256_tokens_like_the_cpu_oracle(reference_positions):
-    """BASELINE config 4's decode on the model it names: 6 layers, 4 heads, width 128, window 128, weights
+    """The 256-token decode of the char-GPT configuration on the model itself: 6 layers, 4 heads, width 128, window 128, weights
     N(0, 0.02) from seed 0 (the model bench.py times), 256 greedy tokens from id 0.  The oracle is the
     reference's loop on the C restatement's cpu device (key/value cache while the window fills, a full forward
     over the last 128 tokens per token after that).  Against it, on the hip device: the same loop with the
@@ -478,7 +478,7 @@ def sampled_like_the_oracle(got: list, want: list, want_rows: list, u, temperatu
 def test_sampling_on_the_device_draws_the_tokens_of_the_cpu_oracle():
     """hip: the one-launch draw (decode_sample: softmax(logits / temperature), running sum, first index beyond
     u * total) against numpy's choice() arithmetic on the same logits and the same uniform number, row by
-    row for vocabularies from 2 to 50304; then the char-GPT of BASELINE config 4 sampling 200 tokens at
+    row for vocabularies from 2 to 50304; then the char-GPT (6 layers, 4 heads, width 128, window 128) sampling 200 tokens at
     temperature 0.7 -- fixed-shape steps eager and as replayed graphs -- against the reference's loop
     (cache, host-side sampling) on the C restatement's cpu device with the same numbers.  A draw may differ
     only where u sits on the boundary between two tokens (1e-5), and says so."""
