@@ -111,6 +111,65 @@ def test_exp_of_minus_inf_and_log_edge_values():
     check(dev(x).exp().numpy(), np.exp(x.astype(np.float64)).astype(np.float32), 1e-6, "exp edge")
 
 
+def test_special_values_follow_the_reference_source_read_as_ieee():
+    """NaN, the infinities, signed zeros, denormals and the extremes through the element-wise ops, the max reductions and
+    argmax.  The reference builds its kernels with -ffast-math (cpu.py:30-41), which leaves NaN and infinite operands to
+    the compiler: the C restatement built with the same flags answers NaN to inf / 0 and to rsqrt(inf), and lets a NaN
+    decide a max or an argmax.  So the oracle here is the reference's *source* read under IEEE rules, evaluated with
+    numpy: x / y, 1 / sqrt(x), cond > 0 ? x : y (relu is where(x, x, 0), buffer.py:338-342), and the scans
+    `if (v > best)` from (-FLT_MAX, 0), which a NaN never enters (cpu_kernel.py:68-148, :459-517)."""
+    require_gpu()
+    vals = np.array([np.nan, np.inf, -np.inf, 0.0, -0.0, 1e-45, -1e-45, 1e-38, 3.4e38, -3.4e38, 1.0, -1.0, 2.5, -2.5, 88.8, -104.0], np.float32)
+    a, b = np.repeat(vals, len(vals)), np.tile(vals, len(vals))
+    ad, bd = dev(a), dev(b)
+
+    def agree(got, want, what, tol=0.0):
+        if hip.COMPILE_ONLY:
+            return
+        want = np.asarray(want, np.float32)
+        same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+        if tol:
+            fin = np.isfinite(got) & np.isfinite(want)
+            same |= fin & (np.abs(got.astype(np.float64) - want) <= tol * np.abs(want) + 1.5e-45)
+        bad = np.flatnonzero(~same)
+        assert not bad.size, f"{what}: " + "; ".join(f"({a[i]}, {b[i]}) -> {got[i]}, expected {want[i]}" for i in bad[:5])
+    with np.errstate(all="ignore"):
+        agree((ad + bd).numpy(), a + b, "add")
+        agree((ad - bd).numpy(), a - b, "sub")
+        agree((ad * bd).numpy(), a * b, "mul")
+        agree((ad / bd).numpy(), a / b, "div", 1e-6)
+        agree((ad > bd).numpy(), (a > b).astype(np.float32), "greater")
+        agree((ad == bd).numpy(), (a == b).astype(np.float32), "equal")
+        agree(ad.where(ad, bd).numpy(), np.where(a > 0, a, b), "where")
+        agree(ad.relu().numpy(), np.where(a > 0, a, np.float32(0)), "relu")
+        agree((-ad).numpy(), -a, "neg")
+        agree(ad.exp().numpy(), np.exp(a.astype(np.float64)), "exp", 1e-6)
+        agree(ad.log().numpy(), np.log(a.astype(np.float64)), "log", 1e-6)
+        agree(ad.sqrt().numpy(), np.sqrt(a), "sqrt", 1e-6)
+        agree(ad.rsqrt().numpy(), 1.0 / np.sqrt(a.astype(np.float64)), "rsqrt", 1e-6)
+    rows = np.stack([np.roll(vals, s) for s in range(len(vals))] + [np.where(np.isnan(np.roll(vals, s)), 1.0, np.roll(vals, s)) for s in range(4)]).astype(np.float32)
+
+    def scan(v):                                   # the reference's loop: (best, index) from (-FLT_MAX, 0), strict '>'
+        best, at = -np.finfo(np.float32).max, 0
+        for i, x in enumerate(v):
+            if x > best:
+                best, at = x, i
+        return best, at
+    rd = dev(rows)
+    for axis in (0, 1):
+        lines = rows.T if axis == 0 else rows
+        want = [scan(v) for v in lines]
+        got_max, got_arg = rd.max(axis).numpy().ravel(), rd.argmax(axis).numpy().ravel()
+        if not hip.COMPILE_ONLY:
+            np.testing.assert_array_equal(got_max, np.array([w[0] for w in want], np.float32), err_msg=f"max over axis {axis}")
+            np.testing.assert_array_equal(got_arg, np.array([w[1] for w in want], np.float32), err_msg=f"argmax over axis {axis}")
+        got_sum = rd.sum(axis).numpy().ravel()
+        with np.errstate(all="ignore"):
+            ref = lines.astype(np.float64).sum(1)
+        if not hip.COMPILE_ONLY:
+            assert (np.isnan(got_sum) == np.isnan(ref)).all() and (got_sum[np.isinf(ref)] == ref[np.isinf(ref)]).all(), f"sum over axis {axis}"
+
+
 def test_where_relu_masked_fill():
     require_gpu()
     c, x, y = f32(64, 50), f32(64, 50), f32(64, 50)
