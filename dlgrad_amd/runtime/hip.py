@@ -357,6 +357,44 @@ class Graph:
             self.arena_id = 0
 
 
+class CapturedStep:
+    """A step function turned into its captured form without the caller handling arenas and captures:
+
+        step = hip.CapturedStep(train_step, before_replay=opt.advance)
+        for _ in range(n):
+            loss = step()              # 1st call: eager inside the graph's arena; 2nd: recorded and run once; later: one replay each
+
+    Every call performs exactly one step.  The value the function returned while it was recorded is returned by
+    every later call: its tensors live at fixed addresses and each replay rewrites them.  before_replay runs ahead of
+    every step after the first (the optimizer's advance(), which writes the next step's constants on the device).
+    What Graph asks of a step holds here too: state at fixed addresses (in-place optimizer), no host transfers, inputs
+    refreshed in place between calls."""
+
+    def __init__(self, fn, before_replay=None) -> None:
+        self.fn, self.before_replay = fn, before_replay
+        self.graph, self.calls, self.result = Graph(), 0, None
+
+    def __call__(self):
+        self.calls += 1
+        if self.calls == 1:
+            with self.graph.arena():
+                return self.fn()
+        if self.before_replay is not None:
+            self.before_replay()
+        if self.calls == 2:
+            with self.graph.capture():
+                self.result = self.fn()
+        self.graph.replay()
+        return self.result
+
+    @property
+    def nodes(self) -> int:
+        return self.graph.nodes
+
+    def close(self) -> None:
+        self.graph.close()
+
+
 # ---- kernel cache -----------------------------------------------------------------------
 
 def code_object(src: str, name: str, l: _ffi.HipLib | None = None, force: bool = False) -> bytes:

@@ -901,6 +901,46 @@ def test_captured_graph_replays_match_eager_steps_bit_for_bit(monkeypatch):
 
 
 @pytest.mark.gpu
+def test_a_step_function_wrapped_for_capture_runs_one_step_per_call(monkeypatch):
+    """hip.CapturedStep: the first call runs the step eagerly inside the graph's arena, the second records it and runs
+    it once, every later call is one replay -- each call exactly one training step, with the bits of the eager
+    steps, and the loss tensor of the recorded call holding each step's loss in turn."""
+    if not hip.available():
+        pytest.skip("no HIP device (graph capture needs one)")
+    monkeypatch.setattr(hip, "EMB_ORDERED", True)
+    cfg = dict(vocab_size=65, block_size=32, n_layer=2, n_head=2, n_embd=64, batch_size=4)
+    rng = np.random.default_rng(5)
+    idx = rng.integers(0, 65, (4, 32)).astype(np.float32)
+    tgt = rng.integers(0, 65, (4, 32)).astype(np.float32)
+
+    def build():
+        model = G.GPT(G.GPTConfig(device="hip", **cfg))
+        G.init_weights_(model, 0)
+        opt = nn.optim.Adam(nn.utils.get_parameters(model), lr=1e-3)
+        ti, tt = Tensor(idx, device="hip"), Tensor(tgt, device="hip")
+
+        def step():
+            opt.zero_grad()
+            _, loss = model(ti, tt)
+            loss.backward()
+            opt.step()
+            return loss
+        return model, opt, step
+
+    eager_model, _, eager_step = build()
+    model, opt, step = build()
+    wrapped = hip.CapturedStep(step, before_replay=opt.advance)
+    for k in range(6):
+        want = float(eager_step().numpy())
+        got = float(wrapped().numpy())
+        assert got == want, f"loss of step {k + 1}"
+        for (name, p), (_, q) in zip(nn.utils.get_state_dict(model).items(), nn.utils.get_state_dict(eager_model).items()):
+            np.testing.assert_array_equal(p.numpy(), q.numpy(), err_msg=f"{name} after step {k + 1}")
+    assert wrapped.calls == 6 and wrapped.nodes > 30
+    wrapped.close()
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("V,P,C,B,T", [(65, 128, 128, 16, 128), (50, 9, 6, 3, 9), (300, 40, 64, 2, 33)])
 def test_token_and_position_embeddings_and_their_sum_in_one_launch(V, P, C, B, T, monkeypatch):
     """hip: nn.embed_tokens is one node and one launch; output and both table gradients have the bits of
