@@ -162,6 +162,37 @@ def run_c2(R: int, C: int, steps: int, warmup: int, events_in_timed_region: bool
             "bytes_per_step": total_bytes, "per_op": per_op, "n_ops": len(ops), "launches_per_step": launches}
 
 
+def run_c2_graph(R: int, C: int, steps: int) -> dict:
+    """The same 26-op suite recorded once as a HIP graph and replayed: what the kernels do at a size where issuing them
+    from Python one by one is what takes the time."""
+    _, _, Buffer, Device, hip = _imports()
+    lib = hip.lib()
+    d = {k: Buffer.from_numpy(v, Device.HIP) for k, v in c2_inputs(R, C).items()}
+    ops = c2_ops(R, C)
+
+    def suite():
+        for _, f, _ in ops:
+            f(d)                                              # (each result goes back to the graph's arena at once)
+    g = hip.Graph()
+    with g.arena():
+        suite()
+    with g.capture():
+        suite()
+    for _ in range(5):
+        g.replay()
+    lib.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        g.replay()
+    lib.sync()
+    wall = time.perf_counter() - t0
+    total_bytes = sum(b for _, _, b in ops)
+    res = {"GBps": round(total_bytes * steps / wall / 1e9, 1), "ms_per_step": round(wall / steps * 1e3, 4), "graph_nodes": g.nodes,
+           "us_per_node": round(wall / steps * 1e6 / max(g.nodes, 1), 2)}
+    g.close()
+    return res
+
+
 def cpu_c2(R: int, C: int, reps: int = 2) -> dict:
     """The same suite on the C restatement of the reference's kernels, one thread."""
     from oracle import cref
@@ -810,7 +841,8 @@ def main() -> None:
                 extra[f"c2_{r2}x{c2}_cache_resident"] = {
                     "GBps": round(e["GBps"], 1), "ms_per_step": round(e["ms_per_step"], 4),
                     "add_same_GBps": round(e["per_op"]["add_same"]["GBps"], 1),
-                    "us_per_launch": round(e["ms_per_step"] * 1e3 / e["launches_per_step"], 2)}
+                    "us_per_launch": round(e["ms_per_step"] * 1e3 / e["launches_per_step"], 2),
+                    "replayed_as_hipgraph": run_c2_graph(r2, c2, max(args.steps, 50))}
             sweep = {}
             for n in (128, 512, 1024, 2048, 4096, 8192):
                 m = run_matmul(n, n, n, max(3, min(args.steps, 10)), 2)
