@@ -495,3 +495,32 @@ def test_first_tile_timing_of_a_process_says_so_once(monkeypatch, tmp_path):
     finally:
         HIP._tuned_table().clear()
         HIP._tuned_table().update(table)
+
+
+def test_tile_names_that_cut_k_are_parsed_and_planned_on_the_host():
+    """Host logic of the product launcher: "base/s" cuts k into s slices across blocks (a workspace and a column-sum
+    launch), "base*g" among g groups of wavefronts inside a block.  Every slice is a whole number of the tile's k
+    steps and none is empty; groups all take the same number of steps, and a k of fewer steps than groups gets fewer
+    groups, down to the plain tile.  Names that are no tile are refused (the tile tables are read through this)."""
+    from dlgrad_amd.codegen import hip_kernel as K
+    from dlgrad_amd.runtime.hip import HIP
+    assert HIP._split_of("128x128/4") == ("128x128", 4) and HIP._groups_of("128x128/4") == 1
+    assert HIP._split_of("64x64k32*4") == ("64x64k32", 1) and HIP._groups_of("64x64k32*4") == 4
+    assert HIP._split_of("64x64") == ("64x64", 1) and HIP._groups_of("64x64") == 1
+    for good in ("64x64", "256x128k32", "128x128/16", "64x64k64*2", "32x32*8", "32x32m16*4"):
+        assert HIP._valid_tile(good), good
+    for bad in ("65x64", "64x64/0", "64x64/x", "64x64*5", "64x64*x", "128x128/2*2", "256x256*2", "", "rows"):
+        assert not HIP._valid_tile(bad), bad
+    for tile, Kd in (("128x128/4", 4096), ("128x128/4", 1030), ("64x64k64/16", 2048), ("64x64m16/3", 700), ("128x64/2", 40)):
+        slices, kchunk = HIP._split_plan(tile, Kd)
+        bk = K.MATMUL_CONFIGS[HIP._split_of(tile)[0]][4]
+        assert kchunk % bk == 0 and (slices - 1) * kchunk < Kd <= slices * kchunk and 1 <= slices <= HIP._split_of(tile)[1], (tile, Kd, slices, kchunk)
+    for tile, Kd, want in (("64x64k64*2", 1024, 2), ("64x64k32*4", 96, 3), ("32x32*8", 40, 3), ("128x128*2", 20, 1), ("64x64*3", 4096, 3), ("32x32m16*4", 1030, 4)):
+        groups, kchunk = HIP._group_plan(tile, Kd)
+        bk = K.MATMUL_CONFIGS[HIP._split_of(tile)[0]][4]
+        assert groups == want and kchunk % bk == 0 and groups * kchunk >= Kd, (tile, Kd, groups, kchunk)
+    # what is offered for timing: split forms only for few-tile products with a long k, and every candidate is a valid tile
+    few = HIP._tile_candidates(512, 512, 1, 2048, True)
+    assert any("/" in t for t in few) and any("*" in t for t in few) and all(HIP._valid_tile(t) for t in few)
+    assert not any("/" in t or "*" in t for t in HIP._tile_candidates(512, 512, 1, 2048, False))
+    assert HIP._splitk_eligible(768, 768, 8192, 1) and not HIP._splitk_eligible(4096, 4096, 4096, 1) and not HIP._splitk_eligible(512, 512, 256, 1)
