@@ -443,7 +443,7 @@ extern "C" __global__ __launch_bounds__(256) void {name}(const float* __restrict
 
 
 @cache
-def reduce_cols_kernel(op: str, vec: int, ty: int = 4, nt: bool = False) -> tuple[str, str, str]:
+def reduce_cols_kernel(op: str, vec: int, ty: int = 4, nt: bool = False, TX: int = 64) -> tuple[str, str, str]:
     """out[o, c, i] = reduce over l in chunk c of x[o, l, i] for an (O, L, I) view, / divisor
     (the non-last-axis case of cpu_kernel.py:68-148, e.g. axis 0 of a matrix).
 
@@ -451,8 +451,9 @@ def reduce_cols_kernel(op: str, vec: int, ty: int = 4, nt: bool = False) -> tupl
     owns 64*vec adjacent columns: lanes read consecutive addresses of one row (coalesced),
     the ty thread rows take every ty-th row of the chunk, and LDS joins them.  L is
     split into `chunks` so that tall, narrow inputs still fill the chip; the launcher
-    reduces the (O, chunks, I) partials with a second call."""
-    name = f"reduce_cols_{op}_v{vec}_y{ty}{'nt' if nt else ''}"
+    reduces the (O, chunks, I) partials with a second call.  TX: lanes along a row (64, or 32 with
+    twice the thread rows: half as many bytes of a row per block, which streams better beyond the caches)."""
+    name = f"reduce_cols_{op}_v{vec}_y{ty}{'nt' if nt else ''}{f'_t{TX}' if TX != 64 else ''}"
     if vec == 4:
         defs = _ld4_define(nt) + """#define VT float4
 #define LD(l) LD4(reinterpret_cast<const float4*>(xp + (u64)(l) * I))
@@ -468,11 +469,11 @@ def reduce_cols_kernel(op: str, vec: int, ty: int = 4, nt: bool = False) -> tupl
 #define STORE(p, r) { (p)[0] = r / divisor; }
 """
     src = f"""{PRELUDE}{_red_defs(op)}{defs}
-extern "C" __global__ __launch_bounds__({64 * ty}) void {name}(const float* __restrict__ x,
+extern "C" __global__ __launch_bounds__({TX * ty}) void {name}(const float* __restrict__ x,
         float* __restrict__ out, u32 L, u32 I, u32 chunk, float divisor) {{
-    __shared__ VT sm[{ty}][64];
+    __shared__ VT sm[{ty}][{TX}];
     const u32 tx = threadIdx.x, ty = threadIdx.y, o = blockIdx.z;
-    const u32 col = (blockIdx.x * 64u + tx) * {vec}u;
+    const u32 col = (blockIdx.x * {TX}u + tx) * {vec}u;
     const u32 l0 = blockIdx.y * chunk, l1 = min(L, l0 + chunk);
     VT a0 = VINIT, a1 = VINIT, a2 = VINIT, a3 = VINIT;
     if (col < I) {{

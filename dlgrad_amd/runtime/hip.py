@@ -615,6 +615,7 @@ ARGMAX_SHORT_ROWS = os.environ.get("DLGRAD_HIP_ARGMAX_SHORT_ROWS", "direct")
 ARGMAX_COL_UNROLL = 8              # rows in flight per thread of the column argmax (8192 x 8192: 50.2 us with 4, 49.5 with 8)
 # blocks of 64 x 16 threads the first stage of a tall column reduction aims for (16384 x 8192 over axis 0: 88.5 us with 8192,
 # 83.6 us = 6.4 TB/s with 2048 -- row chunks of 256 and a quarter of the partials -- 85.8 us with 512)
+REDUCE_COL_TX = int(os.environ.get("DLGRAD_HIP_REDUCE_COL_TX", "0"))          # lanes along a row in the blocks of a tall column reduction (0: chosen by size)
 REDUCE_COL_BLOCKS = int(os.environ.get("DLGRAD_HIP_REDUCE_COL_BLOCKS", "2048"))
 ARGMAX_COL_BLOCKS = 1024           # blocks of 64 x 16 threads the column argmax aims for (8192 x 8192: 65.6 us with 128, 51.5 with 256 or 512, 49.8 with 1024, 57.8 with 2048)
 _permute_plans: dict = _PlanCache()
@@ -959,22 +960,26 @@ class HIP:
     @staticmethod
     def _reduce_cols(kop: str, x_addr: int, O: int, L: int, I: int, divisor: float, out_addr: int) -> None:
         """Up to 512 rows are folded by one launch of 64x16 blocks.  Taller inputs are split
-        into chunks of >= 64 rows (4 loads per thread) sized so that about 8 M threads exist
-        (the measured optimum on a 512 MiB input), which bounds the partials at 1.6 % of the input; the same kernel then folds the
-        (O, chunks, I) partials."""
+        into chunks of >= 64 rows (4 loads per thread) so that about REDUCE_COL_BLOCKS blocks exist, which bounds the
+        partials at under 1 % of the input; the same kernel then folds the (O, chunks, I) partials."""
         vec = 4 if (I % 4 == 0 and x_addr % 16 == 0 and out_addr % 16 == 0) else 1
         bx = (I + 64 * vec - 1) // (64 * vec)
         ty = 16 if L > 64 else 4
         nt = vec == 4 and O * L * I >= NT_STORE_MIN_ELEMENTS
-        k = kernel(K.reduce_cols_kernel, kop, vec, ty, nt)
+        # beyond the caches a 32 x 32 block (512 bytes of a row per block) streams better than 64 x 16 (1 KiB): 16384 x 8192 summed
+        # over axis 0 at 80 % of the HBM peak against 77 %; wider blocks are worse still (128 x 8: 68 %, 256 x 4: 61 %)
+        TX = (REDUCE_COL_TX or (32 if O * L * I >= (1 << 25) else 64)) if (ty == 16 and L > 512) else 64
+        if TX != 64:
+            ty, bx = 1024 // TX, (I + TX * vec - 1) // (TX * vec)
+        k = kernel(K.reduce_cols_kernel, kop, vec, ty, nt, TX)
         chunks = 1 if L <= 512 else max(1, min(REDUCE_COL_BLOCKS // max(1, bx * O), L // 64))
         if chunks == 1:
-            launch(k, (bx, 1, O), (64, ty, 1), x_addr, out_addr, L, I, L, float(divisor))
+            launch(k, (bx, 1, O), (TX, ty, 1), x_addr, out_addr, L, I, L, float(divisor))
             return
-        chunk = ((L + chunks - 1) // chunks + 15) // 16 * 16
+        chunk = ((L + chunks - 1) // chunks + ty - 1) // ty * ty
         chunks = (L + chunk - 1) // chunk
         part = alloc(O * chunks * I)
-        launch(k, (bx, chunks, O), (64, ty, 1), x_addr, part.addr, L, I, chunk, 1.0)
+        launch(k, (bx, chunks, O), (TX, ty, 1), x_addr, part.addr, L, I, chunk, 1.0)
         HIP._reduce_cols(kop, part.addr, O, chunks, I, divisor, out_addr)
 
     @staticmethod
