@@ -334,6 +334,56 @@ def test_scaled_gpt_full_depth_forward_hip_vs_float64():
     tensors_close(lg_hip.reshape(tokens, -1)[rows], lg64.reshape(tokens, -1)[rows], "sampled logit rows")
 
 
+@pytest.mark.gpu
+def test_scaled_gpt_full_depth_backward_agrees_with_differences_of_the_forward(monkeypatch):
+    """The backward pass of the scaled GPT at its own depth and batch (twelve layers, 8 x 1024 tokens, the model
+    bench.py times), held to a property that needs no second implementation: along the direction of the gradient
+    itself, the loss must change by |g| per unit step.  The forward pass at this size is pinned against float64
+    above; here L(theta + e d) - L(theta - e d) over 2 e, with d = g / |g| and e sized for a 1 % change of the loss,
+    must equal |g| to 1 %.  A layer whose backward kernel drops or mis-scales a term (the streaming attention's
+    three gradients, a product read transposed, the cross-entropy rows, an RMSNorm) moves that figure by far more.
+    (With the reference's zero gradient through every mean switched off, so that the backward is the gradient of
+    the forward; the loss is the reference's sum over tokens, its gradient the reference's mean: hence the
+    factor of the token count.)"""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    from dlgrad_amd import ops
+    monkeypatch.setattr(ops, "STRICT_REFERENCE", False)
+    cfg = C5_FULL
+    rng = np.random.default_rng(7)
+    ids = np.minimum(rng.zipf(1.1, (2, cfg["batch_size"], cfg["block_size"])) - 1, cfg["vocab_size"] - 1).astype(np.float32)
+    model = G.GPT(G.GPTConfig(device="hip", **cfg))
+    G.init_weights_(model, 0)
+    idx, tgt = Tensor(ids[0], device="hip"), Tensor(ids[1], device="hip")
+    params = nn.utils.get_parameters(model)
+    tokens = cfg["batch_size"] * cfg["block_size"]
+
+    def loss_only() -> float:
+        with nn.inference():
+            _, loss = model(idx, tgt)
+        return float(loss.numpy())
+    _, loss = model(idx, tgt)
+    loss.backward()
+    l0 = float(loss.numpy())
+    del loss
+    if hip.COMPILE_ONLY:
+        return
+    grads = [p.grad.detach() for p in params]
+    for p in params:
+        p.grad = None
+    norm = float(np.sqrt(sum(float((g * g).sum().numpy()) for g in grads)))
+    assert np.isfinite(norm) and norm > 0
+    eps = 1e-2 * (l0 / tokens) / norm                      # a step that changes the loss per token by about 1 %
+    moved = []
+    for sign in (+1.0, -2.0):                               # theta + e d, then theta - e d
+        for p, g in zip(params, grads):
+            p.data = (p.detach() + g * (sign * eps / norm)).data
+        moved.append(loss_only())
+    slope = (moved[0] - moved[1]) / (2 * eps) / tokens
+    print(f"scaled GPT, 12 layers, batch 8: |g| = {norm:.6e}, slope of the loss along g / |g| = {slope:.6e} (loss per token {l0 / tokens:.4f} -> {moved[0] / tokens:.4f}, {moved[1] / tokens:.4f})")
+    assert abs(slope - norm) <= 1e-2 * norm, (slope, norm)
+
+
 def decode_with_logits(model: G.GPT, first_token: int, n_new: int, reference_positions: bool):
     """The control flow of GPT.generate_greedy_cached (the reference's generate, examples/gpt.py:169-226,
     greedy), keeping the logits every token was chosen from: (ids, [logits (V,) per new token])."""
