@@ -149,6 +149,83 @@ def test_mlp_step_hip_vs_cpu_oracle():
         tensors_close(a, b, f"param {i}")
 
 
+def gan_steps(device):
+    """One discriminator step and one generator step of examples/gan.py (mnist_gan.py:116-126) on seeded weights, noise
+    and images: the two losses, the gradients that reach the generator's first layer, and a parameter of each net
+    after its Adam step."""
+    from examples import gan
+    gen, disc = gan.LinearGen(device), gan.LinearDisc(device)
+    gan.init_weights_(gen, 0, device)
+    gan.init_weights_(disc, 1, device)
+    rng = np.random.default_rng(2)
+    bs = 16
+    real = Tensor((rng.random((bs, 784), dtype=np.float32) * 2 - 1), device=device)
+    noise = [Tensor(rng.uniform(-1, 1, (bs, 128)).astype(np.float32), device=device) for _ in range(2)]
+    opt_g = nn.optim.Adam(nn.utils.get_parameters(gen), lr=0.0005, betas=(0.5, 0.999))
+    opt_d = nn.optim.Adam(nn.utils.get_parameters(disc), lr=0.0005, betas=(0.5, 0.999))
+    d_loss = gan.train_discriminator(disc, opt_d, real, gen(noise[0]).detach())
+    d_grad = disc.net[0].weight.grad.numpy()
+    g_loss = gan.train_generator(disc, opt_g, gen(noise[1]))
+    g_grad = gen.net[0].weight.grad.numpy()
+    return (float(d_loss.numpy()), float(g_loss.numpy()), d_grad, g_grad, disc.net[6].weight.numpy(), gen.net[6].bias.numpy(),
+            gen(noise[0]).numpy())
+
+
+def test_gan_steps_on_cpu_device_match_torch():
+    """The graph of the third example of the reference (two MLPs, leaky ReLU, tanh, the logits form of the binary
+    cross-entropy, Adam with betas (0.5, 0.999)) against PyTorch on the C restatement's device."""
+    from examples import gan
+    d_loss, g_loss, d_grad, g_grad, *_ = gan_steps("cpu")
+    gen, disc = gan.LinearGen("cpu"), gan.LinearDisc("cpu")
+    gan.init_weights_(gen, 0, "cpu")
+    gan.init_weights_(disc, 1, "cpu")
+    rng = np.random.default_rng(2)
+    real = torch.tensor(rng.random((16, 784), dtype=np.float32) * 2 - 1)
+    noise = [torch.tensor(rng.uniform(-1, 1, (16, 128)).astype(np.float32)) for _ in range(2)]
+
+    def net(model, x, params):
+        it = iter(params)
+        for layer in model.net:
+            if isinstance(layer, nn.Linear):
+                w, b = next(it), next(it)
+                x = x @ w.T + b
+            elif layer is Tensor.tanh:
+                x = torch.tanh(x)
+            else:
+                x = torch.nn.functional.leaky_relu(x, 0.2)
+        return x
+    pg = [torch.tensor(p.numpy(), requires_grad=True) for p in nn.utils.get_parameters(gen)]
+    pd = [torch.tensor(p.numpy(), requires_grad=True) for p in nn.utils.get_parameters(disc)]
+    bce = torch.nn.functional.binary_cross_entropy_with_logits
+    fake = net(gen, noise[0], pg).detach()
+    td = (bce(net(disc, real, pd), torch.ones(16, 1)) + bce(net(disc, fake, pd), torch.zeros(16, 1))) / 2
+    td.backward()
+    tensors_close(d_loss, td.detach().numpy(), "discriminator loss")
+    tensors_close(d_grad, pd[0].grad.numpy(), "discriminator gradient", 1e-3)
+    opt = torch.optim.Adam(pd, lr=0.0005, betas=(0.5, 0.999), eps=1e-8)
+    opt.step()
+    for q in pd:
+        q.grad = None
+    tg = bce(net(disc, net(gen, noise[1], pg), pd), torch.ones(16, 1))
+    tg.backward()
+    tensors_close(g_loss, tg.detach().numpy(), "generator loss")
+    tensors_close(g_grad, pg[0].grad.numpy(), "generator gradient", 1e-3)
+
+
+@pytest.mark.gpu
+def test_gan_steps_hip_vs_cpu_oracle():
+    """The same two steps on the hip device against the C restatement's device: losses, gradients, the parameters an
+    Adam step touched (its first step is lr * sign(g): 2e-4 covers a gradient entry of magnitude ~1e-8 changing sign)
+    and the generator's images afterwards."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    c, h = gan_steps("cpu"), gan_steps("hip")
+    names = ("discriminator loss", "generator loss", "discriminator gradient", "generator gradient", "discriminator weight after Adam",
+             "generator bias after Adam", "generated images")
+    for name, a, b in zip(names, h, c):
+        tensors_close(a, b, name, 2e-4 if "after" in name or "images" in name else 1e-4)
+
+
 class ReluBranches:
     """Records the ReLU branch taken per element on one device and imposes it on another.
 
