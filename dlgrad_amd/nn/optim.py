@@ -17,6 +17,13 @@ def _rebind(p: Tensor, new) -> None:
         p.data = new
 
 
+def _adam_multi(**kw):
+    """The hip runtime's update of all parameters by one launch (registered when the runtime is first used)."""
+    from dlgrad_amd.dispatch import dispatcher
+    from dlgrad_amd.helpers import CustomOps
+    return dispatcher.dispatch(CustomOps.ADAM_MULTI_INPLACE, Device.HIP, **kw)
+
+
 class Optimizer:
     def __init__(self, params: list[Tensor], lr: float = 1e-1) -> None:
         self.params = params
@@ -113,14 +120,13 @@ class Adam(Optimizer):
                 self.advance()
             quads = [(p.data, p.grad.data, self.m[id(p)].data, self.v[id(p)].data) for p in self.params
                      if p.grad is not None and p.numel]
-            def base(b):                                 # a pending sum is handed over as its parts: asking for its ptr would run it
-                return b.parts.ptr.addr + 4 * b.offset if getattr(b, "pending", False) else b.ptr.addr
-            if all(not (base(b) & 15) for q in quads for b in q):
-                # every parameter in one launch; the address table is uploaded on the first step only
-                from dlgrad_amd.dispatch import dispatcher
-                from dlgrad_amd.helpers import CustomOps
-                self._table = dispatcher.dispatch(CustomOps.ADAM_MULTI_INPLACE, Device.HIP, tensors=quads,
-                                                  consts=self.consts.data, table=self._table)
+            try:
+                # every parameter in one launch; the address table is uploaded when the tensors have moved.  A pending
+                # sum is handed over as its parts (asking for its ptr would run it)
+                self._table = _adam_multi(tensors=quads, consts=self.consts.data, table=self._table)
+            except ValueError:                           # some tensor is not 16-byte aligned: one launch per parameter
+                pass
+            else:
                 if self._table["frozen"] and self._table not in self._graph_tables:
                     self._graph_tables.append(self._table)         # a captured graph reads it on every replay
                 return

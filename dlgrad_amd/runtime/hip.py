@@ -1579,46 +1579,58 @@ class HIP:
         from dlgrad_amd.buffer import PartialSum
         rows_of = []                                     # per tensor: how many parts the gradient pointer holds, and how far apart
         addrs = []
+        low = 0                                          # the low address bits of all tensors, or-ed
         for pb, gb, mb, vb in tensors:
             if gb.__class__ is PartialSum and gb.pending:
                 g_addr, rows, pitch = gb.parts.ptr.addr + 4 * gb.offset, gb.parts.shape[0], gb.pitch
+                if pitch >= 2 ** 32 or pitch & 3 and not pb.numel & 3:
+                    raise ValueError("adam_multi_inplace: parts of a pending gradient lie too far apart or break the 16-byte alignment")
+                rows_of += (rows, pitch)
             else:
-                g_addr, rows, pitch = gb.ptr.addr, 1, 0
-            if pitch >= 2 ** 32 or pitch & 3 and not pb.numel & 3:
-                raise ValueError("adam_multi_inplace: parts of a pending gradient lie too far apart or break the 16-byte alignment")
-            rows_of += [rows, pitch]
-            addrs += [pb.ptr.addr, g_addr, mb.ptr.addr, vb.ptr.addr]
+                g_addr = gb.ptr.addr
+                rows_of += (1, 0)
+            quad = (pb.ptr.addr, g_addr, mb.ptr.addr, vb.ptr.addr)
+            low |= quad[0] | g_addr | quad[2] | quad[3]
+            addrs += quad
         addrs = tuple(addrs)
-        if any(a & 15 for a in addrs):
+        if low & 15:
             raise ValueError("adam_multi_inplace needs 16-byte aligned tensors")
         key = (addrs, tuple(rows_of))
         if table is None or table["key"] != key:
             nt = len(tensors)
-            sizes = np.array([q[0].numel for q in tensors], dtype=np.uint32)
-            # 256 threads take 256 16-byte items -- or 16 of them, sharing the addition of a gradient that is pending in many parts
-            per_block = np.array([16 if (r > 16 and not n & 3) else 256 for r, n in zip(rows_of[::2], sizes)], dtype=np.int64)
-            nblk = np.maximum(1, (sizes.astype(np.int64) // 4 + per_block - 1) // per_block)
-            first = np.concatenate([[0], np.cumsum(nblk)[:-1]]).astype(np.uint32)
-            owner = np.repeat(np.arange(nt, dtype=np.uint32), nblk)
-            ptrs = np.array(addrs, dtype=np.uint64).reshape(nt, 4).T.reshape(-1)        # four rows: p, g, m, v
-            arrays = [np.ascontiguousarray(a).view(np.float32) for a in (ptrs, sizes, first, owner, np.array(rows_of, dtype=np.uint32))]     # raw bits; rows_of holds (parts, pitch) pairs
-            reuse = (table is not None and not table["frozen"]
-                     and [a.size for a in arrays] == [b.nbytes // 4 for b in table["bufs"]])
-            bufs = table["bufs"] if reuse else [alloc(a.size) for a in arrays]
-
-            def upload(bufs=bufs, arrays=arrays):
-                for b, a in zip(bufs, arrays):
-                    if a.size:
-                        lib().h2d(b.addr, a.ctypes.data, a.nbytes)
-            if capturing():
-                # a captured launch only records where the table is; its contents are written once the
-                # capture has ended, and never again: the graph replays with exactly these addresses
-                _after_capture.append(upload)
-            elif _graph_depth or COMPILE_ONLY:
-                upload()
+            layout = (key[1], tuple(q[0].numel for q in tensors))
+            ptrs = np.array(addrs, dtype=np.uint64).reshape(nt, 4).T.reshape(-1).view(np.float32)        # four rows: p, g, m, v (raw bits)
+            if (table is not None and not table["frozen"] and table["layout"] == layout
+                    and not capturing() and not _graph_depth and not COMPILE_ONLY):
+                # an eager step whose tensors only moved: the sizes and the split into blocks stand, the addresses are sent again
+                HIP._stage_upload(table["bufs"][:1], [ptrs])
+                table["key"] = key
             else:
-                HIP._stage_upload(bufs, arrays)                # an eager step: enqueued, the host does not wait
-            table = {"key": key, "grid": int(nblk.sum()), "nt": nt, "bufs": bufs, "frozen": capturing()}
+                sizes = np.array(layout[1], dtype=np.uint32)
+                # 256 threads take 256 16-byte items -- or 16 of them, sharing the addition of a gradient that is pending in many parts
+                per_block = np.array([16 if (r > 16 and not n & 3) else 256 for r, n in zip(rows_of[::2], sizes)], dtype=np.int64)
+                nblk = np.maximum(1, (sizes.astype(np.int64) // 4 + per_block - 1) // per_block)
+                first = np.concatenate([[0], np.cumsum(nblk)[:-1]]).astype(np.uint32)
+                owner = np.repeat(np.arange(nt, dtype=np.uint32), nblk)
+                arrays = [ptrs] + [np.ascontiguousarray(a).view(np.float32)
+                                   for a in (sizes, first, owner, np.array(rows_of, dtype=np.uint32))]     # raw bits; rows_of holds (parts, pitch) pairs
+                reuse = (table is not None and not table["frozen"]
+                         and [a.size for a in arrays] == [b.nbytes // 4 for b in table["bufs"]])
+                bufs = table["bufs"] if reuse else [alloc(a.size) for a in arrays]
+
+                def upload(bufs=bufs, arrays=arrays):
+                    for b, a in zip(bufs, arrays):
+                        if a.size:
+                            lib().h2d(b.addr, a.ctypes.data, a.nbytes)
+                if capturing():
+                    # a captured launch only records where the table is; its contents are written once the
+                    # capture has ended, and never again: the graph replays with exactly these addresses
+                    _after_capture.append(upload)
+                elif _graph_depth or COMPILE_ONLY:
+                    upload()
+                else:
+                    HIP._stage_upload(bufs, arrays)                # an eager step: enqueued, the host does not wait
+                table = {"key": key, "layout": layout, "grid": int(nblk.sum()), "nt": nt, "bufs": bufs, "frozen": capturing()}
         if table["nt"]:
             b = table["bufs"]
             launch(kernel(K.adam_multi_inplace_kernel), table["grid"], 256, b[0].addr, b[1].addr, b[2].addr, b[3].addr, b[4].addr,

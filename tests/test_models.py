@@ -1238,6 +1238,34 @@ def test_one_launch_adam_over_a_parameter_list_is_bit_identical_to_the_per_tenso
             np.testing.assert_array_equal(a, b)
 
 
+@pytest.mark.gpu
+def test_in_place_adam_takes_a_parameter_off_the_16_byte_grid_with_one_launch_per_tensor():
+    """A parameter that is a view starting 20 bytes into its allocation cannot go through the vectorised one-launch
+    update: the step falls back to one in-place launch per parameter, with the same bits as the aligned copy."""
+    if not (hip.available() or hip.COMPILE_ONLY):
+        pytest.skip("no HIP device")
+    rng = np.random.default_rng(5)
+    whole, other = rng.standard_normal((4, 5)).astype(np.float32), rng.standard_normal((8, 4)).astype(np.float32)
+    grads = [[rng.standard_normal(s).astype(np.float32) for s in ((2, 5), (8, 4))] for _ in range(3)]
+    results = {}
+    for view in (False, True):
+        w = Tensor(whole, device="hip")[1:3] if view else Tensor(whole[1:3].copy(), device="hip")
+        w.requires_grad = True
+        ps = [w, Tensor(other, requires_grad=True, device="hip")]
+        assert bool(hip._addr(w.data) & 15) == view
+        opt = nn.optim.Adam(ps, lr=1e-2, graph_safe=True)
+        n0 = hip.launch_count
+        for g in grads:
+            for p, a in zip(ps, g):
+                p.grad = Tensor(a, device="hip")
+            opt.step()
+        assert hip.launch_count - n0 == (3 * 3 if view else 2 * 3)       # the constants, then each parameter / all at once
+        results[view] = [p.numpy() for p in ps] + [opt.m[id(p)].numpy() for p in ps]
+    if not hip.COMPILE_ONLY:
+        for a, b in zip(results[True], results[False]):
+            np.testing.assert_array_equal(a, b)
+
+
 def gpt_losses(device, cfg_kw, steps, seed=0):
     """Loss before each of `steps` forward + backward + Adam steps on one seeded batch."""
     c = G.GPTConfig(device=device, **cfg_kw)
