@@ -293,10 +293,15 @@ def run_matmul_transposed(n: int) -> dict:
                          (f"{n}_NT_G.Bt", lambda: g @ a.T, "ms_permute_plus_gemm"),
                          (f"{n}_TN_At.G_in_place", lambda: a.matmul_tn(g), "kernel_ms"),
                          (f"{n}_NT_G.Bt_in_place", lambda: g.matmul_nt(a), "kernel_ms")):
-        for _ in range(2):
-            f()
+        f()
+        lib.sync()
+        t_warm = time.perf_counter()                      # the clock warm-up of run_matmul: 50 ms of the product itself, untimed
+        while time.perf_counter() - t_warm < 0.05:
+            for _ in range(4):
+                f()
+            lib.sync()
         timer = EventTimer(lib)
-        for _ in range(5):
+        for _ in range(10):
             timer.run("mm", f)
         lib.sync()
         ms = float(np.mean(timer.collect()["mm"]))
