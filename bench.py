@@ -849,7 +849,7 @@ def main() -> None:
                                           "traffic": None, "kernel": hip.HIP.last_matmul_kernel,
                                           "flops_per_launch": m["flops"], "avg_launch_ms": round(m["kernel_ms"], 4)}}
             gg = run_gpt_graph(max(3, min(args.steps, 20)), 2)
-            g = run_gpt(max(3, min(args.steps, 10)), 2)
+            g = run_gpt(100, 20)
             out["gpt"] = {"metric": "GPT fwd+bwd tokens/s (1 GPU)", "value": round(gg["tokens_per_s"], 1), "unit": "tokens/s",
                           "config": {"workload": "C4 char-GPT vocab 65, block 128, 6 layers, 4 heads, n_embd 128, batch 16; forward + "
                                                  "backward + Adam step, captured once as a HIP graph and replayed per step"},
@@ -909,7 +909,7 @@ def main() -> None:
             out["cpu_baseline"] = cpu_matmul(512)
     elif args.workload == "gpt":
         gg = run_gpt_graph(args.steps, args.warmup)               # the step as it is meant to be run on this device
-        g = run_gpt(max(3, min(args.steps, 10)), 2)               # the same step issued launch by launch from Python
+        g = run_gpt(100, 20)                                      # the same step issued launch by launch from Python
         out = {"metric": "GPT fwd+bwd tokens/s (1 GPU)", "value": gg["tokens_per_s"], "unit": "tokens/s", **base,
                "ms_per_step": gg["ms_per_step"],
                "config": {"workload": "C4 char-GPT vocab 65, block 128, 6 layers, 4 heads, n_embd 128, batch 16; "
